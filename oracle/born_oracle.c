@@ -1,0 +1,512 @@
+/*
+ * born_oracle.c — CPU oracle for the token-sampling path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing the product ships may call into this file:
+ * only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg load it,
+ * and only as the checker / the timed CPU baseline.
+ *
+ * What follows the reference (born-ml/born v0.1.1, paths relative to the
+ * reference root):
+ *   born_oracle_softmax_f32      internal/autodiff/ops/softmax.go:214-238
+ *   born_oracle_log_softmax_f32  internal/nn/cross_entropy.go:126-153
+ *   born_oracle_softmax_via_log  internal/nn/cross_entropy.go:163-170
+ *   born_oracle_argmax           internal/nn/cross_entropy.go:241-251
+ *   born_oracle_exp_f32          internal/autodiff/ops/log.go:159-185
+ *   logits layout                internal/tensor/raw.go:78-105, shape.go:52-63
+ * Go's math.Exp / math.Log are stood in for by glibc exp()/log() (both < 1 ulp
+ * in fp64; the difference vanishes in the fp32 cast for every vector the
+ * reference's tests hold).
+ *
+ * What the reference does NOT contain (its snapshot predates any sampler):
+ * repetition penalty, temperature, top-k, top-p, the inverse-CDF draw and the
+ * speculative accept/reject step.  Their semantics are the ones frozen in
+ * docs/SAMPLING_SPEC.md; parity with "Born's CPU sampler" for those stages is
+ * therefore parity with that specification ("parity unpinned" with respect to
+ * any upstream implementation).  Each of those stages is pinned in
+ * tests/test_oracle_*.py by closed forms, special cases that reduce to the
+ * reference-pinned softmax/argmax, brute force on tiny inputs and an
+ * independent torch restatement.
+ *
+ * Modes of born_oracle_sample / born_oracle_spec_verify:
+ *   0  layer T  — fp64 truth
+ *   1  layer F  — fixed-point realisation (what the HIP kernels must equal bit
+ *                 for bit)
+ *   2  reference-arithmetic baseline (fp64 exp cast to fp32, sequential fp32
+ *      sums, heap top-k) — the timed CPU baseline, never a parity target
+ */
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define BORN_EXPORT __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ */
+/* small helpers                                                       */
+/* ------------------------------------------------------------------ */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* order-preserving fp32 -> uint32 map */
+static inline uint32_t ordkey(float z) {
+    uint32_t b = f2u(z);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+static inline float ordkey_inv(uint32_t k) {
+    return u2f((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+}
+
+/* NaN -> -inf, +inf -> FLT_MAX, -0 -> +0 */
+static inline float canon(float z) {
+    if (z != z) return -INFINITY;
+    if (z > FLT_MAX) return FLT_MAX;
+    if (z == 0.0f) return 0.0f;
+    return z;
+}
+
+static inline float penalise(float x, float r) { return x > 0.0f ? x / r : x * r; }
+
+BORN_EXPORT float born_oracle_expneg(float d) {
+    if (!(d <= 80.0f)) return 0.0f;
+    float x = -d;
+    float k = rintf(x * 1.44269504f);
+    float r = fmaf(k, -0.693145752f, x);
+    r = fmaf(k, -1.42860677e-06f, r);
+    float y = fmaf(1.9875691500e-4f, r, 1.3981999507e-3f);
+    y = fmaf(y, r, 8.3334519073e-3f);
+    y = fmaf(y, r, 4.1665795894e-2f);
+    y = fmaf(y, r, 1.6666665459e-1f);
+    y = fmaf(y, r, 5.0000001201e-1f);
+    float r2 = r * r;
+    y = fmaf(y, r2, r);
+    y = y + 1.0f;
+    return y * u2f((uint32_t)((int)k + 127) << 23);
+}
+
+static inline int bitlen64(uint64_t v) { int n = 0; while (v) { n++; v >>= 1; } return n; }
+BORN_EXPORT int born_oracle_mass_shift(int64_t V) { return 62 - bitlen64((uint64_t)V); }
+
+static inline uint64_t qmass(float z, float m, int S) {
+    float d = (z == m) ? 0.0f : m - z;
+    float e = born_oracle_expneg(d);
+    return (uint64_t)ldexp((double)e, S); /* exact scaling, then truncation */
+}
+static inline float emass(float z, float m) {
+    float d = (z == m) ? 0.0f : m - z;
+    return born_oracle_expneg(d);
+}
+
+static inline uint64_t mix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+BORN_EXPORT float born_oracle_uniform(uint64_t seed, uint64_t step, uint64_t row) {
+    uint64_t x = mix64(mix64(seed ^ (step * 0xD1342543DE82EF95ull)) + row);
+    return (float)(x >> 40) * 0x1p-24f;
+}
+
+/* ------------------------------------------------------------------ */
+/* reference-pinned operators                                          */
+/* ------------------------------------------------------------------ */
+
+/* internal/autodiff/ops/softmax.go:214-238 — 3 passes per row: max, fp64 exp
+ * cast to fp32 with a sequential fp32 sum, divide. */
+BORN_EXPORT void born_oracle_softmax_f32(const float *in, float *out, int64_t B, int64_t V) {
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = in + b * V;
+        float *o = out + b * V;
+        float mx = x[0];
+        for (int64_t j = 1; j < V; j++) if (x[j] > mx) mx = x[j];
+        float s = 0.0f;
+        for (int64_t j = 0; j < V; j++) { o[j] = (float)exp((double)(x[j] - mx)); s += o[j]; }
+        for (int64_t j = 0; j < V; j++) o[j] /= s;
+    }
+}
+
+/* internal/nn/cross_entropy.go:126-153 */
+BORN_EXPORT void born_oracle_log_softmax_f32(const float *in, float *out, int64_t B, int64_t V) {
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = in + b * V;
+        float *o = out + b * V;
+        float mx = x[0];
+        for (int64_t j = 1; j < V; j++) if (x[j] > mx) mx = x[j];
+        float s = 0.0f;
+        for (int64_t j = 0; j < V; j++) s += (float)exp((double)(x[j] - mx));
+        float lse = mx + (float)log((double)s);
+        for (int64_t j = 0; j < V; j++) o[j] = x[j] - lse;
+    }
+}
+
+/* internal/nn/cross_entropy.go:163-170 — softmax as exp(logSoftmax) */
+BORN_EXPORT void born_oracle_softmax_via_log(const float *in, float *out, int64_t B, int64_t V) {
+    born_oracle_log_softmax_f32(in, out, B, V);
+    for (int64_t i = 0; i < B * V; i++) out[i] = (float)exp((double)out[i]);
+}
+
+/* internal/nn/cross_entropy.go:241-251 — strict '>' from index 0 */
+BORN_EXPORT void born_oracle_argmax(const float *in, int64_t B, int64_t V, int64_t stride, int32_t *out) {
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = in + b * stride;
+        int64_t mi = 0;
+        float mv = x[0];
+        for (int64_t j = 1; j < V; j++) if (x[j] > mv) { mv = x[j]; mi = j; }
+        out[b] = (int32_t)mi;
+    }
+}
+
+/* internal/autodiff/ops/log.go:159-185 */
+BORN_EXPORT void born_oracle_exp_f32(const float *in, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = (float)exp((double)in[i]);
+}
+
+/* fp64-accumulated softmax (layer T of the standalone operator checks) */
+BORN_EXPORT void born_oracle_softmax_f64(const float *in, double *out, int64_t B, int64_t V, int64_t stride) {
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = in + b * stride;
+        double *o = out + b * V;
+        float mx = -INFINITY;
+        for (int64_t j = 0; j < V; j++) { float z = canon(x[j]); if (z > mx) mx = z; }
+        double s = 0.0;
+        for (int64_t j = 0; j < V; j++) {
+            float z = canon(x[j]);
+            o[j] = (z == mx) ? 1.0 : exp((double)z - (double)mx);
+            s += o[j];
+        }
+        for (int64_t j = 0; j < V; j++) o[j] /= s;
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* the sampling pipeline (docs/SAMPLING_SPEC.md §2)                    */
+/* ------------------------------------------------------------------ */
+
+static int cmp_u64_desc(const void *a, const void *b) {
+    uint64_t x = *(const uint64_t *)a, y = *(const uint64_t *)b;
+    return x < y ? 1 : (x > y ? -1 : 0);
+}
+
+/* min-heap on uint64 keys, used to keep the k largest keys (mode 2 baseline) */
+static void heap_sift_down(uint64_t *h, int64_t n, int64_t i) {
+    for (;;) {
+        int64_t l = 2 * i + 1, r = l + 1, s = i;
+        if (l < n && h[l] < h[s]) s = l;
+        if (r < n && h[r] < h[s]) s = r;
+        if (s == i) return;
+        uint64_t t = h[i]; h[i] = h[s]; h[s] = t;
+        i = s;
+    }
+}
+
+/* z_j for every j of one row: penalty (unique ids, from the original logit),
+ * temperature, canonicalisation.  `seen` is a V-byte scratch (zeroed on exit).
+ * Returns the number of out-of-range history ids. */
+static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hlen,
+                     float T, float r, float *z, uint8_t *seen) {
+    int64_t bad = 0;
+    for (int64_t j = 0; j < V; j++) z[j] = x[j];
+    if (r != 1.0f) {
+        for (int64_t i = 0; i < hlen; i++) {
+            int32_t t = hist[i];
+            if (t < 0 || t >= V) { bad++; continue; }
+            if (seen[t]) continue;
+            seen[t] = 1;
+            z[t] = penalise(x[t], r);
+        }
+        for (int64_t i = 0; i < hlen; i++) {
+            int32_t t = hist[i];
+            if (t >= 0 && t < V) seen[t] = 0;
+        }
+    } else {
+        for (int64_t i = 0; i < hlen; i++) if (hist[i] < 0 || hist[i] >= V) bad++;
+    }
+    for (int64_t j = 0; j < V; j++) z[j] = canon(z[j] / T);
+    return bad;
+}
+
+/*
+ * born_oracle_sample
+ *   logits [B, row_stride>=V]; history [B, hist_stride] (may be NULL), hist_len
+ *   [B] (NULL => hist_stride entries per row); uniforms [B].
+ * outputs (any may be NULL): tokens[B], probs[B], near[B] (layer T flags: bit 0 =
+ *   the draw lies within 1e-6 of a CDF step, so another correct implementation
+ *   may return a neighbouring token; bit 1 = the top-p cut lies within 1e-6 of a
+ *   CDF step, so the nucleus size may differ by one), n_nucleus[B], and when nuc_cap > 0 the
+ *   first min(n_nucleus, nuc_cap) survivors of each row in rank order:
+ *   nuc_ids[B, nuc_cap], nuc_probs[B, nuc_cap].
+ * returns the number of out-of-range history ids met, or -1 on bad arguments.
+ */
+BORN_EXPORT int64_t born_oracle_sample(
+    const float *logits, int64_t B, int64_t V, int64_t row_stride,
+    const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
+    const float *uniforms, float T, int32_t top_k, float top_p, float rep, int32_t mode,
+    int32_t *tokens, float *probs, uint8_t *near, int32_t *n_nucleus,
+    int64_t nuc_cap, int32_t *nuc_ids, float *nuc_probs)
+{
+    if (!logits || !uniforms || B <= 0 || V <= 0 || row_stride < V) return -1;
+    if (!(T > 0.0f) || !(top_p > 0.0f) || !(rep > 0.0f)) return -1;
+    int64_t k = (top_k <= 0 || top_k >= V) ? V : top_k;
+    int use_p = top_p < 1.0f;
+    int S = born_oracle_mass_shift(V);
+
+    float *z = (float *)malloc(sizeof(float) * (size_t)V);
+    uint8_t *seen = (uint8_t *)calloc((size_t)V, 1);
+    uint64_t *keys = (uint64_t *)malloc(sizeof(uint64_t) * (size_t)V);
+    double *e = (double *)malloc(sizeof(double) * (size_t)k);
+    uint64_t *q = (uint64_t *)malloc(sizeof(uint64_t) * (size_t)k);
+    int64_t bad = 0;
+
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = logits + b * row_stride;
+        int64_t hlen = history ? (hist_len ? hist_len[b] : hist_stride) : 0;
+        bad += row_z(x, V, history ? history + b * hist_stride : NULL, hlen, T, rep, z, seen);
+
+        /* rank order: the k largest 64-bit keys, descending */
+        int64_t n;
+        if (mode == 2 && k < V) {
+            n = k;
+            for (int64_t j = 0; j < k; j++) keys[j] = ((uint64_t)ordkey(z[j]) << 32) | (0xFFFFFFFFu - (uint32_t)j);
+            for (int64_t i = k / 2 - 1; i >= 0; i--) heap_sift_down(keys, k, i);
+            for (int64_t j = k; j < V; j++) {
+                uint64_t kk = ((uint64_t)ordkey(z[j]) << 32) | (0xFFFFFFFFu - (uint32_t)j);
+                if (kk > keys[0]) { keys[0] = kk; heap_sift_down(keys, k, 0); }
+            }
+            qsort(keys, (size_t)k, sizeof(uint64_t), cmp_u64_desc);
+        } else {
+            for (int64_t j = 0; j < V; j++) keys[j] = ((uint64_t)ordkey(z[j]) << 32) | (0xFFFFFFFFu - (uint32_t)j);
+            qsort(keys, (size_t)V, sizeof(uint64_t), cmp_u64_desc);
+            n = k;
+        }
+        float m = ordkey_inv((uint32_t)(keys[0] >> 32));
+        float u = uniforms[b];
+        int64_t np = n, pick = n - 1;
+        int is_near = 0;
+        double Zp_d = 0.0;   /* nucleus normaliser as a double, for probabilities */
+
+        if (mode == 0) {
+            double Zk = 0.0;
+            for (int64_t i = 0; i < n; i++) {
+                float zi = ordkey_inv((uint32_t)(keys[i] >> 32));
+                e[i] = (zi == m) ? 1.0 : exp((double)zi - (double)m);
+                Zk += e[i];
+            }
+            double c = 0.0;
+            int cut_near = 0;
+            if (use_p) {
+                double tp = (double)top_p * Zk;
+                int found = 0;
+                for (int64_t i = 0; i < n; i++) {
+                    c += e[i];
+                    if (fabs(c - tp) < 1e-6 * Zk) cut_near = 1;
+                    if (!found && c >= tp) { np = i + 1; found = 1; }
+                }
+            }
+            double Zp = 0.0;
+            for (int64_t i = 0; i < np; i++) Zp += e[i];
+            double t = (double)u * Zp;
+            /* if the cut itself is within tolerance, Z' may move by one element's mass */
+            double tol = 1e-6 * Zp;
+            if (cut_near) {
+                double delta = e[np - 1];
+                if (np < n && e[np] > delta) delta = e[np];
+                tol += (double)u * delta;
+            }
+            c = 0.0;
+            int found = 0;
+            for (int64_t i = 0; i < np; i++) {
+                c += e[i];
+                if (fabs(c - t) < tol) is_near |= 1;
+                if (!found && c > t) { pick = i; found = 1; }
+            }
+            if (!found) pick = np - 1;
+            if (cut_near) is_near |= 2;
+            Zp_d = Zp;
+        } else if (mode == 1) {
+            uint64_t Zk = 0;
+            for (int64_t i = 0; i < n; i++) {
+                float zi = ordkey_inv((uint32_t)(keys[i] >> 32));
+                q[i] = qmass(zi, m, S);
+                e[i] = (double)emass(zi, m);
+                Zk += q[i];
+            }
+            uint64_t c = 0;
+            if (use_p) {
+                uint64_t tp = (uint64_t)ceil((double)top_p * (double)Zk);
+                if (tp < 1) tp = 1;
+                if (tp > Zk) tp = Zk;
+                for (int64_t i = 0; i < n; i++) { c += q[i]; if (c >= tp) { np = i + 1; break; } }
+            }
+            uint64_t Zp = 0;
+            for (int64_t i = 0; i < np; i++) Zp += q[i];
+            uint64_t td = (uint64_t)floor((double)u * (double)Zp) + 1;
+            if (td > Zp) td = Zp;
+            c = 0;
+            pick = np - 1;
+            for (int64_t i = 0; i < np; i++) { c += q[i]; if (c >= td) { pick = i; break; } }
+            Zp_d = ldexp((double)Zp, -S);
+        } else {
+            /* reference arithmetic: fp64 exp cast to fp32, sequential fp32 sums */
+            float s = 0.0f;
+            for (int64_t i = 0; i < n; i++) {
+                float zi = ordkey_inv((uint32_t)(keys[i] >> 32));
+                float ei = (zi == m) ? 1.0f : (float)exp((double)(zi - m));
+                e[i] = (double)ei;
+                s += ei;
+            }
+            float c = 0.0f;
+            if (use_p) {
+                float tp = top_p * s;
+                for (int64_t i = 0; i < n; i++) { c += (float)e[i]; if (c >= tp) { np = i + 1; break; } }
+            }
+            float Zp = 0.0f;
+            for (int64_t i = 0; i < np; i++) Zp += (float)e[i];
+            float t = u * Zp;
+            c = 0.0f;
+            pick = np - 1;
+            for (int64_t i = 0; i < np; i++) { c += (float)e[i]; if (c > t) { pick = i; break; } }
+            Zp_d = (double)Zp;
+        }
+
+        if (tokens) tokens[b] = (int32_t)(0xFFFFFFFFu - (uint32_t)(keys[pick] & 0xFFFFFFFFu));
+        if (probs) probs[b] = (float)(e[pick] / Zp_d);
+        if (near) near[b] = (uint8_t)is_near;
+        if (n_nucleus) n_nucleus[b] = (int32_t)np;
+        if (nuc_cap > 0 && nuc_ids && nuc_probs) {
+            for (int64_t i = 0; i < nuc_cap; i++) {
+                if (i < np) {
+                    nuc_ids[b * nuc_cap + i] = (int32_t)(0xFFFFFFFFu - (uint32_t)(keys[i] & 0xFFFFFFFFu));
+                    nuc_probs[b * nuc_cap + i] = (float)(e[i] / Zp_d);
+                } else {
+                    nuc_ids[b * nuc_cap + i] = -1;
+                    nuc_probs[b * nuc_cap + i] = 0.0f;
+                }
+            }
+        }
+    }
+    free(z); free(seen); free(keys); free(e); free(q);
+    return bad;
+}
+
+/* ------------------------------------------------------------------ */
+/* speculative accept / reject (docs/SAMPLING_SPEC.md §5)              */
+/* ------------------------------------------------------------------ */
+
+/*
+ * target, draft: [B, G, V] fp32 contiguous; draft_tokens [B, G]; u_acc [B, G];
+ * u_res [B].  outputs: n_accepted[B], next_token[B], near[B] (may be NULL).
+ * mode 0 = layer T, 1 = layer F.  returns number of out-of-range draft tokens
+ * (such a position is rejected with p(d)=q(d)=0), -1 on bad arguments.
+ */
+BORN_EXPORT int64_t born_oracle_spec_verify(
+    const float *target, const float *draft, int64_t B, int64_t G, int64_t V,
+    const int32_t *draft_tokens, const float *u_acc, const float *u_res, float T, int32_t mode,
+    int32_t *n_accepted, int32_t *next_token, uint8_t *near)
+{
+    if (!target || !draft || !draft_tokens || !u_acc || !u_res || B <= 0 || G <= 0 || V <= 0 || !(T > 0.0f)) return -1;
+    int S = born_oracle_mass_shift(V);
+    float *zp = (float *)malloc(sizeof(float) * (size_t)V);
+    float *zq = (float *)malloc(sizeof(float) * (size_t)V);
+    int64_t bad = 0;
+    for (int64_t b = 0; b < B; b++) {
+        int32_t nacc = (int32_t)G, next = -1;
+        int is_near = 0;
+        for (int64_t i = 0; i < G; i++) {
+            const float *xt = target + (b * G + i) * V;
+            const float *xd = draft + (b * G + i) * V;
+            float mp = -INFINITY, mq = -INFINITY;
+            for (int64_t j = 0; j < V; j++) {
+                zp[j] = canon(xt[j] / T); if (zp[j] > mp) mp = zp[j];
+                zq[j] = canon(xd[j] / T); if (zq[j] > mq) mq = zq[j];
+            }
+            int32_t d = draft_tokens[b * G + i];
+            int d_ok = d >= 0 && d < V;
+            if (!d_ok) bad++;
+            float u = u_acc[b * G + i];
+            int accept;
+            if (mode == 0) {
+                double Zp = 0.0, Zq = 0.0;
+                for (int64_t j = 0; j < V; j++) {
+                    Zp += (zp[j] == mp) ? 1.0 : exp((double)zp[j] - (double)mp);
+                    Zq += (zq[j] == mq) ? 1.0 : exp((double)zq[j] - (double)mq);
+                }
+                double pd = d_ok ? ((zp[d] == mp) ? 1.0 : exp((double)zp[d] - (double)mp)) / Zp : 0.0;
+                double qd = d_ok ? ((zq[d] == mq) ? 1.0 : exp((double)zq[d] - (double)mq)) / Zq : 0.0;
+                accept = (double)u * qd < pd;
+                if (fabs((double)u * qd - pd) < 1e-6 * pd) is_near = 1;
+                if (!accept) {
+                    double R = 0.0;
+                    for (int64_t j = 0; j < V; j++) {
+                        double pj = ((zp[j] == mp) ? 1.0 : exp((double)zp[j] - (double)mp)) / Zp;
+                        double qj = ((zq[j] == mq) ? 1.0 : exp((double)zq[j] - (double)mq)) / Zq;
+                        R += pj > qj ? pj - qj : 0.0;
+                    }
+                    double t = (double)u_res[b] * R, c = 0.0;
+                    int found = 0;
+                    next = (int32_t)(V - 1);
+                    for (int64_t j = 0; j < V; j++) {
+                        double pj = ((zp[j] == mp) ? 1.0 : exp((double)zp[j] - (double)mp)) / Zp;
+                        double qj = ((zq[j] == mq) ? 1.0 : exp((double)zq[j] - (double)mq)) / Zq;
+                        c += pj > qj ? pj - qj : 0.0;
+                        if (fabs(c - t) < 1e-6 * R) is_near = 1;
+                        if (!found && c > t) { next = (int32_t)j; found = 1; }
+                    }
+                }
+            } else {
+                uint64_t Zp = 0, Zq = 0;
+                for (int64_t j = 0; j < V; j++) { Zp += qmass(zp[j], mp, S); Zq += qmass(zq[j], mq, S); }
+                uint64_t pd = d_ok ? qmass(zp[d], mp, S) : 0, qd = d_ok ? qmass(zq[d], mq, S) : 0;
+                accept = (double)u * (double)qd * (double)Zp < (double)pd * (double)Zq;
+                if (!accept) {
+                    uint64_t R = 0;
+                    for (int64_t j = 0; j < V; j++) {
+                        double pj = (double)qmass(zp[j], mp, S) / (double)Zp;
+                        double qj = (double)qmass(zq[j], mq, S) / (double)Zq;
+                        double r = pj > qj ? pj - qj : 0.0;
+                        R += (uint64_t)ldexp(r, S);
+                    }
+                    if (R == 0) {
+                        int64_t mi = 0;
+                        for (int64_t j = 1; j < V; j++) if (zp[j] > zp[mi]) mi = j;
+                        next = (int32_t)mi;
+                    } else {
+                        uint64_t td = (uint64_t)floor((double)u_res[b] * (double)R) + 1;
+                        if (td > R) td = R;
+                        uint64_t c = 0;
+                        next = (int32_t)(V - 1);
+                        for (int64_t j = 0; j < V; j++) {
+                            double pj = (double)qmass(zp[j], mp, S) / (double)Zp;
+                            double qj = (double)qmass(zq[j], mq, S) / (double)Zq;
+                            double r = pj > qj ? pj - qj : 0.0;
+                            c += (uint64_t)ldexp(r, S);
+                            if (c >= td) { next = (int32_t)j; break; }
+                        }
+                    }
+                }
+            }
+            if (!accept) { nacc = (int32_t)i; break; }
+        }
+        n_accepted[b] = nacc;
+        next_token[b] = next;
+        if (near) near[b] = (uint8_t)is_near;
+    }
+    free(zp); free(zq);
+    return bad;
+}
+
+/* layer-F row statistics used by the operator checks: m, Z (integer mass sum) */
+BORN_EXPORT void born_oracle_row_stats(const float *logits, int64_t B, int64_t V, int64_t stride, float T,
+                                       float *m_out, uint64_t *Z_out) {
+    int S = born_oracle_mass_shift(V);
+    for (int64_t b = 0; b < B; b++) {
+        const float *x = logits + b * stride;
+        float m = -INFINITY;
+        for (int64_t j = 0; j < V; j++) { float z = canon(x[j] / T); if (z > m) m = z; }
+        uint64_t Z = 0;
+        for (int64_t j = 0; j < V; j++) Z += qmass(canon(x[j] / T), m, S);
+        m_out[b] = m;
+        Z_out[b] = Z;
+    }
+}

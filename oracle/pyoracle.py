@@ -1,0 +1,189 @@
+"""ctypes loader for the CPU oracle (oracle/libborn_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg.  The product package (born_amd/) never imports it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libborn_oracle.so")
+
+MODE_TRUTH = 0      # layer T: fp64
+MODE_FIXED = 1      # layer F: fixed-point realisation (bit-exact target of the HIP kernels)
+MODE_REF32 = 2      # reference arithmetic (timed CPU baseline only)
+
+
+def build(force=False):
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(os.path.join(_HERE, "born_oracle.c")):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libborn_oracle.so"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        f32p, i32p, u8p, f64p, u64p = (C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint8),
+                                      C.POINTER(C.c_double), C.POINTER(C.c_uint64))
+        L.born_oracle_expneg.restype = C.c_float
+        L.born_oracle_expneg.argtypes = [C.c_float]
+        L.born_oracle_mass_shift.restype = C.c_int
+        L.born_oracle_mass_shift.argtypes = [C.c_int64]
+        L.born_oracle_uniform.restype = C.c_float
+        L.born_oracle_uniform.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64]
+        for name in ("born_oracle_softmax_f32", "born_oracle_log_softmax_f32", "born_oracle_softmax_via_log"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [f32p, f32p, C.c_int64, C.c_int64]
+        L.born_oracle_argmax.restype = None
+        L.born_oracle_argmax.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p]
+        L.born_oracle_exp_f32.restype = None
+        L.born_oracle_exp_f32.argtypes = [f32p, f32p, C.c_int64]
+        L.born_oracle_softmax_f64.restype = None
+        L.born_oracle_softmax_f64.argtypes = [f32p, f64p, C.c_int64, C.c_int64, C.c_int64]
+        L.born_oracle_sample.restype = C.c_int64
+        L.born_oracle_sample.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, f32p,
+                                         C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
+                                         i32p, f32p, u8p, i32p, C.c_int64, i32p, f32p]
+        L.born_oracle_spec_verify.restype = C.c_int64
+        L.born_oracle_spec_verify.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int64, i32p, f32p, f32p,
+                                              C.c_float, C.c_int32, i32p, i32p, u8p]
+        L.born_oracle_row_stats.restype = None
+        L.born_oracle_row_stats.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, C.c_float, f32p, u64p]
+        _lib = L
+    return _lib
+
+
+def _p(a, ct):
+    return None if a is None else a.ctypes.data_as(C.POINTER(ct))
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def expneg(d):
+    d = _f32(np.atleast_1d(d))
+    out = np.empty_like(d)
+    L = lib()
+    for i, v in enumerate(d.ravel()):
+        out.ravel()[i] = L.born_oracle_expneg(float(v))
+    return out
+
+
+def uniform(seed, step, row):
+    return lib().born_oracle_uniform(int(seed) & (2**64 - 1), int(step), int(row))
+
+
+def softmax_ref(x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().born_oracle_softmax_f32(_p(x, C.c_float), _p(out, C.c_float), x.shape[0], x.shape[1])
+    return out
+
+
+def log_softmax_ref(x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().born_oracle_log_softmax_f32(_p(x, C.c_float), _p(out, C.c_float), x.shape[0], x.shape[1])
+    return out
+
+
+def softmax_via_log_ref(x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().born_oracle_softmax_via_log(_p(x, C.c_float), _p(out, C.c_float), x.shape[0], x.shape[1])
+    return out
+
+
+def softmax_f64(x):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.float64)
+    lib().born_oracle_softmax_f64(_p(x, C.c_float), _p(out, C.c_double), x.shape[0], x.shape[1], x.shape[1])
+    return out
+
+
+def argmax_ref(x):
+    x = _f32(x)
+    out = np.empty(x.shape[0], dtype=np.int32)
+    lib().born_oracle_argmax(_p(x, C.c_float), x.shape[0], x.shape[1], x.shape[1], _p(out, C.c_int32))
+    return out
+
+
+def exp_ref(x):
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().born_oracle_exp_f32(_p(x, C.c_float), _p(out, C.c_float), x.size)
+    return out
+
+
+def row_stats(x, T=1.0):
+    x = _f32(x)
+    m = np.empty(x.shape[0], dtype=np.float32)
+    Z = np.empty(x.shape[0], dtype=np.uint64)
+    lib().born_oracle_row_stats(_p(x, C.c_float), x.shape[0], x.shape[1], x.shape[1], float(T),
+                                _p(m, C.c_float), _p(Z, C.c_uint64))
+    return m, Z
+
+
+def sample(logits, uniforms, temperature=1.0, top_k=0, top_p=1.0, rep=1.0, history=None, hist_len=None,
+           mode=MODE_TRUTH, nuc_cap=0):
+    """Returns dict(tokens, probs, near, n_nucleus[, nuc_ids, nuc_probs], bad_ids)."""
+    x = _f32(logits)
+    B, V = x.shape
+    u = _f32(uniforms)
+    assert u.shape == (B,)
+    h = hl = None
+    hs = 0
+    if history is not None:
+        h = np.ascontiguousarray(history, dtype=np.int32)
+        assert h.ndim == 2 and h.shape[0] == B
+        hs = h.shape[1]
+        if hist_len is not None:
+            hl = np.ascontiguousarray(hist_len, dtype=np.int32)
+    tokens = np.empty(B, dtype=np.int32)
+    probs = np.empty(B, dtype=np.float32)
+    near = np.zeros(B, dtype=np.uint8)
+    nn = np.empty(B, dtype=np.int32)
+    nid = npr = None
+    if nuc_cap > 0:
+        nid = np.empty((B, nuc_cap), dtype=np.int32)
+        npr = np.empty((B, nuc_cap), dtype=np.float32)
+    bad = lib().born_oracle_sample(_p(x, C.c_float), B, V, V, _p(h, C.c_int32), _p(hl, C.c_int32), hs,
+                                   _p(u, C.c_float), float(temperature), int(top_k), float(top_p), float(rep),
+                                   int(mode), _p(tokens, C.c_int32), _p(probs, C.c_float), _p(near, C.c_uint8),
+                                   _p(nn, C.c_int32), int(nuc_cap), _p(nid, C.c_int32), _p(npr, C.c_float))
+    if bad < 0:
+        raise ValueError("born_oracle_sample: bad arguments")
+    out = dict(tokens=tokens, probs=probs, near=(near & 1).astype(bool), near_cut=(near & 2).astype(bool),
+               n_nucleus=nn, bad_ids=int(bad))
+    if nuc_cap > 0:
+        out["nuc_ids"] = nid
+        out["nuc_probs"] = npr
+    return out
+
+
+def spec_verify(target, draft, draft_tokens, u_acc, u_res, temperature=1.0, mode=MODE_TRUTH):
+    t = _f32(target)
+    d = _f32(draft)
+    B, G, V = t.shape
+    dt = np.ascontiguousarray(draft_tokens, dtype=np.int32)
+    ua = _f32(u_acc)
+    ur = _f32(u_res)
+    nacc = np.empty(B, dtype=np.int32)
+    nxt = np.empty(B, dtype=np.int32)
+    near = np.zeros(B, dtype=np.uint8)
+    bad = lib().born_oracle_spec_verify(_p(t, C.c_float), _p(d, C.c_float), B, G, V, _p(dt, C.c_int32),
+                                        _p(ua, C.c_float), _p(ur, C.c_float), float(temperature), int(mode),
+                                        _p(nacc, C.c_int32), _p(nxt, C.c_int32), _p(near, C.c_uint8))
+    if bad < 0:
+        raise ValueError("born_oracle_spec_verify: bad arguments")
+    return dict(n_accepted=nacc, next_token=nxt, near=near.astype(bool), bad_tokens=int(bad))

@@ -1,0 +1,106 @@
+"""Pins the reference-following part of the oracle against the known-answer vectors the
+reference's own tests hold (tests/golden/reference_kats.json: data only)."""
+import json
+import math
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_kats.json")) as f:
+    KATS = json.load(f)
+
+
+def _expected(case):
+    if "expected" in case:
+        return np.array(case["expected"], dtype=np.float64)
+    expr = case["expected_expr"]
+    if expr in ("exp_ratio", "exp_ratio_of_1_2_3"):
+        e = [math.exp(1.0), math.exp(2.0), math.exp(3.0)]
+        s = sum(e)
+        return np.array([[np.float32(v / s) for v in e]], dtype=np.float64)
+    if expr == "1,e,e*e":
+        return np.array([1.0, np.float32(math.e), np.float32(math.e * math.e)], dtype=np.float64)
+    raise KeyError(expr)
+
+
+def test_softmax_kats(oracle):
+    for case in KATS["softmax"]:
+        x = np.array(case["input"], dtype=np.float32)
+        # ops_test.go exercises softmaxFloat32; cross_entropy_test.go exercises the exp(logSoftmax) form
+        fns = (oracle.softmax_ref, oracle.softmax_f64)
+        if "cross_entropy_test.go" in case["source"]:
+            fns = (oracle.softmax_via_log_ref,) + fns
+        for fn in fns:
+            out = np.asarray(fn(x), dtype=np.float64)
+            if "expected" in case or "expected_expr" in case:
+                assert np.max(np.abs(out - _expected(case))) <= case["tol_abs"], (case["source"], fn.__name__)
+            if "sum_tol" in case:
+                assert abs(out.sum() - 1.0) <= case["sum_tol"]
+            if case.get("finite"):
+                assert np.all(np.isfinite(out))
+
+
+def test_log_softmax_kats(oracle):
+    for case in KATS["log_softmax"]:
+        x = np.array(case["input"], dtype=np.float32)
+        out = oracle.log_softmax_ref(x).astype(np.float64)
+        if "expected" in case:
+            assert np.max(np.abs(out - np.array(case["expected"]))) <= case["tol_abs"], case["source"]
+        if case.get("finite"):
+            assert np.all(np.isfinite(out))
+            loss = -out[0, case["target"]]
+            assert 0.0 <= loss <= case["max_loss"]
+
+
+def test_argmax_kats(oracle):
+    for case in KATS["argmax"]:
+        x = np.array(case["input"], dtype=np.float32)
+        assert oracle.argmax_ref(x).tolist() == case["expected"], case["source"]
+
+
+def test_argmax_tie_rule_and_nan(oracle):
+    # internal/nn/cross_entropy.go:245 uses strict '>' scanning upward: lowest index wins ties,
+    # NaN never wins unless it is at index 0.
+    x = np.array([[5, 5, 5], [1, 7, 7], [np.nan, 9, 1], [1, np.nan, 0], [-np.inf, -np.inf, -np.inf]], dtype=np.float32)
+    assert oracle.argmax_ref(x).tolist() == [0, 1, 0, 0, 0]
+
+
+def test_exp_kats(oracle):
+    for case in KATS["exp"]:
+        x = np.array(case["input"], dtype=np.float32)
+        out = oracle.exp_ref(x).astype(np.float64)
+        assert np.max(np.abs(out - _expected(case))) <= case["tol_abs"]
+
+
+def test_extreme_logits(oracle):
+    for case in KATS["cross_entropy_extremes"]:
+        x = np.array(case["input"], dtype=np.float32)
+        p = oracle.softmax_ref(x)
+        assert oracle.argmax_ref(x)[0] == case["argmax"]
+        assert p[0, case["argmax"]] >= case["p_argmax_min"]
+        ls = oracle.log_softmax_ref(x)
+        assert -ls[0, case["argmax"]] < 0.1          # PerfectPrediction: loss near 0
+        assert -ls[0, 2] > 10.0                      # WorstPrediction: loss high
+
+
+def test_row_independence(oracle):
+    # internal/autodiff/ops/cross_entropy_test.go:168-195: a batch of identical rows gives the single-row result
+    x1 = np.array([[1.0, 2.0, 3.0]], dtype=np.float32)
+    x2 = np.repeat(x1, 2, axis=0)
+    assert np.array_equal(oracle.softmax_ref(x2)[0], oracle.softmax_ref(x1)[0])
+    assert np.array_equal(oracle.softmax_ref(x2)[1], oracle.softmax_ref(x1)[0])
+
+
+def test_expneg_accuracy_and_edges(oracle):
+    d = np.concatenate([np.linspace(0, 80, 4001), np.random.default_rng(1).uniform(0, 40, 4000)]).astype(np.float32)
+    got = oracle.expneg(d).astype(np.float64)
+    want = np.exp(-d.astype(np.float64))
+    rel = np.abs(got - want) / want
+    assert rel.max() < 4e-7, rel.max()
+    assert oracle.expneg(np.float32(0.0))[0] == 1.0
+    assert oracle.expneg(np.float32(80.5))[0] == 0.0
+    assert oracle.expneg(np.float32(np.inf))[0] == 0.0
+    # monotone non-increasing on a dense grid (a sign slip in the range reduction breaks this)
+    g = oracle.expneg(np.linspace(0, 30, 20001).astype(np.float32))
+    assert np.all(np.diff(g) <= 0)
