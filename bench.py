@@ -1,0 +1,149 @@
+#!/usr/bin/env python3
+"""Benchmark of the sampling hot path on one MI355X.
+
+A "step" is one pass of the sampler over one batch of synthetic logits already resident in HBM:
+batch 256 x vocab 128256, temperature 0.7, top-k 50, top-p 0.9, repetition penalty 1.15 over a
+512-token Zipf(1.1) history per row, one seeded uniform per row (configuration 3 of BASELINE.json,
+the one the metric is quoted on).  Prints ONE JSON line.
+
+  value        sampled tokens/s of the whole step (both launches of a step, inputs resident)
+  roofline     the dominant kernel (sample_topk_kernel): algorithmic bytes of one launch divided by
+               its average launch duration, measured here with HIP events on the launch stream
+  cpu_baseline the CPU oracle's reference-arithmetic mode timed on this box's host, one thread,
+               on a bounded sample of the same workload
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C5] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(w, seconds=12.0):
+    """Times the oracle's reference-arithmetic mode (the checker, used here only as the CPU baseline)."""
+    from oracle import pyoracle
+    rows = min(16, w.logits.shape[0])
+    x = np.ascontiguousarray(w.logits[:rows])
+    u = w.uniforms[:rows]
+    h = None if w.history is None else np.ascontiguousarray(w.history[:rows])
+    pyoracle.sample(x, u, w.temperature, w.top_k, w.top_p, w.rep, h, mode=pyoracle.MODE_REF32)   # warm
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        pyoracle.sample(x, u, w.temperature, w.top_k, w.top_p, w.rep, h, mode=pyoracle.MODE_REF32)
+        n += rows
+    dt = time.perf_counter() - t0
+    return {"value": n / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{n} rows of the same workload ({rows}-row slices repeated for {dt:.1f} s), "
+                      "C restatement of a Born-style scalar sampler (fp64 exp cast to fp32, sequential fp32 sums, heap top-k), 1 thread"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--config", default="C3")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; rows are independent, so more GPUs would each take a "
+              "slice of the batch with no exchange. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from born_amd import sampler as S
+    from born_amd import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    gen = {"C1": synth.c1, "C2": synth.c2, "C3": synth.c3, "C5": synth.c5}[args.config]
+    w = gen()
+    B, V = w.logits.shape
+    logits = torch.from_numpy(w.logits).to(dev)
+    uniforms = torch.from_numpy(w.uniforms).to(dev)
+    history = torch.from_numpy(w.history).to(dev) if w.history is not None else None
+    H = 0 if history is None else history.shape[1]
+    tokens = torch.empty(B, dtype=torch.int32, device=dev)
+    probs = torch.empty(B, dtype=torch.float32, device=dev)
+
+    smp = S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k, TopP=w.top_p,
+                                       RepetitionPenalty=w.rep), max_batch=B, max_vocab=V)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        smp.Sample(logits, B, V, history, None, uniforms, tokens, probs, hist_stride=H, stream=stream)
+
+    def timed(k):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(k):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / k            # ms per step
+
+    for _ in range(args.warmup):
+        step()
+    ms = timed(args.steps)
+    smp.Status(stream)
+    counters = smp.Counters(stream)
+    tok_host = tokens.cpu().numpy()
+    assert tok_host.min() >= 0 and tok_host.max() < V
+
+    # dominant kernel alone (the general kernel's early-exit launch left out): roofline of that kernel
+    single_pass = 1 <= w.top_k <= 64
+    if single_pass:
+        smp.SetPath(2)
+        for _ in range(10):
+            step()
+        ms_kernel = timed(args.steps)
+        smp.SetPath(0)
+        kernel_name = "sample_topk_kernel"
+    else:
+        ms_kernel = ms
+        kernel_name = "sample_wide_kernel"
+    alg_bytes = w.algorithmic_bytes()
+    achieved = alg_bytes / (ms_kernel * 1e-3) / 1e9
+
+    out = {
+        "metric": "sampled tokens/s at batch 256 x vocab 128256 (top-k+top-p); achieved HBM GB/s",
+        "value": B / (ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: batch {B} x vocab {V}, T={w.temperature}, top_k={w.top_k}, top_p={w.top_p}, "
+                               f"repetition_penalty={w.rep}, history {H}/row, seeded uniforms; logits resident in HBM",
+                   "seed": synth.BASE_SEED, "fallback_rows_per_step": counters["fallback_rows"] / max(1, args.steps + args.warmup)},
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "kernel_ms": ms_kernel},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,398 @@
+// C ABI over the HIP runtime (include/born_rocm.h).  Host code only: argument checks, the
+// sampler handle with its stream-ordered workspace, and kernel dispatch.
+#include "../../include/born_rocm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+#include "kernels.h"
+
+using namespace born;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+int hip_fail(hipError_t e, const char *what) {
+    return fail(BORN_ROCM_ERR_HIP, "sampler: %s: %s", what, hipGetErrorString(e));
+}
+#define HIP_TRY(expr)                                       \
+    do {                                                    \
+        hipError_t e__ = (expr);                            \
+        if (e__ != hipSuccess) return hip_fail(e__, #expr); \
+    } while (0)
+
+std::once_flag g_cfg_once;
+hipError_t g_cfg_err = hipSuccess;
+
+}  // namespace
+
+struct born_sampler {
+    born_sampler_config cfg;
+    int64_t max_batch, max_vocab;
+    int S_max;                     // segments per row at max_vocab
+    unsigned long long step;       // draws made with the built-in uniform stream
+    int path;                      // 0 = by top_k, 1 = always the general kernel, 2 = single-pass kernel alone
+    // device workspace
+    int *row_flags;
+    unsigned int *row_arrivals;
+    uint2 *cand;
+    int *cand_count;
+    float *seg_thr;
+    int *status;
+    unsigned long long *counters;
+    // argmax partials share cand_count / seg_thr storage; spec-verify statistics:
+    float *sp_mp, *sp_mq;
+    unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd;
+    int64_t spec_rows;
+};
+
+static int fill_defaults(born_sampler_config *c) {
+    if (c->temperature == 0.0f) c->temperature = 1.0f;
+    if (c->top_p == 0.0f) c->top_p = 1.0f;
+    if (c->repetition_penalty == 0.0f) c->repetition_penalty = 1.0f;
+    if (c->top_k < 0) c->top_k = 0;
+    if (!(c->temperature > 0.0f) || !std::isfinite(c->temperature))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: temperature must be > 0 and finite, got %g", (double)c->temperature);
+    if (!(c->top_p > 0.0f) || std::isnan(c->top_p))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: top_p must be > 0, got %g", (double)c->top_p);
+    if (!(c->repetition_penalty > 0.0f) || !std::isfinite(c->repetition_penalty))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: repetition_penalty must be > 0 and finite, got %g",
+                    (double)c->repetition_penalty);
+    return BORN_ROCM_OK;
+}
+
+extern "C" {
+
+const char *born_rocm_last_error(void) { return g_err; }
+
+int born_rocm_device_count(int32_t *count) {
+    if (!count) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: device_count: null output");
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n));
+    *count = n;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_device_name(int32_t device, char *buf, int64_t buf_len) {
+    if (!buf || buf_len <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: device_name: null buffer");
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, device));
+    snprintf(buf, (size_t)buf_len, "%s (%s)", p.name, p.gcnArchName);
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_alloc(int64_t bytes, void **dev_ptr) {
+    if (!dev_ptr || bytes <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: alloc: bytes must be > 0 and the output non-null");
+    HIP_TRY(hipMalloc(dev_ptr, (size_t)bytes));
+    return BORN_ROCM_OK;
+}
+int born_rocm_free(void *dev_ptr) {
+    if (!dev_ptr) return BORN_ROCM_OK;
+    HIP_TRY(hipFree(dev_ptr));
+    return BORN_ROCM_OK;
+}
+int born_rocm_h2d(void *dst_dev, const void *src_host, int64_t bytes, void *stream) {
+    if (!dst_dev || !src_host || bytes < 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: h2d: null pointer or negative size");
+    if (bytes == 0) return BORN_ROCM_OK;
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, (size_t)bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+int born_rocm_d2h(void *dst_host, const void *src_dev, int64_t bytes, void *stream) {
+    if (!dst_host || !src_dev || bytes < 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: d2h: null pointer or negative size");
+    if (bytes == 0) return BORN_ROCM_OK;
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, (size_t)bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+int born_rocm_stream_sync(void *stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, int64_t max_vocab, born_sampler **out) {
+    if (!out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: create: null output");
+    *out = nullptr;
+    if (max_batch <= 0 || max_vocab <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: create: max_batch and max_vocab must be > 0 (got %lld, %lld)",
+                    (long long)max_batch, (long long)max_vocab);
+    if (max_vocab > WIDE_MAX_VOCAB)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: create: max_vocab %lld exceeds the supported %lld",
+                    (long long)max_vocab, (long long)WIDE_MAX_VOCAB);
+    if (max_batch * ((max_vocab + TOPK_SEG - 1) / TOPK_SEG) > (int64_t)0x7FFFFFFF / TOPK_SEG_CAP)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: create: max_batch * segments too large");
+    born_sampler_config c;
+    if (cfg) c = *cfg; else memset(&c, 0, sizeof(c));
+    int rc = fill_defaults(&c);
+    if (rc) return rc;
+
+    std::call_once(g_cfg_once, [] { g_cfg_err = configure_kernels(); });
+    if (g_cfg_err != hipSuccess) return hip_fail(g_cfg_err, "configure_kernels");
+
+    born_sampler *s = new (std::nothrow) born_sampler();
+    if (!s) return fail(BORN_ROCM_ERR_HIP, "sampler: create: out of host memory");
+    memset(s, 0, sizeof(*s));
+    s->cfg = c;
+    s->max_batch = max_batch;
+    s->max_vocab = max_vocab;
+    s->S_max = (int)((max_vocab + TOPK_SEG - 1) / TOPK_SEG);
+    const size_t rows = (size_t)max_batch, segs = rows * (size_t)s->S_max;
+    hipError_t e = hipSuccess;
+    auto alloc = [&](void **p, size_t bytes) {
+        if (e == hipSuccess) e = hipMalloc(p, bytes);
+        if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
+    };
+    alloc((void **)&s->row_flags, rows * sizeof(int));
+    alloc((void **)&s->row_arrivals, rows * sizeof(unsigned int));
+    alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
+    alloc((void **)&s->cand_count, segs * sizeof(int));
+    alloc((void **)&s->seg_thr, segs * sizeof(float));
+    alloc((void **)&s->status, sizeof(int));
+    alloc((void **)&s->counters, 4 * sizeof(unsigned long long));
+    if (e != hipSuccess) {
+        born_rocm_sampler_destroy(s);
+        return hip_fail(e, "workspace allocation");
+    }
+    *out = s;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_destroy(born_sampler *s) {
+    if (!s) return BORN_ROCM_OK;
+    void *ptrs[] = {s->row_flags, s->row_arrivals, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
+                    s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    delete s;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_get_config(const born_sampler *s, born_sampler_config *out) {
+    if (!s || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: get_config: null argument");
+    *out = s->cfg;
+    return BORN_ROCM_OK;
+}
+int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg) {
+    if (!s || !cfg) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_config: null argument");
+    born_sampler_config c = *cfg;
+    int rc = fill_defaults(&c);
+    if (rc) return rc;
+    s->cfg = c;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_set_path(born_sampler *s, int32_t path) {
+    if (!s || path < 0 || path > 2) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
+    s->path = path;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_status(born_sampler *s, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: status: null handle");
+    int st = 0;
+    HIP_TRY(hipMemcpyAsync(&st, s->status, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    if (st) {
+        HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s", (st & 1) ? "out-of-range history id " : "",
+                    (st & 2) ? "out-of-range draft token" : "");
+    }
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
+                               int64_t *general_rows) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: counters: null handle");
+    unsigned long long c[4];
+    HIP_TRY(hipMemcpyAsync(c, s->counters, sizeof(c), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    if (topk_rows) *topk_rows = (int64_t)c[0];
+    if (fallback_rows) *fallback_rows = (int64_t)c[1];
+    if (general_rows) *general_rows = (int64_t)c[2];
+    return BORN_ROCM_OK;
+}
+
+static int check_logits(const char *op, const born_sampler *s, const float *logits, int64_t batch, int64_t vocab,
+                        int64_t row_stride) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: %s: null handle", op);
+    if (!logits) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: %s: null logits", op);
+    if (batch <= 0 || vocab <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: %s: batch and vocab must be > 0 (got %lld, %lld)", op,
+                    (long long)batch, (long long)vocab);
+    if (row_stride < vocab)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: %s: row_stride %lld < vocab %lld", op, (long long)row_stride,
+                    (long long)vocab);
+    if (batch > s->max_batch || vocab > s->max_vocab)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: %s: shape [%lld, %lld] exceeds the handle's [%lld, %lld]", op,
+                    (long long)batch, (long long)vocab, (long long)s->max_batch, (long long)s->max_vocab);
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_argmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     int32_t *tokens_out, void *stream) {
+    int rc = check_logits("argmax", s, logits, batch, vocab, row_stride);
+    if (rc) return rc;
+    if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: argmax: null output");
+    // ARGMAX_SEG == TOPK_SEG, so the per-segment workspace of the handle fits the partials.
+    HIP_TRY(launch_argmax(logits, (int)batch, (int)vocab, row_stride, tokens_out, s->seg_thr, s->cand_count,
+                          s->row_arrivals, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_softmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                      float *out, void *stream) {
+    int rc = check_logits("softmax", s, logits, batch, vocab, row_stride);
+    if (rc) return rc;
+    if (!out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: softmax: null output");
+    HIP_TRY(launch_softmax(logits, (int)batch, (int)vocab, row_stride, out, false, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                          float *out, void *stream) {
+    int rc = check_logits("log_softmax", s, logits, batch, vocab, row_stride);
+    if (rc) return rc;
+    if (!out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: log_softmax: null output");
+    HIP_TRY(launch_softmax(logits, (int)batch, (int)vocab, row_stride, out, true, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                     int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
+                     float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
+    int rc = check_logits("sample", s, logits, batch, vocab, row_stride);
+    if (rc) return rc;
+    if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample: null tokens_out");
+    if (history && hist_stride <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample: history given with hist_stride <= 0");
+    if (!history && hist_len) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample: hist_len given without history");
+    const bool any_nuc = nucleus_len_out || nucleus_ids_out || nucleus_probs_out;
+    if (any_nuc && !(nucleus_len_out && nucleus_ids_out && nucleus_probs_out && nucleus_cap > 0))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample: nucleus outputs must be all null or all set with nucleus_cap > 0");
+    if (row_stride > (int64_t)0x7FFFFFFF || hist_stride > (int64_t)0x7FFFFFFF || nucleus_cap > (int64_t)0x7FFFFFFF)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample: stride too large");
+
+    SampleArgs a;
+    memset(&a, 0, sizeof(a));
+    a.logits = logits;
+    a.row_stride = row_stride;
+    a.B = (int)batch;
+    a.V = (int)vocab;
+    a.history = history;
+    a.hist_len = hist_len;
+    a.hist_stride = history ? hist_stride : 0;
+    a.uniforms = uniforms;
+    a.seed = (unsigned long long)s->cfg.seed;
+    a.step = s->step;
+    a.T = s->cfg.temperature;
+    a.top_p = s->cfg.top_p;
+    a.rep = s->cfg.repetition_penalty;
+    a.top_k = (s->cfg.top_k <= 0 || s->cfg.top_k >= vocab) ? 0 : s->cfg.top_k;
+    a.tokens = tokens_out;
+    a.probs = probs_out;
+    a.nuc_len = nucleus_len_out;
+    a.nuc_ids = nucleus_ids_out;
+    a.nuc_probs = nucleus_probs_out;
+    a.nuc_cap = (int)nucleus_cap;
+    a.row_flags = s->row_flags;
+    a.row_arrivals = s->row_arrivals;
+    a.cand = s->cand;
+    a.cand_count = s->cand_count;
+    a.seg_thr = s->seg_thr;
+    a.S = (int)((vocab + TOPK_SEG - 1) / TOPK_SEG);
+    a.status = s->status;
+    a.counters = s->counters;
+    a.mass_shift = mass_shift(vocab);
+
+    hipStream_t st = (hipStream_t)stream;
+    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K) {
+        HIP_TRY(launch_sample_topk(a, st));
+        // redoes only the rows the first kernel flagged (path 2 leaves them to the caller: measurement only)
+        if (s->path == 0) HIP_TRY(launch_sample_wide(a, true, st));
+    } else {
+        HIP_TRY(launch_sample_wide(a, false, st));
+    }
+    if (!uniforms) s->step++;
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_spec_verify(born_sampler *s, const float *target, const float *draft, int64_t batch, int64_t gamma,
+                          int64_t vocab, const int32_t *draft_tokens, const float *u_accept, const float *u_residual,
+                          int32_t *n_accepted_out, int32_t *next_token_out, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: null handle");
+    if (!target || !draft || !draft_tokens || !u_accept || !u_residual || !n_accepted_out || !next_token_out)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: null pointer");
+    if (batch <= 0 || gamma <= 0 || vocab <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: batch, gamma and vocab must be > 0");
+    if (vocab > s->max_vocab)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: vocab %lld exceeds the handle's %lld", (long long)vocab,
+                    (long long)s->max_vocab);
+    if (batch * gamma > (int64_t)0x7FFFFFFF / 4)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: spec_verify: batch * gamma too large");
+    const int64_t rows = batch * gamma;
+    if (rows > s->spec_rows) {
+        // grow the per-position statistics (stream-ordered use only; the old buffers are idle once synchronised)
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+        void **ps[] = {(void **)&s->sp_mp, (void **)&s->sp_mq, (void **)&s->sp_Zp,
+                       (void **)&s->sp_Zq, (void **)&s->sp_pd, (void **)&s->sp_qd};
+        for (void **p : ps) {
+            if (*p) (void)hipFree(*p);
+            *p = nullptr;
+        }
+        s->spec_rows = 0;
+        HIP_TRY(hipMalloc((void **)&s->sp_mp, (size_t)rows * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&s->sp_mq, (size_t)rows * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&s->sp_Zp, (size_t)rows * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_Zq, (size_t)rows * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_pd, (size_t)rows * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_qd, (size_t)rows * sizeof(unsigned long long)));
+        s->spec_rows = rows;
+    }
+    SpecArgs a;
+    memset(&a, 0, sizeof(a));
+    a.target = target;
+    a.draft = draft;
+    a.B = (int)batch;
+    a.G = (int)gamma;
+    a.V = (int)vocab;
+    a.draft_tokens = draft_tokens;
+    a.u_acc = u_accept;
+    a.u_res = u_residual;
+    a.T = s->cfg.temperature;
+    a.n_accepted = n_accepted_out;
+    a.next_token = next_token_out;
+    a.mp = s->sp_mp; a.mq = s->sp_mq;
+    a.Zp = s->sp_Zp; a.Zq = s->sp_Zq;
+    a.pd = s->sp_pd; a.qd = s->sp_qd;
+    a.status = s->status;
+    a.mass_shift = mass_shift(vocab);
+    HIP_TRY(launch_spec_verify(a, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream) {
+    if (!d_in || !e_out || n <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: expneg: null pointer or n <= 0");
+    HIP_TRY(launch_expneg(d_in, e_out, n, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+int born_rocm_uniforms(int64_t seed, int64_t step, float *u_out, int64_t n, void *stream) {
+    if (!u_out || n <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: uniforms: null pointer or n <= 0");
+    HIP_TRY(launch_uniforms((unsigned long long)seed, (unsigned long long)step, u_out, n, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+}  // extern "C"

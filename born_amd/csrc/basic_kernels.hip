@@ -1,0 +1,168 @@
+// Greedy argmax, softmax / log-softmax and the two exported building blocks.
+//
+// argmax     follows `argmax`, internal/nn/cross_entropy.go:241-251 (strict '>' from index 0)
+// softmax    follows `softmaxFloat32`, internal/autodiff/ops/softmax.go:214-238
+// logsoftmax follows `logSoftmax`, internal/nn/cross_entropy.go:126-153
+#include "dev_common.h"
+#include "kernels.h"
+
+namespace born {
+
+// ---------------------------------------------------------------------------
+// argmax: grid = B * S workgroups of 256 threads, each scanning 8192 logits with
+// 128-bit loads; the last workgroup of a row to arrive merges the S partials.
+// A NaN never wins (the reference's comparisons are false for it) unless it sits
+// at index 0, where the reference's loop returns 0.
+// ---------------------------------------------------------------------------
+
+struct ArgPair {
+    float v;
+    int i;
+};
+__device__ __forceinline__ ArgPair better(ArgPair a, ArgPair b) {
+    // larger value wins; equal values: lower index wins
+    if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+    return a;
+}
+
+__global__ __launch_bounds__(256) void argmax_kernel(const float *__restrict__ logits, int V, long long stride, int S,
+                                                     int *__restrict__ tokens, float *part_val, int *part_idx,
+                                                     unsigned int *arrivals) {
+    __shared__ ArgPair sh[4];
+    __shared__ int is_last;
+    const int row = blockIdx.x / S, seg = blockIdx.x % S;
+    const float *x = logits + (long long)row * stride;
+    const int base = seg * ARGMAX_SEG;
+    const bool vec = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
+    ArgPair best = {-INFINITY, 0x7FFFFFFF};
+#pragma unroll
+    for (int it = 0; it < ARGMAX_SEG / (256 * 4); it++) {
+        int j = base + (it * 256 + (int)threadIdx.x) * 4;
+        float v[4];
+        if (vec && j + 3 < V) {
+            float4 f = *reinterpret_cast<const float4 *>(x + j);
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++) v[c] = (j + c < V) ? x[j + c] : __uint_as_float(0x7FC00000u);
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            // NaN (and padding) compare false everywhere and never enter
+            if (v[c] > best.v || (v[c] == best.v && j + c < best.i)) { best.v = v[c]; best.i = j + c; }
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgPair t = {__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
+        best = better(best, t);
+    }
+    if (lane_id() == 0) sh[wave_id()] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        ArgPair b = sh[0];
+        for (int w = 1; w < 4; w++) b = better(b, sh[w]);
+        part_val[blockIdx.x] = b.v;
+        part_idx[blockIdx.x] = b.i;
+        __threadfence();
+        unsigned int prev = atomicAdd(&arrivals[row], 1u);
+        is_last = (prev == (unsigned int)(S - 1));
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    if (threadIdx.x < WAVE) {
+        ArgPair b = {-INFINITY, 0x7FFFFFFF};
+        for (int s = threadIdx.x; s < S; s += WAVE) {
+            ArgPair t = {load_agent(&part_val[row * S + s]), load_agent(&part_idx[row * S + s])};
+            b = better(b, t);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            ArgPair t = {__shfl_xor(b.v, o, WAVE), __shfl_xor(b.i, o, WAVE)};
+            b = better(b, t);
+        }
+        if (threadIdx.x == 0) {
+            float x0 = x[0];
+            int tok = b.i;
+            if (x0 != x0) tok = 0;                 // NaN at index 0: every later comparison is false
+            if (tok == 0x7FFFFFFF) tok = 0;        // nothing ever compared greater than -inf
+            tokens[row] = tok;
+            arrivals[row] = 0;                     // ready for the next launch on this stream
+        }
+    }
+}
+
+hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
+                         int *part_idx, unsigned int *arrivals, hipStream_t st) {
+    int S = (V + ARGMAX_SEG - 1) / ARGMAX_SEG;
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)(B * S)), dim3(256), 0, st, logits, V, stride, S, tokens,
+                       part_val, part_idx, arrivals);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// softmax / log-softmax: one workgroup (1024 threads) per row, three sweeps
+// (max, integer mass sum, write); sweeps two and three hit L2.
+// ---------------------------------------------------------------------------
+
+template <bool LOG>
+__global__ __launch_bounds__(1024) void softmax_kernel(const float *__restrict__ logits, int V, long long stride,
+                                                       float *__restrict__ out, int S) {
+    __shared__ BlockScratch scr;
+    const int row = blockIdx.x;
+    const float *x = logits + (long long)row * stride;
+    float *o = out + (long long)row * V;
+    float mx = -INFINITY;
+    for (int j = threadIdx.x; j < V; j += 1024) mx = fmaxf(mx, canon(x[j]));
+    const float m = block_max_f32<1024>(mx, &scr);
+    const float scale = mass_scale(S);
+    u64 acc = 0;
+    for (int j = threadIdx.x; j < V; j += 1024) acc += qfix(emass(canon(x[j]), m), scale);
+    u64 Z;
+    block_inclusive_scan_u64<1024>(acc, &scr, &Z);
+    const double Zd = ldexp((double)Z, -S);
+    if (LOG) {
+        const double lz = log(Zd);
+        for (int j = threadIdx.x; j < V; j += 1024) {
+            float z = canon(x[j]);
+            o[j] = (float)(((double)z - (double)m) - lz);
+        }
+    } else {
+        for (int j = threadIdx.x; j < V; j += 1024) o[j] = (float)((double)emass(canon(x[j]), m) / Zd);
+    }
+}
+
+hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
+                          hipStream_t st) {
+    int S = mass_shift(V);
+    if (log_form)
+        hipLaunchKernelGGL(softmax_kernel<true>, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, out, S);
+    else
+        hipLaunchKernelGGL(softmax_kernel<false>, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, out, S);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// exported building blocks
+// ---------------------------------------------------------------------------
+
+__global__ void expneg_kernel(const float *d, float *e, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) e[i] = expneg(d[i]);
+}
+hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st) {
+    hipLaunchKernelGGL(expneg_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, d, e, n);
+    return hipGetLastError();
+}
+
+__global__ void uniforms_kernel(u64 seed, u64 step, float *u, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) u[i] = uniform_of(seed, step, (u64)i);
+}
+hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st) {
+    hipLaunchKernelGGL(uniforms_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, seed, step, u, n);
+    return hipGetLastError();
+}
+
+}  // namespace born

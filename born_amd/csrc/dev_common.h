@@ -1,0 +1,234 @@
+// Device-side building blocks shared by the sampling kernels (gfx950, wave64).
+//
+// Everything numeric here is the fixed-point realisation of docs/SAMPLING_SPEC.md:
+// each floating-point step is a single correctly rounded IEEE operation (the library is
+// built with -ffp-contract=off and correctly rounded fp32 division), every sum is a 64-bit
+// integer sum, so results do not depend on summation order or on the machine.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernels.h"
+
+namespace born {
+
+typedef unsigned long long u64;
+typedef unsigned int u32;
+
+constexpr int WAVE = 64;
+
+// ---- bit patterns ---------------------------------------------------------
+
+__device__ __forceinline__ u32 ordkey(float z) {          // order-preserving fp32 -> uint32
+    u32 b = __float_as_uint(z);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float ordkey_inv(u32 k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+}
+__device__ __forceinline__ u64 make_key64(float z, int id) {   // (z desc, id asc) == key64 desc
+    return ((u64)ordkey(z) << 32) | (u64)(0xFFFFFFFFu - (u32)id);
+}
+__device__ __forceinline__ int key64_id(u64 k) { return (int)(0xFFFFFFFFu - (u32)(k & 0xFFFFFFFFull)); }
+__device__ __forceinline__ float key64_z(u64 k) { return ordkey_inv((u32)(k >> 32)); }
+
+// NaN -> -inf, +inf -> FLT_MAX, -0 -> +0
+__device__ __forceinline__ float canon(float z) {
+    if (z != z) return -INFINITY;
+    if (z > 3.402823466e+38f) return 3.402823466e+38f;
+    if (z == 0.0f) return 0.0f;
+    return z;
+}
+__device__ __forceinline__ float penalise(float x, float r) { return x > 0.0f ? x / r : x * r; }
+
+// z from a (possibly penalised) logit: temperature then canonicalisation
+__device__ __forceinline__ float z_of(float y, float T) { return canon(T == 1.0f ? y : y / T); }
+
+// next representable float below x (x finite or +inf, not NaN); nextbelow(-FLT_MAX) = -inf
+__device__ __forceinline__ float next_below(float x) {
+    if (x == 0.0f) return -1.401298464e-45f;
+    u32 b = __float_as_uint(x);
+    return __uint_as_float((b & 0x80000000u) ? b + 1u : b - 1u);
+}
+
+// ---- the specified exponential and the integer mass ------------------------
+
+__device__ __forceinline__ float expneg(float d) {       // exp(-d), d >= 0; see the spec, section 6
+    if (!(d <= 80.0f)) return 0.0f;
+    float x = -d;
+    float k = rintf(x * 1.44269504f);
+    float r = fmaf(k, -0.693145752f, x);
+    r = fmaf(k, -1.42860677e-06f, r);
+    float y = fmaf(1.9875691500e-4f, r, 1.3981999507e-3f);
+    y = fmaf(y, r, 8.3334519073e-3f);
+    y = fmaf(y, r, 4.1665795894e-2f);
+    y = fmaf(y, r, 1.6666665459e-1f);
+    y = fmaf(y, r, 5.0000001201e-1f);
+    float r2 = r * r;
+    y = fmaf(y, r2, r);
+    y = y + 1.0f;
+    return __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
+}
+__device__ __forceinline__ float emass(float z, float m) {
+    float d = (z == m) ? 0.0f : m - z;
+    return expneg(d);
+}
+// trunc(e * 2^S): e has 24 significant bits, so e * 2^S (S <= 61) is exact in fp32
+__device__ __forceinline__ u64 qfix(float e, float scale) { return (u64)(e * scale); }
+__device__ __forceinline__ float mass_scale(int S) { return __uint_as_float((u32)(S + 127) << 23); }
+
+// ---- built-in uniform stream ------------------------------------------------
+
+__host__ __device__ __forceinline__ u64 mix64(u64 x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+__host__ __device__ __forceinline__ float uniform_of(u64 seed, u64 step, u64 row) {
+    u64 x = mix64(mix64(seed ^ (step * 0xD1342543DE82EF95ull)) + row);
+    return (float)(x >> 40) * 5.9604644775390625e-08f;    // 2^-24
+}
+
+// ---- integer thresholds of the fixed-point pipeline --------------------------
+
+__device__ __forceinline__ u64 top_p_target(float p, u64 Zk) {
+    u64 tp = (u64)ceil((double)p * (double)Zk);
+    if (tp < 1) tp = 1;
+    if (tp > Zk) tp = Zk;
+    return tp;
+}
+__device__ __forceinline__ u64 draw_target(float u, u64 Zp) {
+    u64 td = (u64)floor((double)u * (double)Zp) + 1ull;
+    if (td > Zp) td = Zp;
+    return td;
+}
+__device__ __forceinline__ float prob_of(float e, u64 Zp, int S) {
+    return (float)((double)e / ldexp((double)Zp, -S));
+}
+
+// Loads that must observe what other workgroups wrote before an agent-scope release
+// (per-CU vector L1 is not coherent): relaxed atomic loads at agent scope bypass it.
+__device__ __forceinline__ float load_agent(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int load_agent(const int *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u32 load_agent(const u32 *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u64 load_agent(const u64 *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- wave / block primitives --------------------------------------------------
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }
+__device__ __forceinline__ int wave_id() { return (int)(threadIdx.x >> 6); }
+
+__device__ __forceinline__ float wave_max_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+__device__ __forceinline__ u32 wave_sum_u32(u32 v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ u64 shfl_up_u64(u64 v, int o) {
+    u32 lo = __shfl_up((u32)v, o, WAVE), hi = __shfl_up((u32)(v >> 32), o, WAVE);
+    return ((u64)hi << 32) | lo;
+}
+__device__ __forceinline__ u64 shfl_u64(u64 v, int src) {
+    u32 lo = __shfl((u32)v, src, WAVE), hi = __shfl((u32)(v >> 32), src, WAVE);
+    return ((u64)hi << 32) | lo;
+}
+__device__ __forceinline__ u64 wave_inclusive_scan_u64(u64 v) {
+    int l = lane_id();
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        u64 t = shfl_up_u64(v, o);
+        if (l >= o) v += t;
+    }
+    return v;
+}
+
+// Scratch for block-level collectives: one slot per wave plus broadcast slots.
+struct BlockScratch {
+    u64 w[16];
+    u64 bcast[4];
+};
+
+template <int BLOCK>
+__device__ __forceinline__ float block_max_f32(float v, BlockScratch *s) {
+    constexpr int NW = BLOCK / WAVE;
+    v = wave_max_f32(v);
+    __syncthreads();
+    if (lane_id() == 0) ((float *)s->w)[wave_id()] = v;
+    __syncthreads();
+    float r = ((float *)s->w)[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r = fmaxf(r, ((float *)s->w)[i]);
+    return r;
+}
+
+template <int BLOCK>
+__device__ __forceinline__ u32 block_sum_u32(u32 v, BlockScratch *s) {
+    constexpr int NW = BLOCK / WAVE;
+    v = wave_sum_u32(v);
+    __syncthreads();
+    if (lane_id() == 0) ((u32 *)s->w)[wave_id()] = v;
+    __syncthreads();
+    u32 r = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) r += ((u32 *)s->w)[i];
+    return r;
+}
+
+// Inclusive scan of one u64 per thread across the block; *total receives the block sum.
+template <int BLOCK>
+__device__ __forceinline__ u64 block_inclusive_scan_u64(u64 v, BlockScratch *s, u64 *total) {
+    constexpr int NW = BLOCK / WAVE;
+    u64 inc = wave_inclusive_scan_u64(v);
+    __syncthreads();
+    if (lane_id() == WAVE - 1) s->w[wave_id()] = inc;
+    __syncthreads();
+    u64 off = 0, tot = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+        u64 t = s->w[i];
+        if (i < wave_id()) off += t;
+        tot += t;
+    }
+    *total = tot;
+    return inc + off;
+}
+
+// Bitonic sort of n2 (power of two) u64 keys in LDS, descending.
+template <int BLOCK>
+__device__ __forceinline__ void bitonic_sort_desc(u64 *a, int n2) {
+    for (int k = 2; k <= n2; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < n2; i += BLOCK) {
+                int p = i ^ j;
+                if (p > i) {
+                    u64 x = a[i], y = a[p];
+                    bool first_big = ((i & k) == 0);
+                    if (first_big ? (x < y) : (x > y)) { a[i] = y; a[p] = x; }
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ int next_pow2(int n) {
+    int p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+}  // namespace born

@@ -1,0 +1,89 @@
+// Host-visible launch interface of the HIP kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace born {
+
+// Geometry of the single-pass top-k kernel.
+constexpr int TOPK_BLOCK = 256;            // threads per workgroup (4 waves)
+constexpr int TOPK_F4 = 8;                 // float4 loads per thread
+constexpr int TOPK_SEG = TOPK_BLOCK * TOPK_F4 * 4;   // 8192 logits per workgroup
+constexpr int TOPK_SEG_CAP = 1024;         // candidates one segment may emit
+constexpr int TOPK_ROW_CAP = 2048;         // candidates the row-level finish can hold
+constexpr int TOPK_MAX_K = 64;             // largest top_k served by the single-pass kernel
+
+// Geometry of the general (any k, any p) kernel: one workgroup per row.
+constexpr int WIDE_BLOCK = 1024;
+constexpr int WIDE_BINS = 4096;            // level-0 histogram bins over d = m - z
+constexpr float WIDE_BINS_PER_UNIT = 128.0f;   // 4096 bins cover d in [0, 32)
+constexpr int WIDE_LIST_CAP = 4096;        // elements the in-LDS sort can hold
+constexpr int WIDE_SUB_BINS = 2048;        // radix-descent digit = 11 bits
+constexpr int64_t WIDE_MAX_VOCAB = 524288; // history bitmap must fit LDS next to the histogram
+
+constexpr int ARGMAX_SEG = 8192;
+
+// Integer masses are trunc(e * 2^S) with S chosen so that a whole row sums below 2^62.
+__host__ __device__ inline int mass_shift(long long V) {
+    int n = 0;
+    unsigned long long v = (unsigned long long)V;
+    while (v) { n++; v >>= 1; }
+    return 62 - n;
+}
+
+struct SampleArgs {
+    const float *logits;
+    long long row_stride;
+    int B, V;
+    const int *history;
+    const int *hist_len;
+    long long hist_stride;
+    const float *uniforms;
+    unsigned long long seed, step;
+    float T, top_p, rep;
+    int top_k;                    // 0 = disabled, else 1 <= top_k < V
+    int *tokens;
+    float *probs;
+    int *nuc_len;
+    int *nuc_ids;
+    float *nuc_probs;
+    int nuc_cap;
+    // workspace
+    int *row_flags;               // [B] 1 = row must be redone by the general kernel
+    unsigned int *row_arrivals;   // [B] segment arrival counters (self-resetting)
+    uint2 *cand;                  // [B][S][TOPK_SEG_CAP] (logit bits, id)
+    int *cand_count;              // [B][S]
+    float *seg_thr;               // [B][S]
+    int S;                        // segments per row
+    int *status;                  // device status word
+    unsigned long long *counters; // [0] top-k rows, [1] fallback rows, [2] general rows
+    int mass_shift;
+};
+
+struct SpecArgs {
+    const float *target, *draft;
+    int B, G, V;
+    const int *draft_tokens;
+    const float *u_acc, *u_res;
+    float T;
+    int *n_accepted, *next_token;
+    // workspace: per (b, i) row statistics
+    float *mp, *mq;
+    unsigned long long *Zp, *Zq, *pd, *qd;
+    int *status;
+    int mass_shift;
+};
+
+hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
+                         int *part_idx, unsigned int *arrivals, hipStream_t st);
+hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
+                          hipStream_t st);
+hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
+hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
+hipError_t launch_sample_topk(const SampleArgs &a, hipStream_t st);
+hipError_t launch_sample_wide(const SampleArgs &a, bool fallback_only, hipStream_t st);
+hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);
+size_t wide_lds_bytes(int V);
+hipError_t configure_kernels();   // one-time function attributes (dynamic LDS above 64 KiB)
+
+}  // namespace born

@@ -1,0 +1,139 @@
+/*
+ * born_rocm.h — C ABI of the MI355X (gfx950) token-sampling engine for Born.
+ *
+ * This is the boundary a build-tagged Go package `backend/rocm` binds through cgo
+ * (plain pointers and sizes only; no Go pointer is retained after a call returns).
+ * Born v0.1.1 has no device backend and no sampler, so each entry point cites the
+ * reference interface it stands beside or extends (paths relative to the reference
+ * root).  Semantics of every sampling stage: docs/SAMPLING_SPEC.md.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a BORN_ROCM_ERR_* code; the message
+ *     for the calling thread's last failure is born_rocm_last_error();
+ *   - all device pointers are plain `void*` / typed pointers into HIP device
+ *     memory; `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - logits are fp32, row-major `[batch, vocab]` with a row stride in elements,
+ *     the layout of tensor.RawTensor (internal/tensor/raw.go:78-105, strides
+ *     internal/tensor/shape.go:52-63); token ids are int32, as the reference's
+ *     label tensors are (internal/nn/cross_entropy.go:73, raw.go:167-174);
+ *   - inputs are never modified (the reference's "inputs are immutable unless
+ *     uniquely owned" rule, internal/backend/cpu/backend.go:45-51);
+ *   - launches are asynchronous on `stream`; outputs are valid after the stream
+ *     is synchronised (born_rocm_stream_sync or a born_rocm_d2h on that stream).
+ */
+#ifndef BORN_ROCM_H
+#define BORN_ROCM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BORN_ROCM_OK               0
+#define BORN_ROCM_ERR_ARGUMENT     1   /* programmer error: the Go layer panics "sampler: ..." (internal/backend/cpu/backend.go:36 idiom) */
+#define BORN_ROCM_ERR_HIP          2   /* runtime failure: the Go layer returns an error (internal/tensor/raw.go:89-92 idiom) */
+#define BORN_ROCM_ERR_UNSUPPORTED  3   /* shape outside what the kernels handle (e.g. vocab too large for LDS) */
+#define BORN_ROCM_ERR_DATA         4   /* device-side data error: out-of-range history id / draft token */
+
+/* Sampling configuration.  Mirrors the reference's plain-struct config idiom
+ * (AdamConfig, internal/optim/adam.go:59-63): a zero field means "default", filled
+ * in by born_rocm_sampler_create the way NewAdam fills its defaults
+ * (internal/optim/adam.go:78-91). */
+typedef struct born_sampler_config {
+    float   temperature;          /* 0 => 1.0 ; must be > 0 otherwise */
+    int32_t top_k;                /* <= 0 => disabled */
+    float   top_p;                /* 0 => 1.0 (disabled) ; must be > 0 otherwise; >= 1 disables */
+    float   repetition_penalty;   /* 0 => 1.0 (identity) ; must be > 0 otherwise */
+    int64_t seed;                 /* seed of the built-in uniform stream (used only when `uniforms` is NULL) */
+} born_sampler_config;
+
+typedef struct born_sampler born_sampler;   /* opaque: config + stream-ordered workspace + draw counter */
+
+/* Thread-local message of the last failure on the calling thread ("" if none). */
+const char *born_rocm_last_error(void);
+
+/* Device discovery / selection — extends tensor.Device (internal/tensor/raw.go:10-20), which has no ROCm value. */
+int born_rocm_device_count(int32_t *count);
+int born_rocm_device_name(int32_t device, char *buf, int64_t buf_len);
+
+/* Device buffers — Born's RawTensor is host-only (internal/tensor/raw.go:42-46,139-141); these give the Go
+ * layer its DeviceBuffer handle.  Copies are enqueued on `stream` and are synchronous with respect to the host
+ * when the host pointer is pageable. */
+int born_rocm_alloc(int64_t bytes, void **dev_ptr);
+int born_rocm_free(void *dev_ptr);
+int born_rocm_h2d(void *dst_dev, const void *src_host, int64_t bytes, void *stream);
+int born_rocm_d2h(void *dst_host, const void *src_dev, int64_t bytes, void *stream);
+int born_rocm_stream_sync(void *stream);
+
+/* Sampler handle — the capability object a `SamplerBackend` type assertion would return
+ * (idiom: ReLUBackend, internal/nn/activation.go:8-20).  `max_batch`/`max_vocab` size the workspace;
+ * calls with larger shapes fail with BORN_ROCM_ERR_ARGUMENT.  One handle = one stream at a time. */
+int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, int64_t max_vocab,
+                             born_sampler **out);
+int born_rocm_sampler_destroy(born_sampler *s);
+int born_rocm_sampler_get_config(const born_sampler *s, born_sampler_config *out);   /* after defaults were filled */
+int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg);
+/* Device status since the last call of this function: 0, or BORN_ROCM_ERR_DATA if a kernel met an
+ * out-of-range history id or draft token.  Synchronises `stream`. */
+int born_rocm_sampler_status(born_sampler *s, void *stream);
+/* Work counters accumulated by the kernels (diagnostics): rows sampled by the single-pass top-k kernel,
+ * rows that fell back to the general kernel, rows sampled by the general kernel directly.  Synchronises. */
+int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
+                               int64_t *general_rows);
+
+/* Diagnostics: 0 = choose the kernel from top_k (default), 1 = always use the general kernel, 2 = launch the
+ * single-pass top-k kernel alone (rows it flags are left undone and counted in fallback_rows: for timing that
+ * kernel by itself, never for results).  Both kernels implement the same fixed-point pipeline and must return
+ * identical results; tests compare them. */
+int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
+
+/* Greedy decode: index of the maximum of each row, lowest index on ties — `argmax`,
+ * internal/nn/cross_entropy.go:241-251 (the per-row step of nn.Accuracy, :261-284). */
+int born_rocm_argmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     int32_t *tokens_out, void *stream);
+
+/* Max-shifted softmax / log-softmax over the last dimension —
+ * softmaxFloat32, internal/autodiff/ops/softmax.go:214-238 (ops.Softmax, :268-294);
+ * logSoftmax, internal/nn/cross_entropy.go:126-153.  `out` is `[batch, vocab]` contiguous. */
+int born_rocm_softmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                      float *out, void *stream);
+int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                          float *out, void *stream);
+
+/* One sampling step for `batch` rows: penalty -> temperature -> top-k -> softmax -> top-p -> draw.
+ * No counterpart in the reference snapshot; it consumes the `[batch, vocab]` fp32 output of the last
+ * Linear (internal/nn/linear.go:78-107) where the reference's only consumers are CrossEntropy and
+ * nn.Accuracy (internal/nn/cross_entropy.go:261-284).
+ *   history   int32 [batch, hist_stride] or NULL; hist_len int32 [batch] or NULL (=> hist_stride each)
+ *   uniforms  fp32 [batch] in [0,1) or NULL (=> built-in stream from cfg.seed and the handle's draw counter)
+ *   tokens_out int32 [batch]; probs_out fp32 [batch] or NULL (probability of the sampled token in the
+ *   renormalised nucleus)
+ *   nucleus outputs (all three NULL, or all three set with nucleus_cap > 0): the first
+ *   min(n, nucleus_cap) survivors of each row in rank order; produced when 1 <= top_k <= 4096
+ *   (nucleus_len_out[b] = -1 otherwise). */
+int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
+                     const float *uniforms, int32_t *tokens_out, float *probs_out,
+                     int32_t *nucleus_len_out, int32_t *nucleus_ids_out, float *nucleus_probs_out,
+                     int64_t nucleus_cap, void *stream);
+
+/* Speculative-decoding accept/reject with residual max(0, p - q) resampling.
+ * No counterpart in the reference snapshot.
+ *   target, draft  fp32 [batch, gamma, vocab] contiguous;  draft_tokens int32 [batch, gamma]
+ *   u_accept fp32 [batch, gamma];  u_residual fp32 [batch]
+ *   n_accepted_out int32 [batch];  next_token_out int32 [batch] (-1 when every draft token was accepted) */
+int born_rocm_spec_verify(born_sampler *s, const float *target, const float *draft, int64_t batch,
+                          int64_t gamma, int64_t vocab, const int32_t *draft_tokens, const float *u_accept,
+                          const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out,
+                          void *stream);
+
+/* Building blocks exported for parity tests (device-side evaluation of the specified fp32 exponential and of
+ * the built-in uniform stream). */
+int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream);
+int born_rocm_uniforms(int64_t seed, int64_t step, float *u_out, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BORN_ROCM_H */

@@ -1,0 +1,358 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Bars (docs/SAMPLING_SPEC.md):
+  * against the fixed-point layer of the oracle: token ids, nucleus sizes, accept counts — bit-exact,
+    every row; probabilities bit-exact as fp32;
+  * against the fp64 truth layer: token ids equal except on rows the truth layer flags as drawn within
+    1e-6 of a CDF step (counted, bounded); probabilities within 1e-5 relative.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rocm():
+    from born_amd import sampler as S
+    assert S.DeviceCount() >= 1, "no HIP device visible"
+    return S
+
+
+def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0, max_vocab=None):
+    B, V = x.shape
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=k, TopP=p, RepetitionPenalty=rep), max_batch=B,
+                        max_vocab=max_vocab or V)
+    s.SetPath(path)
+    out = rocm.sample_host(s, x, u, hist, hist_len, nucleus_cap=nuc)
+    out["counters"] = s.Counters()
+    s.Status()
+    s.Close()
+    return out
+
+
+def _check_against_oracle(oracle, rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0,
+                          max_near_frac=1.0):
+    got = _run(rocm, x, u, T, k, p, rep, hist, hist_len, nuc, path)
+    fx = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED, nuc_cap=nuc)
+    tr = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_TRUTH, nuc_cap=nuc)
+    bad = np.nonzero(got["tokens"] != fx["tokens"])[0]
+    assert bad.size == 0, f"token mismatch vs fixed-point oracle at rows {bad[:8]}: {got['tokens'][bad[:8]]} vs {fx['tokens'][bad[:8]]}"
+    assert np.array_equal(got["probs"].view(np.uint32), fx["probs"].view(np.uint32)), "probabilities differ from the fixed-point oracle"
+    diff = got["tokens"] != tr["tokens"]
+    assert not (diff & ~tr["near"]).any(), "token differs from the fp64 truth on a row not flagged near a CDF step"
+    assert tr["near"].mean() <= max_near_frac
+    same = ~diff
+    assert np.allclose(got["probs"][same], tr["probs"][same], rtol=1e-5, atol=0), "probability off by more than 1e-5 relative"
+    if nuc:
+        assert np.array_equal(got["n_nucleus"], fx["n_nucleus"])
+        assert np.array_equal(got["nuc_ids"], fx["nuc_ids"])
+        assert np.array_equal(got["nuc_probs"].view(np.uint32), fx["nuc_probs"].view(np.uint32))
+        ok = ~tr["near_cut"]
+        assert np.array_equal(got["n_nucleus"][ok], tr["n_nucleus"][ok])
+        m = (tr["nuc_ids"][ok] >= 0) & (tr["nuc_ids"][ok] == got["nuc_ids"][ok])
+        assert np.allclose(got["nuc_probs"][ok][m], tr["nuc_probs"][ok][m], rtol=1e-5)
+    return got, fx, tr
+
+
+# ---------------------------------------------------------------- building blocks
+
+def test_expneg_bit_exact(oracle, rocm):
+    from born_amd import _capi
+    d = np.concatenate([np.linspace(0, 90, 20001), np.random.default_rng(0).uniform(0, 40, 50000),
+                        [0.0, 80.0, 80.00001, np.inf]]).astype(np.float32)
+    buf_in = rocm.DeviceBuffer.from_numpy(d)
+    buf_out = rocm.DeviceBuffer(d.nbytes)
+    _capi.check(_capi.lib().born_rocm_expneg(buf_in.ptr, buf_out.ptr, d.size, None))
+    got = buf_out.to_numpy(np.float32, d.shape)
+    want = oracle.expneg(d)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_uniform_stream_bit_exact(oracle, rocm):
+    from born_amd import _capi
+    n = 1000
+    out = rocm.DeviceBuffer(4 * n)
+    for seed, step in [(0, 0), (1234, 7), (-5, 3)]:
+        _capi.check(_capi.lib().born_rocm_uniforms(seed, step, out.ptr, n, None))
+        got = out.to_numpy(np.float32, (n,))
+        want = np.array([oracle.uniform(seed, step, r) for r in range(n)], dtype=np.float32)
+        assert np.array_equal(got, want)
+        assert got.min() >= 0.0 and got.max() < 1.0
+
+
+# ---------------------------------------------------------------- reference-pinned operators
+
+def _argmax(rocm, x, stride=None):
+    B, V = x.shape
+    s = rocm.NewSampler(max_batch=B, max_vocab=V)
+    if stride:
+        xp = np.zeros((B, stride), np.float32)
+        xp[:, :V] = x
+        xp[:, V:] = 1e30              # padding must never be read as data
+        d = rocm.DeviceBuffer.from_numpy(xp)
+    else:
+        d = rocm.DeviceBuffer.from_numpy(x)
+    t = rocm.DeviceBuffer(4 * B)
+    s.Argmax(d, B, V, t, row_stride=stride)
+    s.Argmax(d, B, V, t, row_stride=stride)       # second launch: the arrival counters must have reset themselves
+    return t.to_numpy(np.int32, (B,))
+
+
+def test_argmax_reference_kats_and_tie_rule(oracle, rocm):
+    x = np.array([[1, 2, 3], [3, 1, 2], [2, 3, 1], [1, 1, 3]], dtype=np.float32)        # TestAccuracy vectors
+    assert _argmax(rocm, x).tolist() == [2, 0, 1, 2]
+    x = np.array([[5, 5, 5], [1, 7, 7], [np.nan, 9, 1], [1, np.nan, 0], [-np.inf, -np.inf, -np.inf]], dtype=np.float32)
+    assert _argmax(rocm, x).tolist() == oracle.argmax_ref(x).tolist() == [0, 1, 0, 0, 0]
+
+
+@pytest.mark.parametrize("B,V,stride", [(64, 32000, None), (7, 8193, None), (5, 1001, 1003), (3, 128256, None), (2, 5, 8)])
+def test_argmax_random_and_ties(oracle, rocm, B, V, stride):
+    rng = np.random.default_rng(V)
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    assert np.array_equal(_argmax(rocm, x, stride), oracle.argmax_ref(x))
+    xi = rng.integers(-2, 3, size=(B, V)).astype(np.float32)                              # thousands of ties
+    assert np.array_equal(_argmax(rocm, xi, stride), oracle.argmax_ref(xi))
+
+
+def test_softmax_operators(oracle, rocm):
+    import json, os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")) as f:
+        kats = json.load(f)
+    s = rocm.NewSampler(max_batch=64, max_vocab=32000)
+
+    def soft(x, log=False):
+        B, V = x.shape
+        d, o = rocm.DeviceBuffer.from_numpy(x), rocm.DeviceBuffer(x.nbytes)
+        s.Softmax(d, B, V, o, log=log)
+        return o.to_numpy(np.float32, x.shape)
+
+    for case in kats["softmax"]:
+        x = np.array(case["input"], dtype=np.float32)
+        got = soft(x).astype(np.float64)
+        want = oracle.softmax_ref(x).astype(np.float64)          # the reference's arithmetic
+        assert np.max(np.abs(got - want)) <= 1e-6, case["source"]
+        assert abs(got.sum() - 1.0) <= 1e-6 and np.all(np.isfinite(got))
+    for case in kats["log_softmax"]:
+        x = np.array(case["input"], dtype=np.float32)
+        got = soft(x, log=True).astype(np.float64)
+        assert np.all(np.isfinite(got))
+        assert np.max(np.abs(got - oracle.log_softmax_ref(x))) <= 1e-4 * max(1.0, np.abs(x).max() * 1e-2)
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((64, 32000), dtype=np.float32) * 2).astype(np.float32)
+    got = soft(x)
+    want = oracle.softmax_f64(x)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-30)
+    assert np.max(np.abs(got - oracle.softmax_ref(x))) <= 1e-6
+    lg = soft(x, log=True).astype(np.float64)
+    assert np.max(np.abs(lg - np.log(want))) < 1e-5
+
+
+# ---------------------------------------------------------------- sampling: single-pass top-k kernel
+
+@pytest.mark.parametrize("B,V,T,k,p,rep,H", [
+    (1, 32000, 0.8, 40, 0.95, 1.1, 64),          # C1 shape
+    (32, 128256, 0.7, 50, 0.9, 1.15, 512),       # C3 shape, 32 rows
+    (16, 32000, 1.0, 1, 1.0, 1.3, 16),           # greedy with penalty
+    (16, 8192, 1.3, 64, 0.5, 1.0, 0),
+    (16, 8193, 0.5, 7, 1.0, 0.8, 8),             # tail segment of one element; penalty < 1 boosts
+    (9, 1000, 1.0, 50, 0.9, 1.2, 300),           # fewer lanes than logits per wave
+    (9, 777, 0.9, 64, 0.99, 1.5, 2000),          # history longer than the vocabulary
+    (4, 100, 1.0, 64, 0.9, 1.1, 10),
+    (4, 3, 1.0, 2, 0.9, 1.0, 0),
+])
+def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H):
+    rng = np.random.default_rng(B * 1000003 + V)
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(64, max(k, 1)))
+    c = got["counters"]
+    assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
+
+
+def test_topk_kernel_hist_len_and_strided_rows(oracle, rocm):
+    rng = np.random.default_rng(5)
+    B, V, H = 12, 5000, 40
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+    hl = rng.integers(0, H + 1, size=B).astype(np.int32)
+    _check_against_oracle(oracle, rocm, x, u, 0.9, 20, 0.9, 1.4, hist, hl)
+    # unaligned row stride (scalar load path): rows placed in a wider buffer
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=20, TopP=0.9), max_batch=B, max_vocab=V)
+    xp = np.full((B, V + 3), 99.0, np.float32)
+    xp[:, :V] = x
+    d_x, d_u, d_t = rocm.DeviceBuffer.from_numpy(xp), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer(4 * B)
+    s.Sample(d_x, B, V, None, None, d_u, d_t, row_stride=V + 3)
+    want = oracle.sample(x, u, 0.9, 20, 0.9, mode=oracle.MODE_FIXED)["tokens"]
+    assert np.array_equal(d_t.to_numpy(np.int32, (B,)), want)
+
+
+def test_topk_kernel_ties_and_special_values(oracle, rocm):
+    rng = np.random.default_rng(6)
+    B, V = 24, 20000
+    xi = rng.integers(-3, 4, size=(B, V)).astype(np.float32)           # thousands of exact ties at the cut
+    u = rng.random(B, dtype=np.float32)
+    got, _, _ = _check_against_oracle(oracle, rocm, xi, u, 0.7, 50, 0.9, nuc=64)
+    assert got["counters"]["fallback_rows"] > 0                         # ties overflow the single-pass path
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    x[:, ::7] = -np.inf
+    x[:, 5::11] = np.nan
+    x[0, 100] = np.inf
+    x[1, :] = -np.inf                                                   # nothing finite: uniform over ids
+    x[2, 17:] = -np.inf                                                 # fewer finite logits than top_k
+    x[3, :] = 0.0
+    x[3, 1::2] = -0.0                                                   # -0 ties with +0
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 40, 0.95, nuc=64)
+
+
+def test_topk_and_general_kernels_agree(oracle, rocm):
+    rng = np.random.default_rng(7)
+    B, V, H = 24, 40000, 128
+    x = (rng.standard_normal((B, V), dtype=np.float32) * 2).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+    a = _run(rocm, x, u, 0.7, 50, 0.9, 1.15, hist, nuc=64, path=0)
+    b = _run(rocm, x, u, 0.7, 50, 0.9, 1.15, hist, nuc=64, path=1)
+    assert a["counters"]["topk_rows"] == B and b["counters"]["general_rows"] == B
+    for key in ("tokens", "n_nucleus", "nuc_ids"):
+        assert np.array_equal(a[key], b[key]), key
+    assert np.array_equal(a["probs"].view(np.uint32), b["probs"].view(np.uint32))
+
+
+# ---------------------------------------------------------------- sampling: general kernel
+
+@pytest.mark.parametrize("B,V,T,k,p,rep,H", [
+    (64, 32000, 1.0, 0, 1.0, 1.0, 0),            # C2 multinomial shape
+    (16, 152064, 1.2, 0, 0.99, 1.05, 2048),      # C5 shape, 16 rows
+    (16, 32000, 0.9, 500, 0.9, 1.1, 64),         # top_k above the single-pass limit
+    (8, 50000, 1.0, 20000, 0.8, 1.0, 0),         # top_k too large to list: count descent
+    (8, 50000, 1.0, 20000, 1.0, 1.0, 0),
+    (16, 4097, 0.6, 0, 0.3, 1.0, 0),
+    (16, 1000, 2.0, 100, 1.0, 1.2, 50),
+    (5, 2, 1.0, 0, 0.9, 1.0, 0),
+    (5, 1, 1.0, 0, 0.9, 1.0, 0),
+])
+def test_general_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H):
+    rng = np.random.default_rng(B * 7919 + V + k)
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32) if H else None
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist)
+    assert got["counters"]["general_rows"] == B
+
+
+def test_general_kernel_degenerate_rows(oracle, rocm):
+    rng = np.random.default_rng(8)
+    B, V = 12, 30000
+    u = rng.random(B, dtype=np.float32)
+    x = np.zeros((B, V), np.float32)                                    # every logit equal: radix descent on ids
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 1.0)
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.5)
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 9000, 0.9)
+    xi = rng.integers(-1, 2, size=(B, V)).astype(np.float32)            # three values
+    _check_against_oracle(oracle, rocm, xi, u, 0.8, 0, 0.9)
+    _check_against_oracle(oracle, rocm, xi, u, 0.8, 12345, 0.9)
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    x[:, ::3] = -np.inf
+    x[:, 1::5] = np.nan
+    x[0, :] = -np.inf
+    x[1, 7] = np.inf
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.95)
+    far = rng.standard_normal((B, V), dtype=np.float32) - 200.0         # everything but one far below the maximum
+    far[:, 11] = 0.0
+    _check_against_oracle(oracle, rocm, far, u, 1.0, 0, 1.0)
+
+
+def test_builtin_uniform_stream_in_sample(oracle, rocm):
+    rng = np.random.default_rng(9)
+    B, V = 16, 6000
+    x = rng.standard_normal((B, V), dtype=np.float32)
+    s = rocm.NewSampler(rocm.SamplerConfig(TopK=30, Seed=4242), max_batch=B, max_vocab=V)
+    for step in range(3):
+        got = rocm.sample_host(s, x, None)
+        u = np.array([oracle.uniform(4242, step, r) for r in range(B)], dtype=np.float32)
+        want = oracle.sample(x, u, top_k=30, mode=oracle.MODE_FIXED)
+        assert np.array_equal(got["tokens"], want["tokens"]), step
+
+
+# ---------------------------------------------------------------- speculative accept / reject
+
+def test_spec_verify_against_oracle(oracle, rocm):
+    from born_amd import synth
+    w = synth.c4(rows=16)
+    e = w.extra
+    s = rocm.NewSampler(max_batch=16, max_vocab=32000)
+    got = rocm.verify_host(s, e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"])
+    fx = oracle.spec_verify(e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"], mode=oracle.MODE_FIXED)
+    tr = oracle.spec_verify(e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"], mode=oracle.MODE_TRUTH)
+    assert np.array_equal(got["n_accepted"], fx["n_accepted"]) and np.array_equal(got["next_token"], fx["next_token"])
+    diff = (got["n_accepted"] != tr["n_accepted"]) | (got["next_token"] != tr["next_token"])
+    assert not (diff & ~tr["near"]).any()
+    assert 0 < got["n_accepted"].mean() < 5                               # the workload exercises both outcomes
+    s.Status()
+
+
+def test_spec_verify_special_cases(oracle, rocm):
+    rng = np.random.default_rng(10)
+    B, G, V = 6, 5, 3001                                                   # odd vocabulary: scalar load path
+    t = rng.standard_normal((B, G, V), dtype=np.float32)
+    d = rng.integers(0, V, size=(B, G)).astype(np.int32)
+    ua, ur = rng.random((B, G), dtype=np.float32), rng.random(B, dtype=np.float32)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8), max_batch=B, max_vocab=V)
+    got = rocm.verify_host(s, t, t.copy(), d, ua, ur)                      # identical models accept everything
+    assert np.all(got["n_accepted"] == G) and np.all(got["next_token"] == -1)
+    dr = (t + rng.standard_normal((B, G, V), dtype=np.float32)).astype(np.float32)
+    got = rocm.verify_host(s, t, dr, d, ua, ur)
+    fx = oracle.spec_verify(t, dr, d, ua, ur, temperature=0.8, mode=oracle.MODE_FIXED)
+    assert np.array_equal(got["n_accepted"], fx["n_accepted"]) and np.array_equal(got["next_token"], fx["next_token"])
+    # hand vector: p = [.5 .3 .2], q = [.2 .5 .3], draft token 1 -> accept iff u < 0.6, residual -> id 0
+    s1 = rocm.NewSampler(max_batch=1, max_vocab=3)
+    tt = np.log(np.array([[[5, 3, 2]]], dtype=np.float64)).astype(np.float32)
+    qq = np.log(np.array([[[2, 5, 3]]], dtype=np.float64)).astype(np.float32)
+    r = rocm.verify_host(s1, tt, qq, np.array([[1]], np.int32), np.array([[0.59]], np.float32), np.array([0.7], np.float32))
+    assert r["n_accepted"][0] == 1 and r["next_token"][0] == -1
+    r = rocm.verify_host(s1, tt, qq, np.array([[1]], np.int32), np.array([[0.61]], np.float32), np.array([0.7], np.float32))
+    assert r["n_accepted"][0] == 0 and r["next_token"][0] == 0
+    # out-of-range draft token: rejected, reported through the status word
+    bad = d.copy()
+    bad[2, 0] = V + 5
+    got = rocm.verify_host(s, t, dr, bad, ua, ur)
+    assert got["n_accepted"][2] == 0
+    with pytest.raises(rocm.BornRocmError):
+        s.Status()
+    s.Status()                                                             # the status word clears once read
+
+
+# ---------------------------------------------------------------- error behaviour
+
+def test_argument_errors_panic_like_the_go_layer(rocm):
+    with pytest.raises(rocm.SamplerPanic, match="sampler: temperature"):
+        rocm.NewSampler(rocm.SamplerConfig(Temperature=-1.0))
+    with pytest.raises(rocm.SamplerPanic, match="top_p"):
+        rocm.NewSampler(rocm.SamplerConfig(TopP=-0.5))
+    with pytest.raises(rocm.SamplerPanic, match="repetition_penalty"):
+        rocm.NewSampler(rocm.SamplerConfig(RepetitionPenalty=float("nan")))
+    with pytest.raises(rocm.SamplerPanic):
+        rocm.NewSampler(max_batch=0)
+    s = rocm.NewSampler(max_batch=4, max_vocab=100)
+    cfg = s.Config()
+    assert (cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty) == (1.0, 0, 1.0, 1.0)      # zero => defaults
+    buf = rocm.DeviceBuffer(4 * 4 * 100)
+    tok = rocm.DeviceBuffer(16)
+    with pytest.raises(rocm.SamplerPanic, match="exceeds"):
+        s.Sample(buf, 5, 100, None, None, None, tok)
+    with pytest.raises(rocm.SamplerPanic, match="row_stride"):
+        s.Sample(buf, 4, 100, None, None, None, tok, row_stride=50)
+    with pytest.raises(rocm.SamplerPanic, match="null"):
+        s.Sample(None, 4, 100, None, None, None, tok)
+    with pytest.raises(rocm.SamplerPanic, match="> 0"):
+        s.Sample(buf, 0, 100, None, None, None, tok)
+    # out-of-range history ids: ignored by the kernel, reported by Status
+    x = np.random.default_rng(0).standard_normal((4, 100), dtype=np.float32)
+    h = np.array([[1, 2, 300, -4]] * 4, np.int32)
+    s.SetConfig(rocm.SamplerConfig(TopK=10, RepetitionPenalty=1.2))
+    rocm.sample_host(s, x, np.full(4, 0.5, np.float32), h)
+    with pytest.raises(rocm.BornRocmError, match="history"):
+        s.Status()
