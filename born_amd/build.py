@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libborn_rocm.so")
-SOURCES = ["api.hip", "basic_kernels.hip", "sample_kernels.hip", "spec_kernels.hip"]
+SOURCES = ["api.hip", "basic_kernels.hip", "sample_topk.hip", "sample_wide.hip", "spec_kernels.hip"]
 
 # -ffp-contract=off and correctly rounded fp32 division: every floating-point step of the
 # fixed-point pipeline must be a single IEEE rounding, identical on host and device.
@@ -35,7 +35,7 @@ def build(verbose=False):
     procs = []
     for src in SOURCES:
         obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
-        cmd = [hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc()] + FLAGS + os.environ.get("BORN_EXTRA_HIPCC_FLAGS", "").split() + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

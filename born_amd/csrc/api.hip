@@ -47,7 +47,6 @@ struct born_sampler {
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // 0 = by top_k, 1 = always the general kernel, 2 = single-pass kernel alone
     // device workspace
-    int *row_flags;
     unsigned int *row_arrivals;
     uint2 *cand;
     int *cand_count;
@@ -156,7 +155,6 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
         if (e == hipSuccess) e = hipMalloc(p, bytes);
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
-    alloc((void **)&s->row_flags, rows * sizeof(int));
     alloc((void **)&s->row_arrivals, rows * sizeof(unsigned int));
     alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
     alloc((void **)&s->cand_count, segs * sizeof(int));
@@ -173,7 +171,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->row_flags, s->row_arrivals, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
+    void *ptrs[] = {s->row_arrivals, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -308,7 +306,6 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_ids = nucleus_ids_out;
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
-    a.row_flags = s->row_flags;
     a.row_arrivals = s->row_arrivals;
     a.cand = s->cand;
     a.cand_count = s->cand_count;
@@ -319,9 +316,12 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.mass_shift = mass_shift(vocab);
 
     hipStream_t st = (hipStream_t)stream;
-    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K) {
-        HIP_TRY(launch_sample_topk(a, st));
-        // redoes only the rows the first kernel flagged (path 2 leaves them to the caller: measurement only)
+    // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
+    const bool boosts = history && a.rep < 1.0f;
+    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && !boosts) {
+        HIP_TRY(launch_topk_collect(a, st));
+        // finishes each row from its candidates, or runs the general algorithm on a row that cannot be
+        // proven from them (path 2 stops after the collect kernel: for timing that kernel alone)
         if (s->path == 0) HIP_TRY(launch_sample_wide(a, true, st));
     } else {
         HIP_TRY(launch_sample_wide(a, false, st));

@@ -122,6 +122,33 @@ __device__ __forceinline__ u64 load_agent(const u64 *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Matching stores: relaxed atomic stores at agent scope are written through to the agent's
+// coherence point instead of lingering in an XCD-local L2.
+__device__ __forceinline__ void store_agent(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(int *p, int v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(u64 *p, u64 v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Hand-off between workgroups without a cache-wide fence.  A full agent-scope release/acquire
+// fence on this multi-XCD part writes back and invalidates a whole L2 and costs far more than
+// the kernel it protects.  The producer instead (1) writes its message with store_agent,
+// (2) waits for those stores to complete (workgroup-scope release = wait on the store
+// counters) and joins its workgroup at a barrier, (3) lets one thread bump the arrival counter
+// with an agent-scope atomic.  The consumer that sees the final count reads the message with
+// load_agent only.  Every access to the shared locations is an agent-scope atomic, so each is
+// coherent by itself; the completion wait orders them.
+__device__ __forceinline__ void handoff_complete_stores() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
+__device__ __forceinline__ u32 handoff_arrive(u32 *counter) {
+    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ---- wave / block primitives --------------------------------------------------
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }

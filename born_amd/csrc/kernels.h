@@ -10,7 +10,6 @@ constexpr int TOPK_BLOCK = 256;            // threads per workgroup (4 waves)
 constexpr int TOPK_F4 = 8;                 // float4 loads per thread
 constexpr int TOPK_SEG = TOPK_BLOCK * TOPK_F4 * 4;   // 8192 logits per workgroup
 constexpr int TOPK_SEG_CAP = 1024;         // candidates one segment may emit
-constexpr int TOPK_ROW_CAP = 2048;         // candidates the row-level finish can hold
 constexpr int TOPK_MAX_K = 64;             // largest top_k served by the single-pass kernel
 
 // Geometry of the general (any k, any p) kernel: one workgroup per row.
@@ -49,8 +48,7 @@ struct SampleArgs {
     float *nuc_probs;
     int nuc_cap;
     // workspace
-    int *row_flags;               // [B] 1 = row must be redone by the general kernel
-    unsigned int *row_arrivals;   // [B] segment arrival counters (self-resetting)
+    unsigned int *row_arrivals;   // [B] segment arrival counters of the argmax kernel (self-resetting)
     uint2 *cand;                  // [B][S][TOPK_SEG_CAP] (logit bits, id)
     int *cand_count;              // [B][S]
     float *seg_thr;               // [B][S]
@@ -80,8 +78,8 @@ hipError_t launch_softmax(const float *logits, int B, int V, long long stride, f
                           hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
-hipError_t launch_sample_topk(const SampleArgs &a, hipStream_t st);
-hipError_t launch_sample_wide(const SampleArgs &a, bool fallback_only, hipStream_t st);
+hipError_t launch_topk_collect(const SampleArgs &a, hipStream_t st);
+hipError_t launch_sample_wide(const SampleArgs &a, bool try_candidates, hipStream_t st);
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);
 size_t wide_lds_bytes(int V);
 hipError_t configure_kernels();   // one-time function attributes (dynamic LDS above 64 KiB)

@@ -1,272 +1,17 @@
-// The sampling step: penalty -> temperature -> top-k -> softmax -> top-p -> inverse-CDF draw.
+// General sampling kernel: any top_k / top_p (docs/SAMPLING_SPEC.md, fixed-point layer).
 //
-// Two kernels implement the same fixed-point pipeline (docs/SAMPLING_SPEC.md, layer F) and
-// return bit-identical results for the same row:
-//
-//   sample_topk_kernel  1 <= top_k <= 64.  One HBM pass.  Each workgroup owns an 8192-logit
-//                       segment of one row in registers, derives a threshold that at least
-//                       top_k of its logits reach, emits the few logits at or above it, and
-//                       the last workgroup of the row to arrive finishes the row (sort of the
-//                       survivors, integer CDF, draw).  Rows it cannot prove correct are
-//                       flagged and redone by the general kernel.
-//   sample_wide_kernel  any top_k / top_p.  One workgroup per row; a max sweep, a histogram
-//                       sweep over d = max - z with integer masses, then a sweep that gathers
-//                       only the histogram bins the top-k cut, the top-p cut and the draw fall
-//                       into; those few elements are sorted in LDS and resolved exactly.
-//
-// Logits are read with 128-bit loads and never written.
+// One workgroup (1024 threads) per row.  Sweep 1 finds the row maximum of z, sweep 2 builds a
+// 4096-bin histogram over d = max - z with integer masses (and counts when a top-k cut is needed),
+// then one more sweep gathers only the bins the top-k cut, the top-p cut and the draw fall into;
+// those few elements are sorted in LDS and resolved exactly.  Over-full bins (ties, masked rows)
+// are refined by a radix descent over the 64-bit rank key.  Sweeps 2+ hit L2 / Infinity Cache
+// when the batch fits.  Logits are read with 128-bit loads and never written.
 #include "dev_common.h"
+#include "finish.h"
 #include "kernels.h"
+#include "topk_finish.h"
 
 namespace born {
-
-// ---------------------------------------------------------------------------
-// Shared finish: `list` holds 64-bit keys sorted descending (rank order); the first
-// `ns` are the top-k survivors.  Computes the integer CDF, the top-p cut and the draw.
-// ---------------------------------------------------------------------------
-template <int BLOCK, int ITEMS>
-__device__ void finish_sorted(const u64 *list, int ns, const SampleArgs &a, int row, BlockScratch *scr) {
-    const int tid = threadIdx.x;
-    const float scale = mass_scale(a.mass_shift);
-    const float m = key64_z(list[0]);
-    const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
-    float e[ITEMS];
-    u64 cum[ITEMS];
-    u64 local = 0;
-#pragma unroll
-    for (int it = 0; it < ITEMS; it++) {
-        int i = tid * ITEMS + it;
-        e[it] = 0.0f;
-        if (i < ns) {
-            e[it] = emass(key64_z(list[i]), m);
-            local += qfix(e[it], scale);
-        }
-        cum[it] = local;
-    }
-    u64 Zk;
-    u64 inc = block_inclusive_scan_u64<BLOCK>(local, scr, &Zk);
-    u64 excl = inc - local;
-#pragma unroll
-    for (int it = 0; it < ITEMS; it++) cum[it] += excl;
-
-    int np = ns;
-    u64 Zp = Zk;
-    if (a.top_p < 1.0f) {
-        const u64 tp = top_p_target(a.top_p, Zk);
-        u32 c = 0;
-#pragma unroll
-        for (int it = 0; it < ITEMS; it++) c += (tid * ITEMS + it < ns && cum[it] < tp) ? 1u : 0u;
-        np = (int)block_sum_u32<BLOCK>(c, scr) + 1;
-        __syncthreads();
-#pragma unroll
-        for (int it = 0; it < ITEMS; it++)
-            if (tid * ITEMS + it == np - 1) scr->bcast[0] = cum[it];
-        __syncthreads();
-        Zp = scr->bcast[0];
-    }
-    const u64 td = draw_target(u, Zp);
-    u32 c = 0;
-#pragma unroll
-    for (int it = 0; it < ITEMS; it++) c += (tid * ITEMS + it < np && cum[it] < td) ? 1u : 0u;
-    const int pick = (int)block_sum_u32<BLOCK>(c, scr);
-#pragma unroll
-    for (int it = 0; it < ITEMS; it++) {
-        int i = tid * ITEMS + it;
-        if (i == pick) {
-            a.tokens[row] = key64_id(list[i]);
-            if (a.probs) a.probs[row] = prob_of(e[it], Zp, a.mass_shift);
-        }
-        if (a.nuc_len && i < np && i < a.nuc_cap) {
-            a.nuc_ids[(long long)row * a.nuc_cap + i] = key64_id(list[i]);
-            a.nuc_probs[(long long)row * a.nuc_cap + i] = prob_of(e[it], Zp, a.mass_shift);
-        }
-    }
-    if (a.nuc_len) {
-        if (tid == 0) a.nuc_len[row] = np;
-        for (int i = np + tid; i < a.nuc_cap; i += BLOCK) {
-            a.nuc_ids[(long long)row * a.nuc_cap + i] = -1;
-            a.nuc_probs[(long long)row * a.nuc_cap + i] = 0.0f;
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Single-pass top-k kernel
-// ---------------------------------------------------------------------------
-
-// a-th largest of the 64 keys held one per lane (binary search on the bits; scalar work)
-__device__ __forceinline__ u32 wave_kth_largest(u32 key, int a) {
-    u32 cand = 0;
-#pragma unroll 1
-    for (int bit = 31; bit >= 0; --bit) {
-        u32 t = cand | (1u << bit);
-        int c = __popcll(__ballot(key >= t));
-        if (c >= a) cand = t;
-    }
-    return cand;
-}
-
-__global__ __launch_bounds__(TOPK_BLOCK) void sample_topk_kernel(SampleArgs a) {
-    __shared__ u64 lds[TOPK_ROW_CAP];             // phase 1: uint2 cand[TOPK_SEG_CAP]; finish: u64 list
-    __shared__ u32 bm[TOPK_SEG / 32];
-    __shared__ BlockScratch scr;
-    __shared__ u32 s_wthr[TOPK_BLOCK / WAVE];
-    __shared__ int s_count, s_last, s_n;
-
-    const int tid = threadIdx.x;
-    const int S = a.S;
-    const int row = blockIdx.x / S, seg = blockIdx.x % S;
-    const int V = a.V;
-    const float *x = a.logits + (long long)row * a.row_stride;
-    const int base = seg * TOPK_SEG;
-    const bool vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
-    uint2 *cand = reinterpret_cast<uint2 *>(lds);
-
-    // ---- one pass over the segment: 8 x 128-bit loads per thread, kept in registers
-    float v[TOPK_F4][4];
-#pragma unroll
-    for (int i = 0; i < TOPK_F4; i++) {
-        int j = base + (i * TOPK_BLOCK + tid) * 4;
-        if (vec && j + 3 < V) {
-            float4 f = *reinterpret_cast<const float4 *>(x + j);
-            v[i][0] = f.x; v[i][1] = f.y; v[i][2] = f.z; v[i][3] = f.w;
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; c++) v[i][c] = (j + c < V) ? x[j + c] : -INFINITY;
-        }
-    }
-    float lm = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < TOPK_F4; i++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) lm = fmaxf(lm, v[i][c]);       // fmaxf drops NaN
-
-    // ---- threshold: every wave's a-th largest lane maximum has >= a logits at or above it, so the
-    // minimum over the 4 waves has >= 4a >= top_k of this segment's logits at or above it.
-    const int k = a.top_k;
-    const int aw = (k + 3) >> 2;
-    u32 wk = wave_kth_largest(ordkey(lm), aw);
-    if (tid == 0) s_count = 0;
-    if (lane_id() == 0) s_wthr[wave_id()] = wk;
-    const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
-    const bool has_hist = (a.rep != 1.0f) && hlen > 0;
-    if (has_hist) bm[tid] = 0;                                      // TOPK_SEG / 32 == TOPK_BLOCK words
-    __syncthreads();
-    u32 tk = min(min(s_wthr[0], s_wthr[1]), min(s_wthr[2], s_wthr[3]));
-    float thr = fmaxf(ordkey_inv(tk), -3.402823466e+38f);           // -inf and NaN are never enumerated
-
-    // ---- history tokens of this segment: mark them, and enter their penalised logit as a candidate
-    if (has_hist) {
-        const int *h = a.history + (long long)row * a.hist_stride;
-        for (int i = tid; i < hlen; i += TOPK_BLOCK) {
-            int t = h[i];
-            if (t < 0 || t >= V) {
-                atomicOr(a.status, 1);
-                continue;
-            }
-            int r = t - base;
-            if (r < 0 || r >= TOPK_SEG) continue;
-            u32 bit = 1u << (r & 31);
-            u32 old = atomicOr(&bm[r >> 5], bit);
-            if (old & bit) continue;                               // duplicates do not compound
-            float y = penalise(x[t], a.rep);
-            if (y >= thr) {
-                int pos = atomicAdd(&s_count, 1);
-                if (pos < TOPK_SEG_CAP) cand[pos] = make_uint2(__float_as_uint(y), (u32)t);
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- emit the logits at or above the threshold
-#pragma unroll
-    for (int i = 0; i < TOPK_F4; i++) {
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float xv = v[i][c];
-            if (xv >= thr) {
-                int r = (i * TOPK_BLOCK + tid) * 4 + c;
-                bool skip = has_hist && ((bm[r >> 5] >> (r & 31)) & 1u);
-                if (!skip) {
-                    int pos = atomicAdd(&s_count, 1);
-                    if (pos < TOPK_SEG_CAP) cand[pos] = make_uint2(__float_as_uint(xv), (u32)(base + r));
-                }
-            }
-        }
-    }
-    __syncthreads();
-    const int nseg = s_count;
-    {
-        uint2 *g = a.cand + (long long)blockIdx.x * TOPK_SEG_CAP;
-        for (int i = tid; i < min(nseg, TOPK_SEG_CAP); i += TOPK_BLOCK) g[i] = cand[i];
-        if (tid == 0) {
-            a.cand_count[blockIdx.x] = nseg;
-            a.seg_thr[blockIdx.x] = thr;
-        }
-    }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        unsigned int prev = atomicAdd(&a.row_arrivals[row], 1u);
-        s_last = (prev == (unsigned int)(S - 1));
-        s_n = 0;
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-
-    // ---- row finish (one workgroup per row reaches this point)
-    float t_star = -INFINITY;
-    u32 over = 0;
-    for (int s = tid; s < S; s += TOPK_BLOCK) {
-        t_star = fmaxf(t_star, load_agent(&a.seg_thr[row * S + s]));
-        over |= (load_agent(&a.cand_count[row * S + s]) > TOPK_SEG_CAP) ? 1u : 0u;
-    }
-    t_star = block_max_f32<TOPK_BLOCK>(t_star, &scr);
-    over = block_sum_u32<TOPK_BLOCK>(over, &scr);
-    // Every logit y >= t_star of the row was emitted; any other has z <= z(next_below(t_star)).
-    const u32 ztkey = ordkey(z_of(next_below(t_star), a.T));
-    u64 *list = lds;
-    for (int s = 0; s < S; s++) {
-        const int cnt = min(load_agent(&a.cand_count[row * S + s]), TOPK_SEG_CAP);
-        const u64 *g = reinterpret_cast<const u64 *>(a.cand + (long long)(row * S + s) * TOPK_SEG_CAP);
-        for (int i = tid; i < cnt; i += TOPK_BLOCK) {
-            u64 cv = load_agent(&g[i]);
-            float y = __uint_as_float((u32)(cv & 0xFFFFFFFFull));
-            int id = (int)(cv >> 32);
-            if (y >= t_star) {
-                float z = z_of(y, a.T);
-                if (ordkey(z) > ztkey) {
-                    int pos = atomicAdd(&s_n, 1);
-                    if (pos < TOPK_ROW_CAP) list[pos] = make_key64(z, id);
-                }
-            }
-        }
-    }
-    __syncthreads();
-    const int n = s_n;
-    if (over || n < k || n > TOPK_ROW_CAP) {
-        if (tid == 0) {
-            a.row_flags[row] = 1;
-            a.row_arrivals[row] = 0;
-            atomicAdd(&a.counters[1], 1ull);
-        }
-        return;
-    }
-    const int n2 = next_pow2(n);
-    for (int i = n + tid; i < n2; i += TOPK_BLOCK) list[i] = 0;
-    bitonic_sort_desc<TOPK_BLOCK>(list, n2);
-    finish_sorted<TOPK_BLOCK, 1>(list, k, a, row, &scr);
-    if (tid == 0) {
-        a.row_arrivals[row] = 0;
-        atomicAdd(&a.counters[0], 1ull);
-    }
-}
-
-hipError_t launch_sample_topk(const SampleArgs &a, hipStream_t st) {
-    hipLaunchKernelGGL(sample_topk_kernel, dim3((unsigned)(a.B * a.S)), dim3(TOPK_BLOCK), 0, st, a);
-    return hipGetLastError();
-}
 
 // ---------------------------------------------------------------------------
 // General kernel
@@ -532,7 +277,9 @@ __device__ Found wide_find(const WideCtx &c, WideHeld &held, bool by_count, u64 
     return wide_resolve(c, held.n, b, by_count, target, base_mass, base_cnt);
 }
 
-__global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, int fallback_only) {
+// try_candidates != 0: topk_collect_kernel ran before this launch; finish the row from its candidates
+// if that can be proven correct, otherwise fall through to the general algorithm.
+__global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, int try_candidates) {
     extern __shared__ u64 dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_int[8];
@@ -540,8 +287,13 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, i
 
     const int tid = threadIdx.x;
     const int row = blockIdx.x;
-    if (fallback_only) {
-        if (a.row_flags[row] == 0) return;          // uniform across the workgroup
+    if (try_candidates) {
+        if (topk_try_finish<WIDE_BLOCK>(a, row, dyn + WIDE_BINS, reinterpret_cast<u32 *>(dyn), &scr)) {
+            if (tid == 0) atomicAdd(&a.counters[0], 1ull);
+            return;
+        }
+        if (tid == 0) atomicAdd(&a.counters[1], 1ull);
+        __syncthreads();
     }
     const int V = a.V;
     WideCtx c;
@@ -659,19 +411,16 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, i
             if (a.nuc_len) a.nuc_len[row] = -1;      // the nucleus listing is only produced for small top-k
         }
     }
-    if (tid == 0) {
-        if (fallback_only) a.row_flags[row] = 0;
-        else atomicAdd(&a.counters[2], 1ull);
-    }
+    if (tid == 0 && !try_candidates) atomicAdd(&a.counters[2], 1ull);
 }
 
 size_t wide_lds_bytes(int V) {
     return sizeof(u64) * (WIDE_BINS + WIDE_LIST_CAP) + sizeof(u32) * WIDE_BINS + sizeof(u32) * (size_t)((V + 31) / 32);
 }
 
-hipError_t launch_sample_wide(const SampleArgs &a, bool fallback_only, hipStream_t st) {
+hipError_t launch_sample_wide(const SampleArgs &a, bool try_candidates, hipStream_t st) {
     hipLaunchKernelGGL(sample_wide_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a,
-                       fallback_only ? 1 : 0);
+                       try_candidates ? 1 : 0);
     return hipGetLastError();
 }
 
