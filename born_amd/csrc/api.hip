@@ -48,6 +48,7 @@ struct born_sampler {
     int path;                      // 0 = by top_k, 1 = always the general kernel, 2 = single-pass kernel alone
     // device workspace
     unsigned int *row_arrivals;
+    int *fb_count, *fb_rows;
     uint2 *cand;
     int *cand_count;
     float *seg_thr;
@@ -156,11 +157,13 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
     alloc((void **)&s->row_arrivals, rows * sizeof(unsigned int));
+    alloc((void **)&s->fb_count, sizeof(int));
+    alloc((void **)&s->fb_rows, rows * sizeof(int));
     alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
-    alloc((void **)&s->cand_count, segs * sizeof(int));
+    alloc((void **)&s->cand_count, segs * TOPK_WAVES * sizeof(int));
     alloc((void **)&s->seg_thr, segs * sizeof(float));
     alloc((void **)&s->status, sizeof(int));
-    alloc((void **)&s->counters, 4 * sizeof(unsigned long long));
+    alloc((void **)&s->counters, 64 * sizeof(unsigned long long));   // [0..2] work counters, [8..] phase stamps of debug builds
     if (e != hipSuccess) {
         born_rocm_sampler_destroy(s);
         return hip_fail(e, "workspace allocation");
@@ -171,7 +174,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->row_arrivals, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
+    void *ptrs[] = {s->row_arrivals, s->fb_count, s->fb_rows, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -212,6 +215,15 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     }
     return BORN_ROCM_OK;
 }
+
+#ifdef BORN_PHASE_TIMING
+// debug builds only: raw copy of the counter block (phase time stamps live at [8..])
+int born_rocm_debug_read_counters(born_sampler *s, void *stream, unsigned long long *out, int64_t n) {
+    HIP_TRY(hipMemcpyAsync(out, s->counters, (size_t)n * sizeof(unsigned long long), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+#endif
 
 int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
                                int64_t *general_rows) {
@@ -307,6 +319,8 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
     a.row_arrivals = s->row_arrivals;
+    a.fb_count = s->fb_count;
+    a.fb_rows = s->fb_rows;
     a.cand = s->cand;
     a.cand_count = s->cand_count;
     a.seg_thr = s->seg_thr;
@@ -320,9 +334,12 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     const bool boosts = history && a.rep < 1.0f;
     if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && !boosts) {
         HIP_TRY(launch_topk_collect(a, st));
-        // finishes each row from its candidates, or runs the general algorithm on a row that cannot be
-        // proven from them (path 2 stops after the collect kernel: for timing that kernel alone)
-        if (s->path == 0) HIP_TRY(launch_sample_wide(a, true, st));
+        // the finish proves each row from its candidates or queues it; the general kernel then walks
+        // the queue (path 2 stops after the collect kernel: for timing that kernel alone)
+        if (s->path == 0) {
+            HIP_TRY(launch_topk_finish(a, st));
+            HIP_TRY(launch_sample_wide(a, true, st));
+        }
     } else {
         HIP_TRY(launch_sample_wide(a, false, st));
     }

@@ -149,6 +149,15 @@ __device__ __forceinline__ u32 handoff_arrive(u32 *counter) {
     return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+#ifdef BORN_PHASE_TIMING
+#define BORN_STAMP(args, row, slot)                                                          \
+    do {                                                                                     \
+        if (threadIdx.x == 0 && (row) == 0) (args).counters[8 + (slot)] = wall_clock64();    \
+    } while (0)
+#else
+#define BORN_STAMP(args, row, slot) do {} while (0)
+#endif
+
 // ---- wave / block primitives --------------------------------------------------
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }
@@ -164,6 +173,74 @@ __device__ __forceinline__ u32 wave_sum_u32(u32 v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
     return v;
 }
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
+// load still in flight (its workgroup-scope fence covers global memory), which would serialise
+// a software pipeline that keeps the next tile's loads outstanding across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Cross-lane moves on the DPP path of the vector ALU (no LDS round trip).  CTRL: 0x00-0xFF
+// quad_perm, 0x110+n row_shr:n, 0x140 row_mirror, 0x141 row_half_mirror, 0x142 row_bcast:15,
+// 0x143 row_bcast:31.  Lanes without a valid source (or masked rows) receive `old`.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ u32 dpp_u32(u32 old, u32 src) {
+    return (u32)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, ROW_MASK, 0xF, false);
+}
+
+// Wave-wide maximum / minimum as a wave-uniform value: four DPP steps inside each row of 16
+// lanes, then one lane per row read back.
+__device__ __forceinline__ u32 wave_max_u32(u32 v) {
+    v = max(v, dpp_u32<0xB1>(v, v));
+    v = max(v, dpp_u32<0x4E>(v, v));
+    v = max(v, dpp_u32<0x141>(v, v));
+    v = max(v, dpp_u32<0x140>(v, v));
+    u32 a = (u32)__builtin_amdgcn_readlane((int)v, 0), b = (u32)__builtin_amdgcn_readlane((int)v, 16);
+    u32 c = (u32)__builtin_amdgcn_readlane((int)v, 32), d = (u32)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ u32 wave_min_u32(u32 v) { return ~wave_max_u32(~v); }
+
+// Inclusive prefix sum over the 64 lanes (DPP Hillis-Steele inside rows, then row broadcasts).
+__device__ __forceinline__ u32 wave_inclusive_scan_u32(u32 v) {
+    v += dpp_u32<0x111>(0u, v);
+    v += dpp_u32<0x112>(0u, v);
+    v += dpp_u32<0x114>(0u, v);
+    v += dpp_u32<0x118>(0u, v);
+    v += dpp_u32<0x142, 0xA>(0u, v);
+    v += dpp_u32<0x143, 0xC>(0u, v);
+    return v;
+}
+
+// A key t with at least `a` of the wave's 64 lane keys >= t, as large as a 4-way search between
+// the wave's minimum and maximum key can make it down to a resolution of 2^resolution_bits key
+// units (resolution_bits <= 2 gives the exact a-th largest key).  1 <= a <= 64.  Wave-uniform
+// scalar work; every step issues three independent vector compares.
+__device__ __forceinline__ u32 wave_kth_largest_bound(u32 key, int a, int resolution_bits) {
+    u32 hi = wave_max_u32(key);
+    if (a <= 1) return hi;
+    u32 lo = wave_min_u32(key);                 // all 64 keys are >= lo
+    const u32 res = max(4u, 1u << resolution_bits);
+    while (hi - lo >= res) {
+        const u32 q = (hi - lo) >> 2;            // >= 1
+        const u32 t1 = lo + q, t2 = t1 + q, t3 = t2 + q;        // lo < t1 < t2 < t3 <= hi
+        const int c1 = __popcll(__ballot(key >= t1));
+        const int c2 = __popcll(__ballot(key >= t2));
+        const int c3 = __popcll(__ballot(key >= t3));
+        if (c3 >= a) lo = t3;
+        else if (c2 >= a) { lo = t2; hi = t3 - 1u; }
+        else if (c1 >= a) { lo = t1; hi = t2 - 1u; }
+        else hi = t1 - 1u;
+    }
+    while (hi != lo && resolution_bits <= 2) {   // exact finish over the last few keys
+        const u32 mid = lo + ((hi - lo) >> 1) + 1u;
+        if (__popcll(__ballot(key >= mid)) >= a) lo = mid; else hi = mid - 1u;
+    }
+    return lo;
+}
+
 __device__ __forceinline__ u64 shfl_up_u64(u64 v, int o) {
     u32 lo = __shfl_up((u32)v, o, WAVE), hi = __shfl_up((u32)(v >> 32), o, WAVE);
     return ((u64)hi << 32) | lo;
