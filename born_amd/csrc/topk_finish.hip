@@ -3,7 +3,8 @@
 //
 // With t* = max of the row's segment thresholds, every logit >= t* of the row is among the
 // candidates, so any logit that is not has z <= z(pred(t*)).  The finish
-//   1. gathers the candidates >= t* whose unpenalised z is strictly above that bound;
+//   1. gathers the candidates >= t* whose unpenalised z is strictly above that bound (one thread
+//      per candidate sub-list, whose head it requested together with the counts);
 //   2. shrinks them by unpenalised z to about top_k with the counting argument of the collect
 //      kernel (every wave's a-th largest lane maximum, minimum over the waves = t2);
 //   3. flags the survivors that occur in the row's history (a small hash of the survivors is
@@ -26,7 +27,7 @@ constexpr int FIN_WAVES = FIN_BLOCK / WAVE;
 constexpr int FIN_CAP = 2048;                 // candidates >= t* the finish can hold
 constexpr int FIN_KEEP = 512;                 // survivors of the shrink it can hold
 constexpr int FIN_SLOTS = 2 * FIN_KEEP;       // hash slots (load factor <= 0.5)
-constexpr int FIN_GATHER = 4;                 // candidate loads in flight per thread
+constexpr int FIN_HEAD = 32;                  // entries of its sub-list a thread requests before knowing the count
 __device__ __forceinline__ u32 fin_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 static_assert(FIN_SLOTS == (1 << 10), "fin_hash produces 10 bits");
 
@@ -71,21 +72,24 @@ __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, cons
 
 __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     __shared__ uint2 A[FIN_CAP];               // (logit bits, id) of the candidates >= t*
+    __shared__ u32 Z[FIN_CAP];                 // their unpenalised z as order keys
     __shared__ uint2 Bm[FIN_KEEP];             // survivors of the shrink; .y gets the penalised flag
     __shared__ u64 K[FIN_KEEP];                // their rank keys, 0 = dropped
     __shared__ u64 sorted[WAVE];
     __shared__ u32 tab[FIN_SLOTS];
-    __shared__ int s_off[TOPK_WAVES * WAVE + 1], s_incl[TOPK_WAVES * WAVE], s_wsum[FIN_WAVES];
     __shared__ u32 s_wthr[FIN_WAVES];
+    __shared__ int s_cnt[TOPK_WAVES * WAVE];
     __shared__ int s_n, s_m, s_over, s_valid;
     __shared__ float s_tstar;
 
     const int tid = threadIdx.x, row = blockIdx.x;
     const int S = a.S, V = a.V, k = a.top_k;
-    const int nsub = S * TOPK_WAVES;           // <= 256 sub-lists (one per segment and wave)
+    const int nsub = S * TOPK_WAVES;           // <= 256 sub-lists (one per segment and wave): one per thread
+    static_assert(TOPK_WAVES * WAVE <= FIN_BLOCK, "one thread per candidate sub-list");
 
     BORN_STAMP(a, row, 0);
-    // ---- everything that does not depend on other loads is requested first
+    // ---- requested up front: the sub-list counts, the segment thresholds, the history
+    const uint2 *gr = a.cand + (long long)row * nsub * TOPK_WAVE_CAP;
     int cnt = (tid < nsub) ? a.cand_count[row * nsub + tid] : 0;
     float tseg = (tid < S) ? a.seg_thr[row * S + tid] : -INFINITY;
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
@@ -98,55 +102,64 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
         s_valid = 0;
     }
     for (int i = tid; i < FIN_SLOTS; i += FIN_BLOCK) tab[i] = 0;
-
-    BORN_STAMP(a, row, 1);
-    // ---- offsets of the sub-lists, t*
-    {
-        const int ov = cnt > TOPK_WAVE_CAP;
-        const u32 inc = wave_inclusive_scan_u32((u32)min(cnt, TOPK_WAVE_CAP));
-        s_incl[tid] = (int)inc;
-        if (lane_id() == WAVE - 1) s_wsum[wave_id()] = (int)inc;
-        __syncthreads();                        // also orders the zeroing above
-        if (__ballot(ov) != 0ull && lane_id() == 0) s_over = 1;
-        if (tid < WAVE) {                       // S <= 64
-            float t = wave_max_f32(tseg);
-            if (tid == 0) s_tstar = t;
-        }
-        int off = 0;
-        for (int w = 0; w < wave_id(); w++) off += s_wsum[w];
-        s_off[tid + 1] = s_incl[tid] + off;
-        if (tid == 0) s_off[0] = 0;
+    s_cnt[tid] = min(cnt, TOPK_WAVE_CAP);
+    if (tid < WAVE) {                           // S <= 64
+        float t = wave_max_f32(tseg);
+        if (tid == 0) s_tstar = t;
     }
     __syncthreads();
     const float t_star = s_tstar;
-    const int total = s_off[nsub];
     // Every logit y >= t_star of the row was emitted; any other has z <= z(next_below(t_star)).
     const u32 ztkey = ordkey(z_of(next_below(t_star), a.T));
-    const uint2 *gr = a.cand + (long long)row * nsub * TOPK_WAVE_CAP;
 
-    BORN_STAMP(a, row, 2);
-    // ---- 1. gather the candidates >= t* whose unpenalised z clears the bound
-    for (int i0 = 0; i0 < total; i0 += FIN_BLOCK * FIN_GATHER) {
-        uint2 cv[FIN_GATHER];
+    if (cnt > TOPK_WAVE_CAP) s_over = 1;          // (reset before the barrier above)
+    BORN_STAMP(a, row, 1);
+    // ---- 1. keep the candidates >= t* whose unpenalised z clears the bound
+    // the sub-lists in chunks of FIN_HEAD entries: FIN_HEAD consecutive threads read FIN_HEAD consecutive
+    // entries of one sub-list, every thread has all its loads in flight together, and each wave reserves
+    // its output range with one LDS atomic (one chunk is almost always enough: a wave of the collect
+    // kernel seldom emits more than FIN_HEAD logits)
+    int maxcnt = 0;
+    for (int i = 0; i < nsub; i += 1) maxcnt = max(maxcnt, s_cnt[i]);
+    constexpr int PER = 8;                      // entries per thread and round
+    for (int e0 = 0; e0 < maxcnt; e0 += FIN_HEAD) {
+        for (int base = 0; base < nsub * FIN_HEAD; base += FIN_BLOCK * PER) {
+            uint2 ent[PER];
+            bool have[PER];
 #pragma unroll
-        for (int u = 0; u < FIN_GATHER; u++) {
-            int i = i0 + u * FIN_BLOCK + tid;
-            cv[u] = make_uint2(0xFF800000u, 0u);                    // -inf: filtered below
-            if (i < total) {
-                int lo = 0, hi = nsub;                               // sub-list whose range holds i
-                while (hi - lo > 1) {
-                    int mid = (lo + hi) >> 1;
-                    if (s_off[mid] <= i) lo = mid; else hi = mid;
-                }
-                cv[u] = gr[(long long)lo * TOPK_WAVE_CAP + (i - s_off[lo])];
+            for (int u = 0; u < PER; u++) {
+                const int idx = base + u * FIN_BLOCK + tid;
+                const int sub = idx / FIN_HEAD, e = e0 + idx % FIN_HEAD;
+                have[u] = sub < nsub && e < s_cnt[sub < nsub ? sub : 0];
+                ent[u] = have[u] ? gr[(long long)sub * TOPK_WAVE_CAP + e] : make_uint2(0u, 0u);
             }
-        }
+            u32 zk[PER];
+            u32 pass = 0;
 #pragma unroll
-        for (int u = 0; u < FIN_GATHER; u++) {
-            float y = __uint_as_float(cv[u].x);
-            if (y >= t_star && ordkey(z_of(y, a.T)) > ztkey) {
-                int pos = atomicAdd(&s_n, 1);
-                if (pos < FIN_CAP) A[pos] = cv[u];
+            for (int u = 0; u < PER; u++) {
+                const float y = __uint_as_float(ent[u].x);
+                zk[u] = 0;
+                if (have[u] && y >= t_star) {
+                    zk[u] = ordkey(z_of(y, a.T));
+                    if (zk[u] > ztkey) pass |= 1u << u;
+                }
+            }
+            const u32 mine_n = (u32)__popc(pass);
+            const u32 incl = wave_inclusive_scan_u32(mine_n);
+            const u32 wave_total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
+            u32 wave_base = 0;
+            if (lane_id() == 0 && wave_total) wave_base = (u32)atomicAdd(&s_n, (int)wave_total);
+            wave_base = (u32)__builtin_amdgcn_readfirstlane((int)wave_base);
+            u32 pos = wave_base + incl - mine_n;
+#pragma unroll
+            for (int u = 0; u < PER; u++) {
+                if ((pass >> u) & 1u) {
+                    if (pos < (u32)FIN_CAP) {
+                        A[pos] = ent[u];
+                        Z[pos] = zk[u];
+                    }
+                    pos++;
+                }
             }
         }
     }
@@ -154,13 +167,12 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     const int n = s_n;
     bool ok = !s_over && n >= k && n <= FIN_CAP;
 
-    BORN_STAMP(a, row, 3);
+    BORN_STAMP(a, row, 2);
     // ---- 2. shrink by unpenalised z: t2 has at least top_k candidates at or above it
     u32 t2 = 0;
     if (ok) {
         u32 best = 0;
-        for (int i = lane_id() * FIN_WAVES + wave_id(); i < n; i += FIN_BLOCK)
-            best = max(best, ordkey(z_of(__uint_as_float(A[i].x), a.T)));
+        for (int i = lane_id() * FIN_WAVES + wave_id(); i < n; i += FIN_BLOCK) best = max(best, Z[i]);
         u32 t = wave_kth_largest_bound(best, (k + FIN_WAVES - 1) / FIN_WAVES, 8);
         if (lane_id() == 0) s_wthr[wave_id()] = t;
     }
@@ -168,10 +180,9 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     if (ok) {
         t2 = min(min(s_wthr[0], s_wthr[1]), min(s_wthr[2], s_wthr[3]));
         for (int i = tid; i < n; i += FIN_BLOCK) {
-            uint2 c = A[i];
-            if (ordkey(z_of(__uint_as_float(c.x), a.T)) >= t2) {
+            if (Z[i] >= t2) {
                 int pos = atomicAdd(&s_m, 1);
-                if (pos < FIN_KEEP) Bm[pos] = c;
+                if (pos < FIN_KEEP) Bm[pos] = A[i];
             }
         }
     }
@@ -179,7 +190,7 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     const int m = s_m;
     ok = ok && m <= FIN_KEEP;
 
-    BORN_STAMP(a, row, 4);
+    BORN_STAMP(a, row, 3);
     // ---- 3. history: flag the survivors that were already emitted, report ids out of range
     const bool penal = a.rep != 1.0f && hlen > 0;
     if (ok && penal) {
@@ -209,21 +220,24 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     }
     __syncthreads();
 
-    BORN_STAMP(a, row, 5);
+    BORN_STAMP(a, row, 4);
     // ---- 4. exact z of the survivors; the row is proven if top_k of them stay at or above t2
     if (ok) {
-        int valid = 0;
-        for (int i = tid; i < m; i += FIN_BLOCK) {
+        for (int i0 = 0; i0 < m; i0 += FIN_BLOCK) {
+            const int i = i0 + tid;
+            bool keep = false;
+            if (i < m) {
             uint2 c = Bm[i];
             float y = __uint_as_float(c.x);
             if (c.y & 0x80000000u) y = penalise(y, a.rep);
             float z = z_of(y, a.T);
             u32 zk = ordkey(z);
-            bool keep = zk >= t2 && zk > ztkey;
+            keep = zk >= t2 && zk > ztkey;
             K[i] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
-            valid += keep ? 1 : 0;
+            }
+            const int nk = __popcll(__ballot(keep));                // one uniform add per wave
+            if (lane_id() == 0 && nk) atomicAdd(&s_valid, nk);
         }
-        if (valid) atomicAdd(&s_valid, valid);
     }
     __syncthreads();
     ok = ok && s_valid >= k;
@@ -236,7 +250,7 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
         return;
     }
 
-    BORN_STAMP(a, row, 6);
+    BORN_STAMP(a, row, 5);
     // ---- rank sort: every kept key counts the keys above it (keys are unique); the top_k land in order
     for (int i = tid; i < m; i += FIN_BLOCK) {
         const u64 key = K[i];
@@ -246,11 +260,11 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
         if (r < k) sorted[r] = key;
     }
     __syncthreads();
-    BORN_STAMP(a, row, 7);
+    BORN_STAMP(a, row, 6);
     if (tid < WAVE) finish_sorted_wave(sorted, k, a, row);
-    BORN_STAMP(a, row, 8);
+    BORN_STAMP(a, row, 7);
 #ifdef BORN_PHASE_TIMING
-    if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)m; a.counters[8 + 18] = (u64)total; }
+    if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)m; a.counters[8 + 18] = 0; }
 #endif
     if (tid == 0) atomicAdd(&a.counters[0], 1ull);
 }
