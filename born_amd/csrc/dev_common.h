@@ -218,10 +218,13 @@ __device__ __forceinline__ u32 wave_inclusive_scan_u32(u32 v) {
 // the wave's minimum and maximum key can make it down to a resolution of 2^resolution_bits key
 // units (resolution_bits <= 2 gives the exact a-th largest key).  1 <= a <= 64.  Wave-uniform
 // scalar work; every step issues three independent vector compares.
-__device__ __forceinline__ u32 wave_kth_largest_bound(u32 key, int a, int resolution_bits) {
+// `floor_key` (optional) starts the search there instead of at the wave's minimum; the guarantee then only
+// holds if at least `a` keys reach floor_key (callers that verify the outcome independently may use it).
+__device__ __forceinline__ u32 wave_kth_largest_bound(u32 key, int a, int resolution_bits, u32 floor_key = 0u) {
     u32 hi = wave_max_u32(key);
     if (a <= 1) return hi;
-    u32 lo = wave_min_u32(key);                 // all 64 keys are >= lo
+    u32 lo = max(wave_min_u32(key), floor_key);   // without a floor: all 64 keys are >= lo
+    if (hi < lo) return lo;
     const u32 res = max(4u, 1u << resolution_bits);
     while (hi - lo >= res) {
         const u32 q = (hi - lo) >> 2;            // >= 1

@@ -3,15 +3,16 @@
 //
 // With t* = max of the row's segment thresholds, every logit >= t* of the row is among the
 // candidates, so any logit that is not has z <= z(pred(t*)).  The finish
-//   1. gathers the candidates >= t* whose unpenalised z is strictly above that bound (one thread
-//      per candidate sub-list, whose head it requested together with the counts);
-//   2. shrinks them by unpenalised z to about top_k with the counting argument of the collect
-//      kernel (every wave's a-th largest lane maximum, minimum over the waves = t2);
+//   1. gathers the candidates >= t* (the heads of all candidate sub-lists are requested together
+//      with their counts, so this is one round trip to memory);
+//   2. shrinks them by raw logit (z is monotone in it) to about top_k with the counting argument
+//      of the collect kernel (every wave's a-th largest lane maximum, minimum over the waves = t2);
 //   3. flags the survivors that occur in the row's history (a small hash of the survivors is
 //      probed with the history; duplicates are idempotent) and computes their exact z.  A
 //      penalty >= 1 only lowers a logit, so everything that was cut in step 1 or 2 still has
 //      z below t2 (resp. the bound);
-//   4. accepts the row if at least top_k survivors still have z >= t2 and above the bound: those
+//   4. accepts the row if at least top_k survivors still have z strictly above z(pred(t2)) and
+//      above the bound: those
 //      are then provably the row's top_k; a rank sort orders them and one wave computes the
 //      integer CDF, the top-p cut and the draw.
 // Rows that cannot be proven (candidate overflow, ties across the bound, fewer than top_k finite
@@ -27,9 +28,23 @@ constexpr int FIN_WAVES = FIN_BLOCK / WAVE;
 constexpr int FIN_CAP = 2048;                 // candidates >= t* the finish can hold
 constexpr int FIN_KEEP = 512;                 // survivors of the shrink it can hold
 constexpr int FIN_SLOTS = 2 * FIN_KEEP;       // hash slots (load factor <= 0.5)
-constexpr int FIN_HEAD = 32;                  // entries of its sub-list a thread requests before knowing the count
+constexpr int FIN_PER = 16;                   // candidate entries a thread requests per chunk (the first before it knows the counts)
 __device__ __forceinline__ u32 fin_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 static_assert(FIN_SLOTS == (1 << 10), "fin_hash produces 10 bits");
+
+// Inclusive prefix sum of one u64 (< 2^62) per lane on the DPP path: three 21-bit limbs are scanned
+// as 32-bit values (64 lanes * 2^21 < 2^32) and recombined.
+__device__ __forceinline__ u64 wave_inclusive_scan_u62(u64 q) {
+    const u32 c0 = wave_inclusive_scan_u32((u32)q & 0x1FFFFFu);
+    const u32 c1 = wave_inclusive_scan_u32((u32)(q >> 21) & 0x1FFFFFu);
+    const u32 c2 = wave_inclusive_scan_u32((u32)(q >> 42));
+    return (u64)c0 + ((u64)c1 << 21) + ((u64)c2 << 42);
+}
+__device__ __forceinline__ u64 readlane_u64(u64 v, int lane) {     // lane must be wave-uniform
+    const u32 lo = (u32)__builtin_amdgcn_readlane((int)(u32)v, lane);
+    const u32 hi = (u32)__builtin_amdgcn_readlane((int)(u32)(v >> 32), lane);
+    return ((u64)hi << 32) | lo;
+}
 
 // One wave: integer CDF over the ns <= 64 survivors in `list` (rank order), top-p cut, draw.
 __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, const SampleArgs &a, int row) {
@@ -42,14 +57,14 @@ __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, cons
         e = emass(key64_z(list[l]), m);
         q = qfix(e, mass_scale(a.mass_shift));
     }
-    const u64 cum = wave_inclusive_scan_u64(q);
-    const u64 Zk = shfl_u64(cum, WAVE - 1);
+    const u64 cum = wave_inclusive_scan_u62(q);
+    const u64 Zk = readlane_u64(cum, WAVE - 1);
     int np = ns;
     u64 Zp = Zk;
     if (a.top_p < 1.0f) {
         const u64 tp = top_p_target(a.top_p, Zk);
         np = __popcll(__ballot(l < ns && cum < tp)) + 1;
-        Zp = shfl_u64(cum, np - 1);
+        Zp = readlane_u64(cum, __builtin_amdgcn_readfirstlane(np - 1));
     }
     const u64 td = draw_target(u, Zp);
     const int pick = __popcll(__ballot(l < np && cum < td));
@@ -72,25 +87,37 @@ __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, cons
 
 __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     __shared__ uint2 A[FIN_CAP];               // (logit bits, id) of the candidates >= t*
-    __shared__ u32 Z[FIN_CAP];                 // their unpenalised z as order keys
     __shared__ uint2 Bm[FIN_KEEP];             // survivors of the shrink; .y gets the penalised flag
     __shared__ u64 K[FIN_KEEP];                // their rank keys, 0 = dropped
     __shared__ u64 sorted[WAVE];
     __shared__ u32 tab[FIN_SLOTS];
-    __shared__ u32 s_wthr[FIN_WAVES];
+    __shared__ u32 s_wthr[FIN_WAVES], s_wmax[FIN_WAVES];
     __shared__ int s_cnt[TOPK_WAVES * WAVE];
+    __shared__ int s_rank[FIN_BLOCK];
     __shared__ int s_n, s_m, s_over, s_valid;
     __shared__ float s_tstar;
 
     const int tid = threadIdx.x, row = blockIdx.x;
     const int S = a.S, V = a.V, k = a.top_k;
-    const int nsub = S * TOPK_WAVES;           // <= 256 sub-lists (one per segment and wave): one per thread
-    static_assert(TOPK_WAVES * WAVE <= FIN_BLOCK, "one thread per candidate sub-list");
+    const int nsub = S * TOPK_WAVES;           // <= 256 candidate sub-lists (one per segment and wave)
+    static_assert(TOPK_WAVES * WAVE <= FIN_BLOCK, "one thread per candidate sub-list count");
+    constexpr int PER = FIN_PER;               // entries per thread and chunk
+    // a chunk is FIN_BLOCK * PER entries dealt evenly to the row's sub-lists: `head` consecutive entries each
+    const int head = min(TOPK_WAVE_CAP, FIN_BLOCK * PER / nsub);
+    const float inv_head = 1.0f / (float)head;
 
     BORN_STAMP(a, row, 0);
-    // ---- requested up front: the sub-list counts, the segment thresholds, the history
+    // ---- one round trip: the sub-list counts, the first `head` entries of every sub-list (whatever its
+    // count turns out to be; consecutive threads read consecutive entries), the segment
+    // thresholds, the history
     const uint2 *gr = a.cand + (long long)row * nsub * TOPK_WAVE_CAP;
     int cnt = (tid < nsub) ? a.cand_count[row * nsub + tid] : 0;
+    uint2 ent[PER];
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const int idx = u * FIN_BLOCK + tid, sub = (int)(((float)idx + 0.5f) * inv_head);   // idx / head, exact here
+        ent[u] = sub < nsub ? gr[(long long)sub * TOPK_WAVE_CAP + (idx - sub * head)] : make_uint2(0u, 0u);
+    }
     float tseg = (tid < S) ? a.seg_thr[row * S + tid] : -INFINITY;
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
@@ -103,86 +130,74 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     }
     for (int i = tid; i < FIN_SLOTS; i += FIN_BLOCK) tab[i] = 0;
     s_cnt[tid] = min(cnt, TOPK_WAVE_CAP);
+    {
+        const u32 wm = wave_max_u32((u32)min(cnt, TOPK_WAVE_CAP));
+        if (lane_id() == 0) s_wmax[wave_id()] = wm;
+    }
     if (tid < WAVE) {                           // S <= 64
         float t = wave_max_f32(tseg);
         if (tid == 0) s_tstar = t;
     }
     __syncthreads();
+    if (cnt > TOPK_WAVE_CAP) s_over = 1;        // (reset before the barrier above, read after the next one)
     const float t_star = s_tstar;
+    const int maxcnt = (int)max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
     // Every logit y >= t_star of the row was emitted; any other has z <= z(next_below(t_star)).
     const u32 ztkey = ordkey(z_of(next_below(t_star), a.T));
 
-    if (cnt > TOPK_WAVE_CAP) s_over = 1;          // (reset before the barrier above)
     BORN_STAMP(a, row, 1);
-    // ---- 1. keep the candidates >= t* whose unpenalised z clears the bound
-    // the sub-lists in chunks of FIN_HEAD entries: FIN_HEAD consecutive threads read FIN_HEAD consecutive
-    // entries of one sub-list, every thread has all its loads in flight together, and each wave reserves
-    // its output range with one LDS atomic (one chunk is almost always enough: a wave of the collect
-    // kernel seldom emits more than FIN_HEAD logits)
-    int maxcnt = 0;
-    for (int i = 0; i < nsub; i += 1) maxcnt = max(maxcnt, s_cnt[i]);
-    constexpr int PER = 8;                      // entries per thread and round
-    for (int e0 = 0; e0 < maxcnt; e0 += FIN_HEAD) {
-        for (int base = 0; base < nsub * FIN_HEAD; base += FIN_BLOCK * PER) {
-            uint2 ent[PER];
-            bool have[PER];
+    // ---- 1. keep the candidates >= t*, each wave reserving its output range with one LDS atomic; track the
+    // largest logit key per lane for the shrink.  Chunks after the first are rare (a wave of the collect
+    // kernel seldom emits more than `head` logits).
+    u32 best = 0;
+    for (int e0 = 0; e0 < maxcnt; e0 += head) {
+        u32 pass = 0;
 #pragma unroll
-            for (int u = 0; u < PER; u++) {
-                const int idx = base + u * FIN_BLOCK + tid;
-                const int sub = idx / FIN_HEAD, e = e0 + idx % FIN_HEAD;
-                have[u] = sub < nsub && e < s_cnt[sub < nsub ? sub : 0];
-                ent[u] = have[u] ? gr[(long long)sub * TOPK_WAVE_CAP + e] : make_uint2(0u, 0u);
-            }
-            u32 zk[PER];
-            u32 pass = 0;
-#pragma unroll
-            for (int u = 0; u < PER; u++) {
-                const float y = __uint_as_float(ent[u].x);
-                zk[u] = 0;
-                if (have[u] && y >= t_star) {
-                    zk[u] = ordkey(z_of(y, a.T));
-                    if (zk[u] > ztkey) pass |= 1u << u;
-                }
-            }
-            const u32 mine_n = (u32)__popc(pass);
-            const u32 incl = wave_inclusive_scan_u32(mine_n);
-            const u32 wave_total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
-            u32 wave_base = 0;
-            if (lane_id() == 0 && wave_total) wave_base = (u32)atomicAdd(&s_n, (int)wave_total);
-            wave_base = (u32)__builtin_amdgcn_readfirstlane((int)wave_base);
-            u32 pos = wave_base + incl - mine_n;
-#pragma unroll
-            for (int u = 0; u < PER; u++) {
-                if ((pass >> u) & 1u) {
-                    if (pos < (u32)FIN_CAP) {
-                        A[pos] = ent[u];
-                        Z[pos] = zk[u];
-                    }
-                    pos++;
-                }
+        for (int u = 0; u < PER; u++) {
+            const int idx = u * FIN_BLOCK + tid, sub = (int)(((float)idx + 0.5f) * inv_head), e = e0 + (idx - sub * head);
+            const bool have = sub < nsub && e < s_cnt[sub < nsub ? sub : 0];
+            if (e0 > 0) ent[u] = have ? gr[(long long)sub * TOPK_WAVE_CAP + e] : make_uint2(0u, 0u);
+            if (have && __uint_as_float(ent[u].x) >= t_star) {
+                pass |= 1u << u;
+                best = max(best, ordkey(__uint_as_float(ent[u].x)));
             }
         }
+        const u32 mine_n = (u32)__popc(pass);
+        const u32 incl = wave_inclusive_scan_u32(mine_n);
+        const u32 wave_total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
+        u32 wave_base = 0;
+        if (lane_id() == 0 && wave_total) wave_base = (u32)atomicAdd(&s_n, (int)wave_total);
+        wave_base = (u32)__builtin_amdgcn_readfirstlane((int)wave_base);
+        u32 pos = wave_base + incl - mine_n;
+#pragma unroll
+        for (int u = 0; u < PER; u++) {
+            if ((pass >> u) & 1u) {
+                if (pos < (u32)FIN_CAP) A[pos] = ent[u];
+                pos++;
+            }
+        }
+    }
+    // ---- 2. shrink by the raw logit (z is monotone in it): every wave's a-th largest lane maximum has >= a
+    // candidates at or above it, so t2 = the minimum over the waves has at least top_k
+    {
+        // every candidate is >= t*, so the search starts there; whether top_k survivors remain is verified in step 4
+        u32 t = wave_kth_largest_bound(best, (k + FIN_WAVES - 1) / FIN_WAVES, 12, ordkey(t_star));
+        if (lane_id() == 0) s_wthr[wave_id()] = t;
     }
     __syncthreads();
     const int n = s_n;
     bool ok = !s_over && n >= k && n <= FIN_CAP;
-
+    const u32 t2 = min(min(s_wthr[0], s_wthr[1]), min(s_wthr[2], s_wthr[3]));
+    // A candidate that is cut here has a logit below t2, hence z <= z(next_below(t2)): survivors must end up
+    // strictly above that key and above the row bound.
+    const u32 zb = max(ztkey, ordkey(z_of(next_below(ordkey_inv(t2)), a.T)));
     BORN_STAMP(a, row, 2);
-    // ---- 2. shrink by unpenalised z: t2 has at least top_k candidates at or above it
-    u32 t2 = 0;
     if (ok) {
-        u32 best = 0;
-        for (int i = lane_id() * FIN_WAVES + wave_id(); i < n; i += FIN_BLOCK) best = max(best, Z[i]);
-        u32 t = wave_kth_largest_bound(best, (k + FIN_WAVES - 1) / FIN_WAVES, 8);
-        if (lane_id() == 0) s_wthr[wave_id()] = t;
-    }
-    __syncthreads();
-    if (ok) {
-        t2 = min(min(s_wthr[0], s_wthr[1]), min(s_wthr[2], s_wthr[3]));
         for (int i = tid; i < n; i += FIN_BLOCK) {
-            if (Z[i] >= t2) {
+            const uint2 c = A[i];
+            if (ordkey(__uint_as_float(c.x)) >= t2) {
                 int pos = atomicAdd(&s_m, 1);
-                if (pos < FIN_KEEP) Bm[pos] = A[i];
+                if (pos < FIN_KEEP) Bm[pos] = c;
             }
         }
     }
@@ -221,19 +236,18 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     __syncthreads();
 
     BORN_STAMP(a, row, 4);
-    // ---- 4. exact z of the survivors; the row is proven if top_k of them stay at or above t2
+    // ---- 4. exact z of the survivors; the row is proven if top_k of them stay strictly above the cut keys
     if (ok) {
         for (int i0 = 0; i0 < m; i0 += FIN_BLOCK) {
             const int i = i0 + tid;
             bool keep = false;
             if (i < m) {
-            uint2 c = Bm[i];
-            float y = __uint_as_float(c.x);
-            if (c.y & 0x80000000u) y = penalise(y, a.rep);
-            float z = z_of(y, a.T);
-            u32 zk = ordkey(z);
-            keep = zk >= t2 && zk > ztkey;
-            K[i] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
+                const uint2 c = Bm[i];
+                float y = __uint_as_float(c.x);
+                if (c.y & 0x80000000u) y = penalise(y, a.rep);
+                const float z = z_of(y, a.T);
+                keep = ordkey(z) > zb;
+                K[i] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
             }
             const int nk = __popcll(__ballot(keep));                // one uniform add per wave
             if (lane_id() == 0 && nk) atomicAdd(&s_valid, nk);
@@ -251,13 +265,34 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     }
 
     BORN_STAMP(a, row, 5);
-    // ---- rank sort: every kept key counts the keys above it (keys are unique); the top_k land in order
-    for (int i = tid; i < m; i += FIN_BLOCK) {
-        const u64 key = K[i];
-        if (key == 0ull) continue;
+    // ---- rank sort: every kept key counts the keys above it (keys are unique); the top_k land in order.
+    // With m <= FIN_BLOCK the comparisons of one key are split over FIN_BLOCK / mp threads.
+    if (m <= FIN_BLOCK) {
+        const int mp = next_pow2(m), parts = FIN_BLOCK / mp;
+        const int e = tid & (mp - 1), part = tid / mp;
+        const int len = (m + parts - 1) / parts;
         int r = 0;
-        for (int j = 0; j < m; j++) r += K[j] > key ? 1 : 0;
-        if (r < k) sorted[r] = key;
+        if (e < m) {
+            const u64 key = K[e];
+            const int j1 = min(m, (part + 1) * len);
+#pragma unroll 8
+            for (int j = part * len; j < j1; j++) r += K[j] > key ? 1 : 0;
+        }
+        s_rank[tid] = r;
+        __syncthreads();
+        if (tid < m && K[tid] != 0ull) {
+            int rr = 0;
+            for (int q = 0; q < parts; q++) rr += s_rank[q * mp + tid];
+            if (rr < k) sorted[rr] = K[tid];
+        }
+    } else {
+        for (int i = tid; i < m; i += FIN_BLOCK) {
+            const u64 key = K[i];
+            if (key == 0ull) continue;
+            int r = 0;
+            for (int j = 0; j < m; j++) r += K[j] > key ? 1 : 0;
+            if (r < k) sorted[r] = key;
+        }
     }
     __syncthreads();
     BORN_STAMP(a, row, 6);
