@@ -47,7 +47,6 @@ struct born_sampler {
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // 0 = by top_k, 1 = always the general kernel, 2 = single-pass kernel alone
     // device workspace
-    unsigned int *row_arrivals;
     int *fb_count, *fb_rows;
     uint2 *cand;
     int *cand_count;
@@ -156,7 +155,6 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
         if (e == hipSuccess) e = hipMalloc(p, bytes);
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
-    alloc((void **)&s->row_arrivals, rows * sizeof(unsigned int));
     alloc((void **)&s->fb_count, sizeof(int));
     alloc((void **)&s->fb_rows, rows * sizeof(int));
     alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
@@ -174,7 +172,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->row_arrivals, s->fb_count, s->fb_rows, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
+    void *ptrs[] = {s->fb_count, s->fb_rows, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -260,7 +258,7 @@ int born_rocm_argmax(born_sampler *s, const float *logits, int64_t batch, int64_
     if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: argmax: null output");
     // ARGMAX_SEG == TOPK_SEG, so the per-segment workspace of the handle fits the partials.
     HIP_TRY(launch_argmax(logits, (int)batch, (int)vocab, row_stride, tokens_out, s->seg_thr, s->cand_count,
-                          s->row_arrivals, (hipStream_t)stream));
+                          (hipStream_t)stream));
     return BORN_ROCM_OK;
 }
 
@@ -318,7 +316,6 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_ids = nucleus_ids_out;
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
-    a.row_arrivals = s->row_arrivals;
     a.fb_count = s->fb_count;
     a.fb_rows = s->fb_rows;
     a.cand = s->cand;

@@ -9,10 +9,11 @@
 namespace born {
 
 // ---------------------------------------------------------------------------
-// argmax: grid = B * S workgroups of 256 threads, each scanning 8192 logits with
-// 128-bit loads; the last workgroup of a row to arrive merges the S partials.
-// A NaN never wins (the reference's comparisons are false for it) unless it sits
-// at index 0, where the reference's loop returns 0.
+// argmax: B * S workgroups of 256 threads scan 8192 logits each with 128-bit loads and write one
+// (value, index) partial; a second, tiny launch merges the S partials of each row (a kernel
+// boundary is the cheapest correct way to pass data between workgroups on this multi-XCD part).
+// A NaN never wins (the reference's comparisons are false for it) unless it sits at index 0,
+// where the reference's loop returns 0.
 // ---------------------------------------------------------------------------
 
 struct ArgPair {
@@ -24,12 +25,25 @@ __device__ __forceinline__ ArgPair better(ArgPair a, ArgPair b) {
     if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
     return a;
 }
+__device__ __forceinline__ ArgPair wave_best(ArgPair b) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgPair t = {__shfl_xor(b.v, o, WAVE), __shfl_xor(b.i, o, WAVE)};
+        b = better(b, t);
+    }
+    return b;
+}
+// what the reference's loop returns given the best (value, lowest index) pair over the non-NaN logits
+__device__ __forceinline__ int argmax_token(ArgPair b, float x0) {
+    if (x0 != x0) return 0;                    // NaN at index 0: every later comparison is false
+    if (b.i == 0x7FFFFFFF) return 0;           // nothing ever compared greater than -inf
+    return b.i;
+}
 
-__global__ __launch_bounds__(256) void argmax_kernel(const float *__restrict__ logits, int V, long long stride, int S,
-                                                     int *__restrict__ tokens, float *part_val, int *part_idx,
-                                                     unsigned int *arrivals) {
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float *__restrict__ logits, int V, long long stride,
+                                                             int S, int *__restrict__ tokens, float *part_val,
+                                                             int *part_idx) {
     __shared__ ArgPair sh[4];
-    __shared__ int is_last;
     const int row = blockIdx.x / S, seg = blockIdx.x % S;
     const float *x = logits + (long long)row * stride;
     const int base = seg * ARGMAX_SEG;
@@ -52,52 +66,42 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float *__restrict__ l
             if (v[c] > best.v || (v[c] == best.v && j + c < best.i)) { best.v = v[c]; best.i = j + c; }
         }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        ArgPair t = {__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
-        best = better(best, t);
-    }
+    best = wave_best(best);
     if (lane_id() == 0) sh[wave_id()] = best;
     __syncthreads();
     if (threadIdx.x == 0) {
         ArgPair b = sh[0];
         for (int w = 1; w < 4; w++) b = better(b, sh[w]);
-        part_val[blockIdx.x] = b.v;
-        part_idx[blockIdx.x] = b.i;
-        __threadfence();
-        unsigned int prev = atomicAdd(&arrivals[row], 1u);
-        is_last = (prev == (unsigned int)(S - 1));
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
-    if (threadIdx.x < WAVE) {
-        ArgPair b = {-INFINITY, 0x7FFFFFFF};
-        for (int s = threadIdx.x; s < S; s += WAVE) {
-            ArgPair t = {load_agent(&part_val[row * S + s]), load_agent(&part_idx[row * S + s])};
-            b = better(b, t);
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            ArgPair t = {__shfl_xor(b.v, o, WAVE), __shfl_xor(b.i, o, WAVE)};
-            b = better(b, t);
-        }
-        if (threadIdx.x == 0) {
-            float x0 = x[0];
-            int tok = b.i;
-            if (x0 != x0) tok = 0;                 // NaN at index 0: every later comparison is false
-            if (tok == 0x7FFFFFFF) tok = 0;        // nothing ever compared greater than -inf
-            tokens[row] = tok;
-            arrivals[row] = 0;                     // ready for the next launch on this stream
+        if (S == 1) {
+            tokens[row] = argmax_token(b, x[0]);
+        } else {
+            part_val[blockIdx.x] = b.v;
+            part_idx[blockIdx.x] = b.i;
         }
     }
 }
 
+__global__ __launch_bounds__(64) void argmax_merge_kernel(const float *__restrict__ logits, long long stride, int S,
+                                                          int *__restrict__ tokens, const float *part_val,
+                                                          const int *part_idx) {
+    const int row = blockIdx.x;
+    ArgPair b = {-INFINITY, 0x7FFFFFFF};
+    for (int s = threadIdx.x; s < S; s += WAVE) {
+        ArgPair t = {part_val[row * S + s], part_idx[row * S + s]};
+        b = better(b, t);
+    }
+    b = wave_best(b);
+    if (threadIdx.x == 0) tokens[row] = argmax_token(b, logits[(long long)row * stride]);
+}
+
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
-                         int *part_idx, unsigned int *arrivals, hipStream_t st) {
+                         int *part_idx, hipStream_t st) {
     int S = (V + ARGMAX_SEG - 1) / ARGMAX_SEG;
-    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)(B * S)), dim3(256), 0, st, logits, V, stride, S, tokens,
-                       part_val, part_idx, arrivals);
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3((unsigned)(B * S)), dim3(256), 0, st, logits, V, stride, S, tokens,
+                       part_val, part_idx);
+    if (S > 1)
+        hipLaunchKernelGGL(argmax_merge_kernel, dim3((unsigned)B), dim3(64), 0, st, logits, stride, S, tokens, part_val,
+                           part_idx);
     return hipGetLastError();
 }
 

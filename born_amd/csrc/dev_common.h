@@ -107,48 +107,6 @@ __device__ __forceinline__ float prob_of(float e, u64 Zp, int S) {
     return (float)((double)e / ldexp((double)Zp, -S));
 }
 
-// Loads that must observe what other workgroups wrote before an agent-scope release
-// (per-CU vector L1 is not coherent): relaxed atomic loads at agent scope bypass it.
-__device__ __forceinline__ float load_agent(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ int load_agent(const int *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ u32 load_agent(const u32 *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ u64 load_agent(const u64 *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Matching stores: relaxed atomic stores at agent scope are written through to the agent's
-// coherence point instead of lingering in an XCD-local L2.
-__device__ __forceinline__ void store_agent(float *p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_agent(int *p, int v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_agent(u64 *p, u64 v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Hand-off between workgroups without a cache-wide fence.  A full agent-scope release/acquire
-// fence on this multi-XCD part writes back and invalidates a whole L2 and costs far more than
-// the kernel it protects.  The producer instead (1) writes its message with store_agent,
-// (2) waits for those stores to complete (workgroup-scope release = wait on the store
-// counters) and joins its workgroup at a barrier, (3) lets one thread bump the arrival counter
-// with an agent-scope atomic.  The consumer that sees the final count reads the message with
-// load_agent only.  Every access to the shared locations is an agent-scope atomic, so each is
-// coherent by itself; the completion wait orders them.
-__device__ __forceinline__ void handoff_complete_stores() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-}
-__device__ __forceinline__ u32 handoff_arrive(u32 *counter) {
-    return __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 #ifdef BORN_PHASE_TIMING
 #define BORN_STAMP(args, row, slot)                                                          \
     do {                                                                                     \

@@ -51,7 +51,6 @@ struct SampleArgs {
     float *nuc_probs;
     int nuc_cap;
     // workspace
-    unsigned int *row_arrivals;   // [B] segment arrival counters of the argmax kernel (self-resetting)
     uint2 *cand;                  // [B][S][TOPK_WAVES][TOPK_WAVE_CAP] (logit bits, id)
     int *cand_count;              // [B][S][TOPK_WAVES]
     float *seg_thr;               // [B][S]
@@ -78,7 +77,7 @@ struct SpecArgs {
 };
 
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
-                         int *part_idx, unsigned int *arrivals, hipStream_t st);
+                         int *part_idx, hipStream_t st);
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
                           hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);

@@ -359,3 +359,90 @@ def test_argument_errors_panic_like_the_go_layer(rocm):
     rocm.sample_host(s, x, np.full(4, 0.5, np.float32), h)
     with pytest.raises(rocm.BornRocmError, match="history"):
         s.Status()
+
+
+# ---------------------------------------------------------------- the benchmark configurations
+
+def test_config_c1_steps(oracle, rocm):
+    """C1: batch 1, vocab 32000, fresh logits per step; 40 of the 1000 steps against both oracle layers."""
+    from born_amd import synth
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1), max_batch=1,
+                        max_vocab=32000)
+    near = 0
+    for step in range(40):
+        w = synth.c1(step)
+        got = rocm.sample_host(s, w.logits, w.uniforms, w.history)
+        fx = oracle.sample(w.logits, w.uniforms, 0.8, 40, 0.95, 1.1, w.history, mode=oracle.MODE_FIXED)
+        tr = oracle.sample(w.logits, w.uniforms, 0.8, 40, 0.95, 1.1, w.history, mode=oracle.MODE_TRUTH)
+        assert got["tokens"][0] == fx["tokens"][0] and got["probs"][0] == fx["probs"][0], step
+        assert got["tokens"][0] == tr["tokens"][0] or tr["near"][0]
+        near += int(tr["near"][0])
+    assert near <= 2
+
+
+def test_config_c2_greedy_and_multinomial(oracle, rocm):
+    from born_amd import synth
+    w = synth.c2()
+    assert np.array_equal(_argmax(rocm, w.logits), oracle.argmax_ref(w.logits))
+    got, _, tr = _check_against_oracle(oracle, rocm, w.logits, w.uniforms)          # T=1, full vocabulary
+    assert got["counters"]["general_rows"] == 64
+    assert tr["near"].sum() <= 4
+
+
+def test_config_c3_full_batch(oracle, rocm):
+    """The benchmark configuration at full size: all 256 rows bit-exact against the fixed-point layer,
+    equal to the fp64 truth except on flagged rows, every row served by the single-pass path."""
+    from born_amd import synth
+    w = synth.c3()
+    got, _, tr = _check_against_oracle(oracle, rocm, w.logits, w.uniforms, w.temperature, w.top_k, w.top_p, w.rep,
+                                       w.history, nuc=64)
+    c = got["counters"]
+    assert c["topk_rows"] == 256 and c["fallback_rows"] == 0 and c["general_rows"] == 0
+    print(f"C3: rows flagged near a CDF step by the truth layer: {int(tr['near'].sum())} of 256, "
+          f"tokens differing from the truth layer: {int((got['tokens'] != tr['tokens']).sum())}")
+    assert tr["near"].sum() <= 3
+
+
+def test_config_c4_full(oracle, rocm):
+    from born_amd import synth
+    w = synth.c4()
+    e = w.extra
+    s = rocm.NewSampler(max_batch=64, max_vocab=32000)
+    got = rocm.verify_host(s, e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"])
+    fx = oracle.spec_verify(e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"], mode=oracle.MODE_FIXED)
+    tr = oracle.spec_verify(e["target"], e["draft"], e["draft_tokens"], e["u_acc"], e["u_res"], mode=oracle.MODE_TRUTH)
+    assert np.array_equal(got["n_accepted"], fx["n_accepted"]) and np.array_equal(got["next_token"], fx["next_token"])
+    diff = (got["n_accepted"] != tr["n_accepted"]) | (got["next_token"] != tr["next_token"])
+    assert not (diff & ~tr["near"]).any()
+    # residual CDF steps are ~3e-5 wide at this vocabulary, so a few of the 64 draws land within 1e-6 of one
+    assert tr["near"].sum() <= 8
+    print(f"C4: {int(tr['near'].sum())} of 64 sequences flagged near a boundary, {int(diff.sum())} differ from the truth layer")
+    # every sequence either accepted everything or carries a resampled token of the vocabulary
+    full = got["n_accepted"] == 5
+    assert np.all(got["next_token"][full] == -1) and np.all((got["next_token"][~full] >= 0) & (got["next_token"][~full] < 32000))
+
+
+def test_config_c5_slice_and_full_size_properties(oracle, rocm):
+    """C5 (wide nucleus, vocabulary 152064): 24 rows against the oracle; the full 1024-row batch through
+    size-independent properties (determinism, row independence, range)."""
+    from born_amd import synth
+    w = synth.c5(rows=1024)
+    B, V = w.logits.shape
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=w.temperature, TopP=w.top_p, RepetitionPenalty=w.rep),
+                        max_batch=B, max_vocab=V)
+    full = rocm.sample_host(s, w.logits, w.uniforms, w.history)
+    again = rocm.sample_host(s, w.logits, w.uniforms, w.history)
+    assert np.array_equal(full["tokens"], again["tokens"]) and np.array_equal(full["probs"], again["probs"])
+    assert full["tokens"].min() >= 0 and full["tokens"].max() < V and np.all(full["probs"] > 0)
+    sl = slice(500, 524)
+    part = rocm.sample_host(s, w.logits[sl], w.uniforms[sl], w.history[sl])
+    assert np.array_equal(part["tokens"], full["tokens"][sl])                       # rows are independent
+    fx = oracle.sample(w.logits[sl], w.uniforms[sl], w.temperature, 0, w.top_p, w.rep, w.history[sl], mode=oracle.MODE_FIXED)
+    tr = oracle.sample(w.logits[sl], w.uniforms[sl], w.temperature, 0, w.top_p, w.rep, w.history[sl], mode=oracle.MODE_TRUTH)
+    assert np.array_equal(part["tokens"], fx["tokens"])
+    assert np.array_equal(part["probs"].view(np.uint32), fx["probs"].view(np.uint32))
+    diff = part["tokens"] != tr["tokens"]
+    assert not (diff & ~tr["near"]).any()
+    assert np.allclose(part["probs"][~diff], tr["probs"][~diff], rtol=1e-5)
+    print(f"C5 slice: {int(tr['near'].sum())} of 24 rows flagged near a CDF step, {int(diff.sum())} tokens differ from the truth layer")
+    s.Status()
