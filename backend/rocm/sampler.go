@@ -1,0 +1,183 @@
+//go:build rocm && cgo
+
+// Package rocm is the MI355X (gfx950) token-sampling capability for Born: temperature, top-k, top-p and
+// repetition-penalty sampling plus the speculative-decoding accept/reject step, on logits that stay on the
+// device.  It binds the C ABI of include/born_rocm.h through cgo; every stage is specified in
+// docs/SAMPLING_SPEC.md.
+//
+// Idioms follow the reference: a plain config struct whose zero fields mean "default"
+// (internal/optim/adam.go:59-104), capability discovery by type assertion
+// (internal/nn/activation.go:8-20), panics "sampler: ..." for programmer errors and returned errors for
+// runtime failures (CONTRIBUTING.md:142-162).
+//
+// NOTE: no Go toolchain exists in the image this package was written in; it has been read, not compiled.
+// The Python mirror born_amd/sampler.py exercises the same C ABI calls in the GPU tests.
+package rocm
+
+/*
+#cgo CFLAGS: -I${SRCDIR}/../../include
+#cgo LDFLAGS: -L${SRCDIR}/../../born_amd/lib -lborn_rocm
+#include <stdlib.h>
+#include "born_rocm.h"
+*/
+import "C"
+
+import (
+	"errors"
+	"runtime"
+	"unsafe"
+)
+
+// SamplerConfig mirrors born_sampler_config.  Zero value of a field = default
+// (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off, TopK 0 = off).
+type SamplerConfig struct {
+	Temperature       float32
+	TopK              int
+	TopP              float32
+	RepetitionPenalty float32
+	Seed              int64
+}
+
+// DeviceBuffer is device memory owned by the shim (Born's RawTensor is host-only,
+// internal/tensor/raw.go:42-46).
+type DeviceBuffer struct {
+	ptr   unsafe.Pointer
+	bytes int64
+}
+
+// SamplerBackend is the capability a backend exposes for discovery by type assertion,
+// the way nn.ReLU discovers ReLUBackend (internal/nn/activation.go:41-52).
+type SamplerBackend interface {
+	NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler
+}
+
+// Sampler owns one born_sampler handle (config + stream-ordered workspace + draw counter).
+// One handle serves one stream at a time.
+type Sampler struct {
+	h                  *C.born_sampler
+	maxBatch, maxVocab int
+}
+
+func lastError() string { return C.GoString(C.born_rocm_last_error()) }
+
+// check turns a status code into the reference's error convention.
+func check(rc C.int) error {
+	switch rc {
+	case C.BORN_ROCM_OK:
+		return nil
+	case C.BORN_ROCM_ERR_ARGUMENT:
+		panic(lastError()) // programmer error: "sampler: ..."
+	default:
+		return errors.New(lastError())
+	}
+}
+
+// Alloc returns device memory; Upload/Download copy through the shim (synchronous for pageable memory).
+func Alloc(bytes int64) (DeviceBuffer, error) {
+	var p unsafe.Pointer
+	if err := check(C.born_rocm_alloc(C.int64_t(bytes), &p)); err != nil {
+		return DeviceBuffer{}, err
+	}
+	return DeviceBuffer{ptr: p, bytes: bytes}, nil
+}
+
+func (b DeviceBuffer) Free() error { return check(C.born_rocm_free(b.ptr)) }
+
+func (b DeviceBuffer) Upload(src unsafe.Pointer, bytes int64) error {
+	return check(C.born_rocm_h2d(b.ptr, src, C.int64_t(bytes), nil))
+}
+
+func (b DeviceBuffer) Download(dst unsafe.Pointer, bytes int64) error {
+	return check(C.born_rocm_d2h(dst, b.ptr, C.int64_t(bytes), nil))
+}
+
+// NewSampler fills defaults for zero fields and panics on invalid ones, like NewAdam
+// (internal/optim/adam.go:78-104).
+func NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler {
+	c := C.born_sampler_config{
+		temperature:        C.float(cfg.Temperature),
+		top_k:              C.int32_t(cfg.TopK),
+		top_p:              C.float(cfg.TopP),
+		repetition_penalty: C.float(cfg.RepetitionPenalty),
+		seed:               C.int64_t(cfg.Seed),
+	}
+	var h *C.born_sampler
+	if err := check(C.born_rocm_sampler_create(&c, C.int64_t(maxBatch), C.int64_t(maxVocab), &h)); err != nil {
+		panic("sampler: " + err.Error())
+	}
+	s := &Sampler{h: h, maxBatch: maxBatch, maxVocab: maxVocab}
+	runtime.SetFinalizer(s, func(s *Sampler) { s.Close() })
+	return s
+}
+
+func (s *Sampler) Close() {
+	if s.h != nil {
+		C.born_rocm_sampler_destroy(s.h)
+		s.h = nil
+	}
+}
+
+// Sample draws one token per row from device-resident fp32 logits [batch, vocab].
+// history is int32 [batch, histStride] (zero DeviceBuffer = none), histLen int32 [batch] (zero = all),
+// uniforms fp32 [batch] (zero = built-in stream from cfg.Seed).  Only the 4*batch bytes of token ids cross
+// PCIe.  A returned error with "device reported" means an out-of-range history id was met (and ignored).
+func (s *Sampler) Sample(logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
+	histLen DeviceBuffer, uniforms DeviceBuffer) (tokens []int32, err error) {
+	if batch <= 0 || vocab <= 0 {
+		panic("sampler: Sample: batch and vocab must be > 0")
+	}
+	out, err := Alloc(int64(4 * batch))
+	if err != nil {
+		return nil, err
+	}
+	defer out.Free()
+	if err = check(C.born_rocm_sample(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
+		(*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride), (*C.float)(uniforms.ptr),
+		(*C.int32_t)(out.ptr), nil, nil, nil, nil, 0, nil)); err != nil {
+		return nil, err
+	}
+	tokens = make([]int32, batch)
+	if err = out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil { // synchronises the stream
+		return nil, err
+	}
+	return tokens, check(C.born_rocm_sampler_status(s.h, nil))
+}
+
+// Argmax is the greedy decode: reference argmax per row (internal/nn/cross_entropy.go:241-251).
+func (s *Sampler) Argmax(logits DeviceBuffer, batch, vocab int) ([]int32, error) {
+	out, err := Alloc(int64(4 * batch))
+	if err != nil {
+		return nil, err
+	}
+	defer out.Free()
+	if err = check(C.born_rocm_argmax(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
+		(*C.int32_t)(out.ptr), nil)); err != nil {
+		return nil, err
+	}
+	tokens := make([]int32, batch)
+	return tokens, out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch))
+}
+
+// Verify runs the speculative accept/reject step: target, draft fp32 [batch, gamma, vocab]; draftTokens int32
+// [batch, gamma]; uAccept fp32 [batch, gamma]; uResidual fp32 [batch].  nextToken[b] is -1 when every draft
+// token of sequence b was accepted.
+func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
+	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
+	out, err := Alloc(int64(8 * batch))
+	if err != nil {
+		return nil, nil, err
+	}
+	defer out.Free()
+	na := (*C.int32_t)(out.ptr)
+	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
+	if err = check(C.born_rocm_spec_verify(s.h, (*C.float)(target.ptr), (*C.float)(draft.ptr), C.int64_t(batch),
+		C.int64_t(gamma), C.int64_t(vocab), (*C.int32_t)(draftTokens.ptr), (*C.float)(uAccept.ptr),
+		(*C.float)(uResidual.ptr), na, nt, nil)); err != nil {
+		return nil, nil, err
+	}
+	both := make([]int32, 2*batch)
+	if err = out.Download(unsafe.Pointer(&both[0]), int64(8*batch)); err != nil {
+		return nil, nil, err
+	}
+	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
+}

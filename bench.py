@@ -31,6 +31,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from hardware counters (not measurable from inside this
+# script): two runs `rocprofv3 --pmc FETCH_SIZE --kernel-trace -- python3 bench.py --no-cpu --steps 20
+# --warmup 5 --copy-probe` and the same with WRITE_SIZE; each counter's per-dispatch average for the
+# kernel is scaled by what the same counter reads for the --copy-probe copy of one logits buffer
+# (131 334 144 B read and written): FETCH_SIZE 64152.5 -> factor 1.99925 KiB per unit, WRITE_SIZE
+# 128256.0 -> factor 1.0.  Kernel: FETCH_SIZE 64186.0 -> 131.40 MB read, WRITE_SIZE 2840.8 -> 2.91 MB written.
+PMC_TRAFFIC_BYTES = {("C3", "topk_collect_kernel"): int(64186.0 * 1.99925 * 1024 + 2840.8 * 1024)}
+
 
 def cpu_baseline(w, seconds=12.0):
     """Times the oracle's reference-arithmetic mode (the checker, used here only as the CPU baseline)."""
@@ -60,6 +68,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--rotate", type=int, default=4,
                     help="number of distinct logits buffers cycled through, so that a step never finds its logits in a cache")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a few plain device-to-device copies of one logits buffer (a kernel of known traffic "
+                         "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; rows are independent, so more GPUs would each take a "
@@ -111,6 +122,13 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / k            # ms per step
 
+    if args.copy_probe:
+        dst = torch.empty_like(logits_all[0])
+        for i in range(5):
+            dst.copy_(logits_all[i % nrot])          # reads and writes logits.nbytes each
+        torch.cuda.synchronize()
+        del dst
+
     for _ in range(args.warmup):
         step()
     ms = timed(args.steps)
@@ -151,7 +169,9 @@ def main():
                                f"repetition_penalty={w.rep}, history {H}/row, seeded uniforms; logits resident in HBM",
                    "seed": synth.BASE_SEED, "logits_buffers_rotated": nrot, "fallback_rows_per_step": counters["fallback_rows"] / max(1, args.steps + args.warmup)},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": PMC_TRAFFIC_BYTES.get((args.config, kernel_name)),
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a copy of known size)",
+                     "algorithmic_bytes_per_launch": alg_bytes,
                      "kernel_ms": ms_kernel},
     }
     if not args.no_cpu:

@@ -6,8 +6,8 @@
 // minimum over the four waves is a threshold that at least top_k logits of the segment reach.
 // Each wave then writes the few logits of its lanes at or above the threshold as (raw logit, id)
 // pairs into its own quarter of the segment's candidate area (no cross-wave coordination), with
-// its count; the segment's threshold is stored once.  The row is finished by topk_try_finish()
-// in the next launch (topk_finish.h), which proves from the thresholds that no other logit of
+// its count; the segment's threshold is stored once.  The row is finished by topk_finish_kernel
+// in the next launch (topk_finish.hip), which proves from the thresholds that no other logit of
 // the row can be among the top_k, or hands the row to the general path.
 //
 // Two instantiations: 128-bit loads for 16-byte aligned rows, scalar loads otherwise.

@@ -177,8 +177,9 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
             }
         }
     }
-    // ---- 2. shrink by the raw logit (z is monotone in it): every wave's a-th largest lane maximum has >= a
-    // candidates at or above it, so t2 = the minimum over the waves has at least top_k
+    // ---- 2. shrink by the raw logit (z is monotone in it): t2 = the minimum over the waves of the a-th
+    // largest lane maximum, a = ceil(top_k / waves).  A lane may hold several candidates or none, so t2 is a
+    // cut that usually leaves a little more than top_k, not a guarantee
     {
         // every candidate is >= t*, so the search starts there; whether top_k survivors remain is verified in step 4
         u32 t = wave_kth_largest_bound(best, (k + FIN_WAVES - 1) / FIN_WAVES, 12, ordkey(t_star));

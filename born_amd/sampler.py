@@ -1,4 +1,4 @@
-"""Host-side mirror of the Go package `backend/rocm` (see backend/rocm/*.go and INTEGRATION.md).
+"""Host-side mirror of the Go package `backend/rocm` (backend/rocm/sampler.go).
 
 Names, argument meaning and error behaviour follow the Go layer, which in turn follows the
 reference's idioms: a plain config struct whose zero fields mean "default"

@@ -82,10 +82,10 @@ int born_rocm_sampler_status(born_sampler *s, void *stream);
 int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
                                int64_t *general_rows);
 
-/* Diagnostics: 0 = choose the kernel from top_k (default), 1 = always use the general kernel, 2 = launch the
- * single-pass top-k kernel alone (rows it flags are left undone and counted in fallback_rows: for timing that
- * kernel by itself, never for results).  Both kernels implement the same fixed-point pipeline and must return
- * identical results; tests compare them. */
+/* Diagnostics: 0 = choose the kernels from top_k (default), 1 = always use the general kernel, 2 = launch only
+ * the streaming collect kernel of the single-pass top-k path (no tokens are produced: for timing that kernel
+ * by itself, never for results).  The single-pass path and the general kernel implement the same fixed-point
+ * pipeline and must return identical results; tests compare them. */
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
 
 /* Greedy decode: index of the maximum of each row, lowest index on ties — `argmax`,

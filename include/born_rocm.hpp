@@ -1,0 +1,101 @@
+// born_rocm.hpp — header-only C++ host mirror of the Go package backend/rocm over the C ABI of
+// born_rocm.h: same names, argument meaning and error behaviour (a Go panic is a std::logic_error
+// "sampler: ...", a Go error is a std::runtime_error).  Plumbing only: device pointers in, device
+// pointers out.
+#pragma once
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "born_rocm.h"
+
+namespace born::rocm {
+
+inline void check(int rc) {
+    if (rc == BORN_ROCM_OK) return;
+    std::string msg = born_rocm_last_error();
+    if (rc == BORN_ROCM_ERR_ARGUMENT) throw std::logic_error(msg);   // programmer error
+    throw std::runtime_error(msg);                                    // runtime failure
+}
+
+// Zero value of a field = default, as AdamConfig (internal/optim/adam.go:59-63).
+struct SamplerConfig {
+    float Temperature = 0.0f;
+    int32_t TopK = 0;
+    float TopP = 0.0f;
+    float RepetitionPenalty = 0.0f;
+    int64_t Seed = 0;
+};
+
+class DeviceBuffer {
+public:
+    DeviceBuffer() = default;
+    explicit DeviceBuffer(int64_t bytes) : bytes_(bytes) { check(born_rocm_alloc(bytes, &ptr_)); }
+    DeviceBuffer(const DeviceBuffer &) = delete;
+    DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), bytes_(o.bytes_) { o.ptr_ = nullptr; }
+    ~DeviceBuffer() { if (ptr_) born_rocm_free(ptr_); }
+    void upload(const void *src, int64_t bytes, void *stream = nullptr) { check(born_rocm_h2d(ptr_, src, bytes, stream)); }
+    void download(void *dst, int64_t bytes, void *stream = nullptr) const { check(born_rocm_d2h(dst, ptr_, bytes, stream)); }
+    void *ptr() const { return ptr_; }
+    int64_t bytes() const { return bytes_; }
+
+private:
+    void *ptr_ = nullptr;
+    int64_t bytes_ = 0;
+};
+
+class Sampler {
+public:
+    Sampler(const SamplerConfig &cfg, int64_t max_batch, int64_t max_vocab) {
+        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed};
+        check(born_rocm_sampler_create(&c, max_batch, max_vocab, &h_));
+    }
+    Sampler(const Sampler &) = delete;
+    Sampler &operator=(const Sampler &) = delete;
+    ~Sampler() { born_rocm_sampler_destroy(h_); }
+
+    // One token per row from device-resident logits [batch, vocab]; only the token ids come back to the host.
+    std::vector<int32_t> Sample(const float *logits_dev, int64_t batch, int64_t vocab, const int32_t *history_dev,
+                                int64_t hist_stride, const int32_t *hist_len_dev, const float *uniforms_dev,
+                                void *stream = nullptr) {
+        DeviceBuffer out(4 * batch);
+        check(born_rocm_sample(h_, logits_dev, batch, vocab, vocab, history_dev, hist_len_dev, hist_stride, uniforms_dev,
+                               static_cast<int32_t *>(out.ptr()), nullptr, nullptr, nullptr, nullptr, 0, stream));
+        std::vector<int32_t> tokens(static_cast<size_t>(batch));
+        out.download(tokens.data(), 4 * batch, stream);
+        check(born_rocm_sampler_status(h_, stream));
+        return tokens;
+    }
+
+    std::vector<int32_t> Argmax(const float *logits_dev, int64_t batch, int64_t vocab, void *stream = nullptr) {
+        DeviceBuffer out(4 * batch);
+        check(born_rocm_argmax(h_, logits_dev, batch, vocab, vocab, static_cast<int32_t *>(out.ptr()), stream));
+        std::vector<int32_t> tokens(static_cast<size_t>(batch));
+        out.download(tokens.data(), 4 * batch, stream);
+        return tokens;
+    }
+
+    // Speculative accept/reject; next_token[b] == -1 when every draft token of sequence b was accepted.
+    void Verify(const float *target_dev, const float *draft_dev, int64_t batch, int64_t gamma, int64_t vocab,
+                const int32_t *draft_tokens_dev, const float *u_accept_dev, const float *u_residual_dev,
+                std::vector<int32_t> &n_accepted, std::vector<int32_t> &next_token, void *stream = nullptr) {
+        DeviceBuffer out(8 * batch);
+        int32_t *na = static_cast<int32_t *>(out.ptr());
+        check(born_rocm_spec_verify(h_, target_dev, draft_dev, batch, gamma, vocab, draft_tokens_dev, u_accept_dev,
+                                    u_residual_dev, na, na + batch, stream));
+        std::vector<int32_t> both(static_cast<size_t>(2 * batch));
+        out.download(both.data(), 8 * batch, stream);
+        n_accepted.assign(both.begin(), both.begin() + batch);
+        next_token.assign(both.begin() + batch, both.end());
+        check(born_rocm_sampler_status(h_, stream));
+    }
+
+    born_sampler *handle() const { return h_; }
+
+private:
+    born_sampler *h_ = nullptr;
+};
+
+}  // namespace born::rocm

@@ -95,7 +95,7 @@ def _argmax(rocm, x, stride=None):
         d = rocm.DeviceBuffer.from_numpy(x)
     t = rocm.DeviceBuffer(4 * B)
     s.Argmax(d, B, V, t, row_stride=stride)
-    s.Argmax(d, B, V, t, row_stride=stride)       # second launch: the arrival counters must have reset themselves
+    s.Argmax(d, B, V, t, row_stride=stride)       # second launch: the workspace of the first is reused
     return t.to_numpy(np.int32, (B,))
 
 
