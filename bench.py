@@ -68,10 +68,14 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--rotate", type=int, default=4,
                     help="number of distinct logits buffers cycled through, so that a step never finds its logits in a cache")
+    ap.add_argument("--path", type=int, default=0, help="kernel selection of the sampler (0 = default; 3 = segment kernel + row finish)")
+    ap.add_argument("--kernel-path", type=int, default=None, help="path that launches the dominant kernel alone (5 for path 0, 2 for path 3)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a few plain device-to-device copies of one logits buffer (a kernel of known traffic "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
+    if args.kernel_path is None:
+        args.kernel_path = 2 if args.path == 3 else 5
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; rows are independent, so more GPUs would each take a "
               "slice of the batch with no exchange. Run with --gpus 1.", file=sys.stderr)
@@ -103,6 +107,7 @@ def main():
 
     smp = S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k, TopP=w.top_p,
                                        RepetitionPenalty=w.rep), max_batch=B, max_vocab=V)
+    smp.SetPath(args.path)
     stream = torch.cuda.current_stream().cuda_stream
 
     counter = [0]
@@ -140,12 +145,12 @@ def main():
     # dominant kernel alone (finish and fallback-queue launches left out): roofline of that kernel
     single_pass = 1 <= w.top_k <= 64
     if single_pass:
-        smp.SetPath(2)
+        smp.SetPath(args.kernel_path)
         for _ in range(10):
             step()
         ms_kernel = timed(args.steps)
-        smp.SetPath(0)
-        kernel_name = "topk_collect_kernel"
+        smp.SetPath(args.path)
+        kernel_name = {5: "topk_row_kernel", 2: "topk_collect_kernel"}[args.kernel_path]
     else:
         ms_kernel = ms
         kernel_name = "sample_wide_kernel"

@@ -45,9 +45,10 @@ struct born_sampler {
     int64_t max_batch, max_vocab;
     int S_max;                     // segments per row at max_vocab
     unsigned long long step;       // draws made with the built-in uniform stream
-    int path;                      // 0 = by top_k, 1 = always the general kernel, 2 = single-pass kernel alone
+    int path;                      // see born_rocm_sampler_set_path
+    unsigned queue_epoch;          // steps that used the fallback queue: its counter alternates between two slots
     // device workspace
-    int *fb_count, *fb_rows;
+    int *fb_count, *fb_rows;       // fb_count[2]
     uint2 *cand;
     int *cand_count;
     float *seg_thr;
@@ -155,7 +156,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
         if (e == hipSuccess) e = hipMalloc(p, bytes);
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
-    alloc((void **)&s->fb_count, sizeof(int));
+    alloc((void **)&s->fb_count, 2 * sizeof(int));
     alloc((void **)&s->fb_rows, rows * sizeof(int));
     alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
     alloc((void **)&s->cand_count, segs * TOPK_WAVES * sizeof(int));
@@ -195,7 +196,7 @@ int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg
 }
 
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path) {
-    if (!s || path < 0 || path > 2) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
+    if (!s || path < 0 || path > 5) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
     s->path = path;
     return BORN_ROCM_OK;
 }
@@ -316,7 +317,8 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_ids = nucleus_ids_out;
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
-    a.fb_count = s->fb_count;
+    a.fb_count = s->fb_count + (s->queue_epoch & 1u);
+    a.fb_count_next = s->fb_count + ((s->queue_epoch + 1u) & 1u);
     a.fb_rows = s->fb_rows;
     a.cand = s->cand;
     a.cand_count = s->cand_count;
@@ -330,13 +332,18 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
     const bool boosts = history && a.rep < 1.0f;
     if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && !boosts) {
-        HIP_TRY(launch_topk_collect(a, st));
-        // the finish proves each row from its candidates or queues it; the general kernel then walks
-        // the queue (path 2 stops after the collect kernel: for timing that kernel alone)
-        if (s->path == 0) {
-            HIP_TRY(launch_topk_finish(a, st));
-            HIP_TRY(launch_sample_wide(a, true, st));
+        // Rows that a single-pass kernel cannot prove are queued; the general kernel then walks the queue.
+        // The queue counter of the next step is zeroed by this step's first kernel (the counter of this step
+        // was zeroed by the step before), so no launch is spent on clearing it.
+        const bool by_row = s->path == 0 || s->path == 4 || s->path == 5;
+        if (by_row) {
+            HIP_TRY(launch_topk_row(a, st));                       // one workgroup per row, tail included
+        } else {
+            HIP_TRY(launch_topk_collect(a, st));                   // one workgroup per 8192-logit segment ...
+            if (s->path == 3) HIP_TRY(launch_topk_finish(a, st));  // ... and one per row to finish
         }
+        if (s->path == 0 || s->path == 3 || s->path == 4) HIP_TRY(launch_sample_wide(a, true, st));
+        s->queue_epoch++;
     } else {
         HIP_TRY(launch_sample_wide(a, false, st));
     }

@@ -55,7 +55,8 @@ struct SampleArgs {
     int *cand_count;              // [B][S][TOPK_WAVES]
     float *seg_thr;               // [B][S]
     int S;                        // segments per row
-    int *fb_count;                // number of rows queued for the general kernel (reset by the collect kernel)
+    int *fb_count;                // number of rows queued for the general kernel in this step
+    int *fb_count_next;           // the counter the next step will use: zeroed by the first kernel of this step
     int *fb_rows;                 // [B] the queue
     int *status;                  // device status word
     unsigned long long *counters; // [0] top-k rows, [1] fallback rows, [2] general rows
@@ -84,6 +85,7 @@ hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
 hipError_t launch_topk_collect(const SampleArgs &a, hipStream_t st);
 hipError_t launch_topk_finish(const SampleArgs &a, hipStream_t st);
+hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st);
 hipError_t launch_sample_wide(const SampleArgs &a, bool from_queue, hipStream_t st);
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);
 size_t wide_lds_bytes(int V);

@@ -27,7 +27,10 @@ __global__ __launch_bounds__(TOPK_BLOCK) void topk_collect_kernel(SampleArgs a) 
     const int V = a.V;
     const float *x = a.logits + (long long)row * a.row_stride;
     const int base = seg * TOPK_SEG;
-    if (blockIdx.x == 0 && tid == 0) *a.fb_count = 0;              // the queue of this step starts empty
+    if (blockIdx.x == 0 && tid == 0) {
+        *a.fb_count = 0;              // the queue of this step starts empty (rows are appended by the next launch)
+        *a.fb_count_next = 0;         // and so does the queue of the next step
+    }
 
     float v[TOPK_F4][4];
 #pragma unroll

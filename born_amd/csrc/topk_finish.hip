@@ -20,6 +20,7 @@
 // fallback queue and redone by the general kernel.
 #include "dev_common.h"
 #include "kernels.h"
+#include "topk_tail.h"
 
 namespace born {
 
@@ -31,59 +32,6 @@ constexpr int FIN_SLOTS = 2 * FIN_KEEP;       // hash slots (load factor <= 0.5)
 constexpr int FIN_PER = 16;                   // candidate entries a thread requests per chunk (the first before it knows the counts)
 __device__ __forceinline__ u32 fin_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 static_assert(FIN_SLOTS == (1 << 10), "fin_hash produces 10 bits");
-
-// Inclusive prefix sum of one u64 (< 2^62) per lane on the DPP path: three 21-bit limbs are scanned
-// as 32-bit values (64 lanes * 2^21 < 2^32) and recombined.
-__device__ __forceinline__ u64 wave_inclusive_scan_u62(u64 q) {
-    const u32 c0 = wave_inclusive_scan_u32((u32)q & 0x1FFFFFu);
-    const u32 c1 = wave_inclusive_scan_u32((u32)(q >> 21) & 0x1FFFFFu);
-    const u32 c2 = wave_inclusive_scan_u32((u32)(q >> 42));
-    return (u64)c0 + ((u64)c1 << 21) + ((u64)c2 << 42);
-}
-__device__ __forceinline__ u64 readlane_u64(u64 v, int lane) {     // lane must be wave-uniform
-    const u32 lo = (u32)__builtin_amdgcn_readlane((int)(u32)v, lane);
-    const u32 hi = (u32)__builtin_amdgcn_readlane((int)(u32)(v >> 32), lane);
-    return ((u64)hi << 32) | lo;
-}
-
-// One wave: integer CDF over the ns <= 64 survivors in `list` (rank order), top-p cut, draw.
-__device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, const SampleArgs &a, int row) {
-    const int l = lane_id();
-    const float m = key64_z(list[0]);
-    const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
-    float e = 0.0f;
-    u64 q = 0;
-    if (l < ns) {
-        e = emass(key64_z(list[l]), m);
-        q = qfix(e, mass_scale(a.mass_shift));
-    }
-    const u64 cum = wave_inclusive_scan_u62(q);
-    const u64 Zk = readlane_u64(cum, WAVE - 1);
-    int np = ns;
-    u64 Zp = Zk;
-    if (a.top_p < 1.0f) {
-        const u64 tp = top_p_target(a.top_p, Zk);
-        np = __popcll(__ballot(l < ns && cum < tp)) + 1;
-        Zp = readlane_u64(cum, __builtin_amdgcn_readfirstlane(np - 1));
-    }
-    const u64 td = draw_target(u, Zp);
-    const int pick = __popcll(__ballot(l < np && cum < td));
-    if (l == pick) {
-        a.tokens[row] = key64_id(list[l]);
-        if (a.probs) a.probs[row] = prob_of(e, Zp, a.mass_shift);
-    }
-    if (a.nuc_len) {
-        if (l == 0) a.nuc_len[row] = np;
-        if (l < np && l < a.nuc_cap) {
-            a.nuc_ids[(long long)row * a.nuc_cap + l] = key64_id(list[l]);
-            a.nuc_probs[(long long)row * a.nuc_cap + l] = prob_of(e, Zp, a.mass_shift);
-        }
-        for (int i = np + l; i < a.nuc_cap; i += WAVE) {
-            a.nuc_ids[(long long)row * a.nuc_cap + i] = -1;
-            a.nuc_probs[(long long)row * a.nuc_cap + i] = 0.0f;
-        }
-    }
-}
 
 __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     __shared__ uint2 A[FIN_CAP];               // (logit bits, id) of the candidates >= t*

@@ -82,9 +82,11 @@ int born_rocm_sampler_status(born_sampler *s, void *stream);
 int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
                                int64_t *general_rows);
 
-/* Diagnostics: 0 = choose the kernels from top_k (default), 1 = always use the general kernel, 2 = launch only
- * the streaming collect kernel of the single-pass top-k path (no tokens are produced: for timing that kernel
- * by itself, never for results).  The single-pass path and the general kernel implement the same fixed-point
+/* Diagnostics.  0 = choose the kernels from the configuration (default).  1 = always the general kernel.
+ * For 1 <= top_k <= 64 two single-pass paths exist: 4 = one workgroup per row in one launch (what 0 selects),
+ * 3 = one workgroup per 8192-logit segment followed by a per-row finish.  2 and 5 launch only the streaming
+ * kernel of path 3 resp. 4 and skip the walk of the fallback queue (2 produces no tokens, 5 leaves queued rows
+ * undone): for timing those kernels by themselves, never for results.  All paths implement the same fixed-point
  * pipeline and must return identical results; tests compare them. */
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
 

@@ -148,8 +148,13 @@ def test_softmax_operators(oracle, rocm):
     assert np.max(np.abs(lg - np.log(want))) < 1e-5
 
 
-# ---------------------------------------------------------------- sampling: single-pass top-k kernel
+# ---------------------------------------------------------------- sampling: single-pass top-k kernels
+# path 0 = the default (one workgroup per row, one launch), path 3 = segment kernel + row finish
 
+TOPK_PATHS = [0, 3]
+
+
+@pytest.mark.parametrize("path", TOPK_PATHS)
 @pytest.mark.parametrize("B,V,T,k,p,rep,H", [
     (1, 32000, 0.8, 40, 0.95, 1.1, 64),          # C1 shape
     (32, 128256, 0.7, 50, 0.9, 1.15, 512),       # C3 shape, 32 rows
@@ -161,12 +166,12 @@ def test_softmax_operators(oracle, rocm):
     (4, 100, 1.0, 64, 0.9, 1.1, 10),
     (4, 3, 1.0, 2, 0.9, 1.0, 0),
 ])
-def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H):
+def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
     rng = np.random.default_rng(B * 1000003 + V)
     x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
-    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(64, max(k, 1)))
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(64, max(k, 1)), path=path)
     c = got["counters"]
     if rep < 1.0 and H:          # a boosting penalty is served by the general kernel
         assert c["general_rows"] == B
@@ -174,16 +179,18 @@ def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H):
         assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
 
 
-def test_topk_kernel_hist_len_and_strided_rows(oracle, rocm):
+@pytest.mark.parametrize("path", TOPK_PATHS)
+def test_topk_kernel_hist_len_and_strided_rows(oracle, rocm, path):
     rng = np.random.default_rng(5)
     B, V, H = 12, 5000, 40
     x = rng.standard_normal((B, V), dtype=np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
     hl = rng.integers(0, H + 1, size=B).astype(np.int32)
-    _check_against_oracle(oracle, rocm, x, u, 0.9, 20, 0.9, 1.4, hist, hl)
+    _check_against_oracle(oracle, rocm, x, u, 0.9, 20, 0.9, 1.4, hist, hl, path=path)
     # unaligned row stride (scalar load path): rows placed in a wider buffer
     s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=20, TopP=0.9), max_batch=B, max_vocab=V)
+    s.SetPath(path)
     xp = np.full((B, V + 3), 99.0, np.float32)
     xp[:, :V] = x
     d_x, d_u, d_t = rocm.DeviceBuffer.from_numpy(xp), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer(4 * B)
@@ -192,12 +199,13 @@ def test_topk_kernel_hist_len_and_strided_rows(oracle, rocm):
     assert np.array_equal(d_t.to_numpy(np.int32, (B,)), want)
 
 
-def test_topk_kernel_ties_and_special_values(oracle, rocm):
+@pytest.mark.parametrize("path", TOPK_PATHS)
+def test_topk_kernel_ties_and_special_values(oracle, rocm, path):
     rng = np.random.default_rng(6)
     B, V = 24, 20000
     xi = rng.integers(-3, 4, size=(B, V)).astype(np.float32)           # thousands of exact ties at the cut
     u = rng.random(B, dtype=np.float32)
-    got, _, _ = _check_against_oracle(oracle, rocm, xi, u, 0.7, 50, 0.9, nuc=64)
+    got, _, _ = _check_against_oracle(oracle, rocm, xi, u, 0.7, 50, 0.9, nuc=64, path=path)
     assert got["counters"]["fallback_rows"] > 0                         # ties overflow the single-pass path
     x = rng.standard_normal((B, V), dtype=np.float32)
     x[:, ::7] = -np.inf
@@ -207,16 +215,17 @@ def test_topk_kernel_ties_and_special_values(oracle, rocm):
     x[2, 17:] = -np.inf                                                 # fewer finite logits than top_k
     x[3, :] = 0.0
     x[3, 1::2] = -0.0                                                   # -0 ties with +0
-    _check_against_oracle(oracle, rocm, x, u, 1.0, 40, 0.95, nuc=64)
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 40, 0.95, nuc=64, path=path)
 
 
-def test_topk_and_general_kernels_agree(oracle, rocm):
+@pytest.mark.parametrize("path", TOPK_PATHS)
+def test_topk_and_general_kernels_agree(oracle, rocm, path):
     rng = np.random.default_rng(7)
     B, V, H = 24, 40000, 128
     x = (rng.standard_normal((B, V), dtype=np.float32) * 2).astype(np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
-    a = _run(rocm, x, u, 0.7, 50, 0.9, 1.15, hist, nuc=64, path=0)
+    a = _run(rocm, x, u, 0.7, 50, 0.9, 1.15, hist, nuc=64, path=path)
     b = _run(rocm, x, u, 0.7, 50, 0.9, 1.15, hist, nuc=64, path=1)
     assert a["counters"]["topk_rows"] == B and b["counters"]["general_rows"] == B
     for key in ("tokens", "n_nucleus", "nuc_ids"):
@@ -389,13 +398,14 @@ def test_config_c2_greedy_and_multinomial(oracle, rocm):
     assert tr["near"].sum() <= 4
 
 
-def test_config_c3_full_batch(oracle, rocm):
+@pytest.mark.parametrize("path", TOPK_PATHS)
+def test_config_c3_full_batch(oracle, rocm, path):
     """The benchmark configuration at full size: all 256 rows bit-exact against the fixed-point layer,
     equal to the fp64 truth except on flagged rows, every row served by the single-pass path."""
     from born_amd import synth
     w = synth.c3()
     got, _, tr = _check_against_oracle(oracle, rocm, w.logits, w.uniforms, w.temperature, w.top_k, w.top_p, w.rep,
-                                       w.history, nuc=64)
+                                       w.history, nuc=64, path=path)
     c = got["counters"]
     assert c["topk_rows"] == 256 and c["fallback_rows"] == 0 and c["general_rows"] == 0
     print(f"C3: rows flagged near a CDF step by the truth layer: {int(tr['near'].sum())} of 256, "
