@@ -39,42 +39,55 @@ static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// Loads one stage: ROW_U consecutive blocks of ROW_BLOCK float4 starting at block `it0`.  Blocks that
-// lie wholly inside the row take the vector path; the row's ragged end (and anything past it) is read
-// element by element with -inf fill.
+// Keys.  In the streaming loop a logit is a signed 32-bit key: positive floats keep their bits, negative
+// floats have their magnitude bits flipped, and 0x007FFFFF is added with wrap-around so that +inf becomes
+// INT_MAX and every NaN wraps to the bottom of the range, below -inf (a NaN counts as -inf, and nothing at or
+// below -inf is ever a candidate).  After the loop the sign bit is flipped to get unsigned keys.
+__device__ __forceinline__ int row_skey(float x) {
+    const int b = __float_as_int(x);
+    const u32 m = (u32)(b >> 31) >> 1;                               // 0x7FFFFFFF for negative floats
+    return (int)(((u32)b ^ m) + 0x007FFFFFu);
+}
+__device__ __forceinline__ u32 row_ukey(float x) { return (u32)row_skey(x) ^ 0x80000000u; }
+__device__ __forceinline__ float row_ukey_inv(u32 ku) {              // ku above the key of -inf
+    const u32 s = (ku ^ 0x80000000u) - 0x007FFFFFu;
+    return __uint_as_float((s & 0x80000000u) ? (s ^ 0x7FFFFFFFu) : s);
+}
+
+// One stage = ROW_U consecutive blocks of ROW_BLOCK float4.  row_load_fast: the stage lies wholly inside the
+// row (no branches, so the loads of the next stage can stay in flight while this one is folded).
+__device__ __forceinline__ void row_load_fast(f32x4 (&v)[ROW_U], const float *x, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + ((stage * ROW_U + u) * ROW_BLOCK + tid));
+}
+// row_load_any: the row's ragged end, unaligned rows, and anything past the end (-inf fill).
 template <bool VEC>
-__device__ __forceinline__ void row_load(f32x4 (&v)[ROW_U], const float *x, int V, int it0, int tid) {
-    const int n4full = V >> 2;
-    if (VEC && (it0 + ROW_U) * ROW_BLOCK <= n4full) {               // wave-uniform
+__device__ __forceinline__ void row_load_any(f32x4 (&v)[ROW_U], const float *x, int V, int stage, int tid) {
 #pragma unroll
-        for (int u = 0; u < ROW_U; u++)
-            v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + ((it0 + u) * ROW_BLOCK + tid));
-    } else {
+    for (int u = 0; u < ROW_U; u++) {
+        const int j = ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4;
+        if (VEC && j + 3 < V) {
+            v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x + j));
+        } else {
 #pragma unroll
-        for (int u = 0; u < ROW_U; u++) {
-            const int j = ((it0 + u) * ROW_BLOCK + tid) * 4;
-            if (VEC && j + 3 < V) {
-                v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x + j));
-            } else {
-#pragma unroll
-                for (int c = 0; c < 4; c++) v[u][c] = (j + c < V) ? x[j + c] : -INFINITY;
-            }
+            for (int c = 0; c < 4; c++) v[u][c] = (j + c < V) ? x[j + c] : -INFINITY;
         }
     }
 }
 
-// Folds one stage into the thread's five largest keys.  Slots past the end of the row get key 0,
-// below the key of every float.
+// Folds one stage into the thread's five largest keys (signed, slot number in the low bits).  With RAGGED,
+// slots past the end of the row get INT_MIN.
 template <bool RAGGED>
-__device__ __forceinline__ void row_fold_stage(u32 (&t)[ROW_TOP], const f32x4 (&v)[ROW_U], int V, int it0, int tid, u32 mask) {
+__device__ __forceinline__ void row_fold(int (&t)[ROW_TOP], const f32x4 (&v)[ROW_U], int V, int stage, int tid, int mask) {
 #pragma unroll
     for (int u = 0; u < ROW_U; u++) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const u32 slot = (u32)((it0 + u) * 4 + c);
-            u32 k = (ordkey(fmaxf(v[u][c], -INFINITY)) & ~mask) | slot;          // fmaxf: NaN -> -inf
-            if (RAGGED && ((it0 + u) * ROW_BLOCK + tid) * 4 + c >= V) k = 0u;
-            u32 m;
+            const int slot = (stage * ROW_U + u) * 4 + c;
+            int k = (row_skey(v[u][c]) & ~mask) | slot;
+            if (RAGGED && ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c >= V) k = (int)0x80000000;
+            int m;
             m = min(t[0], k); t[0] = max(t[0], k); k = m;
             m = min(t[1], k); t[1] = max(t[1], k); k = m;
             m = min(t[2], k); t[2] = max(t[2], k); k = m;
@@ -82,13 +95,6 @@ __device__ __forceinline__ void row_fold_stage(u32 (&t)[ROW_TOP], const f32x4 (&
             t[4] = max(t[4], k);
         }
     }
-}
-
-__device__ __forceinline__ void row_fold(u32 (&t)[ROW_TOP], const f32x4 (&v)[ROW_U], int V, int it0, int tid, u32 mask) {
-    if (((it0 + ROW_U) * ROW_BLOCK) * 4 <= V)                       // wave-uniform: no slot of this stage is past the end
-        row_fold_stage<false>(t, v, V, it0, tid, mask);
-    else
-        row_fold_stage<true>(t, v, V, it0, tid, mask);
 }
 
 template <bool VEC>
@@ -126,19 +132,47 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     tab[tid] = 0u;
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
 
-    // ---- the pass over the row: two stages of loads in flight
-    u32 t[ROW_TOP] = {0u, 0u, 0u, 0u, 0u};
+    BORN_STAMP(a, row, 0);
+    // ---- the pass over the row.  Stages that lie wholly inside the row are software-pipelined: the loads of
+    // one stage are in flight while the stage before it is folded.
+    u32 t[ROW_TOP];
     {
+        int ts[ROW_TOP];
+#pragma unroll
+        for (int i = 0; i < ROW_TOP; i++) ts[i] = (int)0x80000000;
+        const int smask = (int)mask;
+        const int nstage = (iters + ROW_U - 1) / ROW_U;
+        const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;  // stages made of whole float4 blocks inside the row
         f32x4 va[ROW_U], vb[ROW_U];
-        row_load<VEC>(va, x, V, 0, tid);
-        for (int it0 = 0; it0 < iters; it0 += 2 * ROW_U) {
-            row_load<VEC>(vb, x, V, it0 + ROW_U, tid);
-            row_fold(t, va, V, it0, tid, mask);
-            row_load<VEC>(va, x, V, it0 + 2 * ROW_U, tid);
-            row_fold(t, vb, V, it0 + ROW_U, tid, mask);
+        int s = 0;
+        if (nfull > 0) {
+            row_load_fast(va, x, 0, tid);
+            while (s + 2 < nfull) {
+                row_load_fast(vb, x, s + 1, tid);
+                row_fold<false>(ts, va, V, s, tid, smask);
+                row_load_fast(va, x, s + 2, tid);
+                row_fold<false>(ts, vb, V, s + 1, tid, smask);
+                s += 2;
+            }
+            if (s + 1 < nfull) {
+                row_load_fast(vb, x, s + 1, tid);
+                row_fold<false>(ts, va, V, s, tid, smask);
+                row_fold<false>(ts, vb, V, s + 1, tid, smask);
+                s += 2;
+            } else {
+                row_fold<false>(ts, va, V, s, tid, smask);
+                s += 1;
+            }
         }
+        for (; s < nstage; s++) {
+            row_load_any<VEC>(va, x, V, s, tid);
+            row_fold<true>(ts, va, V, s, tid, smask);
+        }
+#pragma unroll
+        for (int i = 0; i < ROW_TOP; i++) t[i] = (u32)ts[i] ^ 0x80000000u;   // unsigned keys from here on
     }
 
+    BORN_STAMP(a, row, 1);
     // ---- T0: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
     // need = ceil(top_k / a)-th largest of the wave results
     const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
@@ -189,9 +223,10 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         }
     }
     __syncthreads();
+    BORN_STAMP(a, row, 2);
     const int n = s_n;
     // T0 at or below the key of -inf: fewer than top_k finite logits, or a vocabulary too small for the counting argument
-    bool ok = n >= k && n <= ROW_CAP && T0 > ordkey(-INFINITY);
+    bool ok = n >= k && n <= ROW_CAP && T0 > row_ukey(-INFINITY);
 
     // ---- exact logits back by id; hash of the ids; T1 by counting
     float y = 0.0f;
@@ -213,6 +248,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         if (gt < want && want <= ge) s_t1 = mykey;                   // equal values from equal keys only
     }
     __syncthreads();
+    BORN_STAMP(a, row, 3);
     const u32 T1 = s_t1;                                             // T0 <= T1, truncated
     if (ok && t[ROW_TOP - 1] >= T1) s_sat = 1;                       // this thread may hide a sixth logit >= T1
     // history: flag the candidates that were already emitted, report ids out of range
@@ -236,12 +272,13 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         }
     }
     __syncthreads();
+    BORN_STAMP(a, row, 4);
     ok = ok && !s_sat;
 
     // ---- exact z; the row is proven if top_k candidates stay strictly above the bound.  A logit outside the
     // candidates >= T1 has a key of at most T1 - 1.
     if (ok) {
-        const u32 zb = ordkey(z_of(ordkey_inv(T1 - 1u), a.T));
+        const u32 zb = ordkey(z_of(row_ukey_inv(T1 - 1u), a.T));
         bool keep = false;
         if (tid < n) {
             float yy = y;
@@ -254,6 +291,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         if (lane_id() == 0 && nk) atomicAdd(&s_valid, nk);
     }
     __syncthreads();
+    BORN_STAMP(a, row, 5);
     ok = ok && s_valid >= k;
     if (!ok) {
         if (tid == 0) {
@@ -286,7 +324,12 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         }
     }
     __syncthreads();
+    BORN_STAMP(a, row, 6);
     if (tid < WAVE) finish_sorted_wave(sorted, k, a, row);
+    BORN_STAMP(a, row, 7);
+#ifdef BORN_PHASE_TIMING
+    if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }
+#endif
     if (tid == 0) atomicAdd(&a.counters[0], 1ull);
 }
 
