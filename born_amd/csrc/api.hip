@@ -162,7 +162,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     alloc((void **)&s->cand_count, segs * TOPK_WAVES * sizeof(int));
     alloc((void **)&s->seg_thr, segs * sizeof(float));
     alloc((void **)&s->status, sizeof(int));
-    alloc((void **)&s->counters, 64 * sizeof(unsigned long long));   // [0..2] work counters, [8..] phase stamps of debug builds
+    alloc((void **)&s->counters, (64 + 8 * rows) * sizeof(unsigned long long));   // [0..2] work counters; debug builds: [8..] phase stamps, [64..] per-row stamps
     if (e != hipSuccess) {
         born_rocm_sampler_destroy(s);
         return hip_fail(e, "workspace allocation");

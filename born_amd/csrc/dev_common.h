@@ -111,6 +111,7 @@ __device__ __forceinline__ float prob_of(float e, u64 Zp, int S) {
 #define BORN_STAMP(args, row, slot)                                                          \
     do {                                                                                     \
         if (threadIdx.x == 0 && (row) == 0) (args).counters[8 + (slot)] = wall_clock64();    \
+        if (threadIdx.x == 0) (args).counters[64 + 8 * (row) + (slot)] = wall_clock64();     \
     } while (0)
 #else
 #define BORN_STAMP(args, row, slot) do {} while (0)

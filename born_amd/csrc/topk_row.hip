@@ -1,25 +1,25 @@
 // One-launch sampler for 1 <= top_k <= 64 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
 // of 1024 threads per row.
 //
-// The row is streamed from HBM once with 128-bit non-temporal loads, two stages of loads in flight
-// per thread.  Every thread keeps the five largest of its logits as 32-bit keys: the order-
-// preserving key of the logit with its low bits replaced by the logit's slot number within the
-// thread, so that the id travels with the key through a branch-free min/max network.  With
-// b = number of replaced bits, "truncated key" below means the key with those bits cleared.
+// The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 logits, the
+// loads of one stage in flight while the stage before it is examined.
 //
-//   T0  a truncated key that at least top_k logits of the row reach: every wave takes the a-th
-//       largest of its lane maxima; the w-th largest of the wave results has >= w * a >= top_k.
-//   C   all kept keys >= T0 (about 2-3 top_k), compacted into LDS; their exact logits are read
-//       back by id (the keys lost b bits) while the ids are hashed and probed with the history.
-//   T1  the truncated key of the (top_k + 16)-th largest candidate.  If no thread's fifth key
-//       reaches T1, every logit of the row with truncated key >= T1 is in C; any other logit is
-//       below the float of T1, and so is its z after a penalty (repetition_penalty >= 1 only
-//       lowers a logit) and the monotone division by the temperature.
-//   The row is proven if top_k candidates end up with z strictly above that bound; a rank sort
-//   orders them and one wave computes the integer CDF, the top-p cut and the draw.
-// Rows that cannot be proven (a thread with more than five candidates, fewer than top_k finite
-// logits, heavy ties, penalised tokens dropping below the bound) are appended to the fallback
-// queue, which the general kernel walks in the next launch.
+//   Tw  From the first stage alone: every wave takes the a-th largest of its lane maxima, and the
+//       w-th largest of the wave results has >= w * a >= top_k logits of that stage at or above
+//       it.  So the row's top_k-th largest logit is >= Tw, and only logits >= Tw matter.
+//   L   Every logit >= Tw of the whole row (the first stage included) is appended, exact value
+//       and id, to the list of the wave that met it (ballot + lane rank, no atomics): one
+//       compare per logit in the common case.
+//   T2  Same counting argument over the lists: >= top_k + 16 candidates reach T2 >= Tw.  The
+//       candidates >= T2 (about 2 top_k) are compacted into C.
+//   Any logit outside C is below T2, and so is its z after a penalty (repetition_penalty >= 1
+//   only lowers a logit) and the monotone division by the temperature.  The ids in C are hashed
+//   and probed with the history; the row is proven if top_k candidates end up with z strictly
+//   above that bound.  A rank sort orders them and one wave computes the integer CDF, the top-p
+//   cut and the draw.
+// Rows that cannot be proven (fewer than top_k finite logits, heavy ties, list overflow, penalised
+// tokens dropping below the bound) are appended to the fallback queue, which the general kernel
+// walks in the next launch.
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
@@ -29,33 +29,19 @@ namespace born {
 constexpr int ROW_BLOCK = 1024;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
 constexpr int ROW_U = 4;                      // 128-bit loads per thread and stage
-constexpr int ROW_TOP = 5;                    // keys kept per thread
-constexpr int ROW_CAP = 512;                  // candidates the tail can hold
+constexpr int ROW_WCAP = 256;                 // list entries per wave
+constexpr int ROW_CAP = 512;                  // candidates >= T2 the tail can hold
 constexpr int ROW_SLOTS = 1024;               // hash slots (load factor <= 0.5)
 constexpr int ROW_MARGIN = 16;                // candidates kept beyond top_k
 __device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
 static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
+static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// Keys.  In the streaming loop a logit is a signed 32-bit key: positive floats keep their bits, negative
-// floats have their magnitude bits flipped, and 0x007FFFFF is added with wrap-around so that +inf becomes
-// INT_MAX and every NaN wraps to the bottom of the range, below -inf (a NaN counts as -inf, and nothing at or
-// below -inf is ever a candidate).  After the loop the sign bit is flipped to get unsigned keys.
-__device__ __forceinline__ int row_skey(float x) {
-    const int b = __float_as_int(x);
-    const u32 m = (u32)(b >> 31) >> 1;                               // 0x7FFFFFFF for negative floats
-    return (int)(((u32)b ^ m) + 0x007FFFFFu);
-}
-__device__ __forceinline__ u32 row_ukey(float x) { return (u32)row_skey(x) ^ 0x80000000u; }
-__device__ __forceinline__ float row_ukey_inv(u32 ku) {              // ku above the key of -inf
-    const u32 s = (ku ^ 0x80000000u) - 0x007FFFFFu;
-    return __uint_as_float((s & 0x80000000u) ? (s ^ 0x7FFFFFFFu) : s);
-}
-
 // One stage = ROW_U consecutive blocks of ROW_BLOCK float4.  row_load_fast: the stage lies wholly inside the
-// row (no branches, so the loads of the next stage can stay in flight while this one is folded).
+// row (no branches, so the loads of the next stage can stay in flight while this one is examined).
 __device__ __forceinline__ void row_load_fast(f32x4 (&v)[ROW_U], const float *x, int stage, int tid) {
 #pragma unroll
     for (int u = 0; u < ROW_U; u++)
@@ -76,37 +62,50 @@ __device__ __forceinline__ void row_load_any(f32x4 (&v)[ROW_U], const float *x, 
     }
 }
 
-// Folds one stage into the thread's five largest keys (signed, slot number in the low bits).  With RAGGED,
-// slots past the end of the row get INT_MIN.
-template <bool RAGGED>
-__device__ __forceinline__ void row_fold(int (&t)[ROW_TOP], const f32x4 (&v)[ROW_U], int V, int stage, int tid, int mask) {
+// Appends the logits >= tw of one stage to the wave's list.  tw >= -FLT_MAX, so -inf (the fill past the end of
+// the row included) and NaN never pass.  `count` is wave-uniform.
+__device__ __forceinline__ void row_filter(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid) {
 #pragma unroll
     for (int u = 0; u < ROW_U; u++) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const int slot = (stage * ROW_U + u) * 4 + c;
-            int k = (row_skey(v[u][c]) & ~mask) | slot;
-            if (RAGGED && ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c >= V) k = (int)0x80000000;
-            int m;
-            m = min(t[0], k); t[0] = max(t[0], k); k = m;
-            m = min(t[1], k); t[1] = max(t[1], k); k = m;
-            m = min(t[2], k); t[2] = max(t[2], k); k = m;
-            m = min(t[3], k); t[3] = max(t[3], k); k = m;
-            t[4] = max(t[4], k);
+            const float xv = v[u][c];
+            const bool pass = xv >= tw;
+            const u64 m = __ballot(pass);
+            if (m) {                                                 // wave-uniform
+                if (pass) {
+                    const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+                    if (pos < (u32)ROW_WCAP)
+                        list[pos] = make_uint2(__float_as_uint(xv), (u32)(((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c));
+                }
+                count += (u32)__popcll(m);
+            }
         }
     }
 }
 
+// The need-th largest of the 16 wave results in `wthr` (LDS), computed redundantly by every wave in its first
+// 16 lanes; 0 if fewer than `need` results are non-zero.
+__device__ __forceinline__ u32 row_pick(const u32 *wthr, int need) {
+    const int l = lane_id();
+    const u32 mine = l < ROW_WAVES ? wthr[l] : 0u;
+    int ge = 0;
+#pragma unroll
+    for (int w = 0; w < ROW_WAVES; w++) ge += (wthr[w] >= mine) ? 1 : 0;
+    // a value that at least `need` results reach; the largest such value is the need-th largest
+    return wave_max_u32((l < ROW_WAVES && ge >= need) ? mine : 0u);
+}
+
 template <bool VEC>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
-    __shared__ uint2 C[ROW_CAP];               // (packed key, id); .y bit 31 = id occurs in the history
-    __shared__ u64 K[ROW_CAP];                 // rank keys of the candidates, 0 = dropped
+    __shared__ uint2 L[ROW_WAVES][ROW_WCAP];   // per-wave lists of (logit bits, id) >= Tw
+    __shared__ uint2 C[ROW_CAP];               // candidates >= T2; .y bit 31 = id occurs in the history
+    __shared__ u64 K[ROW_CAP];                 // their rank keys, 0 = dropped
     __shared__ u64 sorted[WAVE];
     __shared__ u32 tab[ROW_SLOTS];
     __shared__ int s_rank[ROW_BLOCK];
-    __shared__ u32 s_wthr[ROW_WAVES];
-    __shared__ u32 s_t1;
-    __shared__ int s_n, s_valid, s_sat;
+    __shared__ u32 s_wthr[ROW_WAVES], s_wthr2[ROW_WAVES];
+    __shared__ int s_n, s_valid, s_over;
 
     const int tid = threadIdx.x, row = blockIdx.x;
     const int V = a.V, k = a.top_k;
@@ -115,8 +114,8 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
 
     const int n4 = (V + 3) >> 2;
     const int iters = (n4 + ROW_BLOCK - 1) / ROW_BLOCK;             // float4 blocks per thread
-    const int idx_bits = 32 - __clz(iters * 4 - 1);                 // slot numbers are < iters * 4
-    const u32 mask = (1u << idx_bits) - 1u;
+    const int nstage = (iters + ROW_U - 1) / ROW_U;
+    const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;      // stages made of whole float4 blocks inside the row
 
     // the history is requested first and used last
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
@@ -126,98 +125,99 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     if (tid == 0) {
         s_n = 0;
         s_valid = 0;
-        s_sat = 0;
-        s_t1 = 0u;
+        s_over = 0;
     }
     tab[tid] = 0u;
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
 
     BORN_STAMP(a, row, 0);
-    // ---- the pass over the row.  Stages that lie wholly inside the row are software-pipelined: the loads of
-    // one stage are in flight while the stage before it is folded.
-    u32 t[ROW_TOP];
-    {
-        int ts[ROW_TOP];
-#pragma unroll
-        for (int i = 0; i < ROW_TOP; i++) ts[i] = (int)0x80000000;
-        const int smask = (int)mask;
-        const int nstage = (iters + ROW_U - 1) / ROW_U;
-        const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;  // stages made of whole float4 blocks inside the row
-        f32x4 va[ROW_U], vb[ROW_U];
-        int s = 0;
-        if (nfull > 0) {
-            row_load_fast(va, x, 0, tid);
-            while (s + 2 < nfull) {
-                row_load_fast(vb, x, s + 1, tid);
-                row_fold<false>(ts, va, V, s, tid, smask);
-                row_load_fast(va, x, s + 2, tid);
-                row_fold<false>(ts, vb, V, s + 1, tid, smask);
-                s += 2;
-            }
-            if (s + 1 < nfull) {
-                row_load_fast(vb, x, s + 1, tid);
-                row_fold<false>(ts, va, V, s, tid, smask);
-                row_fold<false>(ts, vb, V, s + 1, tid, smask);
-                s += 2;
-            } else {
-                row_fold<false>(ts, va, V, s, tid, smask);
-                s += 1;
-            }
-        }
-        for (; s < nstage; s++) {
-            row_load_any<VEC>(va, x, V, s, tid);
-            row_fold<true>(ts, va, V, s, tid, smask);
-        }
-#pragma unroll
-        for (int i = 0; i < ROW_TOP; i++) t[i] = (u32)ts[i] ^ 0x80000000u;   // unsigned keys from here on
-    }
+    f32x4 va[ROW_U], vb[ROW_U];
+    if (nfull > 0) row_load_fast(va, x, 0, tid); else row_load_any<VEC>(va, x, V, 0, tid);
+    if (nfull > 1) row_load_fast(vb, x, 1, tid);                     // in flight during the search for Tw
 
-    BORN_STAMP(a, row, 1);
-    // ---- T0: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
+    // ---- Tw from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
     // need = ceil(top_k / a)-th largest of the wave results
     const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
     const int aw = (k + act - 1) / act;                              // <= 64 as top_k <= 64
     const int need = (k + aw - 1) / aw;                              // <= act
     {
-        const u32 wk = wave_kth_largest_bound(t[0], aw, 12);
+        float lm = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
+        const u32 wk = wave_kth_largest_bound(ordkey(lm), aw, 10);
         if (lane_id() == 0) s_wthr[wave_id()] = wk;
     }
-    __syncthreads();
-    u32 T0;
-    {
-        // every wave ranks the 16 wave results in its first 16 lanes
-        const int l = lane_id();
-        const u32 mine = l < ROW_WAVES ? s_wthr[l] : 0u;
-        int ge = 0;
-#pragma unroll
-        for (int w = 0; w < ROW_WAVES; w++) ge += (s_wthr[w] >= mine) ? 1 : 0;
-        // the need-th largest: the smallest value that at least `need` results reach
-        const u64 okm = __ballot(l < ROW_WAVES && ge >= need);
-        // among the lanes with ge >= need take the largest value
-        const u32 cand = (l < ROW_WAVES && ge >= need) ? mine : 0u;
-        T0 = okm ? wave_max_u32(cand) : 0u;
-        T0 &= ~mask;
-    }
-    // every logit of the row whose truncated key is >= T0 sits in some thread's five keys, unless that thread
-    // has more than five of them (judged against T1 below)
+    lds_barrier();
+    const u32 twkey = row_pick(s_wthr, need);
+    // at or below the key of -inf: fewer than top_k finite logits in the first stage (or a vocabulary too small
+    // for the counting argument); nothing is listed and the row goes to the general kernel
+    const bool have_tw = twkey > ordkey(-INFINITY);
+    const float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
 
-    // ---- C: compact the kept keys >= T0 (a wave reserves its range with one LDS atomic)
+    // ---- the pass over the row
+    uint2 *list = L[wave_id()];
+    u32 count = 0;
+    {
+        int s = 0;
+        if (nfull > 1) {
+            // at the loop head va = stage s and vb = stage s + 1 are both requested
+            while (s + 3 < nfull) {
+                row_filter(va, tw, list, count, s, tid);
+                row_load_fast(va, x, s + 2, tid);
+                row_filter(vb, tw, list, count, s + 1, tid);
+                row_load_fast(vb, x, s + 3, tid);
+                s += 2;
+            }
+            const bool three = s + 2 < nfull;                        // two or three whole stages remain
+            row_filter(va, tw, list, count, s, tid);
+            if (three) row_load_fast(va, x, s + 2, tid);
+            row_filter(vb, tw, list, count, s + 1, tid);
+            if (three) row_filter(va, tw, list, count, s + 2, tid);
+            s = nfull;
+        } else {
+            row_filter(va, tw, list, count, 0, tid);                 // the first stage, whole or ragged
+            s = 1;
+        }
+        for (; s < nstage; s++) {
+            row_load_any<VEC>(va, x, V, s, tid);
+            row_filter(va, tw, list, count, s, tid);
+        }
+    }
+    if (count > (u32)ROW_WCAP && lane_id() == 0) s_over = 1;
+    const int cw = (int)min(count, (u32)ROW_WCAP);
+
+    BORN_STAMP(a, row, 1);
+    // ---- T2 over the lists: a2 lanes per wave, need2-th largest of the wave results.  A wave with fewer than
+    // a2 lanes holding a candidate reports 0.
+    const int want = k + ROW_MARGIN;
+    const int a2 = (want + ROW_WAVES - 1) / ROW_WAVES;
+    const int need2 = (want + a2 - 1) / a2;
+    {
+        u32 best = 0u;
+        for (int e = lane_id(); e < cw; e += WAVE) best = max(best, ordkey(__uint_as_float(list[e].x)));
+        const int lanes = __popcll(__ballot(best != 0u));            // every entry is >= tw
+        const u32 wk = lanes >= a2 ? wave_kth_largest_bound(best, a2, 10, twkey) : 0u;
+        if (lane_id() == 0) s_wthr2[wave_id()] = wk;
+    }
+    __syncthreads();
+    const u32 t2key = max(twkey, row_pick(s_wthr2, need2));         // at least top_k logits reach it either way
+
+    // ---- C: compact the list entries >= T2 (a wave reserves its range with one LDS atomic)
     {
         int cnt = 0;
-#pragma unroll
-        for (int i = 0; i < ROW_TOP; i++) cnt += (t[i] >= T0 && t[i] != 0u) ? 1 : 0;
+        for (int e = lane_id(); e < cw; e += WAVE) cnt += ordkey(__uint_as_float(list[e].x)) >= t2key ? 1 : 0;
         const u32 incl = wave_inclusive_scan_u32((u32)cnt);
         const u32 total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
         u32 base = 0;
         if (lane_id() == 0 && total) base = (u32)atomicAdd(&s_n, (int)total);
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
         u32 pos = base + incl - (u32)cnt;
-#pragma unroll
-        for (int i = 0; i < ROW_TOP; i++) {
-            if (i < cnt) {                                           // the keys are in descending order
-                const u32 slot = t[i] & mask;
-                const u32 id = (((slot >> 2) * ROW_BLOCK + (u32)tid) << 2) + (slot & 3u);
-                if (pos < (u32)ROW_CAP) C[pos] = make_uint2(t[i], id);
+        for (int e = lane_id(); e < cw; e += WAVE) {
+            const uint2 c = list[e];
+            if (ordkey(__uint_as_float(c.x)) >= t2key) {
+                if (pos < (u32)ROW_CAP) C[pos] = c;
                 pos++;
             }
         }
@@ -225,32 +225,15 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     __syncthreads();
     BORN_STAMP(a, row, 2);
     const int n = s_n;
-    // T0 at or below the key of -inf: fewer than top_k finite logits, or a vocabulary too small for the counting argument
-    bool ok = n >= k && n <= ROW_CAP && T0 > row_ukey(-INFINITY);
+    bool ok = have_tw && !s_over && n >= k && n <= ROW_CAP;
 
-    // ---- exact logits back by id; hash of the ids; T1 by counting
-    float y = 0.0f;
-    u32 mykey = 0u, myid = 0u;
+    // ---- hash of the candidate ids
     if (ok && tid < n) {
-        const uint2 c = C[tid];
-        mykey = c.x & ~mask;
-        myid = c.y;
-        y = x[myid];
-        u32 slot = row_hash(myid);
+        u32 slot = row_hash(C[tid].y);
         while (atomicCAS(&tab[slot], 0u, (u32)(tid + 1)) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
-        const int want = min(n, k + ROW_MARGIN);
-        int gt = 0, ge = 0;
-        for (int j = 0; j < n; j++) {
-            const u32 o = C[j].x & ~mask;
-            gt += o > mykey ? 1 : 0;
-            ge += o >= mykey ? 1 : 0;
-        }
-        if (gt < want && want <= ge) s_t1 = mykey;                   // equal values from equal keys only
     }
     __syncthreads();
     BORN_STAMP(a, row, 3);
-    const u32 T1 = s_t1;                                             // T0 <= T1, truncated
-    if (ok && t[ROW_TOP - 1] >= T1) s_sat = 1;                       // this thread may hide a sixth logit >= T1
     // history: flag the candidates that were already emitted, report ids out of range
     const bool penal = a.rep != 1.0f && hlen > 0;
     for (int i = tid; i < hlen; i += ROW_BLOCK) {
@@ -273,19 +256,19 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     }
     __syncthreads();
     BORN_STAMP(a, row, 4);
-    ok = ok && !s_sat;
 
-    // ---- exact z; the row is proven if top_k candidates stay strictly above the bound.  A logit outside the
-    // candidates >= T1 has a key of at most T1 - 1.
+    // ---- exact z; the row is proven if top_k candidates stay strictly above the bound.  A logit outside C has
+    // a key of at most T2 - 1 (T2 > the key of -inf, so that is the key of a float or of -inf).
     if (ok) {
-        const u32 zb = ordkey(z_of(row_ukey_inv(T1 - 1u), a.T));
+        const u32 zb = ordkey(z_of(ordkey_inv(t2key - 1u), a.T));
         bool keep = false;
         if (tid < n) {
-            float yy = y;
-            if (C[tid].y & 0x80000000u) yy = penalise(yy, a.rep);
-            const float z = z_of(yy, a.T);
-            keep = mykey >= T1 && ordkey(z) > zb;
-            K[tid] = keep ? make_key64(z, (int)myid) : 0ull;
+            const uint2 c = C[tid];
+            float y = __uint_as_float(c.x);
+            if (c.y & 0x80000000u) y = penalise(y, a.rep);
+            const float z = z_of(y, a.T);
+            keep = ordkey(z) > zb;
+            K[tid] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
         }
         const int nk = __popcll(__ballot(keep));                     // one uniform add per wave
         if (lane_id() == 0 && nk) atomicAdd(&s_valid, nk);
@@ -329,6 +312,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     BORN_STAMP(a, row, 7);
 #ifdef BORN_PHASE_TIMING
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }
+    if (lane_id() == 0) atomicAdd(&a.counters[8 + 18], (u64)count);
 #endif
     if (tid == 0) atomicAdd(&a.counters[0], 1ull);
 }
