@@ -55,6 +55,7 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     const float inv_head = 1.0f / (float)head;
 
     BORN_STAMP(a, row, 0);
+    const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
     // ---- one round trip: the sub-list counts, the first `head` entries of every sub-list (whatever its
     // count turns out to be; consecutive threads read consecutive entries), the segment
     // thresholds, the history
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(FIN_BLOCK) void topk_finish_kernel(SampleArgs a) {
     }
     __syncthreads();
     BORN_STAMP(a, row, 6);
-    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row);
+    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
     BORN_STAMP(a, row, 7);
 #ifdef BORN_PHASE_TIMING
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)m; a.counters[8 + 18] = 0; }

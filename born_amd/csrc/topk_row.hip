@@ -121,6 +121,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
+    const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
     if (tid == 0) {
         s_n = 0;
@@ -131,9 +132,10 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
 
     BORN_STAMP(a, row, 0);
-    f32x4 va[ROW_U], vb[ROW_U];
+    f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
     if (nfull > 0) row_load_fast(va, x, 0, tid); else row_load_any<VEC>(va, x, V, 0, tid);
     if (nfull > 1) row_load_fast(vb, x, 1, tid);                     // in flight during the search for Tw
+    if (nfull > 2) row_load_fast(vc, x, 2, tid);
 
     // ---- Tw from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
     // need = ceil(top_k / a)-th largest of the wave results
@@ -161,24 +163,31 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     u32 count = 0;
     {
         int s = 0;
-        if (nfull > 1) {
-            // at the loop head va = stage s and vb = stage s + 1 are both requested
-            while (s + 3 < nfull) {
+        if (nfull > 2) {
+            // at the loop head va, vb, vc = stages s, s + 1, s + 2 are requested: two stages stay in flight
+            // while one is examined
+            while (s + 5 < nfull) {
                 row_filter(va, tw, list, count, s, tid);
-                row_load_fast(va, x, s + 2, tid);
+                row_load_fast(va, x, s + 3, tid);
                 row_filter(vb, tw, list, count, s + 1, tid);
-                row_load_fast(vb, x, s + 3, tid);
-                s += 2;
+                row_load_fast(vb, x, s + 4, tid);
+                row_filter(vc, tw, list, count, s + 2, tid);
+                row_load_fast(vc, x, s + 5, tid);
+                s += 3;
             }
-            const bool three = s + 2 < nfull;                        // two or three whole stages remain
+            const int r = nfull - s;                                 // 3, 4 or 5 whole stages remain
             row_filter(va, tw, list, count, s, tid);
-            if (three) row_load_fast(va, x, s + 2, tid);
+            if (r > 3) row_load_fast(va, x, s + 3, tid);
             row_filter(vb, tw, list, count, s + 1, tid);
-            if (three) row_filter(va, tw, list, count, s + 2, tid);
+            if (r > 4) row_load_fast(vb, x, s + 4, tid);
+            row_filter(vc, tw, list, count, s + 2, tid);
+            if (r > 3) row_filter(va, tw, list, count, s + 3, tid);
+            if (r > 4) row_filter(vb, tw, list, count, s + 4, tid);
             s = nfull;
         } else {
             row_filter(va, tw, list, count, 0, tid);                 // the first stage, whole or ragged
-            s = 1;
+            if (nfull > 1) row_filter(vb, tw, list, count, 1, tid);
+            s = nfull > 1 ? 2 : 1;
         }
         for (; s < nstage; s++) {
             row_load_any<VEC>(va, x, V, s, tid);
@@ -308,7 +317,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     }
     __syncthreads();
     BORN_STAMP(a, row, 6);
-    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row);
+    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
     BORN_STAMP(a, row, 7);
 #ifdef BORN_PHASE_TIMING
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }

@@ -20,11 +20,11 @@ __device__ __forceinline__ u64 readlane_u64(u64 v, int lane) {     // lane must 
     return ((u64)hi << 32) | lo;
 }
 
-// One wave: integer CDF over the ns <= 64 survivors in `list` (rank order), top-p cut, draw.
-__device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, const SampleArgs &a, int row) {
+// One wave: integer CDF over the ns <= 64 survivors in `list` (rank order), top-p cut, draw with the row's
+// uniform u (fetched by the caller ahead of time: it is the last dependency of the row).
+__device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, const SampleArgs &a, int row, float u) {
     const int l = lane_id();
     const float m = key64_z(list[0]);
-    const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
     float e = 0.0f;
     u64 q = 0;
     if (l < ns) {
