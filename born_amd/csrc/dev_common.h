@@ -17,6 +17,21 @@ typedef unsigned int u32;
 
 constexpr int WAVE = 64;
 
+// Pointers into LDS (and, where a pointer travels in a struct, into global memory) that keep their address space through structs and calls that are not inlined: a plain
+// pointer there makes the compiler fall back to flat loads, stores and atomics, which are slower than their
+// ds_* forms and also hold up the counters that let global loads stay in flight.
+#define BORN_LDS __attribute__((address_space(3)))
+#define BORN_GLOBAL __attribute__((address_space(1)))
+typedef BORN_LDS u64 lds_u64;
+typedef BORN_LDS u32 lds_u32;
+typedef BORN_LDS int lds_int;
+template <class T>
+__device__ __forceinline__ T lds_add(BORN_LDS T *p, T v) {          // returns the old value
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void lds_min(lds_int *p, int v) { __hip_atomic_fetch_min(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+__device__ __forceinline__ void lds_or(lds_u32 *p, u32 v) { __hip_atomic_fetch_or(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+
 // ---- bit patterns ---------------------------------------------------------
 
 __device__ __forceinline__ u32 ordkey(float z) {          // order-preserving fp32 -> uint32
@@ -118,6 +133,10 @@ __device__ __forceinline__ float prob_of(float e, u64 Zp, int S) {
 #endif
 
 // ---- wave / block primitives --------------------------------------------------
+
+// A value that is the same in every lane, moved to a scalar register (keeps loop invariants out of the vector
+// register file, where a 1024-thread workgroup has only 128 registers per lane).
+__device__ __forceinline__ float uniform_f32(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }
 __device__ __forceinline__ int wave_id() { return (int)(threadIdx.x >> 6); }

@@ -13,44 +13,77 @@ static_assert(WIDE_BINS == WIDE_LIST_CAP, "the histogram scan and the list scan 
 // ---------------------------------------------------------------------------
 
 struct WideCtx {
-    const float *x;
+    const BORN_GLOBAL float *x;
     int V;
     bool vec, has_hist, count_mode;
     float T, rep, m, scale;
-    const u32 *bm;
-    u64 *mass;      // [WIDE_BINS] inclusive cumulative masses after the scan
-    u32 *cnt;       // [WIDE_BINS] inclusive cumulative counts (count_mode only)
-    u64 *list;      // [WIDE_LIST_CAP]
-    BlockScratch *scr;
-    int *s_int;     // [8] shared ints
-    u64 *s_u64;     // [4] shared u64
+    const lds_u32 *bm;
+    lds_u64 *mass;  // [WIDE_BINS] inclusive cumulative masses after the scan
+    lds_u32 *cnt;   // [WIDE_BINS] inclusive cumulative counts (count_mode only)
+    lds_u64 *list;  // [WIDE_LIST_CAP]
+    BORN_LDS BlockScratch *scr;
+    lds_int *s_int; // [8] shared ints
+    lds_u64 *s_u64; // [4] shared u64
 };
 
 __device__ __forceinline__ int wide_bin(float d) {
     return d < 32.0f ? (int)(d * WIDE_BINS_PER_UNIT) : WIDE_BINS - 1;     // monotone in d; inf -> last bin
 }
 
-// Visit every element of the row as (id, z).
+// Visit every element of the row as (id, z).  Aligned rows are read in stages of WIDE_U float4 per thread, the
+// loads of the next stage in flight while this one is visited (the loop body has no branch around a load, so
+// the compiler can wait for exactly the stage it needs); what is left of the row is read block by block.
+constexpr int WIDE_U = 4;
+typedef float wide_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void wide_load_stage(wide_f32x4 (&v)[WIDE_U], const BORN_GLOBAL float *x, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < WIDE_U; u++)
+        v[u] = ((const BORN_GLOBAL wide_f32x4 *)x)[(stage * WIDE_U + u) * WIDE_BLOCK + tid];
+}
+
+template <class F>
+__device__ __forceinline__ void wide_visit4(const WideCtx &c, const wide_f32x4 &q, int j, F &f) {
+    float y[4] = {q[0], q[1], q[2], q[3]};
+    if (c.has_hist) {
+        u32 bits = (c.bm[j >> 5] >> (j & 31)) & 0xFu;
+        if (bits) {
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                if ((bits >> t) & 1u) y[t] = penalise(y[t], c.rep);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) f(j + t, z_of(y[t], c.T));
+}
+
+template <class F>
+__device__ __forceinline__ void wide_visit_stage(const WideCtx &c, const wide_f32x4 (&v)[WIDE_U], int stage, int tid, F &f) {
+#pragma unroll
+    for (int u = 0; u < WIDE_U; u++) wide_visit4(c, v[u], ((stage * WIDE_U + u) * WIDE_BLOCK + tid) << 2, f);
+}
+
 template <class F>
 __device__ __forceinline__ void wide_foreach(const WideCtx &c, F f) {
     const int tid = threadIdx.x;
     if (c.vec) {
         const int n4 = c.V >> 2;
-        const float4 *x4 = reinterpret_cast<const float4 *>(c.x);
-        for (int i = tid; i < n4; i += WIDE_BLOCK) {
-            float4 q = x4[i];
-            int j = i << 2;
-            float y[4] = {q.x, q.y, q.z, q.w};
-            if (c.has_hist) {
-                u32 bits = (c.bm[j >> 5] >> (j & 31)) & 0xFu;
-                if (bits) {
+        const int nfull = n4 / (WIDE_U * WIDE_BLOCK);              // whole stages
+        if (nfull > 0) {
+            wide_f32x4 va[WIDE_U], vb[WIDE_U];
+            wide_load_stage(va, c.x, 0, tid);
+            for (int s = 0; s + 1 < nfull; s++) {
+                wide_load_stage(vb, c.x, s + 1, tid);
+                wide_visit_stage(c, va, s, tid, f);
 #pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        if ((bits >> t) & 1u) y[t] = penalise(y[t], c.rep);
-                }
+                for (int u = 0; u < WIDE_U; u++) va[u] = vb[u];
             }
-#pragma unroll
-            for (int t = 0; t < 4; t++) f(j + t, z_of(y[t], c.T));
+            wide_visit_stage(c, va, nfull - 1, tid, f);
+        }
+        const BORN_GLOBAL wide_f32x4 *x4 = (const BORN_GLOBAL wide_f32x4 *)c.x;
+        for (int i = nfull * WIDE_U * WIDE_BLOCK + tid; i < n4; i += WIDE_BLOCK) {
+            const wide_f32x4 q = x4[i];
+            wide_visit4(c, q, i << 2, f);
         }
         for (int j = (n4 << 2) + tid; j < c.V; j += WIDE_BLOCK) {
             float y = c.x[j];
@@ -68,7 +101,7 @@ __device__ __forceinline__ void wide_foreach(const WideCtx &c, F f) {
 
 // In-place inclusive scan over n (<= WIDE_ITEMS * WIDE_BLOCK) LDS entries, WIDE_ITEMS consecutive per thread.
 template <class T>
-__device__ __forceinline__ void wide_scan_inplace(T *arr, int n, BlockScratch *scr) {
+__device__ __forceinline__ void wide_scan_inplace(BORN_LDS T *arr, int n, BORN_LDS BlockScratch *scr) {
     const int tid = threadIdx.x;
     u64 v[WIDE_ITEMS], local = 0;
 #pragma unroll
@@ -78,7 +111,7 @@ __device__ __forceinline__ void wide_scan_inplace(T *arr, int n, BlockScratch *s
         v[t] = local;
     }
     u64 tot;
-    u64 inc = block_inclusive_scan_u64<WIDE_BLOCK>(local, scr, &tot);
+    u64 inc = block_inclusive_scan_u64<WIDE_BLOCK>(local, (BlockScratch *)scr, &tot);
     u64 excl = inc - local;
 #pragma unroll
     for (int t = 0; t < WIDE_ITEMS; t++) {
@@ -90,7 +123,7 @@ __device__ __forceinline__ void wide_scan_inplace(T *arr, int n, BlockScratch *s
 
 // smallest index with cumulative[idx] >= target (cumulative is inclusive and non-decreasing)
 template <class T>
-__device__ __forceinline__ int first_reaching(const T *cum, int n, u64 target) {
+__device__ __forceinline__ int first_reaching(const BORN_LDS T *cum, int n, u64 target) {
     int lo = 0, hi = n - 1;
     while (lo < hi) {
         int mid = (lo + hi) >> 1;
@@ -106,7 +139,7 @@ struct Found {
 // The sorted list holds (at least) every element of the bins named in `held`; within the run of
 // bin `b` (or over the whole list when b < 0) find the first element at which base + running
 // measure reaches `target`.
-__device__ Found wide_resolve(const WideCtx &c, int n, int b, bool by_count, u64 target, u64 base_mass,
+__device__ __forceinline__ Found wide_resolve(const WideCtx &c, int n, int b, bool by_count, u64 target, u64 base_mass,
                               u64 base_cnt) {
     const int tid = threadIdx.x;
     u64 q[WIDE_ITEMS], cm[WIDE_ITEMS];
@@ -132,8 +165,8 @@ __device__ Found wide_resolve(const WideCtx &c, int n, int b, bool by_count, u64
         cc[t] = lc;
     }
     u64 tot;
-    u64 em = block_inclusive_scan_u64<WIDE_BLOCK>(lm, c.scr, &tot) - lm;
-    u64 ec = block_inclusive_scan_u64<WIDE_BLOCK>((u64)lc, c.scr, &tot) - lc;
+    u64 em = block_inclusive_scan_u64<WIDE_BLOCK>(lm, (BlockScratch *)c.scr, &tot) - lm;
+    u64 ec = block_inclusive_scan_u64<WIDE_BLOCK>((u64)lc, (BlockScratch *)c.scr, &tot) - lc;
     if (tid == 0) c.s_int[0] = 0x7FFFFFFF;
     __syncthreads();
     int mine = 0x7FFFFFFF;
@@ -142,7 +175,7 @@ __device__ Found wide_resolve(const WideCtx &c, int n, int b, bool by_count, u64
         u64 meas = by_count ? base_cnt + ec + cc[t] : base_mass + em + cm[t];
         if (in[t] && meas >= target) mine = tid * WIDE_ITEMS + t;
     }
-    if (mine != 0x7FFFFFFF) atomicMin(&c.s_int[0], mine);
+    if (mine != 0x7FFFFFFF) lds_min(c.s_int, mine);
     __syncthreads();
     const int win = c.s_int[0];
 #pragma unroll
@@ -176,7 +209,7 @@ __device__ __forceinline__ int wide_collect(const WideCtx &c, P pred) {
         u64 key = make_key64(z, j);
         if (pred(wide_bin(d), key)) {
             if (!c.count_mode && qfix(expneg(d), c.scale) == 0) return;
-            int pos = atomicAdd(&c.s_int[1], 1);
+            int pos = lds_add(c.s_int + 1, 1);
             if (pos < WIDE_LIST_CAP) c.list[pos] = key;
         }
     });
@@ -189,14 +222,14 @@ __device__ __forceinline__ int wide_collect(const WideCtx &c, P pred) {
 __device__ __forceinline__ void wide_sort(const WideCtx &c, int n) {
     const int n2 = next_pow2(n);
     for (int i = n + threadIdx.x; i < n2; i += WIDE_BLOCK) c.list[i] = 0;
-    bitonic_sort_desc<WIDE_BLOCK>(c.list, n2);
+    bitonic_sort_desc<WIDE_BLOCK>((u64 *)c.list, n2);
 }
 
 // Radix descent inside one over-full bin: refine by 11 key bits per sweep until the
 // remaining set fits the list.  The sub-histograms live in the list's storage.
-__device__ Found wide_descend(const WideCtx &c, int b, bool by_count, u64 target, u64 base_mass, u64 base_cnt) {
-    u64 *smass = c.list;                                           // [WIDE_SUB_BINS]
-    u32 *scnt = reinterpret_cast<u32 *>(c.list + WIDE_SUB_BINS);   // [WIDE_SUB_BINS]
+__device__ __noinline__ Found wide_descend(const WideCtx &c, int b, bool by_count, u64 target, u64 base_mass, u64 base_cnt) {
+    lds_u64 *smass = c.list;                                       // [WIDE_SUB_BINS]
+    lds_u32 *scnt = (lds_u32 *)(c.list + WIDE_SUB_BINS);           // [WIDE_SUB_BINS]
     u64 prefix = 0;
     int plen = 0;
     for (;;) {
@@ -216,8 +249,8 @@ __device__ Found wide_descend(const WideCtx &c, int b, bool by_count, u64 target
             if (!c.count_mode && q == 0) return;
             int digit = (int)((key >> (64 - plen - db)) & (u64)(nsb - 1));
             int idx = nsb - 1 - digit;                             // larger keys first
-            atomicAdd(&scnt[idx], 1u);
-            atomicAdd(&smass[idx], q);
+            lds_add(scnt + idx, 1u);
+            lds_add(smass + idx, q);
         });
         __syncthreads();
         wide_scan_inplace(smass, nsb, c.scr);
@@ -249,53 +282,62 @@ struct WideHeld {
 };
 
 // Find the element at which the cumulative measure (count or mass, in rank order) first reaches target.
-__device__ Found wide_find(const WideCtx &c, WideHeld &held, bool by_count, u64 target, int hint0, int hint1) {
+__device__ __forceinline__ Found wide_find(const WideCtx &c, WideHeld &held, bool by_count, u64 target, int hint0, int hint1) {
     const int b = by_count ? first_reaching(c.cnt, WIDE_BINS, target) : first_reaching(c.mass, WIDE_BINS, target);
     const u64 base_mass = b ? c.mass[b - 1] : 0ull;
     const u64 base_cnt = (b && c.count_mode) ? c.cnt[b - 1] : 0ull;
+    bool descend = false;
     if (!(held.bin[0] == b || held.bin[1] == b || held.bin[2] == b)) {
+        // gather the target's bin together with the hinted ones; if that overflows the list, the target's bin alone
         int w0 = b, w1 = hint0 >= 0 ? hint0 : b, w2 = hint1 >= 0 ? hint1 : b;
-        int n = wide_collect(c, [&](int bin, u64) { return bin == w0 || bin == w1 || bin == w2; });
-        if (n > WIDE_LIST_CAP && (w1 != b || w2 != b)) {
+        int n;
+        for (;;) {
+            n = wide_collect(c, [&](int bin, u64) { return bin == w0 || bin == w1 || bin == w2; });
+            if (n <= WIDE_LIST_CAP || (w1 == b && w2 == b)) break;
             w1 = w2 = b;
-            n = wide_collect(c, [&](int bin, u64) { return bin == b; });
         }
         if (n > WIDE_LIST_CAP) {
             held.bin[0] = held.bin[1] = held.bin[2] = -1;
             held.n = 0;
-            return wide_descend(c, b, by_count, target, base_mass, base_cnt);
+            descend = true;
+        } else {
+            wide_sort(c, n);
+            held.bin[0] = w0; held.bin[1] = w1; held.bin[2] = w2;
+            held.n = n;
         }
-        wide_sort(c, n);
-        held.bin[0] = w0; held.bin[1] = w1; held.bin[2] = w2;
-        held.n = n;
+    }
+    if (descend) {                       // over-full bin (ties, masked rows): refined out of line, on a copy of the
+        const WideCtx cc = c;            // context so that the original never has its address taken
+        return wide_descend(cc, b, by_count, target, base_mass, base_cnt);
     }
     return wide_resolve(c, held.n, b, by_count, target, base_mass, base_cnt);
 }
 
 // The general algorithm on one row (every thread of the workgroup calls it together).
-__device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, u64 *dyn, BlockScratch &scr, int *s_int, u64 *s_u64,
-                         const bool count_it) {
+__device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds_u64 *dyn, BORN_LDS BlockScratch *scr, lds_int *s_int,
+                                         lds_u64 *s_u64, const bool count_it) {
     const int tid = threadIdx.x;
     const int V = a.V;
     WideCtx c;
-    c.x = a.logits + (long long)row * a.row_stride;
+    c.x = (const BORN_GLOBAL float *)(a.logits + (long long)row * a.row_stride);
     c.V = V;
     c.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
-    c.T = a.T;
-    c.rep = a.rep;
-    c.scale = mass_scale(a.mass_shift);
+    c.T = uniform_f32(a.T);
+    c.rep = uniform_f32(a.rep);
+    c.scale = uniform_f32(mass_scale(a.mass_shift));
     c.mass = dyn;
     c.list = dyn + WIDE_BINS;
-    c.cnt = reinterpret_cast<u32 *>(dyn + WIDE_BINS + WIDE_LIST_CAP);
-    u32 *bm = c.cnt + WIDE_BINS;
+    c.cnt = (lds_u32 *)(dyn + WIDE_BINS + WIDE_LIST_CAP);
+    lds_u32 *bm = c.cnt + WIDE_BINS;
     c.bm = bm;
-    c.scr = &scr;
+    c.scr = scr;
     c.s_int = s_int;
     c.s_u64 = s_u64;
     const int k = a.top_k;
     c.count_mode = k > 0;
     const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
+    BORN_STAMP(a, row, 0);
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     c.has_hist = (a.rep != 1.0f) && hlen > 0;
@@ -307,7 +349,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, u64
         for (int i = tid; i < hlen; i += WIDE_BLOCK) {
             int t = h[i];
             if (t < 0 || t >= V) atomicOr(a.status, 1);
-            else atomicOr(&bm[t >> 5], 1u << (t & 31));
+            else lds_or(bm + (t >> 5), 1u << (t & 31));
         }
         __syncthreads();
     } else if (a.history) {
@@ -318,11 +360,13 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, u64
         }
     }
 
+    BORN_STAMP(a, row, 1);
     // ---- sweep 1: row maximum of z
     float mx = -INFINITY;
     wide_foreach(c, [&](int, float z) { mx = fmaxf(mx, z); });
-    c.m = block_max_f32<WIDE_BLOCK>(mx, &scr);
+    c.m = uniform_f32(block_max_f32<WIDE_BLOCK>(mx, (BlockScratch *)scr));
 
+    BORN_STAMP(a, row, 2);
     // ---- sweep 2: histogram over d = m - z (integer masses; counts only when a top-k cut is needed)
     for (int i = tid; i < WIDE_BINS; i += WIDE_BLOCK) {
         c.mass[i] = 0;
@@ -332,66 +376,83 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, u64
     wide_foreach(c, [&](int, float z) {
         float d = (z == c.m) ? 0.0f : c.m - z;
         int b = wide_bin(d);
-        if (c.count_mode) atomicAdd(&c.cnt[b], 1u);
+        if (c.count_mode) lds_add(c.cnt + b, 1u);
         u64 q = qfix(expneg(d), c.scale);
-        if (q) atomicAdd(&c.mass[b], q);
+        if (q) lds_add(c.mass + b, q);
     });
     __syncthreads();
-    wide_scan_inplace(c.mass, WIDE_BINS, &scr);
-    if (c.count_mode) wide_scan_inplace(c.cnt, WIDE_BINS, &scr);
+    BORN_STAMP(a, row, 3);
+    wide_scan_inplace(c.mass, WIDE_BINS, scr);
+    if (c.count_mode) wide_scan_inplace(c.cnt, WIDE_BINS, scr);
 
-    int token;
-    float prob;
-    bool done = false;
+    BORN_STAMP(a, row, 4);
+    // ---- locate, in this order as far as they apply: the k-th element (by count), the top-p cut and the draw
+    // (by mass).  One call site of wide_find, so that the whole search is inlined once.
+    WideHeld held;
+    held.bin[0] = held.bin[1] = held.bin[2] = -1;
+    held.n = 0;
+    u64 Zk = c.mass[WIDE_BINS - 1], Zp = 0, kcut = 0;
+    Found f;
+    f.key = 0;
+    f.mass = 0;
+    int bk = -1;
+    // a small enough top-k is finished from a sorted list of its k elements (that also yields the nucleus listing)
+    bool listing = false;
     if (c.count_mode) {
-        // Small enough top-k: gather every bin down to the one holding the k-th element, sort, finish.
-        const int bk = first_reaching(c.cnt, WIDE_BINS, (u64)k);
-        if (c.cnt[bk] <= (u32)WIDE_LIST_CAP) {
-            int n = wide_collect(c, [&](int bin, u64) { return bin <= bk; });
-            wide_sort(c, n);
-            finish_sorted<WIDE_BLOCK, WIDE_ITEMS>(c.list, k, a, row, &scr);
-            done = true;
-        } else if (k <= WIDE_LIST_CAP) {
-            // The k-th element's bin is over-full (ties, masked rows): locate the k-th key exactly, then
-            // gather the k elements at or above it.
-            WideHeld held;
-            held.bin[0] = held.bin[1] = held.bin[2] = -1;
-            held.n = 0;
-            const u64 kcut = wide_find(c, held, true, (u64)k, -1, -1).key;
-            int n = wide_collect(c, [&](int, u64 key) { return key >= kcut; });
-            wide_sort(c, min(n, WIDE_LIST_CAP));
-            finish_sorted<WIDE_BLOCK, WIDE_ITEMS>(c.list, k, a, row, &scr);
-            done = true;
-        }
+        bk = first_reaching(c.cnt, WIDE_BINS, (u64)k);
+        listing = c.cnt[bk] <= (u32)WIDE_LIST_CAP;       // every bin down to the k-th element's fits the list
     }
-    if (!done) {
-        WideHeld held;
-        held.bin[0] = held.bin[1] = held.bin[2] = -1;
-        held.n = 0;
-        u64 Zk = c.mass[WIDE_BINS - 1];
-        if (c.count_mode) Zk = wide_find(c, held, true, (u64)k, -1, -1).mass;
-        u64 Zp = Zk;
-        if (a.top_p < 1.0f) {
-            const u64 tp = top_p_target(a.top_p, Zk);
-            // The nucleus mass lies in [tp, mass through the cut's bin]; predict the draw's bin(s) from
+    for (int phase = c.count_mode ? (listing ? 3 : 0) : 1; phase < 3; phase++) {
+        bool by_count = false;
+        u64 target;
+        int h0 = -1, h1 = -1;
+        if (phase == 0) {
+            by_count = true;
+            target = (u64)k;
+        } else if (phase == 1) {
+            if (!(a.top_p < 1.0f)) {
+                Zp = Zk;
+                continue;
+            }
+            target = top_p_target(a.top_p, Zk);
+            // The nucleus mass lies in [target, mass through the cut's bin]; predict the draw's bin(s) from
             // that interval so one sweep gathers the cut's bin and the draw's bin together.
-            const int bp = first_reaching(c.mass, WIDE_BINS, tp);
-            u64 hi = c.mass[bp] < Zk ? c.mass[bp] : Zk;
-            int h0 = first_reaching(c.mass, WIDE_BINS, draw_target(u, tp));
-            int h1 = first_reaching(c.mass, WIDE_BINS, draw_target(u, hi));
+            const int bp = first_reaching(c.mass, WIDE_BINS, target);
+            const u64 hi = c.mass[bp] < Zk ? c.mass[bp] : Zk;
+            h0 = first_reaching(c.mass, WIDE_BINS, draw_target(u, target));
+            h1 = first_reaching(c.mass, WIDE_BINS, draw_target(u, hi));
             if (h1 - h0 > 1) h0 = h1 = -1;
-            Zp = wide_find(c, held, false, tp, h0, h1).mass;
+        } else {
+            BORN_STAMP(a, row, 5);
+            target = draw_target(u, Zp);
         }
-        const u64 td = draw_target(u, Zp);
-        Found f = wide_find(c, held, false, td, -1, -1);
-        token = key64_id(f.key);
-        prob = prob_of(emass(key64_z(f.key), c.m), Zp, a.mass_shift);
-        if (tid == 0) {
-            a.tokens[row] = token;
-            if (a.probs) a.probs[row] = prob;
-            if (a.nuc_len) a.nuc_len[row] = -1;      // the nucleus listing is only produced for small top-k
+        f = wide_find(c, held, by_count, target, h0, h1);
+        if (phase == 0) {
+            // The k-th element's bin is over-full (ties, masked rows): its key is now known exactly
+            Zk = f.mass;
+            if (k <= WIDE_LIST_CAP) {
+                listing = true;
+                kcut = f.key;
+                bk = -1;
+                break;
+            }
+        } else if (phase == 1) {
+            Zp = f.mass;
         }
     }
+    BORN_STAMP(a, row, 6);
+    if (listing) {
+        const int bk_ = bk;
+        const u64 kcut_ = kcut;
+        int n = wide_collect(c, [&](int bin, u64 key) { return bk_ >= 0 ? bin <= bk_ : key >= kcut_; });
+        wide_sort(c, min(n, WIDE_LIST_CAP));
+        finish_sorted<WIDE_BLOCK, WIDE_ITEMS>((const u64 *)c.list, k, a, row, (BlockScratch *)scr);
+    } else if (tid == 0) {
+        a.tokens[row] = key64_id(f.key);
+        if (a.probs) a.probs[row] = prob_of(emass(key64_z(f.key), c.m), Zp, a.mass_shift);
+        if (a.nuc_len) a.nuc_len[row] = -1;              // the nucleus listing is only produced for small top-k
+    }
+    BORN_STAMP(a, row, 7);
     if (tid == 0 && count_it) atomicAdd(&a.counters[2], 1ull);
 }
 
@@ -405,7 +466,8 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, i
     // one call site, so the row routine is inlined and the kernel arguments stay in scalar registers
     const int limit = from_queue ? *a.fb_count : a.B;
     for (int i = blockIdx.x; i < limit; i += gridDim.x) {
-        wide_row(a, from_queue ? a.fb_rows[i] : i, dyn, scr, s_int, s_u64, !from_queue);
+        wide_row(a, from_queue ? a.fb_rows[i] : i, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64,
+                 !from_queue);
         __syncthreads();
     }
 }
