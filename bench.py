@@ -6,13 +6,11 @@ batch 256 x vocab 128256, temperature 0.7, top-k 50, top-p 0.9, repetition penal
 512-token Zipf(1.1) history per row, one seeded uniform per row (configuration 3 of BASELINE.json,
 the one the metric is quoted on).  Prints ONE JSON line.
 
-  value        sampled tokens/s of the whole step (all three launches of a step: collect, finish,
-               fallback queue; inputs resident in HBM, cycled through several buffers so that no
+  value        sampled tokens/s of the whole step (one launch: topk_row_kernel reads every row once
+               and finishes it; inputs resident in HBM, cycled through several buffers so that no
                step finds its logits in the Infinity Cache)
-  roofline     the dominant kernel (topk_collect_kernel, the one pass over the logits):
-               algorithmic bytes of one step divided by that kernel's average launch duration,
-               measured here with HIP events on the launch stream over a second timed loop that
-               launches that kernel alone
+  roofline     that kernel: algorithmic bytes of one step divided by its average launch duration,
+               measured here with HIP events on the launch stream over the timed region
   cpu_baseline the CPU oracle's reference-arithmetic mode timed on this box's host, one thread,
                on a bounded sample of the same workload
 
@@ -37,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # kernel is scaled by what the same counter reads for the --copy-probe copy of one logits buffer
 # (131 334 144 B read and written): FETCH_SIZE 64152.5 -> factor 1.99925 KiB per unit, WRITE_SIZE
 # 128256.0 -> factor 1.0.  Kernel: FETCH_SIZE 64186.0 -> 131.40 MB read, WRITE_SIZE 2840.8 -> 2.91 MB written.
-PMC_TRAFFIC_BYTES = {("C3", "topk_collect_kernel"): int(64186.0 * 1.99925 * 1024 + 2840.8 * 1024)}
+PMC_TRAFFIC_BYTES = {}
 
 
 def cpu_baseline(w, seconds=12.0):
@@ -68,14 +66,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--rotate", type=int, default=4,
                     help="number of distinct logits buffers cycled through, so that a step never finds its logits in a cache")
-    ap.add_argument("--path", type=int, default=0, help="kernel selection of the sampler (0 = default; 3 = segment kernel + row finish)")
-    ap.add_argument("--kernel-path", type=int, default=None, help="path that launches the dominant kernel alone (5 for path 0, 2 for path 3)")
+    ap.add_argument("--path", type=int, default=0, help="kernel selection of the sampler (0 = default; 1 = always the general kernel)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a few plain device-to-device copies of one logits buffer (a kernel of known traffic "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
-    if args.kernel_path is None:
-        args.kernel_path = 2 if args.path == 3 else 5
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; rows are independent, so more GPUs would each take a "
               "slice of the batch with no exchange. Run with --gpus 1.", file=sys.stderr)
@@ -142,18 +137,9 @@ def main():
     tok_host = tokens.cpu().numpy()
     assert tok_host.min() >= 0 and tok_host.max() < V
 
-    # dominant kernel alone (finish and fallback-queue launches left out): roofline of that kernel
-    single_pass = 1 <= w.top_k <= 64
-    if single_pass:
-        smp.SetPath(args.kernel_path)
-        for _ in range(10):
-            step()
-        ms_kernel = timed(args.steps)
-        smp.SetPath(args.path)
-        kernel_name = {5: "topk_row_kernel", 2: "topk_collect_kernel"}[args.kernel_path]
-    else:
-        ms_kernel = ms
-        kernel_name = "sample_wide_kernel"
+    # a step is a single launch, so the step time is the kernel's launch-to-launch duration
+    ms_kernel = ms
+    kernel_name = "topk_row_kernel" if (1 <= w.top_k <= 64 and args.path == 0) else "sample_wide_kernel"
     alg_bytes = w.algorithmic_bytes()
     achieved = alg_bytes / (ms_kernel * 1e-3) / 1e9
 

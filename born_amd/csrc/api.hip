@@ -43,18 +43,15 @@ hipError_t g_cfg_err = hipSuccess;
 struct born_sampler {
     born_sampler_config cfg;
     int64_t max_batch, max_vocab;
-    int S_max;                     // segments per row at max_vocab
+    int S_max;                     // argmax segments per row at max_vocab
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // see born_rocm_sampler_set_path
-    unsigned queue_epoch;          // steps that used the fallback queue: its counter alternates between two slots
     // device workspace
-    int *fb_count, *fb_rows;       // fb_count[2]
-    uint2 *cand;
-    int *cand_count;
-    float *seg_thr;
+    float *arg_val;                // argmax partials [max_batch][S_max]
+    int *arg_idx;
     int *status;
     unsigned long long *counters;
-    // argmax partials share cand_count / seg_thr storage; spec-verify statistics:
+    // spec-verify statistics:
     float *sp_mp, *sp_mq;
     unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd;
     int64_t spec_rows;
@@ -133,7 +130,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     if (max_vocab > WIDE_MAX_VOCAB)
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: create: max_vocab %lld exceeds the supported %lld",
                     (long long)max_vocab, (long long)WIDE_MAX_VOCAB);
-    if (max_batch * ((max_vocab + TOPK_SEG - 1) / TOPK_SEG) > (int64_t)0x7FFFFFFF / TOPK_SEG_CAP)
+    if (max_batch * ((max_vocab + ARGMAX_SEG - 1) / ARGMAX_SEG) > (int64_t)0x7FFFFFFF / 8)
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: create: max_batch * segments too large");
     born_sampler_config c;
     if (cfg) c = *cfg; else memset(&c, 0, sizeof(c));
@@ -149,18 +146,15 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     s->cfg = c;
     s->max_batch = max_batch;
     s->max_vocab = max_vocab;
-    s->S_max = (int)((max_vocab + TOPK_SEG - 1) / TOPK_SEG);
+    s->S_max = (int)((max_vocab + ARGMAX_SEG - 1) / ARGMAX_SEG);
     const size_t rows = (size_t)max_batch, segs = rows * (size_t)s->S_max;
     hipError_t e = hipSuccess;
     auto alloc = [&](void **p, size_t bytes) {
         if (e == hipSuccess) e = hipMalloc(p, bytes);
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
-    alloc((void **)&s->fb_count, 2 * sizeof(int));
-    alloc((void **)&s->fb_rows, rows * sizeof(int));
-    alloc((void **)&s->cand, segs * TOPK_SEG_CAP * sizeof(uint2));
-    alloc((void **)&s->cand_count, segs * TOPK_WAVES * sizeof(int));
-    alloc((void **)&s->seg_thr, segs * sizeof(float));
+    alloc((void **)&s->arg_val, segs * sizeof(float));
+    alloc((void **)&s->arg_idx, segs * sizeof(int));
     alloc((void **)&s->status, sizeof(int));
     alloc((void **)&s->counters, (64 + 8 * rows) * sizeof(unsigned long long));   // [0..2] work counters; debug builds: [8..] phase stamps, [64..] per-row stamps
     if (e != hipSuccess) {
@@ -173,7 +167,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->fb_count, s->fb_rows, s->cand, s->cand_count, s->seg_thr, s->status, s->counters,
+    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -196,7 +190,7 @@ int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg
 }
 
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path) {
-    if (!s || path < 0 || path > 5) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
+    if (!s || path < 0 || path > 1) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
     s->path = path;
     return BORN_ROCM_OK;
 }
@@ -257,8 +251,7 @@ int born_rocm_argmax(born_sampler *s, const float *logits, int64_t batch, int64_
     int rc = check_logits("argmax", s, logits, batch, vocab, row_stride);
     if (rc) return rc;
     if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: argmax: null output");
-    // ARGMAX_SEG == TOPK_SEG, so the per-segment workspace of the handle fits the partials.
-    HIP_TRY(launch_argmax(logits, (int)batch, (int)vocab, row_stride, tokens_out, s->seg_thr, s->cand_count,
+    HIP_TRY(launch_argmax(logits, (int)batch, (int)vocab, row_stride, tokens_out, s->arg_val, s->arg_idx,
                           (hipStream_t)stream));
     return BORN_ROCM_OK;
 }
@@ -317,13 +310,6 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_ids = nucleus_ids_out;
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
-    a.fb_count = s->fb_count + (s->queue_epoch & 1u);
-    a.fb_count_next = s->fb_count + ((s->queue_epoch + 1u) & 1u);
-    a.fb_rows = s->fb_rows;
-    a.cand = s->cand;
-    a.cand_count = s->cand_count;
-    a.seg_thr = s->seg_thr;
-    a.S = (int)((vocab + TOPK_SEG - 1) / TOPK_SEG);
     a.status = s->status;
     a.counters = s->counters;
     a.mass_shift = mass_shift(vocab);
@@ -331,21 +317,10 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     hipStream_t st = (hipStream_t)stream;
     // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
     const bool boosts = history && a.rep < 1.0f;
-    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && !boosts) {
-        // Rows that a single-pass kernel cannot prove are queued; the general kernel then walks the queue.
-        // The queue counter of the next step is zeroed by this step's first kernel (the counter of this step
-        // was zeroed by the step before), so no launch is spent on clearing it.
-        const bool by_row = s->path == 0 || s->path == 4 || s->path == 5;
-        if (by_row) {
-            HIP_TRY(launch_topk_row(a, st));                       // one workgroup per row, tail included
-        } else {
-            HIP_TRY(launch_topk_collect(a, st));                   // one workgroup per 8192-logit segment ...
-            if (s->path == 3) HIP_TRY(launch_topk_finish(a, st));  // ... and one per row to finish
-        }
-        if (s->path == 0 || s->path == 3 || s->path == 4) HIP_TRY(launch_sample_wide(a, true, st));
-        s->queue_epoch++;
+    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
+        HIP_TRY(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
     } else {
-        HIP_TRY(launch_sample_wide(a, false, st));
+        HIP_TRY(launch_sample_wide(a, st));
     }
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;

@@ -5,14 +5,9 @@
 
 namespace born {
 
-// Geometry of the single-pass top-k kernel.
-constexpr int TOPK_BLOCK = 256;            // threads per workgroup (4 waves)
-constexpr int TOPK_F4 = 8;                 // float4 loads per thread
-constexpr int TOPK_SEG = TOPK_BLOCK * TOPK_F4 * 4;   // 8192 logits per workgroup
-constexpr int TOPK_WAVES = TOPK_BLOCK / 64;  // each wave owns a quarter of its segment's candidate area
-constexpr int TOPK_WAVE_CAP = 256;         // candidates one wave may emit
-constexpr int TOPK_SEG_CAP = TOPK_WAVES * TOPK_WAVE_CAP;   // candidate slots per segment
-constexpr int TOPK_MAX_K = 64;             // largest top_k served by the single-pass kernel
+// The single-pass top-k kernel (one workgroup per row).
+constexpr int TOPK_MAX_K = 64;             // largest top_k it serves
+constexpr int ROW_MAX_VOCAB = 393216;      // largest vocabulary it takes (its history bitmap is 48 KiB of LDS)
 
 // Geometry of the general (any k, any p) kernel: one workgroup per row.
 constexpr int WIDE_BINS = 4096;            // level-0 histogram bins over d = m - z
@@ -20,8 +15,6 @@ constexpr float WIDE_BINS_PER_UNIT = 128.0f;   // 4096 bins cover d in [0, 32)
 constexpr int WIDE_LIST_CAP = 4096;        // elements the in-LDS sort can hold
 constexpr int WIDE_SUB_BINS = 2048;        // radix-descent digit = 11 bits
 constexpr int64_t WIDE_MAX_VOCAB = 524288; // history bitmap must fit LDS next to the histogram
-
-constexpr int WIDE_QUEUE_GRID = 64;         // workgroups that walk the fallback queue
 
 constexpr int ARGMAX_SEG = 8192;
 
@@ -51,15 +44,8 @@ struct SampleArgs {
     float *nuc_probs;
     int nuc_cap;
     // workspace
-    uint2 *cand;                  // [B][S][TOPK_WAVES][TOPK_WAVE_CAP] (logit bits, id)
-    int *cand_count;              // [B][S][TOPK_WAVES]
-    float *seg_thr;               // [B][S]
-    int S;                        // segments per row
-    int *fb_count;                // number of rows queued for the general kernel in this step
-    int *fb_count_next;           // the counter the next step will use: zeroed by the first kernel of this step
-    int *fb_rows;                 // [B] the queue
     int *status;                  // device status word
-    unsigned long long *counters; // [0] top-k rows, [1] fallback rows, [2] general rows
+    unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows it finished by exact selection, [2] general rows
     int mass_shift;
 };
 
@@ -83,10 +69,8 @@ hipError_t launch_softmax(const float *logits, int B, int V, long long stride, f
                           hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
-hipError_t launch_topk_collect(const SampleArgs &a, hipStream_t st);
-hipError_t launch_topk_finish(const SampleArgs &a, hipStream_t st);
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st);
-hipError_t launch_sample_wide(const SampleArgs &a, bool from_queue, hipStream_t st);
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st);
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);
 size_t wide_lds_bytes(int V);
 hipError_t configure_kernels();   // one-time function attributes (dynamic LDS above 64 KiB)

@@ -16,29 +16,16 @@ size_t wide_lds_bytes(int V) {
 }
 }  // namespace born
 
-// Two instances: 1024 threads per workgroup for whole batches (most waves to hide the sweeps'
-// latency), 512 for the fallback queue of the top-k path, which is usually empty: with twice the
-// registers per thread that instance needs no scratch memory, so its launch costs little.
 #define BORN_WIDE_BLOCK 1024
 #define BORN_WIDE_NS w1024
-#include "sample_wide_impl.h"
-#undef BORN_WIDE_BLOCK
-#undef BORN_WIDE_NS
-#define BORN_WIDE_BLOCK 512
-#define BORN_WIDE_NS w512
 #include "sample_wide_impl.h"
 #undef BORN_WIDE_BLOCK
 #undef BORN_WIDE_NS
 
 namespace born {
 
-hipError_t launch_sample_wide(const SampleArgs &a, bool from_queue, hipStream_t st) {
-    return from_queue ? w512::launch(a, true, st) : w1024::launch(a, false, st);
-}
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st) { return w1024::launch(a, st); }
 
-hipError_t configure_kernels() {
-    hipError_t e = w1024::configure();
-    return e != hipSuccess ? e : w512::configure();
-}
+hipError_t configure_kernels() { return w1024::configure(); }
 
 }  // namespace born

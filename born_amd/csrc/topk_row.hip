@@ -18,8 +18,11 @@
 //   above that bound.  A rank sort orders them and one wave computes the integer CDF, the top-p
 //   cut and the draw.
 // Rows that cannot be proven (fewer than top_k finite logits, heavy ties, list overflow, penalised
-// tokens dropping below the bound) are appended to the fallback queue, which the general kernel
-// walks in the next launch.
+// tokens dropping below the bound) are finished by the same workgroup with an exact selection that
+// works for any input: a radix descent over the 64-bit rank keys (z descending, id ascending; the
+// keys are unique), 11 bits per sweep of the row, until the top_k keys and the rest of the last
+// bucket fit a list; then the same rank sort and last wave.  The sweeps re-read the row from the
+// caches.
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
@@ -37,6 +40,24 @@ __device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (
 static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
 static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
 static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
+
+// LDS pool (u64 words), laid out once for the proof and once for the exact selection
+constexpr int ROW_POOL = 8000;
+constexpr int OFF_L = 0;                      // [ROW_WAVES][ROW_WCAP] uint2
+constexpr int OFF_C = OFF_L + ROW_WAVES * ROW_WCAP;   // [ROW_CAP] uint2
+constexpr int OFF_K = OFF_C + ROW_CAP;        // [ROW_CAP] u64
+constexpr int OFF_TAB = OFF_K + ROW_CAP;      // [ROW_SLOTS] u32
+constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [WAVE] u64
+static_assert(OFF_SORTED + WAVE <= ROW_POOL, "proof layout fits the pool");
+constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
+constexpr int FB_DIGIT = 11;                  // key bits per sweep
+constexpr int OFF_FB_HIST = FB_BITMAP;        // [1 << FB_DIGIT] u32
+constexpr int OFF_FB_LIST = OFF_FB_HIST + (1 << FB_DIGIT) / 2;
+constexpr int FB_LIST_CAP = 768;
+constexpr int OFF_FB_SORTED = OFF_FB_LIST + FB_LIST_CAP;
+static_assert(OFF_FB_SORTED + WAVE <= ROW_POOL, "selection layout fits the pool");
+static_assert(FB_LIST_CAP <= ROW_BLOCK, "one thread per gathered key");
+static_assert((long long)FB_BITMAP * 64 >= ROW_MAX_VOCAB, "one bitmap bit per id");
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -96,21 +117,151 @@ __device__ __forceinline__ u32 row_pick(const u32 *wthr, int need) {
     return wave_max_u32((l < ROW_WAVES && ge >= need) ? mine : 0u);
 }
 
+// Visits every element of the row as f(id, logit), the loads of one stage in flight while the stage before it
+// is visited.
+template <bool VEC, class F>
+__device__ __forceinline__ void row_foreach(const float *x, int V, int tid, F f) {
+    const int n4 = (V + 3) >> 2;
+    const int nstage = ((n4 + ROW_BLOCK - 1) / ROW_BLOCK + ROW_U - 1) / ROW_U;
+    const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;
+    f32x4 va[ROW_U], vb[ROW_U];
+    auto visit = [&](const f32x4 (&v)[ROW_U], int stage) {
+#pragma unroll
+        for (int u = 0; u < ROW_U; u++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int j = ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c;
+                if (j < V) f(j, v[u][c]);
+            }
+        }
+    };
+    int s = 0;
+    if (nfull > 0) {
+        row_load_fast(va, x, 0, tid);
+        for (; s + 1 < nfull; s++) {
+            row_load_fast(vb, x, s + 1, tid);
+            visit(va, s);
+#pragma unroll
+            for (int u = 0; u < ROW_U; u++) va[u] = vb[u];
+        }
+        visit(va, s);
+        s = nfull;
+    }
+    for (; s < nstage; s++) {
+        row_load_any<VEC>(va, x, V, s, tid);
+        visit(va, s);
+    }
+}
+
+// Exact selection of the row's top_k rank keys for any input (every thread of the workgroup calls it).
+// pool: the workgroup's LDS pool; s_n, s_x: two shared ints.
+template <bool VEC>
+__device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, const float *x, int hlen, const int *h, float u_row,
+                                                 u64 *pool, int *s_n, int *s_x) {
+    const int tid = threadIdx.x, V = a.V, k = a.top_k;
+    u32 *bm = reinterpret_cast<u32 *>(pool);
+    u32 *hist = reinterpret_cast<u32 *>(pool + OFF_FB_HIST);
+    u64 *list = pool + OFF_FB_LIST;
+    u64 *sorted = pool + OFF_FB_SORTED;
+    const bool penal = a.rep != 1.0f && hlen > 0;
+    __syncthreads();                                                 // the proof's use of the pool is over
+    if (penal) {
+        for (int i = tid; i < ((V + 31) >> 5); i += ROW_BLOCK) bm[i] = 0u;
+        __syncthreads();
+        for (int i = tid; i < hlen; i += ROW_BLOCK) {
+            const int t = h[i];
+            if (t >= 0 && t < V) atomicOr(&bm[t >> 5], 1u << (t & 31));
+        }
+        __syncthreads();
+    }
+    auto rank_key = [&](int j, float xv) -> u64 {
+        float y = xv;
+        if (penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, a.rep);
+        return make_key64(z_of(y, a.T), j);
+    };
+    // radix descent: after each sweep the wanted key is the need-th largest inside the bucket `prefix`
+    // (plen leading bits); `above` keys lie above the bucket and belong to the top_k
+    u64 prefix = 0ull;
+    int plen = 0, need = k, above = 0;
+    for (;;) {
+        const int db = min(FB_DIGIT, 64 - plen), nb = 1 << db;
+        for (int i = tid; i < nb; i += ROW_BLOCK) hist[i] = 0u;
+        __syncthreads();
+        {
+            const u64 pf = prefix;
+            const int pl = plen;
+            row_foreach<VEC>(x, V, tid, [&](int j, float xv) {
+                const u64 key = rank_key(j, xv);
+                if (pl == 0 || (key >> (64 - pl)) == pf) atomicAdd(&hist[(u32)(key >> (64 - pl - db)) & (u32)(nb - 1)], 1u);
+            });
+        }
+        __syncthreads();
+        // the largest digit D with (number of keys in digits >= D) >= need: each thread takes two digits, from the top
+        const int d0 = nb - 1 - 2 * tid, d1 = d0 - 1;
+        const u32 c0 = d0 >= 0 ? hist[d0] : 0u, c1 = d1 >= 0 ? hist[d1] : 0u;
+        u32 incl = wave_inclusive_scan_u32(c0 + c1);
+        if (lane_id() == WAVE - 1) s_x[1 + wave_id()] = (int)incl;   // wave totals
+        __syncthreads();
+        u32 base = 0u;
+        for (int w = 0; w < wave_id(); w++) base += (u32)s_x[1 + w];
+        incl += base;
+        const u32 excl = incl - (c0 + c1);
+        __syncthreads();
+        if (excl < (u32)need && (u32)need <= incl) {                 // exactly one thread owns the crossing
+            const bool first = excl + c0 >= (u32)need;
+            s_x[0] = first ? d0 : d1;
+            s_n[0] = (int)(first ? excl : excl + c0);                // keys in the digits above D
+        }
+        __syncthreads();
+        const int D = s_x[0], over = s_n[0];
+        const u32 cntD = hist[D];
+        need -= over;
+        above += over;
+        prefix = (prefix << db) | (u64)D;
+        plen += db;
+        __syncthreads();
+        if (above + (int)cntD <= FB_LIST_CAP || plen == 64) break;
+    }
+    // gather the keys at or above the bucket: `above` + the bucket's, at least top_k of them
+    const u64 lo_key = plen == 64 ? prefix : prefix << (64 - plen);
+    if (tid == 0) s_n[0] = 0;
+    __syncthreads();
+    row_foreach<VEC>(x, V, tid, [&](int j, float xv) {
+        const u64 key = rank_key(j, xv);
+        if (key >= lo_key) {
+            const int pos = atomicAdd(&s_n[0], 1);
+            if (pos < FB_LIST_CAP) list[pos] = key;
+        }
+    });
+    __syncthreads();
+    const int n = min(s_n[0], FB_LIST_CAP);
+    if (tid < n) {
+        const u64 key = list[tid];
+        int r = 0;
+        for (int j = 0; j < n; j++) r += list[j] > key ? 1 : 0;
+        if (r < k) sorted[r] = key;
+    }
+    __syncthreads();
+    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
+    if (tid == 0) atomicAdd(&a.counters[1], 1ull);
+}
+
 template <bool VEC>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
-    __shared__ uint2 L[ROW_WAVES][ROW_WCAP];   // per-wave lists of (logit bits, id) >= Tw
-    __shared__ uint2 C[ROW_CAP];               // candidates >= T2; .y bit 31 = id occurs in the history
-    __shared__ u64 K[ROW_CAP];                 // their rank keys, 0 = dropped
-    __shared__ u64 sorted[WAVE];
-    __shared__ u32 tab[ROW_SLOTS];
+    __shared__ u64 pool[ROW_POOL];
+    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= Tw
+    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);       // candidates >= T2; .y bit 31 = id occurs in the history
+    u64 *const K = pool + OFF_K;                                     // their rank keys, 0 = dropped
+    u32 *const tab = reinterpret_cast<u32 *>(pool + OFF_TAB);
+    u64 *const sorted = pool + OFF_SORTED;
     __shared__ int s_rank[ROW_BLOCK];
     __shared__ u32 s_wthr[ROW_WAVES], s_wthr2[ROW_WAVES];
     __shared__ int s_n, s_valid, s_over;
+    __shared__ int s_x[1 + ROW_WAVES];
 
     const int tid = threadIdx.x, row = blockIdx.x;
     const int V = a.V, k = a.top_k;
     const float *x = a.logits + (long long)row * a.row_stride;
-    if (row == 0 && tid == 0) *a.fb_count_next = 0;                  // the queue slot of the next step starts empty
 
     const int n4 = (V + 3) >> 2;
     const int iters = (n4 + ROW_BLOCK - 1) / ROW_BLOCK;             // float4 blocks per thread
@@ -159,7 +310,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     const float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
 
     // ---- the pass over the row
-    uint2 *list = L[wave_id()];
+    uint2 *list = L + wave_id() * ROW_WCAP;
     u32 count = 0;
     {
         int s = 0;
@@ -226,7 +377,11 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         for (int e = lane_id(); e < cw; e += WAVE) {
             const uint2 c = list[e];
             if (ordkey(__uint_as_float(c.x)) >= t2key) {
-                if (pos < (u32)ROW_CAP) C[pos] = c;
+                if (pos < (u32)ROW_CAP) {
+                    C[pos] = c;
+                    u32 slot = row_hash(c.y);                        // hash of the candidate ids, for the history
+                    while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
+                }
                 pos++;
             }
         }
@@ -236,12 +391,6 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     const int n = s_n;
     bool ok = have_tw && !s_over && n >= k && n <= ROW_CAP;
 
-    // ---- hash of the candidate ids
-    if (ok && tid < n) {
-        u32 slot = row_hash(C[tid].y);
-        while (atomicCAS(&tab[slot], 0u, (u32)(tid + 1)) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
-    }
-    __syncthreads();
     BORN_STAMP(a, row, 3);
     // history: flag the candidates that were already emitted, report ids out of range
     const bool penal = a.rep != 1.0f && hlen > 0;
@@ -285,12 +434,8 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     __syncthreads();
     BORN_STAMP(a, row, 5);
     ok = ok && s_valid >= k;
-    if (!ok) {
-        if (tid == 0) {
-            const int pos = atomicAdd(a.fb_count, 1);
-            a.fb_rows[pos] = row;
-            atomicAdd(&a.counters[1], 1ull);
-        }
+    if (!ok) {                                                       // wave-uniform, workgroup-uniform
+        row_select_exact<VEC>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
         return;
     }
 
