@@ -77,17 +77,16 @@ int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg
 /* Device status since the last call of this function: 0, or BORN_ROCM_ERR_DATA if a kernel met an
  * out-of-range history id or draft token.  Synchronises `stream`. */
 int born_rocm_sampler_status(born_sampler *s, void *stream);
-/* Work counters accumulated by the kernels (diagnostics): rows sampled by the single-pass top-k kernel,
- * rows that fell back to the general kernel, rows sampled by the general kernel directly.  Synchronises. */
+/* Work counters accumulated by the kernels (diagnostics): rows the single-pass top-k kernel settled from its
+ * candidate lists, rows it had to finish by its exact (slower) selection, rows sampled by the general kernel.
+ * Synchronises. */
 int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
                                int64_t *general_rows);
 
-/* Diagnostics.  0 = choose the kernels from the configuration (default).  1 = always the general kernel.
- * For 1 <= top_k <= 64 two single-pass paths exist: 4 = one workgroup per row in one launch (what 0 selects),
- * 3 = one workgroup per 8192-logit segment followed by a per-row finish.  2 and 5 launch only the streaming
- * kernel of path 3 resp. 4 and skip the walk of the fallback queue (2 produces no tokens, 5 leaves queued rows
- * undone): for timing those kernels by themselves, never for results.  All paths implement the same fixed-point
- * pipeline and must return identical results; tests compare them. */
+/* Diagnostics.  0 = choose the kernel from the configuration (default: the single-pass kernel for
+ * 1 <= top_k <= 64 with a penalty >= 1 and a vocabulary of at most 393216, the general kernel otherwise).
+ * 1 = always the general kernel.  Both implement the same fixed-point pipeline and must return identical
+ * results; tests compare them. */
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
 
 /* Greedy decode: index of the maximum of each row, lowest index on ties — `argmax`,
