@@ -53,7 +53,7 @@ struct born_sampler {
     unsigned long long *counters;
     // spec-verify statistics:
     float *sp_mp, *sp_mq;
-    unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd;
+    unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd, *sp_part, *sp_run;
     int64_t spec_rows;
 };
 
@@ -168,7 +168,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
     void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters,
-                    s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd};
+                    s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -344,7 +344,7 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
         // grow the per-position statistics (stream-ordered use only; the old buffers are idle once synchronised)
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
         void **ps[] = {(void **)&s->sp_mp, (void **)&s->sp_mq, (void **)&s->sp_Zp,
-                       (void **)&s->sp_Zq, (void **)&s->sp_pd, (void **)&s->sp_qd};
+                       (void **)&s->sp_Zq, (void **)&s->sp_pd, (void **)&s->sp_qd, (void **)&s->sp_part, (void **)&s->sp_run};
         for (void **p : ps) {
             if (*p) (void)hipFree(*p);
             *p = nullptr;
@@ -356,6 +356,8 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
         HIP_TRY(hipMalloc((void **)&s->sp_Zq, (size_t)rows * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void **)&s->sp_pd, (size_t)rows * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void **)&s->sp_qd, (size_t)rows * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_part, (size_t)rows * SPEC_CHUNKS * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_run, (size_t)rows * SPEC_CHUNKS * 1024 * sizeof(unsigned long long)));
         s->spec_rows = rows;
     }
     SpecArgs a;
@@ -374,6 +376,8 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
     a.mp = s->sp_mp; a.mq = s->sp_mq;
     a.Zp = s->sp_Zp; a.Zq = s->sp_Zq;
     a.pd = s->sp_pd; a.qd = s->sp_qd;
+    a.part = s->sp_part;
+    a.run_mass = s->sp_run;
     a.status = s->status;
     a.mass_shift = mass_shift(vocab);
     HIP_TRY(launch_spec_verify(a, (hipStream_t)stream));

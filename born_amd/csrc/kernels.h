@@ -17,6 +17,7 @@ constexpr int WIDE_SUB_BINS = 2048;        // radix-descent digit = 11 bits
 constexpr int64_t WIDE_MAX_VOCAB = 524288; // history bitmap must fit LDS next to the histogram
 
 constexpr int ARGMAX_SEG = 8192;
+constexpr int SPEC_CHUNKS = 4;              // workgroups per sequence in the residual pass of the speculative step
 
 // Integer masses are trunc(e * 2^S) with S chosen so that a whole row sums below 2^62.
 __host__ __device__ inline int mass_shift(long long V) {
@@ -59,6 +60,8 @@ struct SpecArgs {
     // workspace: per (b, i) row statistics
     float *mp, *mq;
     unsigned long long *Zp, *Zq, *pd, *qd;
+    unsigned long long *part;     // [B][SPEC_CHUNKS] residual mass of each quarter of the rejected row
+    unsigned long long *run_mass; // [B][SPEC_CHUNKS][1024] residual mass of each thread's run of ids
     int *status;
     int mass_shift;
 };

@@ -1,72 +1,96 @@
 // Speculative-decoding accept / reject with residual max(0, p - q) resampling
-// (docs/SAMPLING_SPEC.md section 5, fixed-point layer).
+// (docs/SAMPLING_SPEC.md section 5, fixed-point layer).  Three launches:
 //
-//   spec_stats_kernel   one workgroup per (sequence, position): row maxima and integer
-//                       normalisers of the target and draft distributions, and the two
-//                       masses of the draft token.  Reads each logit row once from HBM
-//                       (the second sweep hits L2).
-//   spec_decide_kernel  one workgroup per sequence: first rejected position, then the
-//                       residual draw over that one row in ascending id order.
+//   spec_stats_kernel     one workgroup per (sequence, position, distribution): row maximum and integer
+//                         normaliser of the target or the draft distribution, and its mass of the draft token.
+//                         Vocabularies of at most 32768 are held in registers, so each logit is read
+//                         from HBM once; larger ones are swept twice (the second sweep hits the caches).
+//   spec_residual_kernel  SPEC_CHUNKS workgroups per sequence: first rejected position (every workgroup
+//                         of a sequence derives it from the statistics), then the integer mass of
+//                         max(0, p - q) over the workgroup's quarter of that one row.
+//   spec_pick_kernel      one workgroup per sequence: the per-thread masses of the quarter the residual
+//                         draw falls into are scanned and the owning thread walks its ids in ascending order.
 #include "dev_common.h"
 #include "kernels.h"
 
 namespace born {
 
 constexpr int SPEC_BLOCK = 1024;
+constexpr int SPEC_NF4 = 8;                   // float4 per thread and array that the stats kernel keeps in registers
+constexpr int SPEC_RESIDENT_V = SPEC_NF4 * SPEC_BLOCK * 4;
+
+typedef float spec_f32x4 __attribute__((ext_vector_type(4)));
 
 template <class F>
-__device__ __forceinline__ void spec_foreach2(const float *xt, const float *xd, int V, bool vec, F f) {
+__device__ __forceinline__ void spec_foreach(const float *x, int V, bool vec, F f) {
     const int tid = threadIdx.x;
     if (vec) {
         const int n4 = V >> 2;
-        const float4 *t4 = reinterpret_cast<const float4 *>(xt);
-        const float4 *d4 = reinterpret_cast<const float4 *>(xd);
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
         for (int i = tid; i < n4; i += SPEC_BLOCK) {
-            float4 a = t4[i], b = d4[i];
-            f(a.x, b.x); f(a.y, b.y); f(a.z, b.z); f(a.w, b.w);
+            float4 q = x4[i];
+            f(q.x); f(q.y); f(q.z); f(q.w);
         }
-        for (int j = (n4 << 2) + tid; j < V; j += SPEC_BLOCK) f(xt[j], xd[j]);
+        for (int j = (n4 << 2) + tid; j < V; j += SPEC_BLOCK) f(x[j]);
     } else {
-        for (int j = tid; j < V; j += SPEC_BLOCK) f(xt[j], xd[j]);
+        for (int j = tid; j < V; j += SPEC_BLOCK) f(x[j]);
     }
 }
 
+// One workgroup per (sequence, position, distribution): blockIdx.x = 2 * row + (0 target | 1 draft).  The two
+// distributions of a position are independent, and twice as many work items spread better over the CUs.
+// RESIDENT: V <= SPEC_RESIDENT_V, V % 4 == 0 and the rows 16-byte aligned.
+template <bool RESIDENT>
 __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     __shared__ BlockScratch scr;
-    const int row = blockIdx.x;
+    const int row = blockIdx.x >> 1, tid = threadIdx.x;
+    const bool is_draft = blockIdx.x & 1;
     const int V = a.V;
-    const float *xt = a.target + (long long)row * V;
-    const float *xd = a.draft + (long long)row * V;
-    const bool vec = ((V & 3) == 0) && ((((uintptr_t)a.target) & 15) == 0) && ((((uintptr_t)a.draft) & 15) == 0);
+    const float *x = (is_draft ? a.draft : a.target) + (long long)row * V;
     const float T = a.T;
-    float mp = -INFINITY, mq = -INFINITY;
-    spec_foreach2(xt, xd, V, vec, [&](float t, float d) {
-        mp = fmaxf(mp, z_of(t, T));
-        mq = fmaxf(mq, z_of(d, T));
-    });
-    mp = block_max_f32<SPEC_BLOCK>(mp, &scr);
-    mq = block_max_f32<SPEC_BLOCK>(mq, &scr);
     const float scale = mass_scale(a.mass_shift);
-    u64 sp = 0, sq = 0;
-    spec_foreach2(xt, xd, V, vec, [&](float t, float d) {
-        sp += qfix(emass(z_of(t, T), mp), scale);
-        sq += qfix(emass(z_of(d, T), mq), scale);
-    });
-    u64 Zp, Zq;
-    block_inclusive_scan_u64<SPEC_BLOCK>(sp, &scr, &Zp);
-    block_inclusive_scan_u64<SPEC_BLOCK>(sq, &scr, &Zq);
-    if (threadIdx.x == 0) {
-        int d = a.draft_tokens[row];
-        u64 pd = 0, qd = 0;
-        if (d >= 0 && d < V) {
-            pd = qfix(emass(z_of(xt[d], T), mp), scale);
-            qd = qfix(emass(z_of(xd[d], T), mq), scale);
-        } else {
-            atomicOr(a.status, 2);
+    float m = -INFINITY;
+    u64 sum = 0;
+    if (RESIDENT) {
+        const int n4 = V >> 2;
+        spec_f32x4 t[SPEC_NF4];
+#pragma unroll
+        for (int i = 0; i < SPEC_NF4; i++) {
+            const int j = i * SPEC_BLOCK + tid;
+            const spec_f32x4 fill = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            t[i] = j < n4 ? __builtin_nontemporal_load(reinterpret_cast<const spec_f32x4 *>(x) + j) : fill;
         }
-        a.mp[row] = mp; a.mq[row] = mq;
-        a.Zp[row] = Zp; a.Zq[row] = Zq;
-        a.pd[row] = pd; a.qd[row] = qd;
+#pragma unroll
+        for (int i = 0; i < SPEC_NF4; i++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                t[i][c] = z_of(t[i][c], T);                          // the -inf fill stays -inf
+                m = fmaxf(m, t[i][c]);
+            }
+        }
+        m = block_max_f32<SPEC_BLOCK>(m, &scr);
+#pragma unroll
+        for (int i = 0; i < SPEC_NF4; i++) {
+            if (i * SPEC_BLOCK + tid < n4) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) sum += qfix(emass(t[i][c], m), scale);
+            }
+        }
+    } else {
+        const bool vec = ((V & 3) == 0) && ((((uintptr_t)a.target) & 15) == 0) && ((((uintptr_t)a.draft) & 15) == 0);
+        spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, z_of(v, T)); });
+        m = block_max_f32<SPEC_BLOCK>(m, &scr);
+        spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(z_of(v, T), m), scale); });
+    }
+    u64 Z;
+    block_inclusive_scan_u64<SPEC_BLOCK>(sum, &scr, &Z);
+    if (tid == 0) {
+        const int dt = a.draft_tokens[row];
+        u64 md = 0;                                                  // mass of the draft token in this distribution
+        if (dt >= 0 && dt < V) md = qfix(emass(z_of(x[dt], T), m), scale);
+        else atomicOr(a.status, 2);
+        if (is_draft) { a.mq[row] = m; a.Zq[row] = Z; a.qd[row] = md; }
+        else { a.mp[row] = m; a.Zp[row] = Z; a.pd[row] = md; }
     }
 }
 
@@ -78,49 +102,121 @@ __device__ __forceinline__ u64 residual_mass(float t, float d, float T, float mp
     return (u64)(r * scale_d);
 }
 
-__global__ __launch_bounds__(SPEC_BLOCK) void spec_decide_kernel(SpecArgs a) {
+// First position of sequence b whose draft token is rejected (G if none): accept iff u * q(d) * Zp < p(d) * Zq.
+// Called by one whole wave: lane i tests positions i, i + 64, ...; the lowest rejecting position wins.
+__device__ __forceinline__ int spec_first_rejection(const SpecArgs &a, int b) {
+    for (int i0 = 0; i0 < a.G; i0 += WAVE) {
+        const int i = i0 + lane_id();
+        bool reject = false;
+        if (i < a.G) {
+            const int row = b * a.G + i;
+            const double lhs = (double)a.u_acc[row] * (double)a.qd[row] * (double)a.Zp[row];
+            const double rhs = (double)a.pd[row] * (double)a.Zq[row];
+            reject = !(lhs < rhs);
+        }
+        const u64 m = __ballot(reject);
+        if (m) return i0 + __builtin_ctzll(m);
+    }
+    return a.G;
+}
+
+// The ids of a row are cut into SPEC_CHUNKS quarters, each quarter into one contiguous run per thread, so that
+// thread order is ascending id order.  Returns the run [j0, j1) of this thread in quarter c.
+__device__ __forceinline__ void spec_run(int V, int c, int tid, int &j0, int &j1) {
+    const int per_chunk = (V + SPEC_CHUNKS - 1) / SPEC_CHUNKS;
+    const int lo = min(c * per_chunk, V), hi = min(lo + per_chunk, V);
+    const int per = (per_chunk + SPEC_BLOCK - 1) / SPEC_BLOCK;
+    j0 = min(lo + tid * per, hi);
+    j1 = min(j0 + per, hi);
+}
+
+struct SpecRow {
+    const float *xt, *xd;
+    float T, mp, mq, scale;
+    double Zp, Zq, scale_d;
+};
+__device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int row) {
+    SpecRow r;
+    r.xt = a.target + (long long)row * a.V;
+    r.xd = a.draft + (long long)row * a.V;
+    r.T = a.T;
+    r.mp = a.mp[row];
+    r.mq = a.mq[row];
+    r.scale = mass_scale(a.mass_shift);
+    r.Zp = (double)a.Zp[row];
+    r.Zq = (double)a.Zq[row];
+    r.scale_d = ldexp(1.0, a.mass_shift);
+    return r;
+}
+constexpr int SPEC_RUN = 8;                   // run lengths up to this are loaded before any arithmetic
+__device__ __forceinline__ u64 spec_run_mass(const SpecRow &r, int j0, int j1) {
+    u64 local = 0;
+    if (j1 - j0 <= SPEC_RUN) {
+        float tv[SPEC_RUN], dv[SPEC_RUN];
+#pragma unroll
+        for (int i = 0; i < SPEC_RUN; i++) {
+            const int j = min(j0 + i, j1 - 1);
+            tv[i] = j0 < j1 ? r.xt[j] : 0.0f;
+            dv[i] = j0 < j1 ? r.xd[j] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < SPEC_RUN; i++)
+            if (j0 + i < j1) local += residual_mass(tv[i], dv[i], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+    } else {
+        for (int j = j0; j < j1; j++) local += residual_mass(r.xt[j], r.xd[j], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+    }
+    return local;
+}
+
+__global__ __launch_bounds__(SPEC_BLOCK) void spec_residual_kernel(SpecArgs a) {
     __shared__ BlockScratch scr;
     __shared__ int s_first;
+    const int b = blockIdx.x / SPEC_CHUNKS, c = blockIdx.x % SPEC_CHUNKS, tid = threadIdx.x;
+    if (tid < WAVE) {
+        const int first = spec_first_rejection(a, b);
+        if (tid == 0) {
+            s_first = first;
+            if (c == 0) {
+                a.n_accepted[b] = first;
+                if (first == a.G) a.next_token[b] = -1;
+            }
+        }
+    }
+    __syncthreads();
+    const int first = s_first;
+    if (first == a.G) return;
+    const SpecRow r = spec_row(a, b * a.G + first);
+    int j0, j1;
+    spec_run(a.V, c, tid, j0, j1);
+    const u64 local = spec_run_mass(r, j0, j1);
+    a.run_mass[(long long)blockIdx.x * SPEC_BLOCK + tid] = local;    // the pick reads the quarter it needs
+    u64 R;
+    block_inclusive_scan_u64<SPEC_BLOCK>(local, &scr, &R);
+    if (tid == 0) a.part[b * SPEC_CHUNKS + c] = R;
+}
+
+__global__ __launch_bounds__(SPEC_BLOCK) void spec_pick_kernel(SpecArgs a) {
+    __shared__ BlockScratch scr;
     __shared__ float s_bv[SPEC_BLOCK / WAVE];
     __shared__ int s_bi[SPEC_BLOCK / WAVE];
     const int b = blockIdx.x, tid = threadIdx.x;
     const int G = a.G, V = a.V;
-    if (tid == 0) {
-        int first = G;
-        for (int i = 0; i < G; i++) {
-            int row = b * G + i;
-            double lhs = (double)a.u_acc[row] * (double)a.qd[row] * (double)a.Zp[row];
-            double rhs = (double)a.pd[row] * (double)a.Zq[row];
-            if (!(lhs < rhs)) { first = i; break; }
-        }
-        s_first = first;
-        a.n_accepted[b] = first;
-        if (first == G) a.next_token[b] = -1;
-    }
-    __syncthreads();
-    const int first = s_first;
+    const int first = a.n_accepted[b];                               // written by the residual launch
     if (first == G) return;
-
     const int row = b * G + first;
-    const float *xt = a.target + (long long)row * V;
-    const float *xd = a.draft + (long long)row * V;
-    const float T = a.T, mp = a.mp[row], mq = a.mq[row];
-    const float scale = mass_scale(a.mass_shift);
-    const double Zp = (double)a.Zp[row], Zq = (double)a.Zq[row];
-    const double scale_d = ldexp(1.0, a.mass_shift);
-    // contiguous id ranges per thread keep the cumulative sum in ascending id order
-    const int chunk = (V + SPEC_BLOCK - 1) / SPEC_BLOCK;
-    const int j0 = min(tid * chunk, V), j1 = min(j0 + chunk, V);
-    u64 local = 0;
-    for (int j = j0; j < j1; j++) local += residual_mass(xt[j], xd[j], T, mp, mq, scale, Zp, Zq, scale_d);
-    u64 R;
-    u64 inc = block_inclusive_scan_u64<SPEC_BLOCK>(local, &scr, &R);
+    u64 part[SPEC_CHUNKS], R = 0;
+#pragma unroll
+    for (int c = 0; c < SPEC_CHUNKS; c++) {
+        part[c] = a.part[b * SPEC_CHUNKS + c];
+        R += part[c];
+    }
     if (R == 0) {
         // residual vanished in fixed point: the target's argmax, lowest id on ties
+        const float *xt = a.target + (long long)row * V;
         float bv = -INFINITY;
         int bi = 0x7FFFFFFF;
         for (int j = tid; j < V; j += SPEC_BLOCK) {
-            float z = z_of(xt[j], T);
+            float z = z_of(xt[j], a.T);
             if (z > bv || (z == bv && j < bi)) { bv = z; bi = j; }
         }
 #pragma unroll
@@ -138,24 +234,47 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_decide_kernel(SpecArgs a) {
         }
         return;
     }
-    const u64 td = draw_target(a.u_res[b], R);
+    const u64 td = draw_target(a.u_res[b], R);                       // 1 <= td <= R
+    int c = 0;
+    u64 before = 0;                                                  // residual mass of the quarters before c
+#pragma unroll
+    for (int i = 0; i < SPEC_CHUNKS - 1; i++) {
+        if (c == i && before + part[i] < td) {
+            before += part[i];
+            c = i + 1;
+        }
+    }
+    const SpecRow r = spec_row(a, row);
+    int j0, j1;
+    spec_run(V, c, tid, j0, j1);
+    const u64 local = a.run_mass[((long long)b * SPEC_CHUNKS + c) * SPEC_BLOCK + tid];
+    u64 Rc;
+    const u64 inc = before + block_inclusive_scan_u64<SPEC_BLOCK>(local, &scr, &Rc);
     const u64 excl = inc - local;
-    if (excl < td && td <= inc) {                     // exactly one thread owns the crossing
-        u64 c = excl;
+    if (excl < td && td <= inc) {                                    // exactly one thread owns the crossing
+        u64 acc = excl;
         int tok = j1 - 1;
         for (int j = j0; j < j1; j++) {
-            c += residual_mass(xt[j], xd[j], T, mp, mq, scale, Zp, Zq, scale_d);
-            if (c >= td) { tok = j; break; }
+            acc += residual_mass(r.xt[j], r.xd[j], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+            if (acc >= td) { tok = j; break; }
         }
         a.next_token[b] = tok;
     }
 }
 
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st) {
-    hipLaunchKernelGGL(spec_stats_kernel, dim3((unsigned)(a.B * a.G)), dim3(SPEC_BLOCK), 0, st, a);
+    const bool resident = a.V <= SPEC_RESIDENT_V && (a.V & 3) == 0 && ((((uintptr_t)a.target) & 15) == 0) &&
+                          ((((uintptr_t)a.draft) & 15) == 0);
+    if (resident)
+        hipLaunchKernelGGL(spec_stats_kernel<true>, dim3((unsigned)(2 * a.B * a.G)), dim3(SPEC_BLOCK), 0, st, a);
+    else
+        hipLaunchKernelGGL(spec_stats_kernel<false>, dim3((unsigned)(2 * a.B * a.G)), dim3(SPEC_BLOCK), 0, st, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(spec_decide_kernel, dim3((unsigned)a.B), dim3(SPEC_BLOCK), 0, st, a);
+    hipLaunchKernelGGL(spec_residual_kernel, dim3((unsigned)(a.B * SPEC_CHUNKS)), dim3(SPEC_BLOCK), 0, st, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(spec_pick_kernel, dim3((unsigned)a.B), dim3(SPEC_BLOCK), 0, st, a);
     return hipGetLastError();
 }
 
