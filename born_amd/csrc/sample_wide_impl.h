@@ -30,7 +30,13 @@ __device__ __forceinline__ int wide_bin(float d) {
     return d < 32.0f ? (int)(d * WIDE_BINS_PER_UNIT) : WIDE_BINS - 1;     // monotone in d; inf -> last bin
 }
 
-// Visit every element of the row as (id, z).  Aligned rows are read in stages of WIDE_U float4 per thread, the
+// z of a penalised logit (uniform branch: no division at temperature 1)
+__device__ __forceinline__ float wide_z(const WideCtx &c, float y) {
+    if (c.T == 1.0f) return canon(y);
+    return canon(y / c.T);
+}
+
+// Visit every element of the row as (id, penalised logit).  Aligned rows are read in stages of WIDE_U float4 per thread, the
 // loads of the next stage in flight while this one is visited (the loop body has no branch around a load, so
 // the compiler can wait for exactly the stage it needs); what is left of the row is read block by block.
 constexpr int WIDE_U = 4;
@@ -54,7 +60,7 @@ __device__ __forceinline__ void wide_visit4(const WideCtx &c, const wide_f32x4 &
         }
     }
 #pragma unroll
-    for (int t = 0; t < 4; t++) f(j + t, z_of(y[t], c.T));
+    for (int t = 0; t < 4; t++) f(j + t, y[t]);
 }
 
 template <class F>
@@ -88,13 +94,13 @@ __device__ __forceinline__ void wide_foreach(const WideCtx &c, F f) {
         for (int j = (n4 << 2) + tid; j < c.V; j += WIDE_BLOCK) {
             float y = c.x[j];
             if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, c.rep);
-            f(j, z_of(y, c.T));
+            f(j, y);
         }
     } else {
         for (int j = tid; j < c.V; j += WIDE_BLOCK) {
             float y = c.x[j];
             if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, c.rep);
-            f(j, z_of(y, c.T));
+            f(j, y);
         }
     }
 }
@@ -203,7 +209,8 @@ template <class P>
 __device__ __forceinline__ int wide_collect(const WideCtx &c, P pred) {
     if (threadIdx.x == 0) c.s_int[1] = 0;
     __syncthreads();
-    wide_foreach(c, [&](int j, float z) {
+    wide_foreach(c, [&](int j, float y) {
+        const float z = wide_z(c, y);
         float d = (z == c.m) ? 0.0f : c.m - z;
         if (!c.count_mode && !(d <= 80.0f)) return;            // zero mass: invisible to mass-only selection
         u64 key = make_key64(z, j);
@@ -240,7 +247,8 @@ __device__ __noinline__ Found wide_descend(const WideCtx &c, int b, bool by_coun
             scnt[i] = 0;
         }
         __syncthreads();
-        wide_foreach(c, [&](int j, float z) {
+        wide_foreach(c, [&](int j, float y) {
+            const float z = wide_z(c, y);
             float d = (z == c.m) ? 0.0f : c.m - z;
             if (wide_bin(d) != b) return;
             u64 key = make_key64(z, j);
@@ -363,8 +371,9 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     BORN_STAMP(a, row, 1);
     // ---- sweep 1: row maximum of z
     float mx = -INFINITY;
-    wide_foreach(c, [&](int, float z) { mx = fmaxf(mx, z); });
-    c.m = uniform_f32(block_max_f32<WIDE_BLOCK>(mx, (BlockScratch *)scr));
+    // (z is a non-decreasing function of the penalised logit, so the maximum is taken before the division)
+    wide_foreach(c, [&](int, float y) { mx = fmaxf(mx, y); });
+    c.m = uniform_f32(wide_z(c, block_max_f32<WIDE_BLOCK>(mx, (BlockScratch *)scr)));
 
     BORN_STAMP(a, row, 2);
     // ---- sweep 2: histogram over d = m - z (integer masses; counts only when a top-k cut is needed)
@@ -373,7 +382,8 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
         c.cnt[i] = 0;
     }
     __syncthreads();
-    wide_foreach(c, [&](int, float z) {
+    wide_foreach(c, [&](int, float y) {
+        const float z = wide_z(c, y);
         float d = (z == c.m) ? 0.0f : c.m - z;
         int b = wide_bin(d);
         if (c.count_mode) lds_add(c.cnt + b, 1u);
