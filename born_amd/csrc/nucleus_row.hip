@@ -1,0 +1,366 @@
+// Sampler for top_k disabled (full-vocabulary multinomial and top-p): one workgroup of 1024 threads per
+// row, three sweeps over the row (docs/SAMPLING_SPEC.md, fixed-point layer).
+//
+//   sweep 1  maximum and smallest finite value of the penalised logits (z is a non-decreasing function of
+//            the penalised logit, so no division is needed yet): m = z(max), and the span of d = m - z.
+//   sweep 2  integer masses trunc(expneg(d) * 2^S) accumulated into 4096 bins that cover exactly that span
+//            (u64 LDS atomics), then an inclusive scan: cumulative mass in rank order, bin by bin.
+//   targets  the top-p cut target ceil(p * Z) and the draw target each fall into one bin; the draw's bin is
+//            predicted from the interval the nucleus mass must lie in, so one gather usually serves both.
+//   sweep 3  gather: a compare of the penalised logit against the wanted bins' value ranges (widened, so
+//            that it can only over-select) stages about 1 % of the row in per-wave LDS lists (ballot + lane
+//            rank); the staged entries are then classified exactly.
+//   resolve  every gathered entry sums the masses of the entries of its bin that rank at or above it; the
+//            first entry in rank order whose cumulative mass reaches a target is found with an LDS max.
+// Rows this cannot settle (a wanted bin too full for the lists: heavy ties, masked rows) are queued for the
+// general kernel, which walks the queue in the next launch.
+#include "dev_common.h"
+#include "kernels.h"
+
+namespace born {
+
+constexpr int NUC_BLOCK = 1024;
+constexpr int NUC_WAVES = NUC_BLOCK / WAVE;
+constexpr int NUC_U = 4;                      // 128-bit loads per thread and stage
+constexpr int NUC_BINS = 4096;
+constexpr int NUC_WCAP = 160;                 // staged entries per wave
+constexpr int NUC_CAP = 1024;                 // gathered entries (one per thread)
+constexpr int NUC_PER = NUC_BINS / NUC_BLOCK; // bins per thread in the scan
+
+typedef float nuc_f32x4 __attribute__((ext_vector_type(4)));
+
+struct NucRow {                               // uniform per workgroup
+    const float *x;
+    int V;
+    bool vec, penal, degenerate;
+    float T, rep, m, scale, range, sbin;
+};
+
+__device__ __forceinline__ float nuc_z(const NucRow &r, float y) {
+    if (r.T == 1.0f) return canon(y);
+    return canon(y / r.T);
+}
+__device__ __forceinline__ float nuc_d(const NucRow &r, float z) { return r.degenerate ? 0.0f : r.m - z; }
+__device__ __forceinline__ int nuc_bin(const NucRow &r, float d) {
+    return d < r.range ? min((int)(d * r.sbin), NUC_BINS - 1) : NUC_BINS - 1;   // monotone in d; NaN and inf -> last bin
+}
+
+// Visits every element of the row as f(id, penalised logit); aligned rows in stages of NUC_U float4 per thread,
+// the next stage's loads in flight while this one is visited.
+template <class F>
+__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
+    const int tid = threadIdx.x;
+    auto visit4 = [&](const nuc_f32x4 &q, int j) {
+        float y[4] = {q[0], q[1], q[2], q[3]};
+        if (r.penal) {
+            const u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
+            if (bits) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    if ((bits >> t) & 1u) y[t] = penalise(y[t], r.rep);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) f(j + t, y[t]);
+    };
+    if (r.vec) {
+        const int n4 = r.V >> 2;
+        const int nfull = n4 / (NUC_U * NUC_BLOCK);
+        const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
+        if (nfull > 0) {
+            nuc_f32x4 va[NUC_U], vb[NUC_U];
+#pragma unroll
+            for (int u = 0; u < NUC_U; u++) va[u] = x4[u * NUC_BLOCK + tid];
+            for (int s = 0; s + 1 < nfull; s++) {
+#pragma unroll
+                for (int u = 0; u < NUC_U; u++) vb[u] = x4[((s + 1) * NUC_U + u) * NUC_BLOCK + tid];
+#pragma unroll
+                for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
+#pragma unroll
+                for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
+            }
+#pragma unroll
+            for (int u = 0; u < NUC_U; u++) visit4(va[u], (((nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+        }
+        for (int i = nfull * NUC_U * NUC_BLOCK + tid; i < n4; i += NUC_BLOCK) {
+            const nuc_f32x4 q = x4[i];
+            visit4(q, i << 2);
+        }
+        for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) {
+            float y = r.x[j];
+            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, r.rep);
+            f(j, y);
+        }
+    } else {
+        for (int j = tid; j < r.V; j += NUC_BLOCK) {
+            float y = r.x[j];
+            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, r.rep);
+            f(j, y);
+        }
+    }
+}
+
+// smallest bin whose inclusive cumulative mass reaches target
+__device__ __forceinline__ int nuc_first_reaching(const u64 *cum, u64 target) {
+    int lo = 0, hi = NUC_BINS - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (cum[mid] >= target) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+}
+
+// Range of penalised logits that can fall into bin w, widened so that it can only over-select.
+__device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, float &yhi) {
+    if (r.degenerate) {
+        ylo = -INFINITY;
+        yhi = INFINITY;
+        return;
+    }
+    const float dlo = (float)w / r.sbin, dhi = (float)(w + 1) / r.sbin;
+    const float sl = 1e-4f + 4e-6f * (fabsf(r.m) + dhi);
+    const float zhi = r.m - dlo + sl, zlo = r.m - dhi - sl;
+    yhi = zhi * r.T;
+    ylo = zlo * r.T;
+    yhi += 4e-6f * fabsf(yhi) + 1e-30f;
+    ylo -= 4e-6f * fabsf(ylo) + 1e-30f;
+    if (w == NUC_BINS - 1) ylo = -INFINITY;                          // the last bin also takes everything beyond the span
+    if (w == 0) yhi = INFINITY;
+}
+
+__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
+    extern __shared__ u64 nuc_dyn[];
+    __shared__ BlockScratch scr;
+    __shared__ int s_n, s_over;
+    __shared__ u64 s_win, s_mass;
+
+    u64 *const mass = nuc_dyn;                                                   // [NUC_BINS] masses, then cumulative
+    uint2 *const stage = reinterpret_cast<uint2 *>(nuc_dyn + NUC_BINS);          // [NUC_WAVES][NUC_WCAP] (logit bits, id)
+    u64 *const fkey = nuc_dyn + NUC_BINS + NUC_WAVES * NUC_WCAP;                 // [NUC_CAP] rank keys of the gathered entries
+    u64 *const fq = fkey + NUC_CAP;                                              // [NUC_CAP] mass | slot << 62
+    u32 *const bm = reinterpret_cast<u32 *>(fq + NUC_CAP);                       // history bitmap, one bit per id
+
+    const int tid = threadIdx.x, row = blockIdx.x;
+    const int V = a.V;
+    if (row == 0 && tid == 0) *a.fb_count_next = 0;                  // the queue of the next step starts empty
+
+    NucRow r;
+    r.x = a.logits + (long long)row * a.row_stride;
+    r.V = V;
+    r.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
+    r.T = a.T;
+    r.rep = a.rep;
+    r.scale = mass_scale(a.mass_shift);
+    const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
+
+    // ---- history bitmap
+    const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
+    const int *h = a.history + (long long)row * a.hist_stride;
+    r.penal = (a.rep != 1.0f) && hlen > 0;
+    if (r.penal)
+        for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
+    for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;
+    if (tid == 0) {
+        s_n = 0;
+        s_over = 0;
+        s_win = 0ull;
+    }
+    __syncthreads();
+    for (int i = tid; i < hlen; i += NUC_BLOCK) {
+        const int t = h[i];
+        if (t < 0 || t >= V) atomicOr(a.status, 1);
+        else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
+    }
+    __syncthreads();
+
+    // ---- sweep 1: maximum and smallest finite penalised logit
+    {
+        float mx = -INFINITY, mn = INFINITY;
+        nuc_foreach(r, bm, [&](int, float y) {
+            mx = fmaxf(mx, y);
+            mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
+        });
+        mx = block_max_f32<NUC_BLOCK>(mx, &scr);
+        mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
+        r.m = uniform_f32(nuc_z(r, mx));
+        r.degenerate = r.m == -INFINITY;                             // nothing finite: every d is 0 by definition
+        const float zmin = mn < INFINITY ? nuc_z(r, mn) : r.m;
+        const float span = r.degenerate ? 0.0f : r.m - zmin;         // >= 0
+        r.range = uniform_f32(fminf(32.0f, span * 1.0001f + 1e-3f));
+        r.sbin = uniform_f32((float)NUC_BINS / r.range);
+    }
+
+    // ---- sweep 2: integer masses by bin
+    nuc_foreach(r, bm, [&](int, float y) {
+        const float d = nuc_d(r, nuc_z(r, y));
+        atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d), r.scale));
+    });
+    __syncthreads();
+    u64 Zk;
+    {
+        u64 v[NUC_PER], local = 0;
+#pragma unroll
+        for (int t = 0; t < NUC_PER; t++) {
+            local += mass[tid * NUC_PER + t];
+            v[t] = local;
+        }
+        const u64 excl = block_inclusive_scan_u64<NUC_BLOCK>(local, &scr, &Zk) - local;
+#pragma unroll
+        for (int t = 0; t < NUC_PER; t++) mass[tid * NUC_PER + t] = v[t] + excl;
+    }
+    __syncthreads();
+    const u64 *cum = mass;
+
+    // ---- the bins to gather: the top-p cut's, and the draw's predicted from the interval [tp, cum[bp]]
+    const bool cut = a.top_p < 1.0f;
+    u64 tp = Zk;
+    int w0, w1, w2;
+    if (cut) {
+        tp = top_p_target(a.top_p, Zk);
+        w0 = nuc_first_reaching(cum, tp);
+        const u64 hi = cum[w0] < Zk ? cum[w0] : Zk;
+        w1 = nuc_first_reaching(cum, draw_target(u, tp));
+        w2 = nuc_first_reaching(cum, draw_target(u, hi));
+        if (w2 - w1 > 1) w1 = w2 = w0;
+    } else {
+        w0 = w1 = w2 = nuc_first_reaching(cum, draw_target(u, Zk));
+    }
+
+    bool ok = true;
+    u64 Zp = Zk, tokkey = 0ull;
+    // One or two rounds: the second only if the draw's bin was not among the predicted ones.
+    for (int round = 0; round < 2; round++) {
+        // ---- sweep 3: stage the logits inside the wanted bins' ranges, then classify them exactly
+        float lo0, hi0, lo1, hi1, lo2, hi2;
+        nuc_range(r, w0, lo0, hi0);
+        nuc_range(r, w1, lo1, hi1);
+        nuc_range(r, w2, lo2, hi2);
+        uint2 *list = stage + wave_id() * NUC_WCAP;
+        u32 count = 0;
+        nuc_foreach(r, bm, [&](int j, float y) {
+            const bool pass = (!(y < lo0) && !(y > hi0)) || (!(y < lo1) && !(y > hi1)) || (!(y < lo2) && !(y > hi2));
+            const u64 mk = __ballot(pass);
+            if (mk) {                                                // wave-uniform
+                if (pass) {
+                    const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                    if (pos < (u32)NUC_WCAP) list[pos] = make_uint2(__float_as_uint(y), (u32)j);
+                }
+                count += (u32)__popcll(mk);
+            }
+        });
+        if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
+        const int cw = (int)min(count, (u32)NUC_WCAP);
+        for (int e0 = 0; e0 < cw; e0 += WAVE) {
+            const int e = e0 + lane_id();
+            bool take = false;
+            u64 key = 0ull, qs = 0ull;
+            if (e < cw) {
+                const uint2 c = list[e];
+                const float z = nuc_z(r, __uint_as_float(c.x));
+                const float d = nuc_d(r, z);
+                const int b = nuc_bin(r, d);
+                const int slot = b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+                if (slot >= 0) {
+                    take = true;
+                    key = make_key64(z, (int)c.y);
+                    qs = qfix(expneg(d), r.scale) | ((u64)slot << 62);
+                }
+            }
+            const u64 mk = __ballot(take);
+            if (mk) {
+                int base = 0;
+                if (lane_id() == 0) base = atomicAdd(&s_n, __popcll(mk));
+                base = __builtin_amdgcn_readfirstlane(base);
+                if (take) {
+                    const int pos = base + (int)__builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                    if (pos < NUC_CAP) {
+                        fkey[pos] = key;
+                        fq[pos] = qs;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int n = s_n;
+        if (s_over || n > NUC_CAP) {
+            ok = false;
+            break;
+        }
+        // ---- resolve: cumulative mass of every entry within its bin, in rank order
+        u64 mykey = 0ull, mine = 0ull;                               // inclusive mass at and above this entry in its bin
+        int myslot = -1;
+        if (tid < n) {
+            mykey = fkey[tid];
+            const u64 q = fq[tid];
+            myslot = (int)(q >> 62);
+            for (int j = 0; j < n; j++) {
+                const u64 kj = fkey[j], qj = fq[j];
+                if ((int)(qj >> 62) == myslot && kj >= mykey) mine += qj & 0x3FFFFFFFFFFFFFFFull;
+            }
+        }
+        // first entry in rank order (largest key) of bin `slot` at which base + cumulative reaches target
+        auto first_at = [&](int slot, u64 base, u64 target, u64 &key_out, u64 &mass_out) {
+            if (myslot == slot && base + mine >= target) atomicMax(&s_win, mykey);
+            __syncthreads();
+            const u64 win = s_win;
+            if (myslot == slot && mykey == win) s_mass = base + mine;
+            __syncthreads();
+            key_out = win;
+            mass_out = s_mass;
+            __syncthreads();
+            if (tid == 0) s_win = 0ull;
+            __syncthreads();
+        };
+        if (round == 0 && cut) {
+            u64 kcut;
+            first_at(0, w0 ? cum[w0 - 1] : 0ull, tp, kcut, Zp);
+            if (kcut == 0ull) {                                      // cannot happen for a consistent histogram: fail safe
+                ok = false;
+                break;
+            }
+        }
+        const u64 td = draw_target(u, Zp);
+        const int bd = nuc_first_reaching(cum, td);
+        const int slot = bd == w0 ? 0 : bd == w1 ? 1 : bd == w2 ? 2 : -1;
+        if (slot >= 0) {
+            u64 mdraw;
+            first_at(slot, bd ? cum[bd - 1] : 0ull, td, tokkey, mdraw);
+            break;
+        }
+        // the prediction missed: gather the draw's bin alone
+        w0 = w1 = w2 = bd;
+        if (tid == 0) s_n = 0;
+        __syncthreads();
+        if (round == 1) ok = false;
+    }
+    if (!ok || tokkey == 0ull) {
+        if (tid == 0) {
+            const int pos = atomicAdd(a.fb_count, 1);
+            a.fb_rows[pos] = row;
+            atomicAdd(&a.counters[1], 1ull);
+        }
+        return;
+    }
+    if (tid == 0) {
+        a.tokens[row] = key64_id(tokkey);
+        if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m), Zp, a.mass_shift);
+        if (a.nuc_len) a.nuc_len[row] = -1;                          // the nucleus listing is only produced for small top-k
+        atomicAdd(&a.counters[2], 1ull);
+    }
+}
+
+size_t nucleus_lds_bytes(int V) {
+    return sizeof(u64) * (NUC_BINS + NUC_WAVES * NUC_WCAP + 2 * NUC_CAP) + sizeof(u32) * (size_t)((V + 31) / 32);
+}
+
+hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st) {
+    hipLaunchKernelGGL(nucleus_row_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a);
+    return hipGetLastError();
+}
+
+hipError_t configure_nucleus() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
+}
+
+}  // namespace born
