@@ -46,9 +46,7 @@ struct born_sampler {
     int S_max;                     // argmax segments per row at max_vocab
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // see born_rocm_sampler_set_path
-    unsigned queue_epoch;          // steps that used the fallback queue: its counter alternates between two slots
     // device workspace
-    int *fb_count, *fb_rows;       // fb_count[2]
     float *arg_val;                // argmax partials [max_batch][S_max]
     int *arg_idx;
     int *status;
@@ -158,8 +156,6 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
         if (e == hipSuccess) e = hipMalloc(p, bytes);
         if (e == hipSuccess) e = hipMemset(*p, 0, bytes);
     };
-    alloc((void **)&s->fb_count, 2 * sizeof(int));
-    alloc((void **)&s->fb_rows, rows * sizeof(int));
     alloc((void **)&s->arg_val, segs * sizeof(float));
     alloc((void **)&s->arg_idx, segs * sizeof(int));
     alloc((void **)&s->status, sizeof(int));
@@ -174,7 +170,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->fb_count, s->fb_rows, s->arg_val, s->arg_idx, s->status, s->counters,
+    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -210,8 +206,8 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (st) {
         HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s", (st & 1) ? "out-of-range history id " : "",
-                    (st & 2) ? "out-of-range draft token" : "");
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s", (st & 1) ? "out-of-range history id " : "",
+                    (st & 2) ? "out-of-range draft token " : "", (st & 4) ? "an internal inconsistency (please report)" : "");
     }
     return BORN_ROCM_OK;
 }
@@ -317,9 +313,6 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.nuc_ids = nucleus_ids_out;
     a.nuc_probs = nucleus_probs_out;
     a.nuc_cap = (int)nucleus_cap;
-    a.fb_count = s->fb_count + (s->queue_epoch & 1u);
-    a.fb_count_next = s->fb_count + ((s->queue_epoch + 1u) & 1u);
-    a.fb_rows = s->fb_rows;
     a.status = s->status;
     a.counters = s->counters;
     a.mass_shift = mass_shift(vocab);
@@ -330,14 +323,9 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
         HIP_TRY(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
     } else if (s->path != 1 && a.top_k == 0) {
-        // no top-k cut: the lean three-sweep kernel; rows it cannot settle are queued and the general kernel walks
-        // the queue.  The queue counter of the next step is zeroed by this step's first kernel (the counter of
-        // this step was zeroed by the step before), so no launch is spent on clearing it.
-        HIP_TRY(launch_nucleus_row(a, st));
-        HIP_TRY(launch_sample_wide(a, true, st));
-        s->queue_epoch++;
+        HIP_TRY(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
     } else {
-        HIP_TRY(launch_sample_wide(a, false, st));
+        HIP_TRY(launch_sample_wide(a, st));
     }
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;

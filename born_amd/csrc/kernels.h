@@ -16,8 +16,6 @@ constexpr int WIDE_LIST_CAP = 4096;        // elements the in-LDS sort can hold
 constexpr int WIDE_SUB_BINS = 2048;        // radix-descent digit = 11 bits
 constexpr int64_t WIDE_MAX_VOCAB = 524288; // history bitmap must fit LDS next to the histogram
 
-constexpr int WIDE_QUEUE_GRID = 32;         // workgroups that walk the queue of rows the nucleus kernel could not settle
-
 constexpr int ARGMAX_SEG = 8192;
 constexpr int SPEC_CHUNKS = 4;              // workgroups per sequence in the residual pass of the speculative step
 
@@ -47,11 +45,8 @@ struct SampleArgs {
     float *nuc_probs;
     int nuc_cap;
     // workspace
-    int *fb_count;                // rows queued for the general kernel in this step (nucleus kernel)
-    int *fb_count_next;           // the counter the next step will use: zeroed by the first kernel of this step
-    int *fb_rows;                 // [B] the queue
     int *status;                  // device status word
-    unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows it finished by exact selection, [2] general rows
+    unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows that needed an exact (slower) refinement, [2] rows sampled without a top-k cut or by the general kernel
     int mass_shift;
 };
 
@@ -78,7 +73,7 @@ hipError_t launch_softmax(const float *logits, int B, int V, long long stride, f
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st);
-hipError_t launch_sample_wide(const SampleArgs &a, bool from_queue, hipStream_t st);
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st);
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st);
 hipError_t configure_nucleus();
 size_t nucleus_lds_bytes(int V);

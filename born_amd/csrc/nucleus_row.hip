@@ -12,8 +12,8 @@
 //            rank); the staged entries are then classified exactly.
 //   resolve  every gathered entry sums the masses of the entries of its bin that rank at or above it; the
 //            first entry in rank order whose cumulative mass reaches a target is found with an LDS max.
-// Rows this cannot settle (a wanted bin too full for the lists: heavy ties, masked rows) are queued for the
-// general kernel, which walks the queue in the next launch.
+// A wanted bin too full for the lists (heavy ties, masked rows) is refined in place by a radix descent over
+// the rank keys of that bin, 11 bits per sweep.
 #include "dev_common.h"
 #include "kernels.h"
 
@@ -142,7 +142,6 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
 
     const int tid = threadIdx.x, row = blockIdx.x;
     const int V = a.V;
-    if (row == 0 && tid == 0) *a.fb_count_next = 0;                  // the queue of the next step starts empty
 
     NucRow r;
     r.x = a.logits + (long long)row * a.row_stride;
@@ -153,6 +152,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     r.scale = mass_scale(a.mass_shift);
     const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
+    BORN_STAMP(a, row, 0);
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
@@ -173,6 +173,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     }
     __syncthreads();
 
+    BORN_STAMP(a, row, 1);
     // ---- sweep 1: maximum and smallest finite penalised logit
     {
         float mx = -INFINITY, mn = INFINITY;
@@ -190,12 +191,14 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
         r.sbin = uniform_f32((float)NUC_BINS / r.range);
     }
 
+    BORN_STAMP(a, row, 2);
     // ---- sweep 2: integer masses by bin
     nuc_foreach(r, bm, [&](int, float y) {
         const float d = nuc_d(r, nuc_z(r, y));
         atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d), r.scale));
     });
     __syncthreads();
+    BORN_STAMP(a, row, 3);
     u64 Zk;
     {
         u64 v[NUC_PER], local = 0;
@@ -226,11 +229,9 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
         w0 = w1 = w2 = nuc_first_reaching(cum, draw_target(u, Zk));
     }
 
-    bool ok = true;
-    u64 Zp = Zk, tokkey = 0ull;
-    // One or two rounds: the second only if the draw's bin was not among the predicted ones.
-    for (int round = 0; round < 2; round++) {
-        // ---- sweep 3: stage the logits inside the wanted bins' ranges, then classify them exactly
+    BORN_STAMP(a, row, 4);
+    // ---- sweep 3: stage the logits inside the wanted bins' ranges, then classify them exactly
+    {
         float lo0, hi0, lo1, hi1, lo2, hi2;
         nuc_range(r, w0, lo0, hi0);
         nuc_range(r, w1, lo1, hi1);
@@ -280,73 +281,147 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
                 }
             }
         }
-        __syncthreads();
-        const int n = s_n;
-        if (s_over || n > NUC_CAP) {
-            ok = false;
-            break;
-        }
-        // ---- resolve: cumulative mass of every entry within its bin, in rank order
-        u64 mykey = 0ull, mine = 0ull;                               // inclusive mass at and above this entry in its bin
-        int myslot = -1;
-        if (tid < n) {
-            mykey = fkey[tid];
-            const u64 q = fq[tid];
-            myslot = (int)(q >> 62);
-            for (int j = 0; j < n; j++) {
-                const u64 kj = fkey[j], qj = fq[j];
-                if ((int)(qj >> 62) == myslot && kj >= mykey) mine += qj & 0x3FFFFFFFFFFFFFFFull;
-            }
-        }
-        // first entry in rank order (largest key) of bin `slot` at which base + cumulative reaches target
-        auto first_at = [&](int slot, u64 base, u64 target, u64 &key_out, u64 &mass_out) {
-            if (myslot == slot && base + mine >= target) atomicMax(&s_win, mykey);
-            __syncthreads();
-            const u64 win = s_win;
-            if (myslot == slot && mykey == win) s_mass = base + mine;
-            __syncthreads();
-            key_out = win;
-            mass_out = s_mass;
-            __syncthreads();
-            if (tid == 0) s_win = 0ull;
-            __syncthreads();
-        };
-        if (round == 0 && cut) {
-            u64 kcut;
-            first_at(0, w0 ? cum[w0 - 1] : 0ull, tp, kcut, Zp);
-            if (kcut == 0ull) {                                      // cannot happen for a consistent histogram: fail safe
-                ok = false;
-                break;
-            }
-        }
-        const u64 td = draw_target(u, Zp);
-        const int bd = nuc_first_reaching(cum, td);
-        const int slot = bd == w0 ? 0 : bd == w1 ? 1 : bd == w2 ? 2 : -1;
-        if (slot >= 0) {
-            u64 mdraw;
-            first_at(slot, bd ? cum[bd - 1] : 0ull, td, tokkey, mdraw);
-            break;
-        }
-        // the prediction missed: gather the draw's bin alone
-        w0 = w1 = w2 = bd;
-        if (tid == 0) s_n = 0;
-        __syncthreads();
-        if (round == 1) ok = false;
     }
-    if (!ok || tokkey == 0ull) {
-        if (tid == 0) {
-            const int pos = atomicAdd(a.fb_count, 1);
-            a.fb_rows[pos] = row;
-            atomicAdd(&a.counters[1], 1ull);
+    __syncthreads();
+    BORN_STAMP(a, row, 5);
+    const bool listed = !s_over && s_n <= NUC_CAP;                   // the wanted bins fit the lists
+    const int n = listed ? s_n : 0;
+    __syncthreads();
+
+    // ---- cumulative mass of every listed entry within its bin, in rank order
+    u64 mykey = 0ull, mine = 0ull;                                   // inclusive mass at and above this entry in its bin
+    int myslot = -1;
+    if (tid < n) {
+        mykey = fkey[tid];
+        myslot = (int)(fq[tid] >> 62);
+        for (int j = 0; j < n; j++) {
+            const u64 kj = fkey[j], qj = fq[j];
+            if ((int)(qj >> 62) == myslot && kj >= mykey) mine += qj & 0x3FFFFFFFFFFFFFFFull;
         }
-        return;
     }
+    __syncthreads();                                                 // the lists may be overwritten from here on
+
+    // ---- the cut, then the draw: each is the first element in rank order of one bin at which the cumulative
+    // mass reaches a target.  A bin that is listed is resolved from `mine`; any other bin (the lists overflowed:
+    // heavy ties, masked rows; or the draw's bin was not the predicted one) by a radix descent over the rank
+    // keys of that bin, 11 bits per sweep, until its bucket fits the list.
+    u64 Zp = Zk, tokkey = 0ull;
+    u64 *const smass = reinterpret_cast<u64 *>(stage);               // [2048] sub-histogram of masses
+    u32 *const scnt = reinterpret_cast<u32 *>(fkey);                 // [2048] and of counts
+    static_assert(NUC_WAVES * NUC_WCAP >= 2048 && NUC_CAP * 2 >= 2048, "the sub-histograms fit the list storage");
+    for (int phase = cut ? 0 : 1; phase < 2; phase++) {
+        const u64 target = phase == 0 ? tp : draw_target(u, Zp);
+        const int b = phase == 0 ? w0 : nuc_first_reaching(cum, target);
+        u64 base = b ? cum[b - 1] : 0ull;
+        const int slot = !listed ? -1 : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+        if (slot < 0) {
+            u64 prefix = 0ull;
+            int plen = 0;
+            for (;;) {
+                const int db = min(11, 64 - plen), nsb = 1 << db;
+                for (int i = tid; i < nsb; i += NUC_BLOCK) {
+                    smass[i] = 0ull;
+                    scnt[i] = 0u;
+                }
+                __syncthreads();
+                {
+                    const u64 pf = prefix;
+                    const int pl = plen;
+                    nuc_foreach(r, bm, [&](int j, float y) {
+                        const float z = nuc_z(r, y);
+                        const float d = nuc_d(r, z);
+                        if (nuc_bin(r, d) != b) return;
+                        const u64 key = make_key64(z, j);
+                        if (pl > 0 && (key >> (64 - pl)) != pf) return;
+                        const int idx = nsb - 1 - (int)((key >> (64 - pl - db)) & (u64)(nsb - 1));   // larger keys first
+                        atomicAdd(&smass[idx], qfix(expneg(d), r.scale));
+                        atomicAdd(&scnt[idx], 1u);
+                    });
+                }
+                __syncthreads();
+                {
+                    // inclusive scan over nsb <= 2048 sub-bins, two per thread
+                    const int i0 = 2 * tid, i1 = i0 + 1;
+                    const u64 c0 = i0 < nsb ? smass[i0] : 0ull, c1 = i1 < nsb ? smass[i1] : 0ull;
+                    u64 tot;
+                    const u64 excl = block_inclusive_scan_u64<NUC_BLOCK>(c0 + c1, &scr, &tot) - (c0 + c1);
+                    if (i0 < nsb) smass[i0] = excl + c0;
+                    if (i1 < nsb) smass[i1] = excl + c0 + c1;
+                }
+                __syncthreads();
+                int lo = 0, hi = nsb - 1;                            // first sub-bin at which base + cumulative reaches target
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (base + smass[mid] >= target) hi = mid; else lo = mid + 1;
+                }
+                const u32 cntb = scnt[lo];
+                base += lo ? smass[lo - 1] : 0ull;
+                prefix = (prefix << db) | (u64)(nsb - 1 - lo);
+                plen += db;
+                __syncthreads();
+                if (cntb <= (u32)NUC_CAP || plen == 64) break;
+            }
+            // list the bucket and sum within it
+            if (tid == 0) s_n = 0;
+            __syncthreads();
+            {
+                const u64 pf = prefix;
+                const int pl = plen;
+                nuc_foreach(r, bm, [&](int j, float y) {
+                    const float z = nuc_z(r, y);
+                    const float d = nuc_d(r, z);
+                    if (nuc_bin(r, d) != b) return;
+                    const u64 key = make_key64(z, j);
+                    if (pl < 64 ? (key >> (64 - pl)) != pf : key != pf) return;
+                    const int pos = atomicAdd(&s_n, 1);
+                    if (pos < NUC_CAP) {
+                        fkey[pos] = key;
+                        fq[pos] = qfix(expneg(d), r.scale);          // slot 0
+                    }
+                });
+            }
+            __syncthreads();
+            const int nb = min(s_n, NUC_CAP);
+            mykey = 0ull;
+            mine = 0ull;
+            myslot = -1;
+            if (tid < nb) {
+                mykey = fkey[tid];
+                myslot = 0;
+                for (int j = 0; j < nb; j++)
+                    if (fkey[j] >= mykey) mine += fq[j];
+            }
+            __syncthreads();
+        }
+        // first entry in rank order (largest key) of the bin at which base + cumulative reaches target
+        const int sl = slot < 0 ? 0 : slot;
+        if (myslot == sl && base + mine >= target) atomicMax(&s_win, mykey);
+        __syncthreads();
+        const u64 win = s_win;
+        if (myslot == sl && mykey == win) s_mass = base + mine;
+        __syncthreads();
+        if (phase == 0) Zp = s_mass;
+        else tokkey = win;
+        __syncthreads();
+        if (tid == 0) s_win = 0ull;
+        __syncthreads();
+        if (win == 0ull) break;                                      // inconsistent histogram: cannot happen
+    }
+    BORN_STAMP(a, row, 6);
     if (tid == 0) {
-        a.tokens[row] = key64_id(tokkey);
-        if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m), Zp, a.mass_shift);
+        if (tokkey == 0ull) {
+            atomicOr(a.status, 4);                                   // internal inconsistency, reported by the status call
+            a.tokens[row] = 0;
+            if (a.probs) a.probs[row] = 0.0f;
+        } else {
+            a.tokens[row] = key64_id(tokkey);
+            if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m), Zp, a.mass_shift);
+        }
         if (a.nuc_len) a.nuc_len[row] = -1;                          // the nucleus listing is only produced for small top-k
-        atomicAdd(&a.counters[2], 1ull);
+        atomicAdd(&a.counters[listed ? 2 : 1], 1ull);
+        if (!listed) atomicAdd(&a.counters[2], 1ull);
     }
+    BORN_STAMP(a, row, 7);
 }
 
 size_t nucleus_lds_bytes(int V) {

@@ -24,7 +24,7 @@ size_t wide_lds_bytes(int V) {
 
 namespace born {
 
-hipError_t launch_sample_wide(const SampleArgs &a, bool from_queue, hipStream_t st) { return w1024::launch(a, from_queue, st); }
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st) { return w1024::launch(a, st); }
 
 hipError_t configure_kernels() { return w1024::configure(); }
 

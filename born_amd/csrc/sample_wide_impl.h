@@ -323,7 +323,7 @@ __device__ __forceinline__ Found wide_find(const WideCtx &c, WideHeld &held, boo
 
 // The general algorithm on one row (every thread of the workgroup calls it together).
 __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds_u64 *dyn, BORN_LDS BlockScratch *scr, lds_int *s_int,
-                                         lds_u64 *s_u64, const bool count_it) {
+                                         lds_u64 *s_u64) {
     const int tid = threadIdx.x;
     const int V = a.V;
     WideCtx c;
@@ -463,27 +463,20 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
         if (a.nuc_len) a.nuc_len[row] = -1;              // the nucleus listing is only produced for small top-k
     }
     BORN_STAMP(a, row, 7);
-    if (tid == 0 && count_it) atomicAdd(&a.counters[2], 1ull);
+    if (tid == 0) atomicAdd(&a.counters[2], 1ull);
 }
 
-// from_queue == 0: one workgroup per row of the batch.  from_queue != 0: the workgroups walk the queue of rows
-// the nucleus kernel could not settle (usually empty: immediate exit).
-__global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a, int from_queue) {
+// One workgroup per row of the batch.
+__global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a) {
     extern __shared__ u64 dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_int[8];
     __shared__ u64 s_u64[4];
-    const int limit = from_queue ? *a.fb_count : a.B;
-    for (int i = blockIdx.x; i < limit; i += gridDim.x) {            // one call site, so the row routine is inlined once
-        wide_row(a, from_queue ? a.fb_rows[i] : i, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64,
-                 !from_queue);
-        __syncthreads();
-    }
+    wide_row(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
 }
 
-hipError_t launch(const SampleArgs &a, bool from_queue, hipStream_t st) {
-    const unsigned grid = from_queue ? (unsigned)(a.B < WIDE_QUEUE_GRID ? a.B : WIDE_QUEUE_GRID) : (unsigned)a.B;
-    hipLaunchKernelGGL(sample_wide_kernel, dim3(grid), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a, from_queue ? 1 : 0);
+hipError_t launch(const SampleArgs &a, hipStream_t st) {
+    hipLaunchKernelGGL(sample_wide_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a);
     return hipGetLastError();
 }
 
