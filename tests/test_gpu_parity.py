@@ -233,8 +233,25 @@ def test_topk_and_general_kernels_agree(oracle, rocm, path):
     assert np.array_equal(a["probs"].view(np.uint32), b["probs"].view(np.uint32))
 
 
-# ---------------------------------------------------------------- sampling: general kernel
+def test_kernel_selection_by_shape(oracle, rocm):
+    """A vocabulary beyond the single-pass kernel's limit takes the general kernel; no top-k cut takes the
+    three-sweep kernel; a general-kernel run of the same input agrees bit for bit."""
+    rng = np.random.default_rng(17)
+    B, V = 2, 400000
+    x = (rng.standard_normal((B, V), dtype=np.float32) * 2).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, 64)).astype(np.int32)
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, 0.9, 50, 0.9, 1.2, hist, nuc=64)
+    assert got["counters"]["general_rows"] == B and got["counters"]["topk_rows"] == 0
+    a = _run(rocm, x, u, 0.9, 0, 0.9, 1.2, hist, path=0)
+    b = _run(rocm, x, u, 0.9, 0, 0.9, 1.2, hist, path=1)
+    assert np.array_equal(a["tokens"], b["tokens"]) and np.array_equal(a["probs"].view(np.uint32), b["probs"].view(np.uint32))
 
+
+# ---------------------------------------------------------------- sampling: kernel without a top-k cut (path 0, top_k 0)
+# and the general kernel (path 0 for top_k > 64, path 1 for everything)
+
+@pytest.mark.parametrize("path", [0, 1])
 @pytest.mark.parametrize("B,V,T,k,p,rep,H", [
     (64, 32000, 1.0, 0, 1.0, 1.0, 0),            # C2 multinomial shape
     (16, 152064, 1.2, 0, 0.99, 1.05, 2048),      # C5 shape, 16 rows
@@ -246,35 +263,38 @@ def test_topk_and_general_kernels_agree(oracle, rocm, path):
     (5, 2, 1.0, 0, 0.9, 1.0, 0),
     (5, 1, 1.0, 0, 0.9, 1.0, 0),
 ])
-def test_general_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H):
+def test_general_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
     rng = np.random.default_rng(B * 7919 + V + k)
     x = rng.standard_normal((B, V), dtype=np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, size=(B, H)).astype(np.int32) if H else None
-    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist)
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, path=path)
     assert got["counters"]["general_rows"] == B
 
 
-def test_general_kernel_degenerate_rows(oracle, rocm):
+@pytest.mark.parametrize("path", [0, 1])
+def test_general_kernel_degenerate_rows(oracle, rocm, path):
     rng = np.random.default_rng(8)
     B, V = 12, 30000
     u = rng.random(B, dtype=np.float32)
     x = np.zeros((B, V), np.float32)                                    # every logit equal: radix descent on ids
-    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 1.0)
-    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.5)
-    _check_against_oracle(oracle, rocm, x, u, 1.0, 9000, 0.9)
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 1.0, path=path)
+    if path == 0:
+        assert got["counters"]["fallback_rows"] == B                    # ... taken by the kernel without a top-k cut
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.5, path=path)
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 9000, 0.9, path=path)
     xi = rng.integers(-1, 2, size=(B, V)).astype(np.float32)            # three values
-    _check_against_oracle(oracle, rocm, xi, u, 0.8, 0, 0.9)
-    _check_against_oracle(oracle, rocm, xi, u, 0.8, 12345, 0.9)
+    _check_against_oracle(oracle, rocm, xi, u, 0.8, 0, 0.9, path=path)
+    _check_against_oracle(oracle, rocm, xi, u, 0.8, 12345, 0.9, path=path)
     x = rng.standard_normal((B, V), dtype=np.float32)
     x[:, ::3] = -np.inf
     x[:, 1::5] = np.nan
     x[0, :] = -np.inf
     x[1, 7] = np.inf
-    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.95)
+    _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.95, path=path)
     far = rng.standard_normal((B, V), dtype=np.float32) - 200.0         # everything but one far below the maximum
     far[:, 11] = 0.0
-    _check_against_oracle(oracle, rocm, far, u, 1.0, 0, 1.0)
+    _check_against_oracle(oracle, rocm, far, u, 1.0, 0, 1.0, path=path)
 
 
 def test_builtin_uniform_stream_in_sample(oracle, rocm):
