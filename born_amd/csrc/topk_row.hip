@@ -299,7 +299,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         for (int u = 0; u < ROW_U; u++)
 #pragma unroll
             for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
-        const u32 wk = wave_kth_largest_bound(ordkey(lm), aw, 10);
+        const u32 wk = wave_kth_largest_bound(ordkey(lm), aw, 14);
         if (lane_id() == 0) s_wthr[wave_id()] = wk;
     }
     lds_barrier();
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         u32 best = 0u;
         for (int e = lane_id(); e < cw; e += WAVE) best = max(best, ordkey(__uint_as_float(list[e].x)));
         const int lanes = __popcll(__ballot(best != 0u));            // every entry is >= tw
-        const u32 wk = lanes >= a2 ? wave_kth_largest_bound(best, a2, 10, twkey) : 0u;
+        const u32 wk = lanes >= a2 ? wave_kth_largest_bound(best, a2, 14, twkey) : 0u;
         if (lane_id() == 0) s_wthr2[wave_id()] = wk;
     }
     __syncthreads();
