@@ -36,7 +36,10 @@ constexpr int ROW_WCAP = 256;                 // list entries per wave
 constexpr int ROW_CAP = 512;                  // candidates >= T2 the tail can hold
 constexpr int ROW_SLOTS = 1024;               // hash slots (load factor <= 0.5)
 constexpr int ROW_MARGIN = 16;                // candidates kept beyond top_k
+constexpr int ROW_HSLOTS = 2048;              // slots of the history hash (at most ROW_BLOCK tokens: load factor <= 0.5)
 __device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
+__device__ __forceinline__ u32 row_hhash(u32 id) { return (id * 2654435761u) >> (32 - 11); }
+static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS == 2 * ROW_BLOCK, "row_hhash produces 11 bits; two slots per thread to clear");
 static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
 static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
 static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
@@ -48,7 +51,8 @@ constexpr int OFF_C = OFF_L + ROW_WAVES * ROW_WCAP;   // [ROW_CAP] uint2
 constexpr int OFF_K = OFF_C + ROW_CAP;        // [ROW_CAP] u64
 constexpr int OFF_TAB = OFF_K + ROW_CAP;      // [ROW_SLOTS] u32
 constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [WAVE] u64
-static_assert(OFF_SORTED + WAVE <= ROW_POOL, "proof layout fits the pool");
+constexpr int OFF_HTAB = OFF_SORTED + WAVE;   // [ROW_HSLOTS] u32
+static_assert(OFF_HTAB + ROW_HSLOTS / 2 <= ROW_POOL, "proof layout fits the pool");
 constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
 constexpr int FB_DIGIT = 11;                  // key bits per sweep
 constexpr int OFF_FB_HIST = FB_BITMAP;        // [1 << FB_DIGIT] u32
@@ -254,6 +258,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     u64 *const K = pool + OFF_K;                                     // their rank keys, 0 = dropped
     u32 *const tab = reinterpret_cast<u32 *>(pool + OFF_TAB);
     u64 *const sorted = pool + OFF_SORTED;
+    u32 *const htab = reinterpret_cast<u32 *>(pool + OFF_HTAB);
     __shared__ int s_rank[ROW_BLOCK];
     __shared__ u32 s_wthr[ROW_WAVES], s_wthr2[ROW_WAVES];
     __shared__ int s_n, s_valid, s_over;
@@ -281,6 +286,12 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     }
     tab[tid] = 0u;
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
+    // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
+    // probe it at the end; a longer one probes a hash of the candidates instead.
+    const bool penal = a.rep != 1.0f && hlen > 0;
+    const bool hfast = penal && hlen <= ROW_BLOCK;
+    htab[tid] = 0u;
+    htab[tid + ROW_BLOCK] = 0u;
 
     BORN_STAMP(a, row, 0);
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
@@ -303,6 +314,18 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         if (lane_id() == 0) s_wthr[wave_id()] = wk;
     }
     lds_barrier();
+    if (hfast && tid < hlen) {
+        if (h0 < 0 || h0 >= V) {
+            atomicOr(a.status, 1);
+        } else {
+            u32 slot = row_hhash((u32)h0);
+            for (;;) {
+                const u32 old = atomicCAS(&htab[slot], 0u, (u32)h0 + 1u);
+                if (old == 0u || old == (u32)h0 + 1u) break;        // inserted, or a duplicate of an earlier occurrence
+                slot = (slot + 1) & (ROW_HSLOTS - 1);
+            }
+        }
+    }
     const u32 twkey = row_pick(s_wthr, need);
     // at or below the key of -inf: fewer than top_k finite logits in the first stage (or a vocabulary too small
     // for the counting argument); nothing is listed and the row goes to the general kernel
@@ -379,8 +402,10 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
             if (ordkey(__uint_as_float(c.x)) >= t2key) {
                 if (pos < (u32)ROW_CAP) {
                     C[pos] = c;
-                    u32 slot = row_hash(c.y);                        // hash of the candidate ids, for the history
-                    while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
+                    if (penal && !hfast) {                           // a long history probes a hash of the candidate ids
+                        u32 slot = row_hash(c.y);
+                        while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
+                    }
                 }
                 pos++;
             }
@@ -392,27 +417,28 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     bool ok = have_tw && !s_over && n >= k && n <= ROW_CAP;
 
     BORN_STAMP(a, row, 3);
-    // history: flag the candidates that were already emitted, report ids out of range
-    const bool penal = a.rep != 1.0f && hlen > 0;
-    for (int i = tid; i < hlen; i += ROW_BLOCK) {
-        const int tk = (i == tid) ? h0 : h[i];
-        if (tk < 0 || tk >= V) {
-            atomicOr(a.status, 1);
-            continue;
-        }
-        if (!(ok && penal)) continue;
-        u32 slot = row_hash((u32)tk);
-        for (;;) {
-            const u32 e = tab[slot];
-            if (e == 0u) break;
-            if ((C[e - 1].y & 0x7FFFFFFFu) == (u32)tk) {
-                atomicOr(&C[e - 1].y, 0x80000000u);
-                break;
+    if (!hfast) {
+        // long (or unpenalised) history: report ids out of range, flag the candidates that were already emitted
+        for (int i = tid; i < hlen; i += ROW_BLOCK) {
+            const int tk = (i == tid) ? h0 : h[i];
+            if (tk < 0 || tk >= V) {
+                atomicOr(a.status, 1);
+                continue;
             }
-            slot = (slot + 1) & (ROW_SLOTS - 1);
+            if (!(ok && penal)) continue;
+            u32 slot = row_hash((u32)tk);
+            for (;;) {
+                const u32 e = tab[slot];
+                if (e == 0u) break;
+                if ((C[e - 1].y & 0x7FFFFFFFu) == (u32)tk) {
+                    atomicOr(&C[e - 1].y, 0x80000000u);
+                    break;
+                }
+                slot = (slot + 1) & (ROW_SLOTS - 1);
+            }
         }
+        __syncthreads();
     }
-    __syncthreads();
     BORN_STAMP(a, row, 4);
 
     // ---- exact z; the row is proven if top_k candidates stay strictly above the bound.  A logit outside C has
@@ -423,7 +449,19 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
         if (tid < n) {
             const uint2 c = C[tid];
             float y = __uint_as_float(c.x);
-            if (c.y & 0x80000000u) y = penalise(y, a.rep);
+            bool seen = (c.y & 0x80000000u) != 0u;
+            if (hfast) {                                             // is the candidate's id in the hashed history?
+                u32 slot = row_hhash(c.y);
+                for (;;) {
+                    const u32 e = htab[slot];
+                    if (e == 0u || e == c.y + 1u) {
+                        seen = e != 0u;
+                        break;
+                    }
+                    slot = (slot + 1) & (ROW_HSLOTS - 1);
+                }
+            }
+            if (seen) y = penalise(y, a.rep);
             const float z = z_of(y, a.T);
             keep = ordkey(z) > zb;
             K[tid] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
