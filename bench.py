@@ -33,9 +33,9 @@ HBM_PEAK_GBS = 8000.0
 # script): two runs `rocprofv3 --pmc FETCH_SIZE --kernel-trace -- python3 bench.py --no-cpu --steps 20
 # --warmup 5 --copy-probe` and the same with WRITE_SIZE; each counter's per-dispatch average for the
 # kernel is scaled by what the same counter reads for the --copy-probe copy of one logits buffer
-# (131 334 144 B read and written): FETCH_SIZE 64153.3 -> factor 1.99921 KiB per unit, WRITE_SIZE
-# 128256.0 -> factor 1.0.  Kernel: FETCH_SIZE 64602.2 -> 132.25 MB read, WRITE_SIZE 24.0 -> 24 KiB written.
-PMC_TRAFFIC_BYTES = {("C3", "topk_row_kernel"): int(64602.2 * (128256 / 64153.3) * 1024 + 24.0 * 1024)}
+# (131 334 144 B read and written): FETCH_SIZE 64152.8 -> factor 1.99923 KiB per unit, WRITE_SIZE
+# 128256.0 -> factor 1.0.  Kernel: FETCH_SIZE 64603.7 -> 132.26 MB read, WRITE_SIZE 24.0 -> 24 KiB written.
+PMC_TRAFFIC_BYTES = {("C3", "topk_row_kernel"): int(64603.7 * (128256 / 64152.8) * 1024 + 24.0 * 1024)}
 
 
 def cpu_baseline(w, seconds=12.0):
