@@ -42,6 +42,8 @@ SYMBOLS = {
     "born_rocm_spec_verify": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_expneg": (C.c_int, [_vp, _vp, _i64, _vp]),
     "born_rocm_uniforms": (C.c_int, [_i64, _i64, _vp, _i64, _vp]),
+    "born_rocm_linear": (C.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _vp]),
+    "born_rocm_matmul": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
 }
 
 _lib = None

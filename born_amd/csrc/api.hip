@@ -400,4 +400,41 @@ int born_rocm_uniforms(int64_t seed, int64_t step, float *u_out, int64_t n, void
     return BORN_ROCM_OK;
 }
 
+static int gemm_entry(const char *what, const float *a, const float *b, const float *bias, float *c, int64_t m,
+                      int64_t k, int64_t n, int64_t lda, int64_t ldb, int64_t ldc, bool bt, void *stream) {
+    if (!a || !b || !c) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: null pointer", what);
+    const int64_t lim = 0x7FFFFFFF;
+    if (m <= 0 || k <= 0 || n <= 0 || m > lim - 256 || k > lim - 64 || n > lim - 256)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "%s: shape [%lld,%lld] @ [%lld,%lld] out of range", what, (long long)m,
+                    (long long)k, (long long)k, (long long)n);
+    if (lda < k || ldb < (bt ? k : n) || ldc < n)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "%s: a row pitch is smaller than the row", what);
+    GemmArgs g;
+    g.a = a;
+    g.b = b;
+    g.bias = bias;
+    g.c = c;
+    g.M = (int)m;
+    g.N = (int)n;
+    g.K = (int)k;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.ldc = ldc;
+    g.vec_a = ((uintptr_t)a & 15) == 0 && (lda & 3) == 0;
+    g.vec_b = ((uintptr_t)b & 15) == 0 && (ldb & 3) == 0;
+    HIP_TRY(launch_gemm_f32(g, bt, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t x_stride, const float *weight,
+                     int64_t out_features, int64_t w_stride, const float *bias, float *out, int64_t out_stride,
+                     void *stream) {
+    return gemm_entry("linear", x, weight, bias, out, batch, in_features, out_features, x_stride, w_stride, out_stride,
+                      true, stream);
+}
+int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                     int64_t ldb, int64_t ldc, void *stream) {
+    return gemm_entry("matmul", a, b, nullptr, c, m, k, n, lda, ldb, ldc, false, stream);
+}
+
 }  // extern "C"

@@ -66,6 +66,16 @@ struct SpecArgs {
     int mass_shift;
 };
 
+// C[M,N] = A[M,K] * B (+ bias[N]); B is [N,K] (b_transposed, the weight of a linear layer) or [K,N].
+struct GemmArgs {
+    const float *a, *b, *bias;    // bias may be null
+    float *c;
+    int M, N, K;
+    long long lda, ldb, ldc;      // row pitches in elements
+    bool vec_a, vec_b;            // 128-bit loads are legal (base 16-byte aligned, pitch a multiple of 4)
+};
+hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st);
+
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st);
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,

@@ -1,0 +1,81 @@
+"""Host-side mirror of the logits producer of the Go package `backend/rocm` (backend/rocm/linear.go).
+
+`Linear` follows nn.Linear of the reference (internal/nn/linear.go:24-140): weight `[out_features,
+in_features]`, bias `[out_features]`, Xavier-uniform weights and zero bias from `NewLinear`
+(internal/nn/init.go:24-42), `Forward` = x @ W^T + b, and the same panics on a shape mismatch.
+`MatMul` follows tensor.Backend.MatMul (internal/tensor/backend.go:20; internal/backend/cpu/matmul.go:13-50):
+2-D operands only, `[m,k] @ [k,n]`.
+
+Operands and results are device memory (a `DeviceBuffer`, a torch CUDA tensor or a raw address): the
+`[batch, vocab]` output of the LM head is what `Sampler.Sample` reads, without a host round trip.
+"""
+import math
+
+import numpy as np
+
+from . import _capi
+from .sampler import DeviceBuffer, SamplerPanic, _check, _ptr
+
+
+class LinearPanic(SamplerPanic):
+    """What the Go layer would panic with ("Linear.Forward: ..." / "matmul: ...")."""
+
+
+def MatMul(a, b, m, k, n, out, k_b=None, stream=None):
+    """out[m,n] = a[m,k] @ b[k_b,n]; panics like the CPU backend when the inner dimensions differ."""
+    if k_b is not None and k_b != k:
+        raise LinearPanic(f"matmul: shape mismatch [{m},{k}] @ [{k_b},{n}]")
+    if min(m, k, n) <= 0:
+        raise LinearPanic(f"matmul: shape mismatch [{m},{k}] @ [{k},{n}]")
+    _check(_capi.lib().born_rocm_matmul(_ptr(a), _ptr(b), _ptr(out), int(m), int(k), int(n), int(k), int(n), int(n), stream))
+    return out
+
+
+class Linear:
+    """y = x @ W^T + b on the device."""
+
+    def __init__(self, in_features, out_features, weight, bias):
+        self.inFeatures, self.outFeatures = int(in_features), int(out_features)
+        self.weight, self.bias = weight, bias
+
+    def InFeatures(self):
+        return self.inFeatures
+
+    def OutFeatures(self):
+        return self.outFeatures
+
+    def Weight(self):
+        return self.weight
+
+    def Bias(self):
+        return self.bias
+
+    def Parameters(self):
+        return [self.weight, self.bias]
+
+    def Forward(self, input, input_shape, out, stream=None):
+        """input: device fp32 `[batch, in_features]` (shape given as `input_shape`); out: device fp32
+        `[batch, out_features]`.  Returns `out`."""
+        if len(input_shape) != 2:
+            raise LinearPanic(f"Linear.Forward: expected 2D input [batch, features], got shape {list(input_shape)}")
+        batch, feat = int(input_shape[0]), int(input_shape[1])
+        if feat != self.inFeatures:
+            raise LinearPanic(f"Linear.Forward: expected input with {self.inFeatures} features, got {feat}")
+        if batch <= 0:
+            raise LinearPanic("Linear.Forward: empty batch")
+        _check(_capi.lib().born_rocm_linear(_ptr(input), batch, self.inFeatures, self.inFeatures, _ptr(self.weight),
+                                            self.outFeatures, self.inFeatures, _ptr(self.bias), _ptr(out),
+                                            self.outFeatures, stream))
+        return out
+
+
+def NewLinear(in_features, out_features, seed=None, stream=None):
+    """Xavier/Glorot-uniform weights in [-sqrt(6/(in+out)), +sqrt(6/(in+out))], zero bias, both uploaded to the
+    device.  The reference draws from the process-global unseeded generator; a seed can be given here."""
+    if in_features <= 0 or out_features <= 0:
+        raise LinearPanic("NewLinear: features must be positive")
+    bound = math.sqrt(6.0 / float(in_features + out_features))
+    rng = np.random.default_rng(seed)
+    w = ((rng.random((out_features, in_features)) * 2.0 - 1.0) * bound).astype(np.float32)
+    b = np.zeros(out_features, dtype=np.float32)
+    return Linear(in_features, out_features, DeviceBuffer.from_numpy(w, stream), DeviceBuffer.from_numpy(b, stream))

@@ -129,6 +129,25 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
                           const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out,
                           void *stream);
 
+/* The logits producer, fp32 on the matrix cores (fp32 operands, fp32 accumulation; the order of the k-sum
+ * differs from the reference's sequential loop, so results agree with it to rounding, not bit for bit).
+ *
+ * born_rocm_linear: out[batch, out_features] = x[batch, in_features] @ weight^T + bias, weight stored
+ * [out_features, in_features] row-major as nn.Linear holds it, bias [out_features] or NULL: Linear.Forward,
+ * internal/nn/linear.go:78-107 (which transposes the weight, calls MatMul and adds the bias).  For the LM
+ * head `out` is the `[batch, vocab]` logits that born_rocm_sample reads, so they never leave the device.
+ *
+ * born_rocm_matmul: c[m,n] = a[m,k] @ b[k,n], all row-major: tensor.Backend.MatMul,
+ * internal/tensor/backend.go:20, CPU form internal/backend/cpu/matmul.go:13-71 (2-D fp32 only).
+ *
+ * Pitches (x_stride, w_stride, out_stride, lda, ldb, ldc) are in elements between consecutive rows.  Inputs
+ * are not modified; `out` / `c` must not overlap them. */
+int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t x_stride, const float *weight,
+                     int64_t out_features, int64_t w_stride, const float *bias, float *out, int64_t out_stride,
+                     void *stream);
+int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                     int64_t ldb, int64_t ldc, void *stream);
+
 /* Building blocks exported for parity tests (device-side evaluation of the specified fp32 exponential and of
  * the built-in uniform stream). */
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream);

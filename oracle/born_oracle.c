@@ -12,6 +12,8 @@
  *   born_oracle_softmax_via_log  internal/nn/cross_entropy.go:163-170
  *   born_oracle_argmax           internal/nn/cross_entropy.go:241-251
  *   born_oracle_exp_f32          internal/autodiff/ops/log.go:159-185
+ *   born_oracle_matmul_f32       internal/backend/cpu/matmul.go:55-71
+ *   born_oracle_linear_f32       internal/nn/linear.go:78-107
  *   logits layout                internal/tensor/raw.go:78-105, shape.go:52-63
  * Go's math.Exp / math.Log are stood in for by glibc exp()/log() (both < 1 ulp
  * in fp64; the difference vanishes in the fp32 cast for every vector the
@@ -161,6 +163,30 @@ BORN_EXPORT void born_oracle_argmax(const float *in, int64_t B, int64_t V, int64
 /* internal/autodiff/ops/log.go:159-185 */
 BORN_EXPORT void born_oracle_exp_f32(const float *in, float *out, int64_t n) {
     for (int64_t i = 0; i < n; i++) out[i] = (float)exp((double)in[i]);
+}
+
+/* internal/backend/cpu/matmul.go:55-71: C[i,j] = sum_k A[i,k] * B[k,j], one fp32 accumulator per element,
+ * k ascending, product and sum each rounded to fp32 (no fused multiply-add: -ffp-contract=off). */
+BORN_EXPORT void born_oracle_matmul_f32(float *c, const float *a, const float *b, int64_t m, int64_t k, int64_t n) {
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t j = 0; j < n; j++) {
+            float sum = 0.0f;
+            for (int64_t kk = 0; kk < k; kk++) sum += a[i * k + kk] * b[kk * n + j];
+            c[i * n + j] = sum;
+        }
+}
+
+/* internal/nn/linear.go:78-107: y = x @ W^T + b with W stored [out_features, in_features]; the reference
+ * forms the transposed view, runs the matmul above and then adds the bias row in fp32 (bias may be NULL here,
+ * for a layer used without one). */
+BORN_EXPORT void born_oracle_linear_f32(float *y, const float *x, const float *w, const float *bias, int64_t batch,
+                                        int64_t in_features, int64_t out_features) {
+    for (int64_t i = 0; i < batch; i++)
+        for (int64_t j = 0; j < out_features; j++) {
+            float sum = 0.0f;
+            for (int64_t kk = 0; kk < in_features; kk++) sum += x[i * in_features + kk] * w[j * in_features + kk];
+            y[i * out_features + j] = bias ? sum + bias[j] : sum;
+        }
 }
 
 /* fp64-accumulated softmax (layer T of the standalone operator checks) */

@@ -47,6 +47,10 @@ def lib():
         L.born_oracle_argmax.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p]
         L.born_oracle_exp_f32.restype = None
         L.born_oracle_exp_f32.argtypes = [f32p, f32p, C.c_int64]
+        L.born_oracle_matmul_f32.restype = None
+        L.born_oracle_matmul_f32.argtypes = [f32p, f32p, f32p, C.c_int64, C.c_int64, C.c_int64]
+        L.born_oracle_linear_f32.restype = None
+        L.born_oracle_linear_f32.argtypes = [f32p, f32p, f32p, f32p, C.c_int64, C.c_int64, C.c_int64]
         L.born_oracle_softmax_f64.restype = None
         L.born_oracle_softmax_f64.argtypes = [f32p, f64p, C.c_int64, C.c_int64, C.c_int64]
         L.born_oracle_sample.restype = C.c_int64
@@ -123,6 +127,35 @@ def exp_ref(x):
     out = np.empty_like(x)
     lib().born_oracle_exp_f32(_p(x, C.c_float), _p(out, C.c_float), x.size)
     return out
+
+
+def matmul_ref(a, b):
+    """The reference's naive fp32 MatMul: [m,k] @ [k,n], sequential k-sum per element."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    m, k = a.shape
+    k2, n = b.shape
+    assert k == k2, "matmul: shape mismatch"
+    c = np.empty((m, n), dtype=np.float32)
+    lib().born_oracle_matmul_f32(_p(c, C.c_float), _p(a, C.c_float), _p(b, C.c_float), m, k, n)
+    return c
+
+
+def linear_ref(x, w, bias=None):
+    """The reference's Linear.Forward: x[batch,in] @ w[out,in]^T + bias[out]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    batch, fin = x.shape
+    fout, fin2 = w.shape
+    assert fin == fin2, "linear: shape mismatch"
+    bp = None
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+        assert bias.shape == (fout,)
+        bp = _p(bias, C.c_float)
+    y = np.empty((batch, fout), dtype=np.float32)
+    lib().born_oracle_linear_f32(_p(y, C.c_float), _p(x, C.c_float), _p(w, C.c_float), bp, batch, fin, fout)
+    return y
 
 
 def row_stats(x, T=1.0):

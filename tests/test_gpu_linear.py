@@ -1,0 +1,220 @@
+"""GPU parity tests of the logits producer (born_rocm_linear / born_rocm_matmul, through the C ABI and its
+Python mirror) against the CPU oracle's restatement of the reference's MatMul and Linear.Forward.
+
+Tolerance (floating point; the order of the k-sum differs between the matrix-core kernel and the
+reference's sequential loop, so agreement is to rounding):
+    |gpu - exact| <= (4 * sqrt(K) + 2) * 2^-24 * (sum_k |a_k| |b_k| + |bias|)
+against an fp64 product, and twice the reference loop's own worst-case bound plus that against the
+oracle.  Integer-valued operands, whose partial sums are all exact in fp32, must match bit for bit.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+EPS = 2.0 ** -24
+
+
+@pytest.fixture(scope="module")
+def rocm():
+    from born_amd import sampler as S
+    assert S.DeviceCount() >= 1, "no HIP device visible"
+    return S
+
+
+@pytest.fixture(scope="module")
+def lin():
+    from born_amd import linear as L
+    return L
+
+
+def _bound(a, bt, bias, K):
+    mag = np.abs(a).astype(np.float64) @ np.abs(bt).astype(np.float64).T
+    if bias is not None:
+        mag = mag + np.abs(bias).astype(np.float64)[None, :]
+    return (4.0 * np.sqrt(K) + 2.0) * EPS * mag + 1e-37
+
+
+def _gpu_linear(rocm, lin, x, w, bias):
+    M, K = x.shape
+    N = w.shape[0]
+    layer = lin.Linear(K, N, rocm.DeviceBuffer.from_numpy(w), None if bias is None else rocm.DeviceBuffer.from_numpy(bias))
+    dx = rocm.DeviceBuffer.from_numpy(x)
+    out = rocm.DeviceBuffer(M * N * 4)
+    layer.Forward(dx, (M, K), out)
+    return out.to_numpy(np.float32, (M, N))
+
+
+def _gpu_matmul(rocm, lin, a, b):
+    M, K = a.shape
+    N = b.shape[1]
+    out = rocm.DeviceBuffer(M * N * 4)
+    lin.MatMul(rocm.DeviceBuffer.from_numpy(a), rocm.DeviceBuffer.from_numpy(b), M, K, N, out, k_b=b.shape[0])
+    return out.to_numpy(np.float32, (M, N))
+
+
+def test_reference_kats(rocm, lin):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_kats.json")) as f:
+        kats = json.load(f)
+    for case in kats["matmul"]:
+        got = _gpu_matmul(rocm, lin, np.array(case["a"], np.float32), np.array(case["b"], np.float32))
+        assert np.max(np.abs(got.astype(np.float64) - np.array(case["expected"]))) <= case["tol_abs"], case["source"]
+    for case in kats["linear"]:
+        bias = None if case["bias"] is None else np.array(case["bias"], np.float32)
+        got = _gpu_linear(rocm, lin, np.array(case["x"], np.float32), np.array(case["weight"], np.float32), bias)
+        assert np.max(np.abs(got.astype(np.float64) - np.array(case["expected"]))) <= case["tol_abs"], case["source"]
+
+
+SHAPES = [(1, 1, 1), (1, 3, 2), (2, 2, 2), (3, 5, 7), (7, 16, 5), (33, 17, 65), (64, 64, 64), (127, 100, 129),
+          (128, 128, 128), (129, 15, 127), (130, 257, 300), (256, 512, 1000), (5, 1000, 1), (300, 33, 31)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_linear_matches_oracle(oracle, rocm, lin, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(M * 1000003 + K * 1009 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    for b in (bias, None):
+        got = _gpu_linear(rocm, lin, x, w, b)
+        exact = x.astype(np.float64) @ w.astype(np.float64).T + (0.0 if b is None else b.astype(np.float64)[None, :])
+        bound = _bound(x, w, b, K)
+        assert np.all(np.abs(got - exact) <= bound), f"{shape}: off the fp64 product by {np.max(np.abs(got - exact) / bound):.2f} bounds"
+        ref = oracle.linear_ref(x, w, b)
+        ref_bound = (K + 2) * EPS * (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T + (0 if b is None else np.abs(b)[None, :]))
+        assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + ref_bound), shape
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_matmul_matches_oracle(oracle, rocm, lin, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(M * 7919 + K * 104729 + N)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    got = _gpu_matmul(rocm, lin, a, b)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    bound = _bound(a, np.ascontiguousarray(b.T), None, K)
+    assert np.all(np.abs(got - exact) <= bound), f"{shape}: off the fp64 product by {np.max(np.abs(got - exact) / bound):.2f} bounds"
+    ref = oracle.matmul_ref(a, b)
+    ref_bound = (K + 2) * EPS * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= bound + ref_bound), shape
+
+
+@pytest.mark.parametrize("shape", [(3, 5, 7), (130, 257, 300), (256, 64, 129)])
+def test_integer_valued_operands_are_bit_exact(oracle, rocm, lin, shape):
+    # every product and partial sum is an integer below 2^24: exact in fp32 whatever the order of the sum
+    M, K, N = shape
+    rng = np.random.default_rng(11)
+    x = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    w = rng.integers(-8, 9, (N, K)).astype(np.float32)
+    bias = rng.integers(-100, 101, N).astype(np.float32)
+    assert np.array_equal(_gpu_linear(rocm, lin, x, w, bias), oracle.linear_ref(x, w, bias))
+    b = np.ascontiguousarray(w.T)
+    assert np.array_equal(_gpu_matmul(rocm, lin, x, b), oracle.matmul_ref(x, b))
+
+
+def test_pitches_and_unaligned_operands(oracle, rocm):
+    # rows wider than the matrix, pitches that are not multiples of 4 elements, bases off 16-byte alignment:
+    # the kernel must take its scalar loads, never read or write outside the rows
+    import ctypes as C
+    from born_amd import _capi
+    rng = np.random.default_rng(5)
+    M, K, N = 70, 37, 150
+    lda, ldw, ldc = 41, 39, 153
+    xa = rng.standard_normal((M, lda)).astype(np.float32)
+    wa = rng.standard_normal((N, ldw)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    for off in (0, 1):                                   # element offset of every base pointer
+        dx = rocm.DeviceBuffer.from_numpy(np.concatenate([np.zeros(off, np.float32), xa.ravel()]))
+        dw = rocm.DeviceBuffer.from_numpy(np.concatenate([np.zeros(off, np.float32), wa.ravel()]))
+        db = rocm.DeviceBuffer.from_numpy(np.concatenate([np.zeros(off, np.float32), bias]))
+        sentinel = np.full(off + M * ldc, -777.0, np.float32)
+        dc = rocm.DeviceBuffer.from_numpy(sentinel)
+        _capi.check(_capi.lib().born_rocm_linear(dx.ptr + 4 * off, M, K, lda, dw.ptr + 4 * off, N, ldw, db.ptr + 4 * off,
+                                                 dc.ptr + 4 * off, ldc, None))
+        out = dc.to_numpy(np.float32, (off + M * ldc,))
+        assert np.all(out[:off] == -777.0)
+        got = out[off:].reshape(M, ldc)
+        assert np.all(got[:, N:] == -777.0), "wrote outside the rows of the output"
+        x, w = xa[:, :K], wa[:, :K]
+        exact = x.astype(np.float64) @ w.astype(np.float64).T + bias[None, :]
+        assert np.all(np.abs(got[:, :N] - exact) <= _bound(x, w, bias, K))
+        # the same operands through matmul: b = w^T stored [K, N] with pitch ldb
+        ldb = N + 3
+        ba = np.zeros((K, ldb), np.float32)
+        ba[:, :N] = w.T
+        dbm = rocm.DeviceBuffer.from_numpy(np.concatenate([np.zeros(off, np.float32), ba.ravel()]))
+        dc2 = rocm.DeviceBuffer.from_numpy(sentinel)
+        _capi.check(_capi.lib().born_rocm_matmul(dx.ptr + 4 * off, dbm.ptr + 4 * off, dc2.ptr + 4 * off, M, K, N, lda, ldb, ldc, None))
+        got2 = dc2.to_numpy(np.float32, (off + M * ldc,))[off:].reshape(M, ldc)
+        assert np.all(got2[:, N:] == -777.0)
+        assert np.all(np.abs(got2[:, :N] - (exact - bias[None, :])) <= _bound(x, w, None, K))
+
+
+def test_argument_errors(rocm, lin):
+    w = rocm.DeviceBuffer(64)
+    layer = lin.Linear(4, 4, w, None)
+    with pytest.raises(lin.LinearPanic, match="expected input with 4 features, got 3"):
+        layer.Forward(w, (1, 3), w)
+    with pytest.raises(lin.LinearPanic, match="expected 2D input"):
+        layer.Forward(w, (4,), w)
+    with pytest.raises(lin.LinearPanic, match="shape mismatch"):
+        lin.MatMul(w, w, 2, 2, 2, w, k_b=3)
+    from born_amd import _capi
+    assert _capi.lib().born_rocm_linear(None, 1, 1, 1, None, 1, 1, None, None, 1, None) == _capi.ERR_ARGUMENT
+    assert _capi.lib().born_rocm_matmul(w.ptr, w.ptr, w.ptr, 2, 2, 2, 1, 2, 2, None) == _capi.ERR_ARGUMENT   # pitch < row
+
+
+def test_lm_head_then_sample_without_leaving_the_device(oracle, rocm, lin):
+    # hidden states -> LM head -> sampler, all on the device; the sampler's tokens are bit-exact against the
+    # oracle run on the logits the device produced, and those logits agree with the oracle's Linear to rounding
+    rng = np.random.default_rng(2025)
+    B, K, V = 48, 256, 32000
+    hidden = rng.standard_normal((B, K)).astype(np.float32)
+    w = (rng.standard_normal((V, K)) * (2.0 / np.sqrt(K))).astype(np.float32)
+    bias = (rng.standard_normal(V) * 0.1).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, (B, 64)).astype(np.int32)
+    layer = lin.Linear(K, V, rocm.DeviceBuffer.from_numpy(w), rocm.DeviceBuffer.from_numpy(bias))
+    logits = rocm.DeviceBuffer(B * V * 4)
+    layer.Forward(rocm.DeviceBuffer.from_numpy(hidden), (B, K), logits)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.7, TopK=50, TopP=0.9, RepetitionPenalty=1.15), max_batch=B, max_vocab=V)
+    tokens = rocm.DeviceBuffer(B * 4)
+    probs = rocm.DeviceBuffer(B * 4)
+    s.Sample(logits, B, V, rocm.DeviceBuffer.from_numpy(hist), None, rocm.DeviceBuffer.from_numpy(u), tokens, probs, hist_stride=64)
+    s.Status()
+    got_tokens = tokens.to_numpy(np.int32, (B,))
+    x = logits.to_numpy(np.float32, (B, V))
+    exact = hidden.astype(np.float64) @ w.astype(np.float64).T + bias[None, :]
+    assert np.all(np.abs(x - exact) <= _bound(hidden, w, bias, K))
+    fx = oracle.sample(x, u, 0.7, 50, 0.9, 1.15, hist, None, mode=oracle.MODE_FIXED)
+    assert np.array_equal(got_tokens, fx["tokens"])
+    s.Close()
+
+
+def test_lm_head_full_size_spot_check(rocm, lin):
+    # batch 256 x hidden 2048 -> vocabulary 128256 (1 GB of weights): 4000 random entries and two whole
+    # columns of tiles against fp64 dot products; every workgroup id mapping (XCD-aware order) is exercised
+    rng = np.random.default_rng(99)
+    M, K, N = 256, 2048, 128256
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((N, K), dtype=np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    got = _gpu_linear(rocm, lin, x, w, bias)
+    rows = rng.integers(0, M, 4000)
+    cols = rng.integers(0, N, 4000)
+    exact = np.einsum("ik,ik->i", x[rows].astype(np.float64), w[cols].astype(np.float64)) + bias[cols]
+    mag = np.einsum("ik,ik->i", np.abs(x[rows]).astype(np.float64), np.abs(w[cols]).astype(np.float64)) + np.abs(bias[cols])
+    assert np.all(np.abs(got[rows, cols] - exact) <= (4 * np.sqrt(K) + 2) * EPS * mag)
+    for c0 in (0, N - 300):                                # first tiles and the ragged last ones, all rows
+        sl = slice(c0, c0 + 300)
+        ex = x.astype(np.float64) @ w[sl].astype(np.float64).T + bias[sl][None, :]
+        assert np.all(np.abs(got[:, sl] - ex) <= _bound(x, w[sl], bias[sl], K))
+    # every output element was written: a checksum of all rows against the fp64 product with the column sum of W
+    colsum = w.astype(np.float64).sum(axis=0)
+    want = x.astype(np.float64) @ colsum + bias.astype(np.float64).sum()
+    scale = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).sum(axis=0)
+    assert np.all(np.abs(got.astype(np.float64).sum(axis=1) - want) <= (4 * np.sqrt(K) + 2) * EPS * scale)

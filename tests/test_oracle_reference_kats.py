@@ -104,3 +104,44 @@ def test_expneg_accuracy_and_edges(oracle):
     # monotone non-increasing on a dense grid (a sign slip in the range reduction breaks this)
     g = oracle.expneg(np.linspace(0, 30, 20001).astype(np.float32))
     assert np.all(np.diff(g) <= 0)
+
+
+def test_matmul_kats(oracle):
+    for case in KATS["matmul"]:
+        a = np.array(case["a"], dtype=np.float32)
+        b = np.array(case["b"], dtype=np.float32)
+        out = oracle.matmul_ref(a, b).astype(np.float64)
+        assert out.shape == (a.shape[0], b.shape[1])
+        assert np.max(np.abs(out - np.array(case["expected"], dtype=np.float64))) <= case["tol_abs"], case["source"]
+
+
+def test_linear_kats(oracle):
+    for case in KATS["linear"]:
+        x = np.array(case["x"], dtype=np.float32)
+        w = np.array(case["weight"], dtype=np.float32)
+        bias = None if case["bias"] is None else np.array(case["bias"], dtype=np.float32)
+        out = oracle.linear_ref(x, w, bias).astype(np.float64)
+        assert out.shape == (x.shape[0], w.shape[0])
+        assert np.max(np.abs(out - np.array(case["expected"], dtype=np.float64))) <= case["tol_abs"], case["source"]
+
+
+def test_matmul_and_linear_against_what_the_mathematics_fixes(oracle):
+    # Checks a transposed operand, a dropped bias, a wrong pitch or a dropped k-term would fail:
+    # non-square shapes against an fp64 product, the transposition identity, bias as a rank-1 update.
+    rng = np.random.default_rng(7)
+    for (m, k, n) in [(1, 1, 1), (3, 5, 7), (7, 3, 5), (16, 33, 9), (5, 257, 11)]:
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((k, n)).astype(np.float32)
+        c = oracle.matmul_ref(a, b)
+        c64 = a.astype(np.float64) @ b.astype(np.float64)
+        bound = (k + 1) * 2.0 ** -24 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+        assert np.all(np.abs(c - c64) <= bound), (m, k, n)
+        # integer-valued operands: every partial sum is exact in fp32
+        ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        bi = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        assert np.array_equal(oracle.matmul_ref(ai, bi), (ai.astype(np.int64) @ bi.astype(np.int64)).astype(np.float32))
+        # Linear.Forward is MatMul with the transposed weight (same k order, so bit for bit), plus the bias
+        w = np.ascontiguousarray(b.T)
+        bias = rng.standard_normal(n).astype(np.float32)
+        assert np.array_equal(oracle.linear_ref(a, w, None), c)
+        assert np.array_equal(oracle.linear_ref(a, w, bias), c + bias[None, :])
