@@ -5,13 +5,16 @@
 //   BT = false  B is given as [K,N] (N contiguous): the backend's MatMul
 //               (reference: internal/backend/cpu/matmul.go:13-71)
 //
-// One workgroup of 256 threads (4 waves, 2 x 2) computes a 128 x 128 tile of C; each wave owns 64 x 64 of it
-// as 2 x 2 blocks of 32 x 32, 64 accumulator registers per lane.  K advances in slices of 16: the slice after
-// the current one is fetched from global memory into registers (128-bit loads) while the current one is
-// multiplied out of LDS, then written to the other LDS buffer; one barrier per slice.  In LDS a tile row holds
-// its 16 k-values contiguously (pitch 20 floats, so that the 128-bit operand reads of 16 lanes cover all banks);
-// within a group of 8 k-values lanes 0-31 feed k..k+3 and lanes 32-63 feed k+4..k+7 to four consecutive MFMAs
-// (the order of the k-sum is free, both operands use the same one).
+// One workgroup of 256 threads (4 waves) computes a BM x 128 tile of C, BM = 128, 64 or 32 chosen from M: a
+// decode batch of a few rows is bound by streaming the weights once, and a tile as tall as the batch keeps the
+// matrix cores from multiplying padding.  Waves own 64 x 64 (BM = 128, 2 x 2 waves), 64 x 32 or 32 x 32 (4 waves
+// side by side) of the tile as blocks of 32 x 32, 16 accumulator registers per lane and block.
+//
+// K advances in slices of 32.  Two slices are in flight in registers (128-bit global loads issued two
+// multiplies ahead), one is being multiplied out of LDS and one is being written to the other LDS buffer; one
+// barrier per slice.  In LDS a tile row holds its 32 k-values contiguously (pitch 36 floats, so that the 128-bit
+// operand reads of 16 lanes cover all banks); within a group of 8 k-values lanes 0-31 feed k..k+3 and lanes
+// 32-63 feed k+4..k+7 to four consecutive MFMAs (the order of the k-sum is free, both operands use the same one).
 //
 // Workgroup ids are dealt round-robin to the 8 XCDs; the tile order makes the workgroups that share a tile
 // column of B (all M-tiles of that column) land on the same XCD back to back, so that B is fetched from HBM
@@ -24,11 +27,15 @@ namespace born {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GM = 128, GN = 128, GK = 16;
-constexpr int GPITCH = 20;                    // floats per LDS tile row ([row][k] layout)
-constexpr int GPITCH_N = 132;                 // floats per LDS k-row ([k][n] layout of B when BT = false)
+constexpr int GN = 128, GK = 32;
+constexpr int GPITCH = GK + 4;                // floats per LDS tile row ([row][k] layout)
+constexpr int GPITCH_N = GN + 4;              // floats per LDS k-row ([k][n] layout of B when BT = false)
 constexpr int GEMM_THREADS = 256;
+constexpr int LQ = GK / 4;                    // 128-bit loads per tile row and slice
+constexpr int LROWS = GEMM_THREADS / LQ;      // tile rows one pass of the workgroup's loads covers (32)
+constexpr int BPASS = GN / LROWS;             // passes over B per slice (4; also GK / 8 k-rows of the [k][n] form)
 constexpr int NUM_XCD = 8;
+static_assert(GK / 8 == BPASS && LROWS == 32, "loader geometry");
 
 // Four consecutive k-values of one tile row; zero outside the matrix.
 __device__ __forceinline__ f32x4 gemm_load_k4(const float *base, long long ld, int row, int rows, int k, int K, bool vec) {
@@ -61,25 +68,29 @@ __device__ __forceinline__ f32x4 gemm_load_n4(const float *base, long long ld, i
     return v;
 }
 
-template <bool BT>
+// FAST: every 128-bit load is legal and K is a multiple of the slice, so the loads need no guards (rows past
+// the matrix are clamped onto its last row: their products land in accumulators that are never stored).
+template <bool BT, bool FAST, int BM>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
+    constexpr int APASS = BM / LROWS;
+    constexpr int WGM = BM == 128 ? 2 : 1, WGN = 4 / WGM;            // waves along M and N
+    constexpr int IB = BM / (32 * WGM), JB = GN / (32 * WGN);        // 32 x 32 blocks per wave along M and N
     constexpr int B_WORDS = BT ? GN * GPITCH : GK * GPITCH_N;
-    __shared__ __attribute__((aligned(16))) float As[2][GM * GPITCH];
+    __shared__ __attribute__((aligned(16))) float As[2][BM * GPITCH];
     __shared__ __attribute__((aligned(16))) float Bs[2][B_WORDS];
 
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int r = lane & 31, h = lane >> 5;
 
     // tile of this workgroup
-    const int mt = (g.M + GM - 1) / GM;
+    const int mt = (g.M + BM - 1) / BM;
     const int nt = (g.N + GN - 1) / GN;
     int tile_m, tile_n;
     {
         const int id = blockIdx.x;
-        const int total = mt * nt;
         const int full = (nt / NUM_XCD) * NUM_XCD * mt;              // ids covered by whole groups of 8 tile columns
         if (id < full) {
             const int xcd = id % NUM_XCD, s = id / NUM_XCD;
@@ -90,91 +101,126 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
             tile_m = s % mt;
             tile_n = (nt / NUM_XCD) * NUM_XCD + s / mt;
         }
-        if (id >= total) return;
+        if (id >= mt * nt) return;
     }
-    const int m0 = tile_m * GM, n0 = tile_n * GN;
+    const int m0 = tile_m * BM, n0 = tile_n * GN;
 
     // loader coordinates
-    const int lrow = tid >> 2, lk = (tid & 3) * 4;                   // [row][k] tiles: rows lrow, lrow + 64
-    const int nk_row = tid >> 5, nn4 = (tid & 31) * 4;               // [k][n] tile of B: k-rows nk_row, nk_row + 8
+    const int lrow = tid / LQ, lk = (tid % LQ) * 4;                  // [row][k] tiles: rows lrow + 32 * i
+    const int nk_row = tid >> 5, nn4 = (tid & 31) * 4;               // [k][n] tile of B: k-rows nk_row + 8 * i
 
     const int nslice = (g.K + GK - 1) / GK;
-    f32x4 ra[2], rb[2];
-    auto fetch = [&](int slice) {
+    f32x4 ra[2][APASS], rb[2][BPASS];                                // two slices in flight
+    const float *fa[APASS], *fb[BPASS];                              // FAST: this thread's load addresses at slice 0
+    long long fstep_b = 0;
+    if (FAST) {
+#pragma unroll
+        for (int i = 0; i < APASS; i++) fa[i] = g.a + (long long)min(m0 + lrow + LROWS * i, g.M - 1) * g.lda + lk;
+#pragma unroll
+        for (int i = 0; i < BPASS; i++) {
+            if (BT)
+                fb[i] = g.b + (long long)min(n0 + lrow + LROWS * i, g.N - 1) * g.ldb + lk;
+            else
+                fb[i] = g.b + (long long)(nk_row + 8 * i) * g.ldb + min(n0 + nn4, g.N - 4);
+        }
+        fstep_b = BT ? GK : (long long)GK * g.ldb;
+    }
+    auto fetch = [&](f32x4 (&qa)[APASS], f32x4 (&qb)[BPASS], int slice) {
+        if (FAST) {
+#pragma unroll
+            for (int i = 0; i < APASS; i++) qa[i] = *reinterpret_cast<const f32x4 *>(fa[i] + (long long)slice * GK);
+#pragma unroll
+            for (int i = 0; i < BPASS; i++) qb[i] = *reinterpret_cast<const f32x4 *>(fb[i] + slice * fstep_b);
+            return;
+        }
         const int k0 = slice * GK;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            ra[i] = gemm_load_k4(g.a, g.lda, m0 + lrow + 64 * i, g.M, k0 + lk, g.K, g.vec_a);
+        for (int i = 0; i < APASS; i++) qa[i] = gemm_load_k4(g.a, g.lda, m0 + lrow + LROWS * i, g.M, k0 + lk, g.K, g.vec_a);
+#pragma unroll
+        for (int i = 0; i < BPASS; i++) {
             if (BT)
-                rb[i] = gemm_load_k4(g.b, g.ldb, n0 + lrow + 64 * i, g.N, k0 + lk, g.K, g.vec_b);
+                qb[i] = gemm_load_k4(g.b, g.ldb, n0 + lrow + LROWS * i, g.N, k0 + lk, g.K, g.vec_b);
             else
-                rb[i] = gemm_load_n4(g.b, g.ldb, k0 + nk_row + 8 * i, g.K, n0 + nn4, g.N, g.vec_b);
+                qb[i] = gemm_load_n4(g.b, g.ldb, k0 + nk_row + 8 * i, g.K, n0 + nn4, g.N, g.vec_b);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](const f32x4 (&qa)[APASS], const f32x4 (&qb)[BPASS], int buf) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *reinterpret_cast<f32x4 *>(&As[buf][(lrow + 64 * i) * GPITCH + lk]) = ra[i];
+        for (int i = 0; i < APASS; i++) *reinterpret_cast<f32x4 *>(&As[buf][(lrow + LROWS * i) * GPITCH + lk]) = qa[i];
+#pragma unroll
+        for (int i = 0; i < BPASS; i++) {
             if (BT)
-                *reinterpret_cast<f32x4 *>(&Bs[buf][(lrow + 64 * i) * GPITCH + lk]) = rb[i];
+                *reinterpret_cast<f32x4 *>(&Bs[buf][(lrow + LROWS * i) * GPITCH + lk]) = qb[i];
             else
-                *reinterpret_cast<f32x4 *>(&Bs[buf][(nk_row + 8 * i) * GPITCH_N + nn4]) = rb[i];
+                *reinterpret_cast<f32x4 *>(&Bs[buf][(nk_row + 8 * i) * GPITCH_N + nn4]) = qb[i];
         }
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[IB][JB];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < IB; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < JB; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int s = 0; s < nslice; s++) {
-        const int buf = s & 1;
-        fetch(min(s + 1, nslice - 1));                               // in flight during the multiply (the last one is unused)
+    auto multiply = [&](int buf) {
 #pragma unroll
-        for (int kg = 0; kg < 2; kg++) {
-            f32x4 af[2], bf[2];
+        for (int kg = 0; kg < GK / 8; kg++) {
+            f32x4 af[IB], bf[JB];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                af[i] = *reinterpret_cast<const f32x4 *>(&As[buf][(wm * 64 + i * 32 + r) * GPITCH + kg * 8 + h * 4]);
+            for (int i = 0; i < IB; i++)
+                af[i] = *reinterpret_cast<const f32x4 *>(&As[buf][((wm * IB + i) * 32 + r) * GPITCH + kg * 8 + h * 4]);
             if (BT) {
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-                    bf[j] = *reinterpret_cast<const f32x4 *>(&Bs[buf][(wn * 64 + j * 32 + r) * GPITCH + kg * 8 + h * 4]);
+                for (int j = 0; j < JB; j++)
+                    bf[j] = *reinterpret_cast<const f32x4 *>(&Bs[buf][((wn * JB + j) * 32 + r) * GPITCH + kg * 8 + h * 4]);
             } else {
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < JB; j++)
 #pragma unroll
-                    for (int kk = 0; kk < 4; kk++) bf[j][kk] = Bs[buf][(kg * 8 + h * 4 + kk) * GPITCH_N + wn * 64 + j * 32 + r];
+                    for (int kk = 0; kk < 4; kk++) bf[j][kk] = Bs[buf][(kg * 8 + h * 4 + kk) * GPITCH_N + (wn * JB + j) * 32 + r];
             }
 #pragma unroll
             for (int kk = 0; kk < 4; kk++)
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < IB; i++)
 #pragma unroll
-                    for (int j = 0; j < 2; j++)
+                    for (int j = 0; j < JB; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][kk], bf[j][kk], acc[i][j], 0, 0, 0);
         }
-        stash(buf ^ 1);
+    };
+    // One step: slice s is multiplied out of LDS buffer s & 1 while the loads of slice s + 2 are issued into the
+    // register set P; set Q holds slice s + 1 (issued one step ago) and goes to the other LDS buffer afterwards.
+    // Slices past the end are clamped onto the last one: loaded again, never multiplied.
+    auto step = [&](int s, f32x4 (&pa)[APASS], f32x4 (&pb)[BPASS], const f32x4 (&qa)[APASS], const f32x4 (&qb)[BPASS]) {
+        fetch(pa, pb, min(s + 2, nslice - 1));
+        __builtin_amdgcn_sched_barrier(0);                           // keep the loads up here, ahead of the multiply
+        multiply(s & 1);
+        stash(qa, qb, (s & 1) ^ 1);
         __syncthreads();
+    };
+
+    fetch(ra[0], rb[0], 0);
+    fetch(ra[1], rb[1], min(1, nslice - 1));
+    stash(ra[0], rb[0], 0);
+    __syncthreads();
+    for (int s = 0; s < nslice; s += 2) {
+        step(s, ra[0], rb[0], ra[1], rb[1]);
+        if (s + 1 < nslice) step(s + 1, ra[1], rb[1], ra[0], rb[0]);  // uniform
     }
 
     // C: accumulator v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4, column r of its 32 x 32 block
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int col = n0 + wn * 64 + j * 32 + r;
+    for (int j = 0; j < JB; j++) {
+        const int col = n0 + (wn * JB + j) * 32 + r;
         if (col >= g.N) continue;
         const float bias = g.bias ? g.bias[col] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < IB; i++) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
                 if (row < g.M) {
                     const float sum = acc[i][j][v];
                     g.c[(long long)row * g.ldc + col] = g.bias ? sum + bias : sum;
@@ -184,14 +230,34 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     }
 }
 
-hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
-    const long long mt = (g.M + GM - 1) / GM, nt = (g.N + GN - 1) / GN;
-    const long long grid = mt * nt;
-    if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
-    if (b_transposed)
-        hipLaunchKernelGGL(gemm_f32_kernel<true>, dim3((unsigned)grid), dim3(GEMM_THREADS), 0, st, g);
+template <bool BT, bool FAST>
+static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
+    const long long nt = (g.N + GN - 1) / GN;
+    const dim3 bl(GEMM_THREADS);
+    if (bm == 32)
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32>), dim3((unsigned)(nt * ((g.M + 31) / 32))), bl, 0, st, g);
+    else if (bm == 64)
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64>), dim3((unsigned)(nt * ((g.M + 63) / 64))), bl, 0, st, g);
     else
-        hipLaunchKernelGGL(gemm_f32_kernel<false>, dim3((unsigned)grid), dim3(GEMM_THREADS), 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 128>), dim3((unsigned)(nt * ((g.M + 127) / 128))), bl, 0, st, g);
+}
+
+hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
+    const int bm = g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
+    const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
+    if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
+    const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
+    if (b_transposed) {
+        if (fast)
+            launch_gemm_bm<true, true>(g, bm, st);
+        else
+            launch_gemm_bm<true, false>(g, bm, st);
+    } else {
+        if (fast)
+            launch_gemm_bm<false, true>(g, bm, st);
+        else
+            launch_gemm_bm<false, false>(g, bm, st);
+    }
     return hipGetLastError();
 }
 
