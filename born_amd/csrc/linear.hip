@@ -5,10 +5,11 @@
 //   BT = false  B is given as [K,N] (N contiguous): the backend's MatMul
 //               (reference: internal/backend/cpu/matmul.go:13-71)
 //
-// One workgroup of 256 threads (4 waves) computes a BM x 128 tile of C, BM = 128, 64 or 32 chosen from M: a
-// decode batch of a few rows is bound by streaming the weights once, and a tile as tall as the batch keeps the
-// matrix cores from multiplying padding.  Waves own 64 x 64 (BM = 128, 2 x 2 waves), 64 x 32 or 32 x 32 (4 waves
-// side by side) of the tile as blocks of 32 x 32, 16 accumulator registers per lane and block.
+// One workgroup of 256 threads (4 waves) computes a BM x 128 tile of C, BM = 128, 64, 32 or 16 chosen from M:
+// a decode batch of a few rows is bound by streaming the weights once, and a tile as tall as the batch keeps
+// the matrix cores from multiplying padding.  Waves own 64 x 64 (BM = 128, 2 x 2 waves), 64 x 32 or 32 x 32
+// (4 waves side by side) of the tile as blocks of 32 x 32, 16 accumulator registers per lane and block; the
+// 16-row tile uses v_mfma_f32_16x16x4_f32 instead, two 16 x 16 blocks per wave.
 //
 // K advances in slices of 32.  Two slices are in flight in registers (128-bit global loads issued two
 // multiplies ahead), one is being multiplied out of LDS and one is being written to the other LDS buffer; one
@@ -72,11 +73,13 @@ __device__ __forceinline__ f32x4 gemm_load_n4(const float *base, long long ld, i
 // the matrix are clamped onto its last row: their products land in accumulators that are never stored).
 template <bool BT, bool FAST, int BM>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
-    constexpr int APASS = BM / LROWS;
+    constexpr bool SMALL = BM == 16;                                 // 16-row tile: v_mfma_f32_16x16x4_f32, two 16-column blocks per wave
+    constexpr int AROWS = SMALL ? LROWS : BM;                        // tile rows of A loaded and kept in LDS
+    constexpr int APASS = AROWS / LROWS;
     constexpr int WGM = BM == 128 ? 2 : 1, WGN = 4 / WGM;            // waves along M and N
-    constexpr int IB = BM / (32 * WGM), JB = GN / (32 * WGN);        // 32 x 32 blocks per wave along M and N
+    constexpr int IB = SMALL ? 1 : BM / (32 * WGM), JB = GN / (32 * WGN);   // 32 x 32 blocks per wave along M and N
     constexpr int B_WORDS = BT ? GN * GPITCH : GK * GPITCH_N;
-    __shared__ __attribute__((aligned(16))) float As[2][BM * GPITCH];
+    __shared__ __attribute__((aligned(16))) float As[2][AROWS * GPITCH];
     __shared__ __attribute__((aligned(16))) float Bs[2][B_WORDS];
 
     const int tid = threadIdx.x;
@@ -110,6 +113,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     const int nk_row = tid >> 5, nn4 = (tid & 31) * 4;               // [k][n] tile of B: k-rows nk_row + 8 * i
 
     const int nslice = (g.K + GK - 1) / GK;
+    // Every workgroup walks the slices of K from a different starting slice (and wraps): workgroups running
+    // at the same time then read different columns of B, whose rows are a large power of two apart for the
+    // usual K, instead of all crowding the same few memory channels.
+    const int rot = (int)(blockIdx.x % (unsigned)nslice);
     f32x4 ra[2][APASS], rb[2][BPASS];                                // two slices in flight
     const float *fa[APASS], *fb[BPASS];                              // FAST: this thread's load addresses at slice 0
     long long fstep_b = 0;
@@ -125,7 +132,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
         }
         fstep_b = BT ? GK : (long long)GK * g.ldb;
     }
-    auto fetch = [&](f32x4 (&qa)[APASS], f32x4 (&qb)[BPASS], int slice) {
+    auto fetch = [&](f32x4 (&qa)[APASS], f32x4 (&qb)[BPASS], int step_no) {
+        int slice = step_no + rot;
+        slice = slice >= nslice ? slice - nslice : slice;
         if (FAST) {
 #pragma unroll
             for (int i = 0; i < APASS; i++) qa[i] = *reinterpret_cast<const f32x4 *>(fa[i] + (long long)slice * GK);
@@ -156,6 +165,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
         }
     };
 
+    f32x4 acc16[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};  // SMALL: columns wn * 32 + 16 * jb + lane % 16
+    const int j16 = lane & 15, q16 = lane >> 4;
     f32x16 acc[IB][JB];
 #pragma unroll
     for (int i = 0; i < IB; i++)
@@ -165,6 +176,29 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     auto multiply = [&](int buf) {
+        if (SMALL) {
+            // lane (j, q) feeds k-values kg * 16 + 4 q .. + 3 of row j to four consecutive MFMAs
+#pragma unroll
+            for (int kg = 0; kg < GK / 16; kg++) {
+                const f32x4 af = *reinterpret_cast<const f32x4 *>(&As[buf][j16 * GPITCH + kg * 16 + q16 * 4]);
+                f32x4 bf[2];
+#pragma unroll
+                for (int jb = 0; jb < 2; jb++) {
+                    if (BT) {
+                        bf[jb] = *reinterpret_cast<const f32x4 *>(&Bs[buf][(wn * 32 + jb * 16 + j16) * GPITCH + kg * 16 + q16 * 4]);
+                    } else {
+#pragma unroll
+                        for (int kk = 0; kk < 4; kk++) bf[jb][kk] = Bs[buf][(kg * 16 + q16 * 4 + kk) * GPITCH_N + wn * 32 + jb * 16 + j16];
+                    }
+                }
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for (int jb = 0; jb < 2; jb++)
+                        acc16[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[kk], bf[jb][kk], acc16[jb], 0, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int kg = 0; kg < GK / 8; kg++) {
             f32x4 af[IB], bf[JB];
@@ -210,6 +244,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
         if (s + 1 < nslice) step(s + 1, ra[1], rb[1], ra[0], rb[0]);  // uniform
     }
 
+    if (SMALL) {                                                     // accumulator v of lane (j, q) is row 4 q + v, column j of its block
+#pragma unroll
+        for (int jb = 0; jb < 2; jb++) {
+            const int col = n0 + wn * 32 + jb * 16 + j16;
+            if (col >= g.N) continue;
+            const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = m0 + 4 * q16 + v;
+                if (row < g.M) g.c[(long long)row * g.ldc + col] = g.bias ? acc16[jb][v] + bias : acc16[jb][v];
+            }
+        }
+        return;
+    }
     // C: accumulator v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4, column r of its 32 x 32 block
 #pragma unroll
     for (int j = 0; j < JB; j++) {
@@ -234,7 +282,9 @@ template <bool BT, bool FAST>
 static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
     const long long nt = (g.N + GN - 1) / GN;
     const dim3 bl(GEMM_THREADS);
-    if (bm == 32)
+    if (bm == 16)
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 16>), dim3((unsigned)(nt * ((g.M + 15) / 16))), bl, 0, st, g);
+    else if (bm == 32)
         hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32>), dim3((unsigned)(nt * ((g.M + 31) / 32))), bl, 0, st, g);
     else if (bm == 64)
         hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64>), dim3((unsigned)(nt * ((g.M + 63) / 64))), bl, 0, st, g);
@@ -243,7 +293,7 @@ static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
 }
 
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
-    const int bm = g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
+    const int bm = g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
