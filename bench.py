@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_FP32_PEAK_TFLOPS = 157.3
 
 # HBM bytes per launch of the dominant kernel, from hardware counters (not measurable from inside this
 # script): two runs `rocprofv3 --pmc FETCH_SIZE --kernel-trace -- python3 bench.py --no-cpu --steps 20
@@ -77,6 +78,51 @@ def cpu_baseline(w, seconds=12.0):
     return out
 
 
+def producer_leg(torch, dev, smp, sample_step, B, V, hidden, logits_all, stream, iters):
+    """The logits producer in front of the sampler: x[B, hidden] @ W[V, hidden]^T + b on the fp32 matrix cores
+    (born_rocm_linear), written into the buffers the sampling step reads.  Random-init weights of the LM-head
+    shape; reported beside the headline metric, never part of it."""
+    from born_amd import linear as L
+    g = torch.Generator(device=dev)
+    g.manual_seed(20251125)
+    x = torch.randn(B, hidden, device=dev, generator=g)
+    wgt = torch.randn(V, hidden, device=dev, generator=g) * (1.5 / hidden ** 0.5)
+    bias = torch.zeros(V, device=dev)
+    layer = L.Linear(hidden, V, wgt, bias)
+    scratch = torch.empty(B, V, device=dev)          # the logits the head produces and the chained sampling step reads
+
+    def head():
+        layer.Forward(x, (B, hidden), scratch, stream=stream)
+
+    def timed(fn, k):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(k):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / k
+
+    for _ in range(3):
+        head()
+    ms_head = timed(head, iters)
+
+    def both():
+        head()
+        sample_step(scratch)
+
+    both()
+    ms_both = timed(both, iters)
+    flops = 2.0 * B * hidden * V
+    tf = flops / (ms_head * 1e-3) / 1e12
+    return {"kernel": "gemm_f32_kernel", "workload": f"LM head: [{B}, {hidden}] @ [{V}, {hidden}]^T + bias, fp32 in / fp32 accumulate / fp32 out",
+            "ms": ms_head, "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                        "frac": tf / MFMA_FP32_PEAK_TFLOPS},
+            "weight_stream_GBs": V * hidden * 4 / (ms_head * 1e-3) / 1e9,
+            "ms_head_plus_sampling_step": ms_both, "tokens_per_s_head_plus_sampling": B / (ms_both * 1e-3), "iters": iters}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -87,6 +133,9 @@ def main():
     ap.add_argument("--rotate", type=int, default=4,
                     help="number of distinct logits buffers cycled through, so that a step never finds its logits in a cache")
     ap.add_argument("--path", type=int, default=0, help="kernel selection of the sampler (0 = default; 1 = always the general kernel)")
+    ap.add_argument("--no-producer", action="store_true",
+                    help="skip the LM-head leg (hidden states -> logits on the device, then the same sampling step)")
+    ap.add_argument("--hidden", type=int, default=4096, help="hidden size of the LM-head leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a few plain device-to-device copies of one logits buffer (a kernel of known traffic "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -127,9 +176,10 @@ def main():
 
     counter = [0]
 
-    def step():
-        lg = logits_all[counter[0] % nrot]
-        counter[0] += 1
+    def step(lg=None):
+        if lg is None:
+            lg = logits_all[counter[0] % nrot]
+            counter[0] += 1
         smp.Sample(lg, B, V, history, None, uniforms, tokens, probs, hist_stride=H, stream=stream)
 
     def timed(k):
@@ -185,6 +235,8 @@ def main():
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "kernel_ms": ms_kernel},
     }
+    if not args.no_producer:
+        out["producer"] = producer_leg(torch, dev, smp, step, B, V, args.hidden, logits_all, stream, max(5, args.steps // 10))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))

@@ -98,4 +98,31 @@ private:
     born_sampler *h_ = nullptr;
 };
 
+// nn.Linear on the device (internal/nn/linear.go:24-140): y = x @ W^T + b, W [out_features, in_features]
+// row-major, b [out_features] or none.  The parameters are caller-owned device memory.
+class Linear {
+public:
+    Linear(int64_t in_features, int64_t out_features, const float *weight_dev, const float *bias_dev)
+        : in_(in_features), out_(out_features), w_(weight_dev), b_(bias_dev) {}
+    int64_t InFeatures() const { return in_; }
+    int64_t OutFeatures() const { return out_; }
+    // out_dev[batch, out_features]; throws like the reference panics when `features` is not in_features
+    void Forward(const float *input_dev, int64_t batch, int64_t features, float *out_dev, void *stream = nullptr) const {
+        if (features != in_)
+            throw std::invalid_argument("Linear.Forward: expected input with " + std::to_string(in_) + " features, got " +
+                                        std::to_string(features));
+        check(born_rocm_linear(input_dev, batch, in_, in_, w_, out_, in_, b_, out_dev, out_, stream));
+    }
+
+private:
+    int64_t in_, out_;
+    const float *w_, *b_;
+};
+
+// tensor.Backend.MatMul (internal/tensor/backend.go:20): c[m,n] = a[m,k] @ b[k,n], row-major device memory.
+inline void MatMul(const float *a_dev, const float *b_dev, float *c_dev, int64_t m, int64_t k, int64_t n,
+                   void *stream = nullptr) {
+    check(born_rocm_matmul(a_dev, b_dev, c_dev, m, k, n, k, n, n, stream));
+}
+
 }  // namespace born::rocm
