@@ -11,9 +11,9 @@
 // (4 waves side by side) of the tile as blocks of 32 x 32, 16 accumulator registers per lane and block; the
 // 16-row tile uses v_mfma_f32_16x16x4_f32 instead, two 16 x 16 blocks per wave.
 //
-// K advances in slices of 32.  Two slices are in flight in registers (128-bit global loads issued two
-// multiplies ahead), one is being multiplied out of LDS and one is being written to the other LDS buffer; one
-// barrier per slice.  In LDS a tile row holds its 32 k-values contiguously (pitch 36 floats, so that the 128-bit
+// K advances in slices of 32.  In gemm_f32_kernel two slices are in flight in registers (128-bit global loads
+// issued two multiplies ahead), one is being multiplied out of LDS and one is being written to the other LDS
+// buffer; one barrier per slice.  gemm_f32_dma_kernel (further down) loads straight into LDS instead.  In LDS a tile row holds its 32 k-values contiguously (pitch 36 floats, so that the 128-bit
 // operand reads of 16 lanes cover all banks); within a group of 8 k-values lanes 0-31 feed k..k+3 and lanes
 // 32-63 feed k+4..k+7 to four consecutive MFMAs (the order of the k-sum is free, both operands use the same one).
 //
@@ -278,6 +278,144 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     }
 }
 
+// The same tile computation for W[N,K] operands whose loads need no guards, with the global loads written
+// straight into LDS (global_load_lds_dwordx4) instead of through registers: an fp32 32x32x2 MFMA writes an
+// accumulator register every issue cycle, so every other register write (a returning global load, an LDS
+// operand read) takes a cycle from the matrix pipe; this form has none for the global side.
+// A direct load puts lane l's 16 bytes at LDS address base + 16 l, so a wave instruction fills 64 consecutive
+// 16-byte slots and the layout cannot be padded.  Slot of (row, c = k / 4) is 8 row + (c ^ ((row >> 1) & 7)):
+// the operand reads of 16 consecutive rows at one c then fall into 16 different bank groups.  Each lane picks
+// the global address that belongs to its slot: a wave instruction still reads 8 rows x 128 contiguous bytes.
+template <int BM, int KS>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_dma_kernel(GemmArgs g) {
+    constexpr int WGM = BM == 128 ? 2 : 1, WGN = 4 / WGM;
+    constexpr int IB = BM / (32 * WGM), JB = GN / (32 * WGN);
+    constexpr int SL = KS / 4;                                       // 16-byte slots per tile row and slice
+    constexpr int SWS = SL == 8 ? 1 : 2;                             // swizzle of row: (row >> SWS) & (SL - 1)
+    constexpr int AJ = BM * SL / 256, BJ = GN * SL / 256;            // direct loads per wave and slice: A, B
+    __shared__ __attribute__((aligned(16))) float As0[BM * KS], As1[BM * KS], Bs0[GN * KS], Bs1[GN * KS];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int r = lane & 31, h = lane >> 5;
+
+    const int mt = (g.M + BM - 1) / BM;
+    const int nt = (g.N + GN - 1) / GN;
+    int tile_m, tile_n;
+    {
+        const int id = blockIdx.x;
+        const int full = (nt / NUM_XCD) * NUM_XCD * mt;
+        if (id < full) {
+            const int xcd = id % NUM_XCD, s = id / NUM_XCD;
+            tile_m = s % mt;
+            tile_n = (s / mt) * NUM_XCD + xcd;
+        } else {
+            const int s = id - full;
+            tile_m = s % mt;
+            tile_n = (nt / NUM_XCD) * NUM_XCD + s / mt;
+        }
+        if (id >= mt * nt) return;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * GN;
+    const int nslice = g.K / KS;
+    const int rot = (int)(blockIdx.x % (unsigned)nslice);
+
+    const int lr = lane / SL, lc = lane % SL;
+    const float *pa[AJ], *pb[BJ];
+#pragma unroll
+    for (int j = 0; j < AJ; j++) {
+        const int row = (wave * AJ + j) * (64 / SL) + lr;
+        pa[j] = g.a + (long long)min(m0 + row, g.M - 1) * g.lda + ((lc ^ ((row >> SWS) & (SL - 1))) << 2);
+    }
+#pragma unroll
+    for (int j = 0; j < BJ; j++) {
+        const int row = (wave * BJ + j) * (64 / SL) + lr;
+        pb[j] = g.b + (long long)min(n0 + row, g.N - 1) * g.ldb + ((lc ^ ((row >> SWS) & (SL - 1))) << 2);
+    }
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    auto dma = [&](float *as, float *bs, int step_no) {
+        int slice = step_no + rot;
+        slice = slice >= nslice ? slice - nslice : slice;
+        const long long off = (long long)slice * KS;
+#pragma unroll
+        for (int j = 0; j < AJ; j++)
+            __builtin_amdgcn_global_load_lds((gptr_t)(pa[j] + off), (lptr_t)(as + (wave * AJ + j) * 256), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < BJ; j++)
+            __builtin_amdgcn_global_load_lds((gptr_t)(pb[j] + off), (lptr_t)(bs + (wave * BJ + j) * 256), 16, 0, 0);
+    };
+
+    f32x16 acc[IB][JB];
+#pragma unroll
+    for (int i = 0; i < IB; i++)
+#pragma unroll
+        for (int j = 0; j < JB; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+    const int sw = (r >> SWS) & (SL - 1);                                    // tile rows of a wave start at multiples of 32
+    auto multiply = [&](const float *as, const float *bs) {
+        f32x4 af[2][IB], bf[2][JB];                                  // operands of group kg + 1 are read while group kg is multiplied
+        auto frag = [&](int kg, f32x4 (&fa)[IB], f32x4 (&fb)[JB]) {
+            const int cs = ((kg * 2 + h) ^ sw) << 2;
+#pragma unroll
+            for (int i = 0; i < IB; i++) fa[i] = *reinterpret_cast<const f32x4 *>(&as[((wm * IB + i) * 32 + r) * KS + cs]);
+#pragma unroll
+            for (int j = 0; j < JB; j++) fb[j] = *reinterpret_cast<const f32x4 *>(&bs[((wn * JB + j) * 32 + r) * KS + cs]);
+        };
+        frag(0, af[0], bf[0]);
+#pragma unroll
+        for (int kg = 0; kg < KS / 8; kg++) {
+            if (kg + 1 < KS / 8) frag(kg + 1, af[(kg + 1) & 1], bf[(kg + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);                       // reads first: they land during the MFMAs below
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int i = 0; i < IB; i++)
+#pragma unroll
+                    for (int j = 0; j < JB; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kg & 1][i][kk], bf[kg & 1][j][kk], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    // slice s is multiplied out of one LDS buffer while the direct loads of slice s + 1 fill the other; the
+    // barrier (which also waits for this wave's loads) ends the step
+    dma(As0, Bs0, 0);
+    __syncthreads();
+    for (int s = 0; s < nslice; s += 2) {
+        dma(As1, Bs1, min(s + 1, nslice - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(As0, Bs0);
+        __syncthreads();
+        if (s + 1 < nslice) {                                        // uniform
+            dma(As0, Bs0, min(s + 2, nslice - 1));
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(As1, Bs1);
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < JB; j++) {
+        const int col = n0 + (wn * JB + j) * 32 + r;
+        if (col >= g.N) continue;
+        const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+        for (int i = 0; i < IB; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                if (row < g.M) {
+                    const float sum = acc[i][j][v];
+                    g.c[(long long)row * g.ldc + col] = g.bias ? sum + bias : sum;
+                }
+            }
+        }
+    }
+}
+
 template <bool BT, bool FAST>
 static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
     const long long nt = (g.N + GN - 1) / GN;
@@ -297,7 +435,15 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
-    if (b_transposed) {
+    if (b_transposed && fast && bm >= 32) {
+        const dim3 gr((unsigned)grid), bl(GEMM_THREADS);
+        if (bm == 128)
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<128, GK>), gr, bl, 0, st, g);
+        else if (bm == 64)
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<64, GK>), gr, bl, 0, st, g);
+        else
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<32, GK>), gr, bl, 0, st, g);
+    } else if (b_transposed) {
         if (fast)
             launch_gemm_bm<true, true>(g, bm, st);
         else
