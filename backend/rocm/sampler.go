@@ -181,3 +181,29 @@ func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, dr
 	}
 	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
 }
+
+// VerifyBonus is Verify for a target that scored gamma+1 positions: `target` is [batch, gamma+1, vocab] and its
+// last position is the bonus distribution, so a sequence whose draft tokens are all accepted gets its next
+// token from it (nextToken is never -1).
+func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
+	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
+	out, err := Alloc(int64(8 * batch))
+	if err != nil {
+		return nil, nil, err
+	}
+	defer out.Free()
+	na := (*C.int32_t)(out.ptr)
+	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
+	seq := C.int64_t((gamma + 1) * vocab)
+	bonus := (*C.float)(unsafe.Add(target.ptr, 4*gamma*vocab))
+	if err = check(C.born_rocm_spec_verify_bonus(s.h, (*C.float)(target.ptr), seq, (*C.float)(draft.ptr),
+		C.int64_t(gamma*vocab), bonus, seq, C.int64_t(batch), C.int64_t(gamma), C.int64_t(vocab),
+		(*C.int32_t)(draftTokens.ptr), (*C.float)(uAccept.ptr), (*C.float)(uResidual.ptr), na, nt, nil)); err != nil {
+		return nil, nil, err
+	}
+	both := make([]int32, 2*batch)
+	if err = out.Download(unsafe.Pointer(&both[0]), int64(8*batch)); err != nil {
+		return nil, nil, err
+	}
+	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
+}

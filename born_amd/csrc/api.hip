@@ -52,8 +52,8 @@ struct born_sampler {
     int *status;
     unsigned long long *counters;
     // spec-verify statistics:
-    float *sp_mp, *sp_mq;
-    unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd, *sp_part, *sp_run;
+    float *sp_mp, *sp_mq, *sp_mb;
+    unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd, *sp_part, *sp_run, *sp_Zb;
     int64_t spec_rows;
 };
 
@@ -171,7 +171,8 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
     void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters,
-                    s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run};
+                    s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run,
+                    s->sp_mb,     s->sp_Zb};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     delete s;
@@ -331,9 +332,10 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     return BORN_ROCM_OK;
 }
 
-int born_rocm_spec_verify(born_sampler *s, const float *target, const float *draft, int64_t batch, int64_t gamma,
-                          int64_t vocab, const int32_t *draft_tokens, const float *u_accept, const float *u_residual,
-                          int32_t *n_accepted_out, int32_t *next_token_out, void *stream) {
+static int spec_verify_impl(born_sampler *s, const float *target, int64_t target_seq_stride, const float *draft,
+                            int64_t draft_seq_stride, const float *bonus, int64_t bonus_stride, int64_t batch,
+                            int64_t gamma, int64_t vocab, const int32_t *draft_tokens, const float *u_accept,
+                            const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out, void *stream) {
     if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: null handle");
     if (!target || !draft || !draft_tokens || !u_accept || !u_residual || !n_accepted_out || !next_token_out)
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: null pointer");
@@ -342,14 +344,16 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
     if (vocab > s->max_vocab)
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: vocab %lld exceeds the handle's %lld", (long long)vocab,
                     (long long)s->max_vocab);
-    if (batch * gamma > (int64_t)0x7FFFFFFF / 4)
+    if (target_seq_stride < gamma * vocab || draft_seq_stride < gamma * vocab || (bonus && bonus_stride < vocab))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: a sequence stride is smaller than the sequence");
+    if (batch * (gamma + 1) > (int64_t)0x7FFFFFFF / 4)
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: spec_verify: batch * gamma too large");
     const int64_t rows = batch * gamma;
     if (rows > s->spec_rows) {
         // grow the per-position statistics (stream-ordered use only; the old buffers are idle once synchronised)
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        void **ps[] = {(void **)&s->sp_mp, (void **)&s->sp_mq, (void **)&s->sp_Zp,
-                       (void **)&s->sp_Zq, (void **)&s->sp_pd, (void **)&s->sp_qd, (void **)&s->sp_part, (void **)&s->sp_run};
+        void **ps[] = {(void **)&s->sp_mp, (void **)&s->sp_mq, (void **)&s->sp_Zp, (void **)&s->sp_Zq, (void **)&s->sp_pd,
+                       (void **)&s->sp_qd, (void **)&s->sp_part, (void **)&s->sp_run, (void **)&s->sp_mb, (void **)&s->sp_Zb};
         for (void **p : ps) {
             if (*p) (void)hipFree(*p);
             *p = nullptr;
@@ -363,12 +367,18 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
         HIP_TRY(hipMalloc((void **)&s->sp_qd, (size_t)rows * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void **)&s->sp_part, (size_t)rows * SPEC_CHUNKS * sizeof(unsigned long long)));
         HIP_TRY(hipMalloc((void **)&s->sp_run, (size_t)rows * SPEC_CHUNKS * 1024 * sizeof(unsigned long long)));
+        HIP_TRY(hipMalloc((void **)&s->sp_mb, (size_t)rows * sizeof(float)));                 // rows >= batch
+        HIP_TRY(hipMalloc((void **)&s->sp_Zb, (size_t)rows * sizeof(unsigned long long)));
         s->spec_rows = rows;
     }
     SpecArgs a;
     memset(&a, 0, sizeof(a));
     a.target = target;
     a.draft = draft;
+    a.bonus = bonus;
+    a.t_seq = target_seq_stride;
+    a.d_seq = draft_seq_stride;
+    a.b_seq = bonus_stride;
     a.B = (int)batch;
     a.G = (int)gamma;
     a.V = (int)vocab;
@@ -381,12 +391,29 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
     a.mp = s->sp_mp; a.mq = s->sp_mq;
     a.Zp = s->sp_Zp; a.Zq = s->sp_Zq;
     a.pd = s->sp_pd; a.qd = s->sp_qd;
+    a.mb = s->sp_mb; a.Zb = s->sp_Zb;
     a.part = s->sp_part;
     a.run_mass = s->sp_run;
     a.status = s->status;
     a.mass_shift = mass_shift(vocab);
     HIP_TRY(launch_spec_verify(a, (hipStream_t)stream));
     return BORN_ROCM_OK;
+}
+
+int born_rocm_spec_verify(born_sampler *s, const float *target, const float *draft, int64_t batch, int64_t gamma,
+                          int64_t vocab, const int32_t *draft_tokens, const float *u_accept, const float *u_residual,
+                          int32_t *n_accepted_out, int32_t *next_token_out, void *stream) {
+    return spec_verify_impl(s, target, gamma * vocab, draft, gamma * vocab, nullptr, 0, batch, gamma, vocab, draft_tokens,
+                            u_accept, u_residual, n_accepted_out, next_token_out, stream);
+}
+
+int born_rocm_spec_verify_bonus(born_sampler *s, const float *target, int64_t target_seq_stride, const float *draft,
+                                int64_t draft_seq_stride, const float *bonus, int64_t bonus_stride, int64_t batch,
+                                int64_t gamma, int64_t vocab, const int32_t *draft_tokens, const float *u_accept,
+                                const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out, void *stream) {
+    if (!bonus) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: spec_verify: null bonus rows");
+    return spec_verify_impl(s, target, target_seq_stride, draft, draft_seq_stride, bonus, bonus_stride, batch, gamma, vocab,
+                            draft_tokens, u_accept, u_residual, n_accepted_out, next_token_out, stream);
 }
 
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream) {

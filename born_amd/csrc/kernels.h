@@ -52,6 +52,8 @@ struct SampleArgs {
 
 struct SpecArgs {
     const float *target, *draft;
+    const float *bonus;           // [B] rows of the target at position G (drawn from when nothing is rejected), or null
+    long long t_seq, d_seq, b_seq;   // elements between consecutive sequences of target, draft, bonus
     int B, G, V;
     const int *draft_tokens;
     const float *u_acc, *u_res;
@@ -60,10 +62,13 @@ struct SpecArgs {
     // workspace: per (b, i) row statistics
     float *mp, *mq;
     unsigned long long *Zp, *Zq, *pd, *qd;
+    float *mb;                    // [B] statistics of the bonus rows
+    unsigned long long *Zb;
     unsigned long long *part;     // [B][SPEC_CHUNKS] residual mass of each quarter of the rejected row
     unsigned long long *run_mass; // [B][SPEC_CHUNKS][1024] residual mass of each thread's run of ids
     int *status;
     int mass_shift;
+    int aligned;                  // set by the launcher: every row starts 16-byte aligned and V % 4 == 0
 };
 
 // C[M,N] = A[M,K] * B (+ bias[N]); B is [N,K] (b_transposed, the weight of a linear layer) or [K,N].

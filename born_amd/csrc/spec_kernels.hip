@@ -10,6 +10,8 @@
 //                         max(0, p - q) over the workgroup's quarter of that one row.
 //   spec_pick_kernel      one workgroup per sequence: the per-thread masses of the quarter the residual
 //                         draw falls into are scanned and the owning thread walks its ids in ascending order.
+// With bonus rows (the target's distribution one position past the draft) a sequence without a rejection draws
+// its next token from that row the same way: the "residual" is then the row's own integer masses.
 #include "dev_common.h"
 #include "kernels.h"
 
@@ -43,10 +45,14 @@ __device__ __forceinline__ void spec_foreach(const float *x, int V, bool vec, F 
 template <bool RESIDENT>
 __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     __shared__ BlockScratch scr;
-    const int row = blockIdx.x >> 1, tid = threadIdx.x;
-    const bool is_draft = blockIdx.x & 1;
+    const int tid = threadIdx.x;
     const int V = a.V;
-    const float *x = (is_draft ? a.draft : a.target) + (long long)row * V;
+    const bool is_bonus = (int)blockIdx.x >= 2 * a.B * a.G;          // the workgroups after the (position, distribution) pairs
+    const int row = is_bonus ? (int)blockIdx.x - 2 * a.B * a.G : (int)(blockIdx.x >> 1);   // bonus: the sequence
+    const bool is_draft = !is_bonus && (blockIdx.x & 1);
+    const float *x = is_bonus ? a.bonus + (long long)row * a.b_seq
+                              : (is_draft ? a.draft + (long long)(row / a.G) * a.d_seq : a.target + (long long)(row / a.G) * a.t_seq) +
+                                    (long long)(row % a.G) * V;
     const float T = a.T;
     const float scale = mass_scale(a.mass_shift);
     float m = -INFINITY;
@@ -77,14 +83,17 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
             }
         }
     } else {
-        const bool vec = ((V & 3) == 0) && ((((uintptr_t)a.target) & 15) == 0) && ((((uintptr_t)a.draft) & 15) == 0);
+        const bool vec = a.aligned != 0;
         spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, z_of(v, T)); });
         m = block_max_f32<SPEC_BLOCK>(m, &scr);
         spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(z_of(v, T), m), scale); });
     }
     u64 Z;
     block_inclusive_scan_u64<SPEC_BLOCK>(sum, &scr, &Z);
-    if (tid == 0) {
+    if (tid == 0 && is_bonus) {
+        a.mb[row] = m;
+        a.Zb[row] = Z;
+    } else if (tid == 0) {
         const int dt = a.draft_tokens[row];
         u64 md = 0;                                                  // mass of the draft token in this distribution
         if (dt >= 0 && dt < V) md = qfix(emass(z_of(x[dt], T), m), scale);
@@ -134,19 +143,33 @@ struct SpecRow {
     const float *xt, *xd;
     float T, mp, mq, scale;
     double Zp, Zq, scale_d;
+    bool plain;                   // bonus row: the mass of id j is the row's own integer mass, there is no draft
 };
-__device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int row) {
+// Position i of sequence b; i == G is the bonus row.
+__device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
     SpecRow r;
-    r.xt = a.target + (long long)row * a.V;
-    r.xd = a.draft + (long long)row * a.V;
     r.T = a.T;
-    r.mp = a.mp[row];
-    r.mq = a.mq[row];
     r.scale = mass_scale(a.mass_shift);
-    r.Zp = (double)a.Zp[row];
-    r.Zq = (double)a.Zq[row];
     r.scale_d = ldexp(1.0, a.mass_shift);
+    r.plain = i == a.G;
+    if (r.plain) {
+        r.xt = r.xd = a.bonus + (long long)b * a.b_seq;
+        r.mp = r.mq = a.mb[b];
+        r.Zp = r.Zq = 1.0;
+    } else {
+        const int row = b * a.G + i;
+        r.xt = a.target + (long long)b * a.t_seq + (long long)i * a.V;
+        r.xd = a.draft + (long long)b * a.d_seq + (long long)i * a.V;
+        r.mp = a.mp[row];
+        r.mq = a.mq[row];
+        r.Zp = (double)a.Zp[row];
+        r.Zq = (double)a.Zq[row];
+    }
     return r;
+}
+__device__ __forceinline__ u64 spec_mass(const SpecRow &r, float t, float d) {
+    if (r.plain) return qfix(emass(z_of(t, r.T), r.mp), r.scale);    // uniform per row
+    return residual_mass(t, d, r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
 }
 constexpr int SPEC_RUN = 8;                   // run lengths up to this are loaded before any arithmetic
 __device__ __forceinline__ u64 spec_run_mass(const SpecRow &r, int j0, int j1) {
@@ -161,9 +184,9 @@ __device__ __forceinline__ u64 spec_run_mass(const SpecRow &r, int j0, int j1) {
         }
 #pragma unroll
         for (int i = 0; i < SPEC_RUN; i++)
-            if (j0 + i < j1) local += residual_mass(tv[i], dv[i], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+            if (j0 + i < j1) local += spec_mass(r, tv[i], dv[i]);
     } else {
-        for (int j = j0; j < j1; j++) local += residual_mass(r.xt[j], r.xd[j], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+        for (int j = j0; j < j1; j++) local += spec_mass(r, r.xt[j], r.xd[j]);
     }
     return local;
 }
@@ -178,14 +201,14 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_residual_kernel(SpecArgs a) {
             s_first = first;
             if (c == 0) {
                 a.n_accepted[b] = first;
-                if (first == a.G) a.next_token[b] = -1;
+                if (first == a.G && !a.bonus) a.next_token[b] = -1;
             }
         }
     }
     __syncthreads();
     const int first = s_first;
-    if (first == a.G) return;
-    const SpecRow r = spec_row(a, b * a.G + first);
+    if (first == a.G && !a.bonus) return;
+    const SpecRow r = spec_row(a, b, first);
     int j0, j1;
     spec_run(a.V, c, tid, j0, j1);
     const u64 local = spec_run_mass(r, j0, j1);
@@ -202,8 +225,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_pick_kernel(SpecArgs a) {
     const int b = blockIdx.x, tid = threadIdx.x;
     const int G = a.G, V = a.V;
     const int first = a.n_accepted[b];                               // written by the residual launch
-    if (first == G) return;
-    const int row = b * G + first;
+    if (first == G && !a.bonus) return;
     u64 part[SPEC_CHUNKS], R = 0;
 #pragma unroll
     for (int c = 0; c < SPEC_CHUNKS; c++) {
@@ -212,7 +234,8 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_pick_kernel(SpecArgs a) {
     }
     if (R == 0) {
         // residual vanished in fixed point: the target's argmax, lowest id on ties
-        const float *xt = a.target + (long long)row * V;
+        // (never a bonus row: its maximum alone has mass 2^S)
+        const float *xt = a.target + (long long)b * a.t_seq + (long long)first * V;
         float bv = -INFINITY;
         int bi = 0x7FFFFFFF;
         for (int j = tid; j < V; j += SPEC_BLOCK) {
@@ -244,7 +267,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_pick_kernel(SpecArgs a) {
             c = i + 1;
         }
     }
-    const SpecRow r = spec_row(a, row);
+    const SpecRow r = spec_row(a, b, first);
     int j0, j1;
     spec_run(V, c, tid, j0, j1);
     const u64 local = a.run_mass[((long long)b * SPEC_CHUNKS + c) * SPEC_BLOCK + tid];
@@ -255,20 +278,23 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_pick_kernel(SpecArgs a) {
         u64 acc = excl;
         int tok = j1 - 1;
         for (int j = j0; j < j1; j++) {
-            acc += residual_mass(r.xt[j], r.xd[j], r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+            acc += spec_mass(r, r.xt[j], r.xd[j]);
             if (acc >= td) { tok = j; break; }
         }
         a.next_token[b] = tok;
     }
 }
 
-hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st) {
-    const bool resident = a.V <= SPEC_RESIDENT_V && (a.V & 3) == 0 && ((((uintptr_t)a.target) & 15) == 0) &&
-                          ((((uintptr_t)a.draft) & 15) == 0);
+hipError_t launch_spec_verify(const SpecArgs &args, hipStream_t st) {
+    SpecArgs a = args;
+    a.aligned = (a.V & 3) == 0 && ((((uintptr_t)a.target) | ((uintptr_t)a.draft) | ((uintptr_t)a.bonus)) & 15) == 0 &&
+                ((a.t_seq | a.d_seq | (a.bonus ? a.b_seq : 0)) & 3) == 0;
+    const bool resident = a.V <= SPEC_RESIDENT_V && a.aligned;
+    const unsigned stats_grid = (unsigned)(2 * a.B * a.G + (a.bonus ? a.B : 0));
     if (resident)
-        hipLaunchKernelGGL(spec_stats_kernel<true>, dim3((unsigned)(2 * a.B * a.G)), dim3(SPEC_BLOCK), 0, st, a);
+        hipLaunchKernelGGL(spec_stats_kernel<true>, dim3(stats_grid), dim3(SPEC_BLOCK), 0, st, a);
     else
-        hipLaunchKernelGGL(spec_stats_kernel<false>, dim3((unsigned)(2 * a.B * a.G)), dim3(SPEC_BLOCK), 0, st, a);
+        hipLaunchKernelGGL(spec_stats_kernel<false>, dim3(stats_grid), dim3(SPEC_BLOCK), 0, st, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(spec_residual_kernel, dim3((unsigned)(a.B * SPEC_CHUNKS)), dim3(SPEC_BLOCK), 0, st, a);

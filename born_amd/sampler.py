@@ -182,6 +182,15 @@ class Sampler:
                                                  _ptr(draftTokens), _ptr(uAccept), _ptr(uResidual),
                                                  _ptr(nAccepted_out), _ptr(nextToken_out), stream))
 
+    def VerifyBonus(self, target, targetSeqStride, draft, draftSeqStride, bonus, bonusStride, batch, gamma, vocab,
+                    draftTokens, uAccept, uResidual, nAccepted_out, nextToken_out, stream=None):
+        """Verify with the bonus draw: `bonus` = the target's logits one position past the draft, per sequence;
+        `target`, `draft`, `bonus` are raw device addresses (ints) or buffers, strides in elements."""
+        _check(_capi.lib().born_rocm_spec_verify_bonus(self._h, _ptr(target), int(targetSeqStride), _ptr(draft),
+                                                       int(draftSeqStride), _ptr(bonus), int(bonusStride), batch, gamma,
+                                                       vocab, _ptr(draftTokens), _ptr(uAccept), _ptr(uResidual),
+                                                       _ptr(nAccepted_out), _ptr(nextToken_out), stream))
+
 
 def NewSampler(cfg=None, max_batch=256, max_vocab=131072):
     """Mirrors `rocm.NewSampler(cfg)`: fills defaults for zero fields, panics on invalid ones."""
@@ -219,8 +228,20 @@ def sample_host(sampler, logits, uniforms=None, history=None, hist_len=None, nuc
     return out
 
 
-def verify_host(sampler, target, draft, draft_tokens, u_acc, u_res):
+def verify_host(sampler, target, draft, draft_tokens, u_acc, u_res, bonus=False):
+    """bonus=True: `target` is [B, G + 1, V], its last position being the bonus distribution."""
     t = np.ascontiguousarray(target, dtype=np.float32)
+    if bonus:
+        B, G1, V = t.shape
+        G = G1 - 1
+        d_t = DeviceBuffer.from_numpy(t)
+        d_d = DeviceBuffer.from_numpy(np.ascontiguousarray(draft, dtype=np.float32))
+        d_tok = DeviceBuffer.from_numpy(np.ascontiguousarray(draft_tokens, dtype=np.int32))
+        d_ua = DeviceBuffer.from_numpy(np.ascontiguousarray(u_acc, dtype=np.float32))
+        d_ur = DeviceBuffer.from_numpy(np.ascontiguousarray(u_res, dtype=np.float32))
+        d_na, d_nt = DeviceBuffer(4 * B), DeviceBuffer(4 * B)
+        sampler.VerifyBonus(d_t, G1 * V, d_d, G * V, d_t.ptr + 4 * G * V, G1 * V, B, G, V, d_tok, d_ua, d_ur, d_na, d_nt)
+        return dict(n_accepted=d_na.to_numpy(np.int32, (B,)), next_token=d_nt.to_numpy(np.int32, (B,)))
     B, G, V = t.shape
     d_t = DeviceBuffer.from_numpy(t)
     d_d = DeviceBuffer.from_numpy(np.ascontiguousarray(draft, dtype=np.float32))

@@ -129,6 +129,18 @@ int born_rocm_spec_verify(born_sampler *s, const float *target, const float *dra
                           const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out,
                           void *stream);
 
+/* The same step with the bonus draw: `bonus` holds, per sequence, the target's logits one position past the
+ * draft (fp32 [vocab], `bonus_stride` elements apart).  A sequence whose draft tokens are all accepted then
+ * gets next_token = a draw from softmax(bonus / T) by inverse CDF in ascending id order with u_residual[b]
+ * (never -1).  Sequence strides (elements between consecutive sequences) let target and bonus alias one
+ * [batch, gamma + 1, vocab] tensor: target_seq_stride = bonus_stride = (gamma + 1) * vocab,
+ * bonus = target + gamma * vocab.  No counterpart in the reference snapshot. */
+int born_rocm_spec_verify_bonus(born_sampler *s, const float *target, int64_t target_seq_stride, const float *draft,
+                                int64_t draft_seq_stride, const float *bonus, int64_t bonus_stride, int64_t batch,
+                                int64_t gamma, int64_t vocab, const int32_t *draft_tokens, const float *u_accept,
+                                const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out,
+                                void *stream);
+
 /* The logits producer, fp32 on the matrix cores (fp32 operands, fp32 accumulation; the order of the k-sum
  * differs from the reference's sequential loop, so results agree with it to rounding, not bit for bit).
  *

@@ -92,6 +92,23 @@ public:
         check(born_rocm_sampler_status(h_, stream));
     }
 
+    // Verify for a target of gamma + 1 positions per sequence ([batch, gamma + 1, vocab]): its last position is the
+    // bonus distribution a fully accepted sequence draws its next token from (next_token is then never -1).
+    void VerifyBonus(const float *target_dev, const float *draft_dev, int64_t batch, int64_t gamma, int64_t vocab,
+                     const int32_t *draft_tokens_dev, const float *u_accept_dev, const float *u_residual_dev,
+                     std::vector<int32_t> &n_accepted, std::vector<int32_t> &next_token, void *stream = nullptr) {
+        DeviceBuffer out(8 * batch);
+        int32_t *na = static_cast<int32_t *>(out.ptr());
+        const int64_t seq = (gamma + 1) * vocab;
+        check(born_rocm_spec_verify_bonus(h_, target_dev, seq, draft_dev, gamma * vocab, target_dev + gamma * vocab, seq, batch,
+                                          gamma, vocab, draft_tokens_dev, u_accept_dev, u_residual_dev, na, na + batch, stream));
+        std::vector<int32_t> both(static_cast<size_t>(2 * batch));
+        out.download(both.data(), 8 * batch, stream);
+        n_accepted.assign(both.begin(), both.begin() + batch);
+        next_token.assign(both.begin() + batch, both.end());
+        check(born_rocm_sampler_status(h_, stream));
+    }
+
     born_sampler *handle() const { return h_; }
 
 private:

@@ -522,6 +522,46 @@ BORN_EXPORT int64_t born_oracle_spec_verify(
     return bad;
 }
 
+/* Bonus draw of the speculative step (docs/SAMPLING_SPEC.md section 5): for every sequence whose draft tokens
+ * were all accepted (n_accepted[b] == G), next_token[b] = a draw from softmax(bonus[b] / T) by inverse CDF in
+ * ascending id order with u_res[b].  mode 0: fp64; mode 1: integer masses. */
+BORN_EXPORT void born_oracle_spec_bonus_draw(const float *bonus, int64_t B, int64_t V, int64_t stride, int64_t G,
+                                             const float *u_res, float T, int32_t mode, const int32_t *n_accepted,
+                                             int32_t *next_token, uint8_t *near) {
+    int S = born_oracle_mass_shift(V);
+    float *z = (float *)malloc(sizeof(float) * (size_t)V);
+    for (int64_t b = 0; b < B; b++) {
+        if (n_accepted[b] != (int32_t)G) continue;
+        const float *x = bonus + b * stride;
+        float m = -INFINITY;
+        for (int64_t j = 0; j < V; j++) { z[j] = canon(x[j] / T); if (z[j] > m) m = z[j]; }
+        int32_t next = (int32_t)(V - 1);
+        if (mode == 0) {
+            double Z = 0.0;
+            for (int64_t j = 0; j < V; j++) Z += (z[j] == m) ? 1.0 : exp((double)z[j] - (double)m);
+            double t = (double)u_res[b] * Z, c = 0.0;
+            int found = 0;
+            for (int64_t j = 0; j < V; j++) {
+                c += (z[j] == m) ? 1.0 : exp((double)z[j] - (double)m);
+                if (near && fabs(c - t) < 1e-6 * Z) near[b] = 1;
+                if (!found && c > t) { next = (int32_t)j; found = 1; }
+            }
+        } else {
+            uint64_t Z = 0;
+            for (int64_t j = 0; j < V; j++) Z += qmass(z[j], m, S);
+            uint64_t td = (uint64_t)floor((double)u_res[b] * (double)Z) + 1;
+            if (td > Z) td = Z;
+            uint64_t c = 0;
+            for (int64_t j = 0; j < V; j++) {
+                c += qmass(z[j], m, S);
+                if (c >= td) { next = (int32_t)j; break; }
+            }
+        }
+        next_token[b] = next;
+    }
+    free(z);
+}
+
 /* layer-F row statistics used by the operator checks: m, Z (integer mass sum) */
 BORN_EXPORT void born_oracle_row_stats(const float *logits, int64_t B, int64_t V, int64_t stride, float T,
                                        float *m_out, uint64_t *Z_out) {

@@ -60,6 +60,9 @@ def lib():
         L.born_oracle_spec_verify.restype = C.c_int64
         L.born_oracle_spec_verify.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int64, i32p, f32p, f32p,
                                               C.c_float, C.c_int32, i32p, i32p, u8p]
+        L.born_oracle_spec_bonus_draw.restype = None
+        L.born_oracle_spec_bonus_draw.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, f32p, C.c_float,
+                                                  C.c_int32, i32p, i32p, u8p]
         L.born_oracle_row_stats.restype = None
         L.born_oracle_row_stats.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, C.c_float, f32p, u64p]
         _lib = L
@@ -204,7 +207,8 @@ def sample(logits, uniforms, temperature=1.0, top_k=0, top_p=1.0, rep=1.0, histo
     return out
 
 
-def spec_verify(target, draft, draft_tokens, u_acc, u_res, temperature=1.0, mode=MODE_TRUTH):
+def spec_verify(target, draft, draft_tokens, u_acc, u_res, temperature=1.0, mode=MODE_TRUTH, bonus=None):
+    """bonus: fp32 [B, V], the target's logits one position past the draft (drawn from when nothing is rejected)."""
     t = _f32(target)
     d = _f32(draft)
     B, G, V = t.shape
@@ -219,4 +223,9 @@ def spec_verify(target, draft, draft_tokens, u_acc, u_res, temperature=1.0, mode
                                         _p(nacc, C.c_int32), _p(nxt, C.c_int32), _p(near, C.c_uint8))
     if bad < 0:
         raise ValueError("born_oracle_spec_verify: bad arguments")
+    if bonus is not None:
+        bn = _f32(bonus)
+        assert bn.shape == (B, V)
+        lib().born_oracle_spec_bonus_draw(_p(bn, C.c_float), B, V, V, G, _p(ur, C.c_float), float(temperature), int(mode),
+                                          _p(nacc, C.c_int32), _p(nxt, C.c_int32), _p(near, C.c_uint8))
     return dict(n_accepted=nacc, next_token=nxt, near=near.astype(bool), bad_tokens=int(bad))

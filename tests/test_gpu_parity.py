@@ -357,6 +357,44 @@ def test_spec_verify_special_cases(oracle, rocm):
     s.Status()                                                             # the status word clears once read
 
 
+def test_spec_verify_bonus_draw(oracle, rocm):
+    # target given as [B, G + 1, V] (the bonus row is the last position, addressed through sequence strides)
+    rng = np.random.default_rng(31)
+    for (B, G, V, T) in [(24, 4, 32000, 1.0), (7, 3, 3001, 0.8), (3, 2, 40000, 1.3)]:   # resident / scalar / two-sweep rows
+        t = rng.standard_normal((B, G + 1, V), dtype=np.float32)
+        dr = t[:, :G].copy()
+        half = B // 2
+        dr[half:] += (0.6 * rng.standard_normal((B - half, G, V))).astype(np.float32)   # first half: identical models
+        d = rng.integers(0, V, size=(B, G)).astype(np.int32)
+        ua, ur = rng.random((B, G), dtype=np.float32), rng.random(B, dtype=np.float32)
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T), max_batch=B, max_vocab=V)
+        got = rocm.verify_host(s, t, dr, d, ua, ur, bonus=True)
+        tt, bonus = np.ascontiguousarray(t[:, :G]), np.ascontiguousarray(t[:, G])
+        fx = oracle.spec_verify(tt, dr, d, ua, ur, temperature=T, mode=oracle.MODE_FIXED, bonus=bonus)
+        tr = oracle.spec_verify(tt, dr, d, ua, ur, temperature=T, mode=oracle.MODE_TRUTH, bonus=bonus)
+        assert np.array_equal(got["n_accepted"], fx["n_accepted"]), (B, G, V)
+        assert np.array_equal(got["next_token"], fx["next_token"]), (B, G, V)
+        diff = (got["n_accepted"] != tr["n_accepted"]) | (got["next_token"] != tr["next_token"])
+        assert not (diff & ~tr["near"]).any()
+        assert np.all(got["n_accepted"][:half] == G) and np.all(got["next_token"] >= 0)
+        # without bonus rows the same call leaves -1 for the fully accepted sequences
+        plain = rocm.verify_host(s, tt, dr, d, ua, ur)
+        assert np.array_equal(plain["n_accepted"], got["n_accepted"])
+        assert np.all(plain["next_token"][:half] == -1)
+        rej = got["n_accepted"] < G
+        assert np.array_equal(plain["next_token"][rej], got["next_token"][rej])
+        s.Status()
+        s.Close()
+    # uniform bonus row: token = floor(u V)
+    B, G, V = 4, 1, 1000
+    t = np.zeros((B, G + 1, V), np.float32)
+    t[:, 0] = rng.standard_normal((B, V), dtype=np.float32)
+    ur = np.array([0.0, 0.4995, 0.5005, 0.9999], np.float32)
+    s = rocm.NewSampler(max_batch=B, max_vocab=V)
+    got = rocm.verify_host(s, t, t[:, :1].copy(), np.zeros((B, 1), np.int32), np.full((B, 1), 0.5, np.float32), ur, bonus=True)
+    assert got["next_token"].tolist() == [0, 499, 500, 999]
+
+
 # ---------------------------------------------------------------- error behaviour
 
 def test_argument_errors_panic_like_the_go_layer(rocm):

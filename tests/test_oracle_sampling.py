@@ -321,3 +321,55 @@ def test_spec_layers_agree_except_flagged(oracle):
     assert not (diff & ~a["near"]).any()
     r = oracle.spec_verify(t, dr, np.full((B, G), V + 3, np.int32), ua, ur, mode=1)
     assert r["bad_tokens"] == B and np.all(r["n_accepted"] == 0)
+
+
+def test_spec_bonus_draw_closed_forms(oracle):
+    # identical models accept everything; the next token then comes from the bonus row by inverse CDF in
+    # ascending id order.  Closed forms: uniform logits -> floor(u V); one-hot -> that id; p = [.5 .3 .2].
+    rng = np.random.default_rng(21)
+    B, G, V = 5, 3, 8
+    t = rng.normal(0, 1, size=(B, G, V)).astype(np.float32)
+    d = rng.integers(0, V, size=(B, G)).astype(np.int32)
+    ua = rng.random((B, G), dtype=np.float32)
+    ur = np.array([0.0, 0.124, 0.126, 0.6, 0.9999], np.float32)
+    for mode in (0, 1):
+        r = oracle.spec_verify(t, t.copy(), d, ua, ur, mode=mode, bonus=np.zeros((B, V), np.float32))
+        assert np.all(r["n_accepted"] == G)
+        assert r["next_token"].tolist() == [0, 0, 1, 4, 7], mode
+        onehot = np.full((B, V), -1e30, np.float32)
+        onehot[np.arange(B), [3, 0, 7, 5, 2]] = 1.5
+        r = oracle.spec_verify(t, t.copy(), d, ua, ur, mode=mode, bonus=onehot)
+        assert r["next_token"].tolist() == [3, 0, 7, 5, 2], mode
+    p532 = np.tile(LOG(5, 3, 2), (4, 1))
+    t3 = rng.normal(0, 1, size=(4, 2, 3)).astype(np.float32)
+    d3 = rng.integers(0, 3, size=(4, 2)).astype(np.int32)
+    for mode in (0, 1):
+        r = oracle.spec_verify(t3, t3.copy(), d3, rng.random((4, 2), dtype=np.float32),
+                               np.array([0.49, 0.51, 0.79, 0.81], np.float32), mode=mode, bonus=p532)
+        assert r["next_token"].tolist() == [0, 1, 1, 2], mode
+    # a rejected sequence ignores the bonus row: same answer with and without it
+    dr = (t + rng.normal(0, 2.0, size=t.shape)).astype(np.float32)
+    a = oracle.spec_verify(t, dr, d, ua, ur, mode=1)
+    b = oracle.spec_verify(t, dr, d, ua, ur, mode=1, bonus=rng.normal(0, 1, size=(B, V)).astype(np.float32))
+    rej = a["n_accepted"] < G
+    assert rej.any() and np.array_equal(a["n_accepted"], b["n_accepted"])
+    assert np.array_equal(a["next_token"][rej], b["next_token"][rej]) and np.all(b["next_token"][~rej] >= 0)
+
+
+def test_spec_bonus_draw_law_and_brute_force(oracle):
+    # the law of the bonus token is softmax(bonus / T); both layers agree with a numpy cumsum except when flagged
+    rng = np.random.default_rng(22)
+    V, N, T = 7, 30000, 0.8
+    bl = rng.normal(0, 1.5, size=V).astype(np.float32)
+    p = np.exp(bl.astype(np.float64) / np.float32(T)); p /= p.sum()
+    t = np.zeros((N, 1, V), np.float32)
+    d = np.zeros((N, 1), np.int32)
+    ur = rng.random(N, dtype=np.float32)
+    bonus = np.broadcast_to(bl, (N, V)).copy()
+    want = np.searchsorted(np.cumsum(p), ur.astype(np.float64), side="right").clip(0, V - 1)
+    for mode in (0, 1):
+        r = oracle.spec_verify(t, t.copy(), d, np.full((N, 1), 0.5, np.float32), ur, temperature=T, mode=mode, bonus=bonus)
+        assert np.all(r["n_accepted"] == 1)
+        counts = np.bincount(r["next_token"], minlength=V)
+        assert ((counts - N * p) ** 2 / (N * p)).sum() < 30.0, mode
+        assert (r["next_token"] != want).mean() < 1e-3, mode
