@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libborn_rocm.so")
-SOURCES = ["api.hip", "basic_kernels.hip", "topk_row.hip", "nucleus_row.hip", "sample_wide.hip", "spec_kernels.hip", "linear.hip"]
+SOURCES = ["api.hip", "basic_kernels.hip", "topk_row.hip", "nucleus_row.hip", "sample_wide.hip", "spec_kernels.hip", "linear.hip", "tensor_ops.hip"]
 
 # -ffp-contract=off and correctly rounded fp32 division: every floating-point step of the
 # fixed-point pipeline must be a single IEEE rounding, identical on host and device.

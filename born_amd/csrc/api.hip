@@ -465,3 +465,182 @@ int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_
 }
 
 }  // extern "C"
+
+namespace {
+
+// "[2 3]" as Go prints a Shape with %v
+void shape_str(char *buf, size_t cap, const int64_t *shape, int32_t nd) {
+    size_t k = 0;
+    k += (size_t)snprintf(buf + k, cap - k, "[");
+    for (int32_t i = 0; i < nd && k < cap; i++) k += (size_t)snprintf(buf + k, cap - k, i ? " %lld" : "%lld", (long long)shape[i]);
+    if (k < cap) snprintf(buf + k, cap - k, "]");
+}
+
+int check_shape(const char *op, const int64_t *shape, int32_t nd) {
+    if (nd < 0 || nd > TENSOR_MAX_DIMS || (nd > 0 && !shape))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "%s: between 0 and %d dimensions are supported", op, TENSOR_MAX_DIMS);
+    for (int32_t i = 0; i < nd; i++)
+        if (shape[i] <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: invalid shape: dimension %d is %lld", op, i, (long long)shape[i]);
+    return BORN_ROCM_OK;
+}
+
+// internal/tensor/shape.go:83-118
+int broadcast_shapes(const char *op, const int64_t *as, int32_t an, const int64_t *bs, int32_t bn, int64_t *out) {
+    const int32_t n = an > bn ? an : bn;
+    for (int32_t i = 0; i < n; i++) {
+        const int32_t ai = an - 1 - i, bi = bn - 1 - i;
+        const int64_t ad = ai >= 0 ? as[ai] : 1, bd = bi >= 0 ? bs[bi] : 1;
+        if (ad == bd || bd == 1) out[n - 1 - i] = ad;
+        else if (ad == 1) out[n - 1 - i] = bd;
+        else {
+            char sa[160], sb[160];
+            shape_str(sa, sizeof sa, as, an);
+            shape_str(sb, sizeof sb, bs, bn);
+            return fail(BORN_ROCM_ERR_ARGUMENT, "%s: shapes not compatible for broadcasting: %s vs %s (dimension %d: %lld vs %lld)",
+                        op, sa, sb, n - 1 - i, (long long)ad, (long long)bd);
+        }
+    }
+    return BORN_ROCM_OK;
+}
+
+// Drops dimensions of size 1 and merges neighbours that both operands walk contiguously.
+void collapse(TensorIndexArgs &t, bool two) {
+    int k = 0;
+    for (int d = 0; d < t.nd; d++) {
+        if (t.shape[d] == 1) continue;
+        if (k > 0 && t.sa[k - 1] == t.sa[d] * t.shape[d] && (!two || t.sb[k - 1] == t.sb[d] * t.shape[d])) {
+            t.shape[k - 1] *= t.shape[d];
+            t.sa[k - 1] = t.sa[d];
+            t.sb[k - 1] = t.sb[d];
+        } else {
+            t.shape[k] = t.shape[d];
+            t.sa[k] = t.sa[d];
+            t.sb[k] = t.sb[d];
+            k++;
+        }
+    }
+    if (k == 0) {
+        t.shape[0] = 1;
+        t.sa[0] = t.sb[0] = 0;
+        k = 1;
+    }
+    t.nd = k;
+}
+
+int binary_entry(const char *op_name, int op, const float *a, const int64_t *as, int32_t an, const float *b, const int64_t *bs,
+                 int32_t bn, float *out, void *stream) {
+    if (!a || !b || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: null pointer", op_name);
+    int rc = check_shape(op_name, as, an);
+    if (rc == BORN_ROCM_OK) rc = check_shape(op_name, bs, bn);
+    if (rc != BORN_ROCM_OK) return rc;
+    TensorIndexArgs t;
+    memset(&t, 0, sizeof t);
+    int64_t os[TENSOR_MAX_DIMS];
+    rc = broadcast_shapes(op_name, as, an, bs, bn, os);
+    if (rc != BORN_ROCM_OK) return rc;
+    t.nd = an > bn ? an : bn;
+    long long ra = 1, rb = 1;
+    t.n = 1;
+    for (int i = 0; i < t.nd; i++) {
+        const int d = t.nd - 1 - i, ai = an - 1 - i, bi = bn - 1 - i;
+        const int64_t ad = ai >= 0 ? as[ai] : 1, bd = bi >= 0 ? bs[bi] : 1;
+        t.shape[d] = os[d];
+        t.sa[d] = ad == 1 ? 0 : ra;
+        t.sb[d] = bd == 1 ? 0 : rb;
+        ra *= ad;
+        rb *= bd;
+        t.n *= os[d];
+    }
+    if (t.nd == 0) {
+        t.nd = 1;
+        t.shape[0] = 1;
+    }
+    collapse(t, true);
+    HIP_TRY(launch_tensor_binary(op, t, a, b, out, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int born_rocm_broadcast_shape(const int64_t *a_shape, int32_t a_ndim, const int64_t *b_shape, int32_t b_ndim,
+                              int64_t *out_shape) {
+    if (!out_shape) return fail(BORN_ROCM_ERR_ARGUMENT, "broadcast: null output");
+    int rc = check_shape("broadcast", a_shape, a_ndim);
+    if (rc == BORN_ROCM_OK) rc = check_shape("broadcast", b_shape, b_ndim);
+    if (rc != BORN_ROCM_OK) return rc;
+    return broadcast_shapes("broadcast", a_shape, a_ndim, b_shape, b_ndim, out_shape);
+}
+int born_rocm_add(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream) {
+    return binary_entry("add", 0, a, a_shape, a_ndim, b, b_shape, b_ndim, out, stream);
+}
+int born_rocm_sub(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream) {
+    return binary_entry("sub", 1, a, a_shape, a_ndim, b, b_shape, b_ndim, out, stream);
+}
+int born_rocm_mul(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream) {
+    return binary_entry("mul", 2, a, a_shape, a_ndim, b, b_shape, b_ndim, out, stream);
+}
+int born_rocm_div(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream) {
+    return binary_entry("div", 3, a, a_shape, a_ndim, b, b_shape, b_ndim, out, stream);
+}
+
+int born_rocm_transpose(const float *in, const int64_t *shape, int32_t ndim, const int32_t *axes, float *out, void *stream) {
+    if (!in || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "transpose: null pointer");
+    int rc = check_shape("transpose", shape, ndim);
+    if (rc != BORN_ROCM_OK) return rc;
+    int32_t ax[TENSOR_MAX_DIMS];
+    bool seen[TENSOR_MAX_DIMS] = {false};
+    for (int32_t i = 0; i < ndim; i++) {
+        ax[i] = axes ? axes[i] : ndim - 1 - i;                      // default: reverse all dimensions
+        if (ax[i] < 0 || ax[i] >= ndim) return fail(BORN_ROCM_ERR_ARGUMENT, "transpose: invalid axis %d for %dD tensor", ax[i], ndim);
+        if (seen[ax[i]]) return fail(BORN_ROCM_ERR_ARGUMENT, "transpose: duplicate axis %d", ax[i]);
+        seen[ax[i]] = true;
+    }
+    long long src_stride[TENSOR_MAX_DIMS];
+    long long run = 1;
+    for (int32_t d = ndim - 1; d >= 0; d--) {
+        src_stride[d] = run;
+        run *= shape[d];
+    }
+    TensorIndexArgs t;
+    memset(&t, 0, sizeof t);
+    t.nd = ndim;
+    t.n = run;
+    for (int32_t i = 0; i < ndim; i++) {
+        t.shape[i] = shape[ax[i]];
+        t.sa[i] = src_stride[ax[i]];
+    }
+    if (t.nd == 0) {
+        t.nd = 1;
+        t.shape[0] = 1;
+    }
+    collapse(t, false);
+    HIP_TRY(launch_tensor_transpose(t, in, out, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_reshape(const float *in, const int64_t *shape, int32_t ndim, const int64_t *new_shape, int32_t new_ndim,
+                      float *out, void *stream) {
+    if (!in || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "reshape: null pointer");
+    int rc = check_shape("reshape", shape, ndim);
+    if (rc == BORN_ROCM_OK) rc = check_shape("reshape", new_shape, new_ndim);
+    if (rc != BORN_ROCM_OK) return rc;
+    long long n0 = 1, n1 = 1;
+    for (int32_t i = 0; i < ndim; i++) n0 *= shape[i];
+    for (int32_t i = 0; i < new_ndim; i++) n1 *= new_shape[i];
+    if (n0 != n1) {
+        char sa[160], sb[160];
+        shape_str(sa, sizeof sa, shape, ndim);
+        shape_str(sb, sizeof sb, new_shape, new_ndim);
+        return fail(BORN_ROCM_ERR_ARGUMENT, "reshape: incompatible shapes: %s -> %s (different number of elements)", sa, sb);
+    }
+    if (in != out) HIP_TRY(hipMemcpyAsync(out, in, (size_t)n0 * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+}  // extern "C"

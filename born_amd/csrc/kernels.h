@@ -81,6 +81,17 @@ struct GemmArgs {
 };
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st);
 
+// Index map of an element-wise or shape operation over a (collapsed) result of nd dimensions: shape[d] and,
+// per operand, the element stride that result dimension d walks in it (0 where the operand is broadcast).
+constexpr int TENSOR_MAX_DIMS = 8;
+struct TensorIndexArgs {
+    long long n;                  // result elements
+    int nd;
+    long long shape[TENSOR_MAX_DIMS], sa[TENSOR_MAX_DIMS], sb[TENSOR_MAX_DIMS];
+};
+hipError_t launch_tensor_binary(int op, const TensorIndexArgs &t, const float *a, const float *b, float *out, hipStream_t st);
+hipError_t launch_tensor_transpose(const TensorIndexArgs &t, const float *in, float *out, hipStream_t st);
+
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st);
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,

@@ -42,7 +42,11 @@ __device__ __forceinline__ void spec_foreach(const float *x, int V, bool vec, F 
 // One workgroup per (sequence, position, distribution): blockIdx.x = 2 * row + (0 target | 1 draft).  The two
 // distributions of a position are independent, and twice as many work items spread better over the CUs.
 // RESIDENT: V <= SPEC_RESIDENT_V, V % 4 == 0 and the rows 16-byte aligned.
-template <bool RESIDENT>
+// z = canon(x / T); UNIT: T == 1, where the division is the identity and is not computed at all.
+template <bool UNIT>
+__device__ __forceinline__ float spec_z(float x, float T) { return UNIT ? canon(x) : z_of(x, T); }
+
+template <bool RESIDENT, bool UNIT>
 __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     __shared__ BlockScratch scr;
     const int tid = threadIdx.x;
@@ -70,7 +74,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
         for (int i = 0; i < SPEC_NF4; i++) {
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                t[i][c] = z_of(t[i][c], T);                          // the -inf fill stays -inf
+                t[i][c] = spec_z<UNIT>(t[i][c], T);                  // the -inf fill stays -inf
                 m = fmaxf(m, t[i][c]);
             }
         }
@@ -84,9 +88,9 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
         }
     } else {
         const bool vec = a.aligned != 0;
-        spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, z_of(v, T)); });
+        spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, spec_z<UNIT>(v, T)); });
         m = block_max_f32<SPEC_BLOCK>(m, &scr);
-        spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(z_of(v, T), m), scale); });
+        spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(spec_z<UNIT>(v, T), m), scale); });
     }
     u64 Z;
     block_inclusive_scan_u64<SPEC_BLOCK>(sum, &scr, &Z);
@@ -103,10 +107,11 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     }
 }
 
-__device__ __forceinline__ u64 residual_mass(float t, float d, float T, float mp, float mq, float scale, double Zp,
-                                             double Zq, double scale_d) {
-    double pj = (double)qfix(emass(z_of(t, T), mp), scale) / Zp;
-    double qj = (double)qfix(emass(z_of(d, T), mq), scale) / Zq;
+// ip = 1 / Zp and iq = 1 / Zq are formed once per row; each product below is one fp64 rounding.
+__device__ __forceinline__ u64 residual_mass(float t, float d, float T, float mp, float mq, float scale, double ip,
+                                             double iq, double scale_d) {
+    double pj = (double)qfix(emass(z_of(t, T), mp), scale) * ip;
+    double qj = (double)qfix(emass(z_of(d, T), mq), scale) * iq;
     double r = pj > qj ? pj - qj : 0.0;
     return (u64)(r * scale_d);
 }
@@ -142,7 +147,7 @@ __device__ __forceinline__ void spec_run(int V, int c, int tid, int &j0, int &j1
 struct SpecRow {
     const float *xt, *xd;
     float T, mp, mq, scale;
-    double Zp, Zq, scale_d;
+    double Zp, Zq, scale_d;       // Zp, Zq: reciprocals of the integer normalisers
     bool plain;                   // bonus row: the mass of id j is the row's own integer mass, there is no draft
 };
 // Position i of sequence b; i == G is the bonus row.
@@ -162,8 +167,8 @@ __device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
         r.xd = a.draft + (long long)b * a.d_seq + (long long)i * a.V;
         r.mp = a.mp[row];
         r.mq = a.mq[row];
-        r.Zp = (double)a.Zp[row];
-        r.Zq = (double)a.Zq[row];
+        r.Zp = 1.0 / (double)a.Zp[row];
+        r.Zq = 1.0 / (double)a.Zq[row];
     }
     return r;
 }
@@ -291,10 +296,18 @@ hipError_t launch_spec_verify(const SpecArgs &args, hipStream_t st) {
                 ((a.t_seq | a.d_seq | (a.bonus ? a.b_seq : 0)) & 3) == 0;
     const bool resident = a.V <= SPEC_RESIDENT_V && a.aligned;
     const unsigned stats_grid = (unsigned)(2 * a.B * a.G + (a.bonus ? a.B : 0));
-    if (resident)
-        hipLaunchKernelGGL(spec_stats_kernel<true>, dim3(stats_grid), dim3(SPEC_BLOCK), 0, st, a);
-    else
-        hipLaunchKernelGGL(spec_stats_kernel<false>, dim3(stats_grid), dim3(SPEC_BLOCK), 0, st, a);
+    const dim3 sg(stats_grid), sb(SPEC_BLOCK);
+    if (resident) {
+        if (a.T == 1.0f)
+            hipLaunchKernelGGL((spec_stats_kernel<true, true>), sg, sb, 0, st, a);
+        else
+            hipLaunchKernelGGL((spec_stats_kernel<true, false>), sg, sb, 0, st, a);
+    } else {
+        if (a.T == 1.0f)
+            hipLaunchKernelGGL((spec_stats_kernel<false, true>), sg, sb, 0, st, a);
+        else
+            hipLaunchKernelGGL((spec_stats_kernel<false, false>), sg, sb, 0, st, a);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(spec_residual_kernel, dim3((unsigned)(a.B * SPEC_CHUNKS)), dim3(SPEC_BLOCK), 0, st, a);

@@ -160,6 +160,37 @@ int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t
 int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
                      int64_t ldb, int64_t ldc, void *stream);
 
+/* The element-wise and shape operations of tensor.Backend (internal/tensor/backend.go:12-33) on fp32 device
+ * memory.  Operands are row-major and contiguous; shapes are given as arrays of `ndim` extents (0 <= ndim <= 8,
+ * every extent > 0).  `out` is contiguous in the result's shape and must not overlap an operand.
+ *
+ * born_rocm_add / sub / mul / div: NumPy-style broadcasting — Add/Sub/Mul/Div,
+ * internal/backend/cpu/backend.go:32-134; the result shape is that of tensor.BroadcastShapes,
+ * internal/tensor/shape.go:83-118, which born_rocm_broadcast_shape evaluates on the host (out_shape receives
+ * max(a_ndim, b_ndim) extents).  Incompatible shapes return BORN_ROCM_ERR_ARGUMENT with the reference's
+ * message ("add: shapes not compatible for broadcasting: [2 3] vs [4] (dimension 1: 3 vs 4)").  Each result
+ * element is one IEEE fp32 operation, so results equal the CPU backend's bit for bit.
+ *
+ * born_rocm_transpose: out = in with its dimensions permuted, result extent i = shape[axes[i]]; axes == NULL
+ * reverses all dimensions — Transpose, internal/backend/cpu/backend.go:164-209 (same validation messages).
+ *
+ * born_rocm_reshape: same elements in row-major order under a new shape; like the reference (which copies,
+ * internal/backend/cpu/backend.go:137-161) it fills `out`, or does nothing when out == in. */
+int born_rocm_broadcast_shape(const int64_t *a_shape, int32_t a_ndim, const int64_t *b_shape, int32_t b_ndim,
+                              int64_t *out_shape);
+int born_rocm_add(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream);
+int born_rocm_sub(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream);
+int born_rocm_mul(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream);
+int born_rocm_div(const float *a, const int64_t *a_shape, int32_t a_ndim, const float *b, const int64_t *b_shape,
+                  int32_t b_ndim, float *out, void *stream);
+int born_rocm_transpose(const float *in, const int64_t *shape, int32_t ndim, const int32_t *axes, float *out,
+                        void *stream);
+int born_rocm_reshape(const float *in, const int64_t *shape, int32_t ndim, const int64_t *new_shape, int32_t new_ndim,
+                      float *out, void *stream);
+
 /* Building blocks exported for parity tests (device-side evaluation of the specified fp32 exponential and of
  * the built-in uniform stream). */
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream);

@@ -14,6 +14,9 @@
  *   born_oracle_exp_f32          internal/autodiff/ops/log.go:159-185
  *   born_oracle_matmul_f32       internal/backend/cpu/matmul.go:55-71
  *   born_oracle_linear_f32       internal/nn/linear.go:78-107
+ *   born_oracle_binary_f32       internal/backend/cpu/backend.go:32-134, ops_float32.go:61-112,
+ *                                broadcast_helpers.go:9-56, internal/tensor/shape.go:83-118
+ *   born_oracle_transpose_f32    internal/backend/cpu/backend.go:164-209, ops_float32.go:115-151
  *   logits layout                internal/tensor/raw.go:78-105, shape.go:52-63
  * Go's math.Exp / math.Log are stood in for by glibc exp()/log() (both < 1 ulp
  * in fp64; the difference vanishes in the fp32 cast for every vector the
@@ -187,6 +190,77 @@ BORN_EXPORT void born_oracle_linear_f32(float *y, const float *x, const float *w
             for (int64_t kk = 0; kk < in_features; kk++) sum += x[i * in_features + kk] * w[j * in_features + kk];
             y[i * out_features + j] = bias ? sum + bias[j] : sum;
         }
+}
+
+/* Element-wise a (op) b with NumPy-style broadcasting, op 0 add, 1 sub, 2 mul, 3 div.
+ * Shape rule: internal/tensor/shape.go:83-118 (align the shapes at the last dimension; extents must be equal or
+ * one of them 1).  Indexing: broadcast_helpers.go:9-56 (an operand's stride is 0 along a dimension it is
+ * broadcast over; the flat source index is the sum of output coordinate x stride), loop ops_float32.go:61-112.
+ * out_shape receives max(an, bn) extents.  Returns 0, or -1 if the shapes do not broadcast / too many dims. */
+BORN_EXPORT int born_oracle_binary_f32(int op, const float *a, const int64_t *as, int an, const float *b,
+                                       const int64_t *bs, int bn, float *out, int64_t *out_shape) {
+    enum { MAXD = 8 };
+    int nd = an > bn ? an : bn;
+    if (an < 0 || bn < 0 || nd > MAXD) return -1;
+    int64_t os[MAXD], ostr[MAXD], astr[MAXD], bstr[MAXD];
+    for (int i = 0; i < nd; i++) {
+        int ai = an - 1 - i, bi = bn - 1 - i;
+        int64_t ad = ai >= 0 ? as[ai] : 1, bd = bi >= 0 ? bs[bi] : 1;
+        if (ad == bd) os[nd - 1 - i] = ad;
+        else if (ad == 1) os[nd - 1 - i] = bd;
+        else if (bd == 1) os[nd - 1 - i] = ad;
+        else return -1;
+    }
+    int64_t n = 1, ra = 1, rb = 1;
+    for (int d = nd - 1; d >= 0; d--) {
+        int ai = d - (nd - an), bi = d - (nd - bn);
+        ostr[d] = n;
+        n *= os[d];
+        astr[d] = (ai < 0 || as[ai] == 1) ? 0 : ra;
+        bstr[d] = (bi < 0 || bs[bi] == 1) ? 0 : rb;
+        if (ai >= 0) ra *= as[ai];
+        if (bi >= 0) rb *= bs[bi];
+    }
+    if (out_shape) for (int d = 0; d < nd; d++) out_shape[d] = os[d];
+    for (int64_t i = 0; i < n; i++) {
+        int64_t rem = i, ia = 0, ib = 0;
+        for (int d = 0; d < nd; d++) {
+            int64_t coord = rem / ostr[d];
+            rem %= ostr[d];
+            ia += coord * astr[d];
+            ib += coord * bstr[d];
+        }
+        float x = a[ia], y = b[ib];
+        out[i] = op == 0 ? x + y : op == 1 ? x - y : op == 2 ? x * y : x / y;
+    }
+    return 0;
+}
+
+/* Transpose by an axis permutation (axes == NULL: reverse all dimensions): every source element i is sent to
+ * the destination position of its permuted coordinates, ops_float32.go:115-151; validation
+ * backend.go:169-190.  Returns 0, or -1 on an invalid permutation. */
+BORN_EXPORT int born_oracle_transpose_f32(const float *src, const int64_t *shape, int nd, const int32_t *axes,
+                                          float *dst) {
+    enum { MAXD = 8 };
+    if (nd < 0 || nd > MAXD) return -1;
+    int ax[MAXD], seen[MAXD] = {0};
+    int64_t sstr[MAXD], dshape[MAXD], dstr[MAXD], n = 1;
+    for (int i = 0; i < nd; i++) {
+        ax[i] = axes ? axes[i] : nd - 1 - i;
+        if (ax[i] < 0 || ax[i] >= nd || seen[ax[i]]) return -1;
+        seen[ax[i]] = 1;
+    }
+    for (int d = nd - 1; d >= 0; d--) { sstr[d] = n; n *= shape[d]; }
+    for (int i = 0; i < nd; i++) dshape[i] = shape[ax[i]];
+    int64_t run = 1;
+    for (int d = nd - 1; d >= 0; d--) { dstr[d] = run; run *= dshape[d]; }
+    for (int64_t i = 0; i < n; i++) {
+        int64_t coords[MAXD], rem = i, di = 0;
+        for (int d = 0; d < nd; d++) { coords[d] = rem / sstr[d]; rem %= sstr[d]; }
+        for (int d = 0; d < nd; d++) di += coords[ax[d]] * dstr[d];
+        dst[di] = src[i];
+    }
+    return 0;
 }
 
 /* fp64-accumulated softmax (layer T of the standalone operator checks) */
@@ -487,9 +561,10 @@ BORN_EXPORT int64_t born_oracle_spec_verify(
                 accept = (double)u * (double)qd * (double)Zp < (double)pd * (double)Zq;
                 if (!accept) {
                     uint64_t R = 0;
+                    const double ip = 1.0 / (double)Zp, iq = 1.0 / (double)Zq;
                     for (int64_t j = 0; j < V; j++) {
-                        double pj = (double)qmass(zp[j], mp, S) / (double)Zp;
-                        double qj = (double)qmass(zq[j], mq, S) / (double)Zq;
+                        double pj = (double)qmass(zp[j], mp, S) * ip;
+                        double qj = (double)qmass(zq[j], mq, S) * iq;
                         double r = pj > qj ? pj - qj : 0.0;
                         R += (uint64_t)ldexp(r, S);
                     }
@@ -503,8 +578,8 @@ BORN_EXPORT int64_t born_oracle_spec_verify(
                         uint64_t c = 0;
                         next = (int32_t)(V - 1);
                         for (int64_t j = 0; j < V; j++) {
-                            double pj = (double)qmass(zp[j], mp, S) / (double)Zp;
-                            double qj = (double)qmass(zq[j], mq, S) / (double)Zq;
+                            double pj = (double)qmass(zp[j], mp, S) * ip;
+                            double qj = (double)qmass(zq[j], mq, S) * iq;
                             double r = pj > qj ? pj - qj : 0.0;
                             c += (uint64_t)ldexp(r, S);
                             if (c >= td) { next = (int32_t)j; break; }

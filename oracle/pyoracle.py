@@ -34,6 +34,7 @@ def lib():
         L = C.CDLL(_SO)
         f32p, i32p, u8p, f64p, u64p = (C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint8),
                                       C.POINTER(C.c_double), C.POINTER(C.c_uint64))
+        i64p = C.POINTER(C.c_int64)
         L.born_oracle_expneg.restype = C.c_float
         L.born_oracle_expneg.argtypes = [C.c_float]
         L.born_oracle_mass_shift.restype = C.c_int
@@ -51,6 +52,10 @@ def lib():
         L.born_oracle_matmul_f32.argtypes = [f32p, f32p, f32p, C.c_int64, C.c_int64, C.c_int64]
         L.born_oracle_linear_f32.restype = None
         L.born_oracle_linear_f32.argtypes = [f32p, f32p, f32p, f32p, C.c_int64, C.c_int64, C.c_int64]
+        L.born_oracle_binary_f32.restype = C.c_int
+        L.born_oracle_binary_f32.argtypes = [C.c_int, f32p, i64p, C.c_int, f32p, i64p, C.c_int, f32p, i64p]
+        L.born_oracle_transpose_f32.restype = C.c_int
+        L.born_oracle_transpose_f32.argtypes = [f32p, i64p, C.c_int, i32p, f32p]
         L.born_oracle_softmax_f64.restype = None
         L.born_oracle_softmax_f64.argtypes = [f32p, f64p, C.c_int64, C.c_int64, C.c_int64]
         L.born_oracle_sample.restype = C.c_int64
@@ -159,6 +164,46 @@ def linear_ref(x, w, bias=None):
     y = np.empty((batch, fout), dtype=np.float32)
     lib().born_oracle_linear_f32(_p(y, C.c_float), _p(x, C.c_float), _p(w, C.c_float), bp, batch, fin, fout)
     return y
+
+
+def binary_ref(op, a, b):
+    """The reference's Add/Sub/Mul/Div ("add", "sub", "mul", "div") with broadcasting; raises ValueError when
+    the shapes do not broadcast (where the reference panics)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    nd = max(a.ndim, b.ndim)
+    ash = np.array(a.shape if a.ndim else [], dtype=np.int64)
+    bsh = np.array(b.shape if b.ndim else [], dtype=np.int64)
+    osh = np.zeros(max(nd, 1), dtype=np.int64)
+    # the result is allocated at the largest size the rule can produce, then cut to the shape returned
+    cap = 1
+    for i in range(nd):
+        ad = a.shape[a.ndim - 1 - i] if i < a.ndim else 1
+        bd = b.shape[b.ndim - 1 - i] if i < b.ndim else 1
+        cap *= max(ad, bd)
+    out = np.empty(cap, dtype=np.float32)
+    rc = lib().born_oracle_binary_f32(["add", "sub", "mul", "div"].index(op), _p(a, C.c_float), _p(ash, C.c_int64), a.ndim,
+                                      _p(b, C.c_float), _p(bsh, C.c_int64), b.ndim, _p(out, C.c_float), _p(osh, C.c_int64))
+    if rc != 0:
+        raise ValueError(f"{op}: shapes not compatible for broadcasting: {list(a.shape)} vs {list(b.shape)}")
+    shape = tuple(int(d) for d in osh[:nd])
+    return out[:int(np.prod(shape, dtype=np.int64)) if nd else 1].reshape(shape)
+
+
+def transpose_ref(x, axes=None):
+    """The reference's Transpose (axes None: reverse all dimensions); raises ValueError on a bad permutation."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    sh = np.array(x.shape if x.ndim else [], dtype=np.int64)
+    ax = None if axes is None else np.array(list(axes), dtype=np.int32)
+    if ax is not None and len(ax) != x.ndim:
+        raise ValueError(f"transpose: axes length {len(ax)} != ndim {x.ndim}")
+    out = np.empty(x.size, dtype=np.float32)
+    rc = lib().born_oracle_transpose_f32(_p(x, C.c_float), _p(sh, C.c_int64), x.ndim, None if ax is None else _p(ax, C.c_int32),
+                                         _p(out, C.c_float))
+    if rc != 0:
+        raise ValueError("transpose: invalid permutation")
+    order = list(range(x.ndim - 1, -1, -1)) if axes is None else list(axes)
+    return out.reshape(tuple(x.shape[i] for i in order))
 
 
 def row_stats(x, T=1.0):

@@ -1,0 +1,163 @@
+"""GPU parity tests of the tensor.Backend operations on device memory (born_rocm_add/sub/mul/div with
+broadcasting, born_rocm_transpose, born_rocm_reshape, and MatMul through the same interface) against the CPU
+oracle's restatement of the reference's CPU backend.  Every result element is a single IEEE fp32 operation, so
+the bar is bit-exact (MatMul: the tolerance of tests/test_gpu_linear.py)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+OPS = ["add", "sub", "mul", "div"]
+
+
+@pytest.fixture(scope="module")
+def be():
+    from born_amd import backend as B
+    return B
+
+
+@pytest.fixture(scope="module")
+def rocm(be):
+    return be.New()
+
+
+def _call(be, rocm, op, a, b):
+    fn = {"add": rocm.Add, "sub": rocm.Sub, "mul": rocm.Mul, "div": rocm.Div}[op]
+    return fn(be.DeviceTensor.from_numpy(a), be.DeviceTensor.from_numpy(b))
+
+
+def test_backend_identity(rocm):
+    assert rocm.Name() == "ROCm" and rocm.Device() == "ROCm"
+
+
+def test_reference_kats(be, rocm):
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_kats.json")) as f:
+        kats = json.load(f)
+    for case in kats["binary"]:
+        a = np.array(case["a"], dtype=np.float32).reshape(case["a_shape"])
+        b = np.array(case["b"], dtype=np.float32).reshape(case["b_shape"])
+        out = _call(be, rocm, case["op"], a, b)
+        assert list(out.Shape()) == case["shape"] and out.numpy().ravel().tolist() == case["expected"], case["source"]
+    for case in kats["transpose"]:
+        x = np.array(case["data"], dtype=np.float32).reshape(case["shape"])
+        out = rocm.Transpose(be.DeviceTensor.from_numpy(x), *(case["axes"] or []))
+        assert list(out.Shape()) == case["out_shape"] and out.numpy().ravel().tolist() == case["expected"], case["source"]
+    for case in kats["reshape"]:
+        x = np.array(case["data"], dtype=np.float32).reshape(case["shape"])
+        out = rocm.Reshape(be.DeviceTensor.from_numpy(x), case["new_shape"])
+        assert list(out.Shape()) == case["new_shape"] and out.numpy().ravel().tolist() == case["expected"], case["source"]
+    for case in kats["matmul"]:
+        out = rocm.MatMul(be.DeviceTensor.from_numpy(np.array(case["a"], np.float32)), be.DeviceTensor.from_numpy(np.array(case["b"], np.float32)))
+        assert np.max(np.abs(out.numpy().astype(np.float64) - np.array(case["expected"]))) <= case["tol_abs"], case["source"]
+
+
+BROADCASTS = [((4, 5), (4, 5)), ((1000, 257), (1000, 257)), ((4, 5), (5,)), ((300, 4097), (4097,)), ((4, 1), (5,)),
+              ((777, 1), (1, 1300)), ((1,), (3, 2)), ((2, 3, 4), (3, 1)), ((2, 1, 4), (5, 1)), ((3, 1, 2, 1), (4, 1, 5)),
+              ((), (2, 3)), ((2, 3), ()), ((6,), (1, 1, 6)), ((5, 1, 7, 1, 3), (2, 1, 6, 1)), ((64, 1, 33), (64, 50, 1)),
+              ((2, 2, 2, 2, 2, 2, 2, 3), (2, 1, 2, 1, 2, 1, 2, 3))]
+
+
+@pytest.mark.parametrize("shapes", BROADCASTS)
+def test_binary_ops_bit_exact(oracle, be, rocm, shapes):
+    sa, sb = shapes
+    rng = np.random.default_rng(len(sa) * 131 + len(sb) * 17 + int(np.prod(sa + sb + (1,))) % 1000)
+    a = rng.standard_normal(sa).astype(np.float32)
+    b = (rng.standard_normal(sb) + 0.25).astype(np.float32)
+    for op in OPS:
+        want = oracle.binary_ref(op, a, b)
+        got = _call(be, rocm, op, a, b)
+        assert got.Shape() == want.shape, (op, sa, sb)
+        assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32)), (op, sa, sb)
+
+
+def test_binary_special_values(oracle, be, rocm):
+    v = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 3.4e38, 1e-45, -1e-45, 7.0, 1e-30], np.float32)
+    a = np.repeat(v, v.size).reshape(v.size, v.size)
+    for op in OPS:
+        with np.errstate(all="ignore"):
+            want = oracle.binary_ref(op, a, v)
+        got = _call(be, rocm, op, a, v).numpy()
+        same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+        assert same.all(), op
+
+
+def test_unaligned_operands_take_the_scalar_route(oracle, be, rocm):
+    from born_amd import _capi
+    import ctypes as C
+    rng = np.random.default_rng(8)
+    n = 10007
+    a = rng.standard_normal(n + 1).astype(np.float32)
+    b = rng.standard_normal(n + 1).astype(np.float32)
+    da, db = be.DeviceBuffer.from_numpy(a), be.DeviceBuffer.from_numpy(b)
+    out = be.DeviceBuffer.from_numpy(np.full(n + 2, -5.0, np.float32))
+    sh = (C.c_int64 * 1)(n)
+    _capi.check(_capi.lib().born_rocm_sub(da.ptr + 4, sh, 1, db.ptr + 4, sh, 1, out.ptr + 4, None))
+    got = out.to_numpy(np.float32, (n + 2,))
+    assert got[0] == -5.0 and got[-1] == -5.0
+    assert np.array_equal(got[1:-1], a[1:] - b[1:])
+
+
+TRANSPOSES = [((2, 3), None), ((1000, 513), None), ((64, 64), (1, 0)), ((2, 3, 4), None), ((2, 3, 4), (0, 2, 1)),
+              ((5, 300, 129), (0, 2, 1)), ((2, 3, 4), (1, 0, 2)), ((2, 3, 4, 5), (3, 1, 0, 2)), ((7,), None), ((1, 5), (1, 0)),
+              ((3, 4, 5, 6), (0, 1, 3, 2)), ((2, 3, 4), (0, 1, 2)), ((6, 1, 7), (2, 1, 0))]
+
+
+@pytest.mark.parametrize("case", TRANSPOSES)
+def test_transpose_bit_exact(oracle, be, rocm, case):
+    shape, axes = case
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    want = oracle.transpose_ref(x, axes)
+    got = rocm.Transpose(be.DeviceTensor.from_numpy(x), *(axes or []))
+    assert got.Shape() == want.shape
+    assert np.array_equal(got.numpy(), want)
+
+
+def test_reshape_keeps_row_major_order(be, rocm):
+    x = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    out = rocm.Reshape(be.DeviceTensor.from_numpy(x), (6, 4))
+    assert out.Shape() == (6, 4) and np.array_equal(out.numpy().ravel(), x.ravel())
+    out = rocm.Reshape(be.DeviceTensor.from_numpy(x), (24,))
+    assert np.array_equal(out.numpy(), x.ravel())
+
+
+def test_panics_carry_the_reference_messages(be, rocm):
+    t23 = be.DeviceTensor.from_numpy(np.zeros((2, 3), np.float32))
+    t4 = be.DeviceTensor.from_numpy(np.zeros((4,), np.float32))
+    with pytest.raises(be.BackendPanic, match=r"add: shapes not compatible for broadcasting: \[2 3\] vs \[4\] \(dimension 1: 3 vs 4\)"):
+        rocm.Add(t23, t4)
+    with pytest.raises(be.BackendPanic, match=r"div: shapes not compatible for broadcasting"):
+        rocm.Div(t23, t4)
+    with pytest.raises(be.BackendPanic, match=r"reshape: incompatible shapes: \[2 3\] -> \[4 2\] \(different number of elements\)"):
+        rocm.Reshape(t23, (4, 2))
+    with pytest.raises(be.BackendPanic, match=r"transpose: axes length 1 != ndim 2"):
+        rocm.Transpose(t23, 0)
+    with pytest.raises(be.BackendPanic, match=r"transpose: duplicate axis 0"):
+        rocm.Transpose(t23, 0, 0)
+    with pytest.raises(be.BackendPanic, match=r"transpose: invalid axis 2 for 2D tensor"):
+        rocm.Transpose(t23, 0, 2)
+    with pytest.raises(be.BackendPanic, match=r"matmul: shape mismatch \[2,3\] @ \[4,1\]"):
+        rocm.MatMul(t23, be.DeviceTensor.from_numpy(np.zeros((4, 1), np.float32)))
+    with pytest.raises(be.BackendPanic, match=r"matmul: only 2D tensors supported, got 2D and 1D"):
+        rocm.MatMul(t23, t4)
+
+
+def test_linear_forward_as_the_reference_composes_it(oracle, be, rocm):
+    # Linear.Forward = Transpose, MatMul, Reshape of the bias, Add (internal/nn/linear.go:89-104), op by op on the device
+    rng = np.random.default_rng(77)
+    B, K, N = 37, 96, 205
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    wT = rocm.Transpose(be.DeviceTensor.from_numpy(w))
+    y = rocm.MatMul(be.DeviceTensor.from_numpy(x), wT)
+    y = rocm.Add(y, rocm.Reshape(be.DeviceTensor.from_numpy(bias), (1, N)))
+    got = y.numpy()
+    exact = x.astype(np.float64) @ w.astype(np.float64).T + bias[None, :]
+    mag = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T + np.abs(bias)[None, :]
+    assert np.all(np.abs(got - exact) <= (4 * np.sqrt(K) + 2) * 2.0 ** -24 * mag)
+    ref = oracle.linear_ref(x, w, bias)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= (4 * np.sqrt(K) + K + 4) * 2.0 ** -24 * mag)

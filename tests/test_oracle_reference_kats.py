@@ -145,3 +145,44 @@ def test_matmul_and_linear_against_what_the_mathematics_fixes(oracle):
         bias = rng.standard_normal(n).astype(np.float32)
         assert np.array_equal(oracle.linear_ref(a, w, None), c)
         assert np.array_equal(oracle.linear_ref(a, w, bias), c + bias[None, :])
+
+
+def test_binary_reshape_transpose_kats(oracle):
+    for case in KATS["binary"]:
+        a = np.array(case["a"], dtype=np.float32).reshape(case["a_shape"])
+        b = np.array(case["b"], dtype=np.float32).reshape(case["b_shape"])
+        out = oracle.binary_ref(case["op"], a, b)
+        assert list(out.shape) == case["shape"], case["source"]
+        assert out.ravel().tolist() == case["expected"], case["source"]
+    for case in KATS["transpose"]:
+        x = np.array(case["data"], dtype=np.float32).reshape(case["shape"])
+        out = oracle.transpose_ref(x, case["axes"])
+        assert list(out.shape) == case["out_shape"] and out.ravel().tolist() == case["expected"], case["source"]
+    for case in KATS["reshape"]:          # a reshape keeps the row-major element order: nothing to restate beyond the copy
+        x = np.array(case["data"], dtype=np.float32).reshape(case["shape"])
+        assert x.reshape(case["new_shape"]).ravel().tolist() == case["expected"], case["source"]
+
+
+def test_binary_and_transpose_against_numpy(oracle):
+    # NumPy's broadcasting and transpose are the library routines these operations reduce to; a wrong stride,
+    # a swapped operand or an inverted permutation fails on non-square, non-commutative cases
+    import pytest
+    rng = np.random.default_rng(3)
+    shapes = [((4, 5), (4, 5)), ((4, 5), (5,)), ((4, 1), (5,)), ((1,), (3, 2)), ((2, 3, 4), (3, 1)), ((2, 1, 4), (5, 1)),
+              ((3, 1, 2, 1), (4, 1, 5)), ((), (2, 3)), ((2, 3), ()), ((6,), (1, 1, 6))]
+    fns = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+    for sa, sb in shapes:
+        a = rng.standard_normal(sa).astype(np.float32)
+        b = (rng.standard_normal(sb) + 3.0).astype(np.float32)
+        for op, fn in fns.items():
+            want = fn(a, b)
+            got = oracle.binary_ref(op, a, b)
+            assert got.shape == want.shape and np.array_equal(got.view(np.uint32), want.view(np.uint32)), (op, sa, sb)
+    with pytest.raises(ValueError):
+        oracle.binary_ref("add", np.zeros((2, 3), np.float32), np.zeros((4,), np.float32))
+    for shape, axes in [((2, 3), None), ((2, 3, 4), None), ((2, 3, 4), (0, 2, 1)), ((2, 3, 4), (1, 0, 2)), ((2, 3, 4, 5), (3, 1, 0, 2)),
+                        ((7,), None), ((1, 5), (1, 0))]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        assert np.array_equal(oracle.transpose_ref(x, axes), np.transpose(x, axes)), (shape, axes)
+    with pytest.raises(ValueError):
+        oracle.transpose_ref(np.zeros((2, 3), np.float32), (0, 0))
