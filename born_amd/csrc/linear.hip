@@ -113,10 +113,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     const int nk_row = tid >> 5, nn4 = (tid & 31) * 4;               // [k][n] tile of B: k-rows nk_row + 8 * i
 
     const int nslice = (g.K + GK - 1) / GK;
-    // Every workgroup walks the slices of K from a different starting slice (and wraps): workgroups running
+    // Every tile column walks the slices of K from a different starting slice (and wraps): workgroups running
     // at the same time then read different columns of B, whose rows are a large power of two apart for the
-    // usual K, instead of all crowding the same few memory channels.
-    const int rot = (int)(blockIdx.x % (unsigned)nslice);
+    // usual K, instead of all crowding the same few memory channels.  The M-tiles of one tile column share the
+    // start, so that they read the same slices of B at about the same time (from L2 the second time).
+    const int rot = (int)((unsigned)tile_n % (unsigned)nslice);
     f32x4 ra[2][APASS], rb[2][BPASS];                                // two slices in flight
     const float *fa[APASS], *fb[BPASS];                              // FAST: this thread's load addresses at slice 0
     long long fstep_b = 0;
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_dma_kernel(GemmArgs g) 
     }
     const int m0 = tile_m * BM, n0 = tile_n * GN;
     const int nslice = g.K / KS;
-    const int rot = (int)(blockIdx.x % (unsigned)nslice);
+    const int rot = (int)((unsigned)tile_n % (unsigned)nslice);   // per tile column, shared by its M-tiles (see gemm_f32_kernel)
 
     const int lr = lane / SL, lc = lane % SL;
     const float *pa[AJ], *pb[BJ];
