@@ -49,3 +49,49 @@ def test_product_package_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f
+
+
+def test_broadcast_shape_rule_on_the_host():
+    # born_rocm_broadcast_shape is pure host logic (tensor.BroadcastShapes, internal/tensor/shape.go:83-118):
+    # checked here against numpy's rule, with the reference's message for incompatible shapes
+    import numpy as np
+    from born_amd import _capi
+    L = _capi.lib()
+
+    def arr(shape):
+        return (ctypes.c_int64 * max(len(shape), 1))(*shape)
+
+    cases = [((2, 3), (2, 3)), ((3, 1), (4,)), ((2, 3), (1,)), ((2, 1, 4), (5, 1)), ((), (2, 3)), ((7,), ()), ((1, 1, 6), (6,)),
+             ((3, 1, 2, 1), (4, 1, 5))]
+    for a, b in cases:
+        nd = max(len(a), len(b))
+        out = (ctypes.c_int64 * max(nd, 1))()
+        assert L.born_rocm_broadcast_shape(arr(a), len(a), arr(b), len(b), out) == _capi.OK, (a, b)
+        assert tuple(out[i] for i in range(nd)) == np.broadcast_shapes(a, b), (a, b)
+    out = (ctypes.c_int64 * 2)()
+    assert L.born_rocm_broadcast_shape(arr((2, 3)), 2, arr((4,)), 1, out) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_last_error() == b"broadcast: shapes not compatible for broadcasting: [2 3] vs [4] (dimension 1: 3 vs 4)"
+    assert L.born_rocm_broadcast_shape(arr((2, 0)), 2, arr((4,)), 1, out) == _capi.ERR_ARGUMENT      # empty extent
+    assert L.born_rocm_broadcast_shape(arr((1,) * 9), 9, arr((4,)), 1, out) == _capi.ERR_ARGUMENT    # too many dimensions
+
+
+def test_producer_and_backend_argument_checks_need_no_gpu():
+    from born_amd import _capi
+    L = _capi.lib()
+    one = (ctypes.c_int64 * 1)(4)
+    assert L.born_rocm_linear(None, 1, 1, 1, None, 1, 1, None, None, 1, None) == _capi.ERR_ARGUMENT
+    assert b"linear: null pointer" in L.born_rocm_last_error()
+    buf = ctypes.create_string_buffer(64)                 # never dereferenced: the checks below fail first
+    p = ctypes.addressof(buf)
+    assert L.born_rocm_matmul(p, p, p, 2, 0, 2, 2, 2, 2, None) == _capi.ERR_ARGUMENT
+    assert b"matmul: shape" in L.born_rocm_last_error()
+    assert L.born_rocm_matmul(p, p, p, 2, 2, 2, 1, 2, 2, None) == _capi.ERR_ARGUMENT
+    assert b"row pitch" in L.born_rocm_last_error()
+    assert L.born_rocm_add(None, one, 1, None, one, 1, None, None) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_transpose(p, (ctypes.c_int64 * 2)(2, 3), 2, (ctypes.c_int32 * 2)(0, 0), p, None) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_last_error() == b"transpose: duplicate axis 0"
+    assert L.born_rocm_transpose(p, (ctypes.c_int64 * 2)(2, 3), 2, (ctypes.c_int32 * 2)(0, 2), p, None) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_last_error() == b"transpose: invalid axis 2 for 2D tensor"
+    assert L.born_rocm_reshape(p, (ctypes.c_int64 * 2)(2, 3), 2, (ctypes.c_int64 * 2)(4, 2), 2, p, None) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_last_error() == b"reshape: incompatible shapes: [2 3] -> [4 2] (different number of elements)"
+    assert L.born_rocm_spec_verify_bonus(None, None, 0, None, 0, None, 0, 1, 1, 1, None, None, None, None, None, None) == _capi.ERR_ARGUMENT
