@@ -91,6 +91,34 @@ func (l *Linear) Forward(input DeviceBuffer, shape []int, out DeviceBuffer, stre
 		(*C.float)(l.bias.ptr), (*C.float)(out.ptr), C.int64_t(l.outFeatures), stream))
 }
 
+// ForwardArgmax is greedy decoding fused into the layer: tokens[b] = argmax_j Forward(input)[b][j] with the
+// reference's tie rule (internal/nn/cross_entropy.go:241-251), the [batch, out_features] logits never written.
+// The sampler handle provides the per-row workspace (batch <= its maxBatch).
+func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]int32, error) {
+	if len(shape) != 2 {
+		panic(fmt.Sprintf("Linear.Forward: expected 2D input [batch, features], got shape %v", shape))
+	}
+	if shape[1] != l.inFeatures {
+		panic(fmt.Sprintf("Linear.Forward: expected input with %d features, got %d", l.inFeatures, shape[1]))
+	}
+	batch := shape[0]
+	out, err := Alloc(int64(4 * batch))
+	if err != nil {
+		return nil, err
+	}
+	defer out.Free()
+	if err = check(C.born_rocm_linear_argmax(s.h, (*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
+		C.int64_t(l.inFeatures), (*C.float)(l.weight.ptr), C.int64_t(l.outFeatures), C.int64_t(l.inFeatures),
+		(*C.float)(l.bias.ptr), (*C.int32_t)(out.ptr), nil)); err != nil {
+		return nil, err
+	}
+	tokens := make([]int32, batch)
+	if err = out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil {
+		return nil, err
+	}
+	return tokens, nil
+}
+
 // MatMul computes c[m,n] = a[m,k] @ b[k,n] (tensor.Backend.MatMul, internal/tensor/backend.go:20; the CPU
 // form and its panics: internal/backend/cpu/matmul.go:13-50).  aShape and bShape are the 2-D shapes.
 func MatMul(a DeviceBuffer, aShape []int, b DeviceBuffer, bShape []int, c DeviceBuffer, stream unsafe.Pointer) error {

@@ -51,6 +51,7 @@ struct born_sampler {
     int *arg_idx;
     int *status;
     unsigned long long *counters;
+    unsigned long long *lm_best;   // [max_batch] packed (value, ~column) keys of the greedy-decode LM head
     // spec-verify statistics:
     float *sp_mp, *sp_mq, *sp_mb;
     unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd, *sp_part, *sp_run, *sp_Zb;
@@ -159,6 +160,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     alloc((void **)&s->arg_val, segs * sizeof(float));
     alloc((void **)&s->arg_idx, segs * sizeof(int));
     alloc((void **)&s->status, sizeof(int));
+    alloc((void **)&s->lm_best, rows * LM_BEST_PITCH * sizeof(unsigned long long));
     alloc((void **)&s->counters, (64 + 8 * rows) * sizeof(unsigned long long));   // [0..2] work counters; debug builds: [8..] phase stamps, [64..] per-row stamps
     if (e != hipSuccess) {
         born_rocm_sampler_destroy(s);
@@ -170,7 +172,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters,
+    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters, s->lm_best,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run,
                     s->sp_mb,     s->sp_Zb};
     for (void *p : ptrs)
@@ -427,9 +429,11 @@ int born_rocm_uniforms(int64_t seed, int64_t step, float *u_out, int64_t n, void
     return BORN_ROCM_OK;
 }
 
+// `best` / `tokens` set: the greedy-decode epilogue (c unused); otherwise the product is stored to c.
 static int gemm_entry(const char *what, const float *a, const float *b, const float *bias, float *c, int64_t m,
-                      int64_t k, int64_t n, int64_t lda, int64_t ldb, int64_t ldc, bool bt, void *stream) {
-    if (!a || !b || !c) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: null pointer", what);
+                      int64_t k, int64_t n, int64_t lda, int64_t ldb, int64_t ldc, bool bt, void *stream,
+                      unsigned long long *best = nullptr, int32_t *tokens = nullptr) {
+    if (!a || !b || (!c && !best)) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: null pointer", what);
     const int64_t lim = 0x7FFFFFFF;
     if (m <= 0 || k <= 0 || n <= 0 || m > lim - 256 || k > lim - 64 || n > lim - 256)
         return fail(BORN_ROCM_ERR_ARGUMENT, "%s: shape [%lld,%lld] @ [%lld,%lld] out of range", what, (long long)m,
@@ -437,6 +441,9 @@ static int gemm_entry(const char *what, const float *a, const float *b, const fl
     if (lda < k || ldb < (bt ? k : n) || ldc < n)
         return fail(BORN_ROCM_ERR_ARGUMENT, "%s: a row pitch is smaller than the row", what);
     GemmArgs g;
+    memset(&g, 0, sizeof g);
+    g.best = best;
+    g.tokens = tokens;
     g.a = a;
     g.b = b;
     g.bias = bias;
@@ -462,6 +469,17 @@ int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t
 int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
                      int64_t ldb, int64_t ldc, void *stream) {
     return gemm_entry("matmul", a, b, nullptr, c, m, k, n, lda, ldb, ldc, false, stream);
+}
+int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
+                            const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
+                            int32_t *tokens_out, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_argmax: null handle");
+    if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_argmax: null pointer");
+    if (batch > s->max_batch)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "linear_argmax: batch %lld exceeds the handle's %lld", (long long)batch,
+                    (long long)s->max_batch);
+    return gemm_entry("linear_argmax", x, weight, bias, nullptr, batch, in_features, out_features, x_stride, w_stride,
+                      out_features, true, stream, s->lm_best, tokens_out);
 }
 
 }  // extern "C"

@@ -78,7 +78,10 @@ struct GemmArgs {
     int M, N, K;
     long long lda, ldb, ldc;      // row pitches in elements
     bool vec_a, vec_b;            // 128-bit loads are legal (base 16-byte aligned, pitch a multiple of 4)
+    unsigned long long *best;     // non-null: keep only each row's largest result as a packed key (c unused), keys LM_BEST_PITCH words apart ..
+    int *tokens;                  // .. and write its column here
 };
+constexpr int LM_BEST_PITCH = 16;
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st);
 
 // Index map of an element-wise or shape operation over a (collapsed) result of nd dimensions: shape[d] and,

@@ -69,9 +69,116 @@ __device__ __forceinline__ f32x4 gemm_load_n4(const float *base, long long ld, i
     return v;
 }
 
+// What a tile does with its results.  EPI 0: adds the bias and stores them.  EPI 1 (greedy decode fused into
+// the LM head): keeps only the largest logit of every row as a packed key, value in the high word, ~column in
+// the low word, merged across tiles with a 64-bit atomic max, so the logits are never written.  The key order
+// is the reference's argmax (internal/nn/cross_entropy.go:241-251): larger value wins, the lower index on equal
+// values (-0 equals +0), a NaN never wins, except at index 0 where the reference returns 0 whatever follows.
+__device__ __forceinline__ u64 gemm_argmax_key(float v, int col) {
+    if (v != v) return col == 0 ? ~0ull : 0ull;
+    v = v == 0.0f ? 0.0f : v;
+    return ((u64)ordkey(v) << 32) | (u64)(0xFFFFFFFFu - (u32)col);
+}
+__device__ __forceinline__ u64 gemm_max_u64(u64 a, u64 b) { return a > b ? a : b; }
+// The keys of consecutive rows sit a cache line apart, and a tile first looks at the key it would have to beat:
+// the value only ever grows, so a tile that does not beat what it reads (however stale) cannot win, and all but
+// the first few tiles of a row skip the atomic.
+constexpr int GEMM_BEST_PITCH = LM_BEST_PITCH; // u64 words between the keys of consecutive rows (a 128-byte line each)
+__device__ __forceinline__ void gemm_offer_key(u64 *best, int row, u64 key) {
+    u64 *p = best + (long long)row * GEMM_BEST_PITCH;
+    if (key > __builtin_nontemporal_load(p)) atomicMax(p, key);
+}
+__device__ __forceinline__ u64 gemm_shfl_xor_u64(u64 x, int o) {
+    const u32 lo = (u32)__shfl_xor((int)(u32)x, o, WAVE), hi = (u32)__shfl_xor((int)(u32)(x >> 32), o, WAVE);
+    return ((u64)hi << 32) | lo;
+}
+
+// 32 x 32 blocks: accumulator v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4, column r of its block
+template <int EPI, int IB, int JB>
+__device__ __forceinline__ void gemm_finish32(const GemmArgs &g, const f32x16 (&acc)[IB][JB], int m0, int n0, int wm,
+                                              int wn, int r, int h) {
+    if (EPI == 0) {
+#pragma unroll
+        for (int j = 0; j < JB; j++) {
+            const int col = n0 + (wn * JB + j) * 32 + r;
+            if (col >= g.N) continue;
+            const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int i = 0; i < IB; i++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                    if (row < g.M) {
+                        const float sum = acc[i][j][v];
+                        g.c[(long long)row * g.ldc + col] = g.bias ? sum + bias : sum;
+                    }
+                }
+            }
+        }
+    } else {
+        float bias[JB];
+#pragma unroll
+        for (int j = 0; j < JB; j++) {
+            const int col = n0 + (wn * JB + j) * 32 + r;
+            bias[j] = (g.bias && col < g.N) ? g.bias[col] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < IB; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                if (m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + (v & 3) >= g.M) continue;   // past the batch for both h: wave-uniform
+                u64 key = 0ull;
+#pragma unroll
+                for (int j = 0; j < JB; j++) {
+                    const int col = n0 + (wn * JB + j) * 32 + r;
+                    const float sum = acc[i][j][v];
+                    if (col < g.N) key = gemm_max_u64(key, gemm_argmax_key(g.bias ? sum + bias[j] : sum, col));
+                }
+#pragma unroll
+                for (int o = 16; o > 0; o >>= 1) key = gemm_max_u64(key, gemm_shfl_xor_u64(key, o));   // the 32 lanes of this h
+                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                if (r == 0 && row < g.M && key) gemm_offer_key(g.best, row, key);
+            }
+        }
+    }
+}
+// 16 x 16 blocks: accumulator v of lane (j, q) is row 4 q + v, column j of its block
+template <int EPI>
+__device__ __forceinline__ void gemm_finish16(const GemmArgs &g, const f32x4 (&acc16)[2], int m0, int n0, int wn, int j16,
+                                              int q16) {
+    if (EPI == 0) {
+#pragma unroll
+        for (int jb = 0; jb < 2; jb++) {
+            const int col = n0 + wn * 32 + jb * 16 + j16;
+            if (col >= g.N) continue;
+            const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = m0 + 4 * q16 + v;
+                if (row < g.M) g.c[(long long)row * g.ldc + col] = g.bias ? acc16[jb][v] + bias : acc16[jb][v];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            if (m0 + v >= g.M) continue;                              // past the batch for every q: wave-uniform
+            u64 key = 0ull;
+#pragma unroll
+            for (int jb = 0; jb < 2; jb++) {
+                const int col = n0 + wn * 32 + jb * 16 + j16;
+                if (col < g.N) key = gemm_max_u64(key, gemm_argmax_key(g.bias ? acc16[jb][v] + g.bias[col] : acc16[jb][v], col));
+            }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) key = gemm_max_u64(key, gemm_shfl_xor_u64(key, o));         // the 16 lanes of this q
+            const int row = m0 + 4 * q16 + v;
+            if (j16 == 0 && row < g.M && key) gemm_offer_key(g.best, row, key);
+        }
+    }
+}
+
 // FAST: every 128-bit load is legal and K is a multiple of the slice, so the loads need no guards (rows past
 // the matrix are clamped onto its last row: their products land in accumulators that are never stored).
-template <bool BT, bool FAST, int BM>
+template <bool BT, bool FAST, int BM, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     constexpr bool SMALL = BM == 16;                                 // 16-row tile: v_mfma_f32_16x16x4_f32, two 16-column blocks per wave
     constexpr int AROWS = SMALL ? LROWS : BM;                        // tile rows of A loaded and kept in LDS
@@ -245,38 +352,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
         if (s + 1 < nslice) step(s + 1, ra[1], rb[1], ra[0], rb[0]);  // uniform
     }
 
-    if (SMALL) {                                                     // accumulator v of lane (j, q) is row 4 q + v, column j of its block
-#pragma unroll
-        for (int jb = 0; jb < 2; jb++) {
-            const int col = n0 + wn * 32 + jb * 16 + j16;
-            if (col >= g.N) continue;
-            const float bias = g.bias ? g.bias[col] : 0.f;
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int row = m0 + 4 * q16 + v;
-                if (row < g.M) g.c[(long long)row * g.ldc + col] = g.bias ? acc16[jb][v] + bias : acc16[jb][v];
-            }
-        }
-        return;
-    }
-    // C: accumulator v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4, column r of its 32 x 32 block
-#pragma unroll
-    for (int j = 0; j < JB; j++) {
-        const int col = n0 + (wn * JB + j) * 32 + r;
-        if (col >= g.N) continue;
-        const float bias = g.bias ? g.bias[col] : 0.f;
-#pragma unroll
-        for (int i = 0; i < IB; i++) {
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
-                if (row < g.M) {
-                    const float sum = acc[i][j][v];
-                    g.c[(long long)row * g.ldc + col] = g.bias ? sum + bias : sum;
-                }
-            }
-        }
-    }
+    if (SMALL)
+        gemm_finish16<EPI>(g, acc16, m0, n0, wn, j16, q16);
+    else
+        gemm_finish32<EPI, IB, JB>(g, acc, m0, n0, wm, wn, r, h);
 }
 
 // The same tile computation for W[N,K] operands whose loads need no guards, with the global loads written
@@ -287,7 +366,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
 // 16-byte slots and the layout cannot be padded.  Slot of (row, c = k / 4) is 8 row + (c ^ ((row >> 1) & 7)):
 // the operand reads of 16 consecutive rows at one c then fall into 16 different bank groups.  Each lane picks
 // the global address that belongs to its slot: a wave instruction still reads 8 rows x 128 contiguous bytes.
-template <int BM, int KS>
+template <int BM, int KS, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_dma_kernel(GemmArgs g) {
     constexpr int WGM = BM == 128 ? 2 : 1, WGN = 4 / WGM;
     constexpr int IB = BM / (32 * WGM), JB = GN / (32 * WGN);
@@ -398,37 +477,50 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_dma_kernel(GemmArgs g) 
         }
     }
 
-#pragma unroll
-    for (int j = 0; j < JB; j++) {
-        const int col = n0 + (wn * JB + j) * 32 + r;
-        if (col >= g.N) continue;
-        const float bias = g.bias ? g.bias[col] : 0.f;
-#pragma unroll
-        for (int i = 0; i < IB; i++) {
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
-                if (row < g.M) {
-                    const float sum = acc[i][j][v];
-                    g.c[(long long)row * g.ldc + col] = g.bias ? sum + bias : sum;
-                }
-            }
-        }
-    }
+    gemm_finish32<EPI, IB, JB>(g, acc, m0, n0, wm, wn, r, h);
 }
 
-template <bool BT, bool FAST>
+template <bool BT, bool FAST, int EPI>
 static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
     const long long nt = (g.N + GN - 1) / GN;
     const dim3 bl(GEMM_THREADS);
     if (bm == 16)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 16>), dim3((unsigned)(nt * ((g.M + 15) / 16))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 16, EPI>), dim3((unsigned)(nt * ((g.M + 15) / 16))), bl, 0, st, g);
     else if (bm == 32)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32>), dim3((unsigned)(nt * ((g.M + 31) / 32))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32, EPI>), dim3((unsigned)(nt * ((g.M + 31) / 32))), bl, 0, st, g);
     else if (bm == 64)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64>), dim3((unsigned)(nt * ((g.M + 63) / 64))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64, EPI>), dim3((unsigned)(nt * ((g.M + 63) / 64))), bl, 0, st, g);
     else
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 128>), dim3((unsigned)(nt * ((g.M + 127) / 128))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 128, EPI>), dim3((unsigned)(nt * ((g.M + 127) / 128))), bl, 0, st, g);
+}
+
+template <int EPI>
+static void launch_gemm_nt(const GemmArgs &g, int bm, long long grid, bool fast, hipStream_t st) {
+    if (fast && bm >= 32) {
+        const dim3 gr((unsigned)grid), bl(GEMM_THREADS);
+        if (bm == 128)
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<128, GK, EPI>), gr, bl, 0, st, g);
+        else if (bm == 64)
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<64, GK, EPI>), gr, bl, 0, st, g);
+        else
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<32, GK, EPI>), gr, bl, 0, st, g);
+    } else if (fast) {
+        launch_gemm_bm<true, true, EPI>(g, bm, st);
+    } else {
+        launch_gemm_bm<true, false, EPI>(g, bm, st);
+    }
+}
+
+// Greedy decode fused into the LM head: the keys are 0 ("nothing seen") when a call starts; the tiny launch
+// that turns the winning key of every row into its token id also puts the 0 back for the next call.
+__global__ void argmax_keys_token_kernel(u64 *best, int *tokens, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        u64 *p = best + (long long)i * GEMM_BEST_PITCH;
+        const u64 k = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tokens[i] = k ? (int)(0xFFFFFFFFu - (u32)k) : 0;
+        *p = 0ull;
+    }
 }
 
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
@@ -436,24 +528,17 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
-    if (b_transposed && fast && bm >= 32) {
-        const dim3 gr((unsigned)grid), bl(GEMM_THREADS);
-        if (bm == 128)
-            hipLaunchKernelGGL((gemm_f32_dma_kernel<128, GK>), gr, bl, 0, st, g);
-        else if (bm == 64)
-            hipLaunchKernelGGL((gemm_f32_dma_kernel<64, GK>), gr, bl, 0, st, g);
-        else
-            hipLaunchKernelGGL((gemm_f32_dma_kernel<32, GK>), gr, bl, 0, st, g);
+    if (g.best) {                                                    // argmax epilogue: W[N,K] form only
+        if (!b_transposed || !g.tokens) return hipErrorInvalidValue;
+        launch_gemm_nt<1>(g, bm, grid, fast, st);
+        hipLaunchKernelGGL(argmax_keys_token_kernel, dim3((unsigned)((g.M + 255) / 256)), dim3(256), 0, st, g.best, g.tokens, g.M);
     } else if (b_transposed) {
-        if (fast)
-            launch_gemm_bm<true, true>(g, bm, st);
-        else
-            launch_gemm_bm<true, false>(g, bm, st);
+        launch_gemm_nt<0>(g, bm, grid, fast, st);
     } else {
         if (fast)
-            launch_gemm_bm<false, true>(g, bm, st);
+            launch_gemm_bm<false, true, 0>(g, bm, st);
         else
-            launch_gemm_bm<false, false>(g, bm, st);
+            launch_gemm_bm<false, false, 0>(g, bm, st);
     }
     return hipGetLastError();
 }

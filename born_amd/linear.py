@@ -69,6 +69,20 @@ class Linear:
         return out
 
 
+def ForwardArgmax(sampler, layer, input, input_shape, tokens_out, stream=None):
+    """Greedy decode fused into the LM head: tokens_out[b] = argmax of layer.Forward(input)[b], the logits never
+    written (born_rocm_linear_argmax).  `sampler` provides the per-row workspace."""
+    if len(input_shape) != 2:
+        raise LinearPanic(f"Linear.Forward: expected 2D input [batch, features], got shape {list(input_shape)}")
+    batch, feat = int(input_shape[0]), int(input_shape[1])
+    if feat != layer.inFeatures:
+        raise LinearPanic(f"Linear.Forward: expected input with {layer.inFeatures} features, got {feat}")
+    _check(_capi.lib().born_rocm_linear_argmax(sampler._h, _ptr(input), batch, layer.inFeatures, layer.inFeatures,
+                                               _ptr(layer.weight), layer.outFeatures, layer.inFeatures, _ptr(layer.bias),
+                                               _ptr(tokens_out), stream))
+    return tokens_out
+
+
 def NewLinear(in_features, out_features, seed=None, stream=None):
     """Xavier/Glorot-uniform weights in [-sqrt(6/(in+out)), +sqrt(6/(in+out))], zero bias, both uploaded to the
     device.  The reference draws from the process-global unseeded generator; a seed can be given here."""

@@ -160,6 +160,16 @@ int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t
 int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
                      int64_t ldb, int64_t ldc, void *stream);
 
+/* Greedy decode fused into the LM head: tokens_out[b] = argmax_j (x[b] @ weight[j]^T + bias[j]) without the
+ * [batch, out_features] logits ever being written: every tile of the product keeps its rows' largest value and
+ * the tiles are merged by a 64-bit atomic max.  Same arithmetic as born_rocm_linear followed by
+ * born_rocm_argmax and the same token ids, including the reference's tie rule (`argmax`,
+ * internal/nn/cross_entropy.go:241-251; Linear.Forward, internal/nn/linear.go:78-107).  The handle provides the
+ * per-row workspace (batch <= its max_batch); one call at a time per handle. */
+int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
+                            const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
+                            int32_t *tokens_out, void *stream);
+
 /* The element-wise and shape operations of tensor.Backend (internal/tensor/backend.go:12-33) on fp32 device
  * memory.  Operands are row-major and contiguous; shapes are given as arrays of `ndim` extents (0 <= ndim <= 8,
  * every extent > 0).  `out` is contiguous in the result's shape and must not overlap an operand.

@@ -220,3 +220,58 @@ def test_lm_head_full_size_spot_check(rocm, lin):
     want = x.astype(np.float64) @ colsum + bias.astype(np.float64).sum()
     scale = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).sum(axis=0)
     assert np.all(np.abs(got.astype(np.float64).sum(axis=1) - want) <= (4 * np.sqrt(K) + 2) * EPS * scale)
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 300), (5, 1000, 77), (16, 128, 260), (17, 96, 132), (48, 64, 256), (65, 32, 128),
+                                   (130, 257, 300), (256, 512, 1000), (12, 4096, 32000)])
+def test_lm_head_argmax_fused_equals_linear_then_argmax(oracle, rocm, lin, shape):
+    # tokens of the fused call == argmax kernel over the materialised logits of the same GEMM (bit-identical
+    # arithmetic), == the oracle's argmax over those logits
+    M, K, N = shape
+    rng = np.random.default_rng(M * 31 + K * 7 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    s = rocm.NewSampler(max_batch=M, max_vocab=N)
+    for b in (bias, None):
+        layer = lin.Linear(K, N, rocm.DeviceBuffer.from_numpy(w), None if b is None else rocm.DeviceBuffer.from_numpy(b))
+        dx = rocm.DeviceBuffer.from_numpy(x)
+        logits = rocm.DeviceBuffer(M * N * 4)
+        layer.Forward(dx, (M, K), logits)
+        tok_ref = rocm.DeviceBuffer(4 * M)
+        s.Argmax(logits, M, N, tok_ref)
+        tok = rocm.DeviceBuffer(4 * M)
+        lin.ForwardArgmax(s, layer, dx, (M, K), tok)
+        got = tok.to_numpy(np.int32, (M,))
+        assert np.array_equal(got, tok_ref.to_numpy(np.int32, (M,))), shape
+        assert np.array_equal(got, oracle.argmax_ref(logits.to_numpy(np.float32, (M, N)))), shape
+    s.Close()
+
+
+def test_lm_head_argmax_tie_and_nan_rules(oracle, rocm, lin):
+    # integer-valued operands make exact ties; NaN never wins except at column 0; -0 equals +0; an all -inf row
+    M, K, N = 6, 32, 300
+    x = np.zeros((M, K), np.float32)
+    w = np.zeros((N, K), np.float32)
+    x[:, 0] = 1.0
+    w[:, 0] = -5.0
+    w[[7, 150, 299], 0] = 3.0                      # rows 0..: three equal maxima -> lowest column 7
+    bias = np.zeros((M, N), np.float32)
+    cases = []
+    b0 = np.zeros(N, np.float32); cases.append(b0)                                    # tie -> 7
+    b1 = b0.copy(); b1[200] = np.nan; cases.append(b1)                                # NaN elsewhere ignored -> 7
+    b2 = b0.copy(); b2[0] = np.nan; cases.append(b2)                                  # NaN at column 0 -> 0
+    b3 = np.full(N, -np.inf, np.float32); cases.append(b3)                            # all -inf -> 0
+    b4 = b3.copy(); b4[[40, 41]] = [5.0 - 0.0, 5.0]; cases.append(b4)                 # two finite: w*x + b = 0 at both? no: -5+5 = 0 vs 0 -> tie -> 40
+    b5 = np.full(N, np.nan, np.float32); cases.append(b5)                             # all NaN -> 0
+    s = rocm.NewSampler(max_batch=M, max_vocab=N)
+    for b in cases:
+        layer = lin.Linear(K, N, rocm.DeviceBuffer.from_numpy(w), rocm.DeviceBuffer.from_numpy(b))
+        dx = rocm.DeviceBuffer.from_numpy(x)
+        tok = rocm.DeviceBuffer(4 * M)
+        lin.ForwardArgmax(s, layer, dx, (M, K), tok)
+        with np.errstate(all="ignore"):
+            logits = oracle.linear_ref(x, w, b)
+        want = oracle.argmax_ref(logits)
+        assert np.array_equal(tok.to_numpy(np.int32, (M,)), want), (b[:3], want)
+    s.Close()
