@@ -275,3 +275,64 @@ def test_lm_head_argmax_tie_and_nan_rules(oracle, rocm, lin):
         want = oracle.argmax_ref(logits)
         assert np.array_equal(tok.to_numpy(np.int32, (M,)), want), (b[:3], want)
     s.Close()
+
+
+def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin):
+    # the decode step (LM head -> sampler, two launches) captured once into a HIP graph and replayed with new
+    # activations and uniforms in the same buffers; every replay is checked against the eager calls and the
+    # oracle, with eager work and synchronisations between the replays.  The HIP runtime is driven through
+    # ctypes (the library itself exports no graph calls).
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    def ok(rc):
+        assert rc == 0, f"HIP error {rc}"
+    rng = np.random.default_rng(404)
+    B, K, V = 4, 256, 32000
+    w = rocm.DeviceBuffer.from_numpy((rng.standard_normal((V, K)) * (2.0 / np.sqrt(K))).astype(np.float32))
+    bias = rocm.DeviceBuffer.from_numpy((0.1 * rng.standard_normal(V)).astype(np.float32))
+    hist_h = rng.integers(0, V, (B, 32)).astype(np.int32)
+    hist = rocm.DeviceBuffer.from_numpy(hist_h)
+    x, u = rocm.DeviceBuffer(B * K * 4), rocm.DeviceBuffer(B * 4)
+    logits, tokens, probs = rocm.DeviceBuffer(B * V * 4), rocm.DeviceBuffer(B * 4), rocm.DeviceBuffer(B * 4)
+    layer = lin.Linear(K, V, w, bias)
+    smp = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1), max_batch=B, max_vocab=V)
+
+    def step(stream):
+        layer.Forward(x, (B, K), logits, stream=stream)
+        smp.Sample(logits, B, V, hist, None, u, tokens, probs, hist_stride=32, stream=stream)
+
+    def upload(buf, a):
+        from born_amd import _capi
+        _capi.check(_capi.lib().born_rocm_h2d(buf.ptr, a.ctypes.data, a.nbytes, None))
+
+    stream = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(stream)))
+    upload(x, np.zeros((B, K), np.float32))
+    upload(u, np.zeros(B, np.float32))
+    step(stream)                                                  # warm-up outside the capture
+    ok(hip.hipStreamSynchronize(stream))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(stream, 0))                      # hipStreamCaptureModeGlobal
+    step(stream)
+    ok(hip.hipStreamEndCapture(stream, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)))
+    for it in range(4):
+        xh = rng.standard_normal((B, K)).astype(np.float32)
+        uh = rng.random(B, dtype=np.float32)
+        upload(x, xh)
+        upload(u, uh)
+        ok(hip.hipGraphLaunch(gexec, stream))
+        ok(hip.hipStreamSynchronize(stream))
+        got_tok, got_logits = tokens.to_numpy(np.int32, (B,)), logits.to_numpy(np.float32, (B, V))
+        upload(tokens, np.full(B, -1, np.int32))
+        step(None)                                                # the same step, eagerly, on the null stream
+        ok(hip.hipDeviceSynchronize())
+        assert np.array_equal(got_tok, tokens.to_numpy(np.int32, (B,))), it
+        assert np.array_equal(got_logits, logits.to_numpy(np.float32, (B, V))), it
+        want = oracle.sample(got_logits, uh, 0.8, 40, 0.95, 1.1, hist_h, None, mode=oracle.MODE_FIXED)
+        assert np.array_equal(got_tok, want["tokens"]), it
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(stream))
+    smp.Status()
+    smp.Close()
