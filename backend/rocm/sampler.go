@@ -207,3 +207,32 @@ func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab in
 	}
 	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
 }
+
+// RowConfigs carries a configuration per row of a batch (continuous batching): device arrays of `batch` values,
+// fp32 for Temperatures / TopPs / Penalties, int32 for TopKs; a zero DeviceBuffer means "the sampler's value for
+// every row".  Values mean what the SamplerConfig fields mean after defaults.
+type RowConfigs struct {
+	Temperatures, TopKs, TopPs, Penalties DeviceBuffer
+}
+
+// SampleRows is Sample with a configuration per row.  A row with invalid values yields token 0 and an error
+// from the status check that follows the copy of the tokens.
+func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
+	histLen, uniforms DeviceBuffer, rows RowConfigs) ([]int32, error) {
+	out, err := Alloc(int64(4 * batch))
+	if err != nil {
+		return nil, err
+	}
+	defer out.Free()
+	if err = check(C.born_rocm_sample_rows(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
+		C.int64_t(vocab), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
+		(*C.float)(uniforms.ptr), (*C.float)(rows.Temperatures.ptr), (*C.int32_t)(rows.TopKs.ptr),
+		(*C.float)(rows.TopPs.ptr), (*C.float)(rows.Penalties.ptr), (*C.int32_t)(out.ptr), nil, nil)); err != nil {
+		return nil, err
+	}
+	tokens := make([]int32, batch)
+	if err = out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil {
+		return nil, err
+	}
+	return tokens, check(C.born_rocm_sampler_status(s.h, nil))
+}

@@ -209,8 +209,9 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (st) {
         HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s", (st & 1) ? "out-of-range history id " : "",
-                    (st & 2) ? "out-of-range draft token " : "", (st & 4) ? "an internal inconsistency (please report)" : "");
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s", (st & 1) ? "out-of-range history id " : "",
+                    (st & 2) ? "out-of-range draft token " : "", (st & 8) ? "invalid per-row configuration " : "",
+                    (st & 4) ? "an internal inconsistency (please report)" : "");
     }
     return BORN_ROCM_OK;
 }
@@ -279,10 +280,11 @@ int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, i
     return BORN_ROCM_OK;
 }
 
-int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
-                     const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
-                     int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
-                     float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
+static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                       const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                       const float *row_T, const int32_t *row_k, const float *row_p, const float *row_rep,
+                       int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
+                       float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
     int rc = check_logits("sample", s, logits, batch, vocab, row_stride);
     if (rc) return rc;
     if (!tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample: null tokens_out");
@@ -321,17 +323,48 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     a.mass_shift = mass_shift(vocab);
 
     hipStream_t st = (hipStream_t)stream;
-    // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
-    const bool boosts = history && a.rep < 1.0f;
-    if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
-        HIP_TRY(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
-    } else if (s->path != 1 && a.top_k == 0) {
-        HIP_TRY(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
+    if (row_T || row_k || row_p || row_rep) {
+        // every kernel over the whole batch: each workgroup takes its row only if the row's configuration is its own
+        RowConfigs rows;
+        rows.T = row_T;
+        rows.k = row_k;
+        rows.p = row_p;
+        rows.rep = row_rep;
+        rows.path = s->path;
+        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) HIP_TRY(launch_topk_row(a, st, &rows));
+        if (s->path != 1) HIP_TRY(launch_nucleus_row(a, st, &rows));
+        HIP_TRY(launch_sample_wide(a, st, &rows));
     } else {
-        HIP_TRY(launch_sample_wide(a, st));
+        // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
+        const bool boosts = history && a.rep < 1.0f;
+        if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
+            HIP_TRY(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
+        } else if (s->path != 1 && a.top_k == 0) {
+            HIP_TRY(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
+        } else {
+            HIP_TRY(launch_sample_wide(a, st));
+        }
     }
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;
+}
+
+int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                     int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
+                     float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
+    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, nullptr, nullptr,
+                       nullptr, nullptr, tokens_out, probs_out, nucleus_len_out, nucleus_ids_out, nucleus_probs_out,
+                       nucleus_cap, stream);
+}
+
+int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                          const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                          const float *temperature_rows, const int32_t *top_k_rows, const float *top_p_rows,
+                          const float *repetition_penalty_rows, int32_t *tokens_out, float *probs_out, void *stream) {
+    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, temperature_rows,
+                       top_k_rows, top_p_rows, repetition_penalty_rows, tokens_out, probs_out, nullptr, nullptr, nullptr, 0,
+                       stream);
 }
 
 static int spec_verify_impl(born_sampler *s, const float *target, int64_t target_seq_stride, const float *draft,

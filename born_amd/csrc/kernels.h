@@ -50,6 +50,14 @@ struct SampleArgs {
     int mass_shift;
 };
 
+// Per-row configurations (device arrays of B values, each optional): a second argument of the per-row kernel
+// instances only, so that the uniform instances keep their argument block (and register allocation) as it is.
+struct RowConfigs {
+    const float *T, *p, *rep;
+    const int *k;
+    int path;                     // the handle's kernel selection (1 = always the general kernel)
+};
+
 struct SpecArgs {
     const float *target, *draft;
     const float *bonus;           // [B] rows of the target at position G (drawn from when nothing is rejected), or null
@@ -101,9 +109,9 @@ hipError_t launch_softmax(const float *logits, int B, int V, long long stride, f
                           hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
-hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st);
-hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st);
-hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st);
+hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
+hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
 hipError_t configure_nucleus();
 size_t nucleus_lds_bytes(int V);
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);

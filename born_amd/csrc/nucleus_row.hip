@@ -16,6 +16,7 @@
 // the rank keys of that bin, 11 bits per sweep.
 #include "dev_common.h"
 #include "kernels.h"
+#include "row_config.h"
 
 namespace born {
 
@@ -128,7 +129,8 @@ __device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, fl
     if (w == 0) yhi = INFINITY;
 }
 
-__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
+// cfg_T, cfg_p, cfg_rep: the row's temperature, top_p and repetition penalty (the handle's, or the row's own).
+__device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep) {
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over;
@@ -147,8 +149,8 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     r.x = a.logits + (long long)row * a.row_stride;
     r.V = V;
     r.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
-    r.T = a.T;
-    r.rep = a.rep;
+    r.T = cfg_T;
+    r.rep = cfg_rep;
     r.scale = mass_scale(a.mass_shift);
     const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
-    r.penal = (a.rep != 1.0f) && hlen > 0;
+    r.penal = (cfg_rep != 1.0f) && hlen > 0;
     if (r.penal)
         for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
     for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;
@@ -215,11 +217,11 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     const u64 *cum = mass;
 
     // ---- the bins to gather: the top-p cut's, and the draw's predicted from the interval [tp, cum[bp]]
-    const bool cut = a.top_p < 1.0f;
+    const bool cut = cfg_p < 1.0f;
     u64 tp = Zk;
     int w0, w1, w2;
     if (cut) {
-        tp = top_p_target(a.top_p, Zk);
+        tp = top_p_target(cfg_p, Zk);
         w0 = nuc_first_reaching(cum, tp);
         const u64 hi = cum[w0] < Zk ? cum[w0] : Zk;
         w1 = nuc_first_reaching(cum, draw_target(u, tp));
@@ -424,18 +426,36 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
     BORN_STAMP(a, row, 7);
 }
 
+__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
+    nucleus_row_body(a, a.T, a.top_p, a.rep);
+}
+// The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
+__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs a, RowConfigs rc) {
+    float T, p, rep;
+    int k;
+    bool invalid;
+    if (!row_config_values(a, rc, (int)blockIdx.x, ROUTE_NUCLEUS, T, k, p, rep, invalid)) return;   // workgroup-uniform, before any barrier
+    nucleus_row_body(a, T, p, rep);
+}
+
 size_t nucleus_lds_bytes(int V) {
     return sizeof(u64) * (NUC_BINS + NUC_WAVES * NUC_WCAP + 2 * NUC_CAP) + sizeof(u32) * (size_t)((V + 31) / 32);
 }
 
-hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st) {
-    hipLaunchKernelGGL(nucleus_row_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a);
+hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
+    if (rows)
+        hipLaunchKernelGGL(nucleus_row_rows_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a, *rows);
+    else
+        hipLaunchKernelGGL(nucleus_row_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a);
     return hipGetLastError();
 }
 
 hipError_t configure_nucleus() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_rows_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
 }
 
 }  // namespace born

@@ -9,6 +9,7 @@
 #include "dev_common.h"
 #include "finish.h"
 #include "kernels.h"
+#include "row_config.h"
 
 namespace born {
 size_t wide_lds_bytes(int V) {
@@ -24,7 +25,7 @@ size_t wide_lds_bytes(int V) {
 
 namespace born {
 
-hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st) { return w1024::launch(a, st); }
+hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) { return w1024::launch(a, st, rows); }
 
 hipError_t configure_kernels() { return w1024::configure(); }
 

@@ -474,14 +474,40 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a) {
     __shared__ u64 s_u64[4];
     wide_row(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
 }
+// The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own;
+// rows whose configuration is invalid end here, reported through the status word.
+__global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_rows_kernel(SampleArgs a, RowConfigs rc) {
+    extern __shared__ u64 dyn[];
+    __shared__ BlockScratch scr;
+    __shared__ int s_int[8];
+    __shared__ u64 s_u64[4];
+    bool invalid;
+    if (!row_config(a, rc, (int)blockIdx.x, ROUTE_GENERAL, invalid)) return;   // workgroup-uniform, before any barrier
+    if (invalid) {
+        if (threadIdx.x == 0) {
+            atomicOr(a.status, 8);
+            a.tokens[blockIdx.x] = 0;
+            if (a.probs) a.probs[blockIdx.x] = 0.0f;
+            if (a.nuc_len) a.nuc_len[blockIdx.x] = -1;
+        }
+        return;
+    }
+    wide_row(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
+}
 
-hipError_t launch(const SampleArgs &a, hipStream_t st) {
-    hipLaunchKernelGGL(sample_wide_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a);
+hipError_t launch(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
+    if (rows)
+        hipLaunchKernelGGL(sample_wide_rows_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a, *rows);
+    else
+        hipLaunchKernelGGL(sample_wide_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a);
     return hipGetLastError();
 }
 
 hipError_t configure() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(sample_wide_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_wide_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)wide_lds_bytes((int)WIDE_MAX_VOCAB));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(sample_wide_rows_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)wide_lds_bytes((int)WIDE_MAX_VOCAB));
 }
 

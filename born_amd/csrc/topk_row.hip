@@ -26,6 +26,7 @@
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
+#include "row_config.h"
 
 namespace born {
 
@@ -251,7 +252,7 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
 }
 
 template <bool VEC>
-__global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
+__device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ u64 pool[ROW_POOL];
     uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= Tw
     uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);       // candidates >= T2; .y bit 31 = id occurs in the history
@@ -509,12 +510,31 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     if (tid == 0) atomicAdd(&a.counters[0], 1ull);
 }
 
-hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st) {
+template <bool VEC>
+__global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
+    topk_row_body<VEC>(a);
+}
+// The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
+template <bool VEC>
+__global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, RowConfigs rc) {
+    bool invalid;
+    if (!row_config(a, rc, (int)blockIdx.x, ROUTE_TOPK, invalid)) return;   // workgroup-uniform, before any barrier
+    topk_row_body<VEC>(a);
+}
+
+hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
     const bool vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
-    if (vec)
-        hipLaunchKernelGGL(topk_row_kernel<true>, dim3((unsigned)a.B), dim3(ROW_BLOCK), 0, st, a);
-    else
-        hipLaunchKernelGGL(topk_row_kernel<false>, dim3((unsigned)a.B), dim3(ROW_BLOCK), 0, st, a);
+    const dim3 gr((unsigned)a.B), bl(ROW_BLOCK);
+    if (rows) {
+        if (vec)
+            hipLaunchKernelGGL(topk_row_rows_kernel<true>, gr, bl, 0, st, a, *rows);
+        else
+            hipLaunchKernelGGL(topk_row_rows_kernel<false>, gr, bl, 0, st, a, *rows);
+    } else if (vec) {
+        hipLaunchKernelGGL(topk_row_kernel<true>, gr, bl, 0, st, a);
+    } else {
+        hipLaunchKernelGGL(topk_row_kernel<false>, gr, bl, 0, st, a);
+    }
     return hipGetLastError();
 }
 

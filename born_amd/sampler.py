@@ -176,6 +176,15 @@ class Sampler:
                                             _ptr(tokens_out), _ptr(probs_out), _ptr(nl), _ptr(ni), _ptr(npb),
                                             cap, stream))
 
+    def SampleRows(self, logits, batch, vocab, history, histLen, uniforms, temperatures, topKs, topPs, penalties,
+                   tokens_out, probs_out=None, row_stride=None, hist_stride=0, stream=None):
+        """Sample with a configuration per row: device arrays of `batch` values, each may be None (=> the
+        handle's value)."""
+        _check(_capi.lib().born_rocm_sample_rows(self._h, _ptr(logits), batch, vocab, row_stride or vocab,
+                                                 _ptr(history), _ptr(histLen), hist_stride, _ptr(uniforms),
+                                                 _ptr(temperatures), _ptr(topKs), _ptr(topPs), _ptr(penalties),
+                                                 _ptr(tokens_out), _ptr(probs_out), stream))
+
     def Verify(self, target, draft, batch, gamma, vocab, draftTokens, uAccept, uResidual, nAccepted_out,
                nextToken_out, stream=None):
         _check(_capi.lib().born_rocm_spec_verify(self._h, _ptr(target), _ptr(draft), batch, gamma, vocab,

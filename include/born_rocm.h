@@ -119,6 +119,19 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
                      int32_t *nucleus_len_out, int32_t *nucleus_ids_out, float *nucleus_probs_out,
                      int64_t nucleus_cap, void *stream);
 
+/* The same step with a configuration per row (continuous batching: requests with different settings share a
+ * batch).  temperature_rows / top_p_rows / repetition_penalty_rows fp32 [batch], top_k_rows int32 [batch], all on
+ * the device, each may be NULL (=> the handle's value for every row).  Values mean what the fields of
+ * born_sampler_config mean after defaults (top_k <= 0 or >= vocab: no top-k cut; top_p = 1: no top-p cut;
+ * repetition_penalty = 1: none).  A row whose values are invalid (temperature or penalty not positive and finite,
+ * top_p outside (0, 1]) gets token 0 and BORN_ROCM_ERR_DATA from born_rocm_sampler_status.  Every row's result
+ * equals what born_rocm_sample returns for that row under a handle configured with the row's values.  No
+ * counterpart in the reference snapshot. */
+int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                          const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                          const float *temperature_rows, const int32_t *top_k_rows, const float *top_p_rows,
+                          const float *repetition_penalty_rows, int32_t *tokens_out, float *probs_out, void *stream);
+
 /* Speculative-decoding accept/reject with residual max(0, p - q) resampling.
  * No counterpart in the reference snapshot.
  *   target, draft  fp32 [batch, gamma, vocab] contiguous;  draft_tokens int32 [batch, gamma]

@@ -395,6 +395,70 @@ def test_spec_verify_bonus_draw(oracle, rocm):
     assert got["next_token"].tolist() == [0, 499, 500, 999]
 
 
+# ---------------------------------------------------------------- a configuration per row
+
+def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0):
+    B, V = x.shape
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=7, TopP=0.8, RepetitionPenalty=1.3), max_batch=B, max_vocab=V)
+    s.SetPath(path)
+    dev = lambda a, dt: None if a is None else rocm.DeviceBuffer.from_numpy(np.ascontiguousarray(a, dtype=dt))
+    tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
+    s.SampleRows(dev(x, np.float32), B, V, dev(hist, np.int32), None, dev(u, np.float32), dev(Ts, np.float32), dev(ks, np.int32),
+                 dev(ps, np.float32), dev(reps, np.float32), tok, pr, hist_stride=0 if hist is None else hist.shape[1])
+    return s, tok.to_numpy(np.int32, (B,)), pr.to_numpy(np.float32, (B,))
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
+    # one batch, every row its own settings, covering the three kernels' territories (top-k <= 64, no top-k cut,
+    # top-k > 64, a boosting penalty < 1); each row must equal the oracle under that row's settings
+    rng = np.random.default_rng(77)
+    B, V, H = 24, 9000, 48
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, (B, H)).astype(np.int32)
+    Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 300, V, V + 5, -3], B).astype(np.int32)
+    ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
+    reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
+    s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path)
+    s.Status()
+    for b in range(B):
+        want = oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(ks[b]), float(ps[b]), float(reps[b]), hist[b:b + 1], None,
+                             mode=oracle.MODE_FIXED)
+        assert tok[b] == want["tokens"][0], (b, Ts[b], ks[b], ps[b], reps[b])
+        assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], b
+    # arrays left out fall back to the handle's values (T 0.9, top_k 7, top_p 0.8, penalty 1.3)
+    s2, tok2, pr2 = _sample_rows(rocm, x, u, hist, None, ks, None, None, path)
+    s2.Status()
+    for b in range(B):
+        want = oracle.sample(x[b:b + 1], u[b:b + 1], 0.9, int(ks[b]), 0.8, 1.3, hist[b:b + 1], None, mode=oracle.MODE_FIXED)
+        assert tok2[b] == want["tokens"][0], b
+    if path == 0:
+        c = s.Counters()
+        assert c["topk_rows"] > 0 and c["general_rows"] > 0                 # more than one kernel took rows
+    s.Close()
+    s2.Close()
+
+
+def test_per_row_invalid_configuration_is_reported(oracle, rocm):
+    rng = np.random.default_rng(78)
+    B, V = 6, 3000
+    x = rng.standard_normal((B, V)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    Ts = np.array([1.0, 0.0, 1.0, np.nan, 0.7, 1.0], np.float32)
+    ps = np.array([0.9, 0.9, 1.5, 0.9, 0.9, 0.0], np.float32)
+    ks = np.array([10, 10, 10, 10, 0, 10], np.int32)
+    s, tok, pr = _sample_rows(rocm, x, u, None, Ts, ks, ps, None)
+    with pytest.raises(rocm.BornRocmError, match="invalid per-row configuration"):
+        s.Status()
+    for b in (0, 4):                                                         # the valid rows are unaffected
+        want = oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(ks[b]), float(ps[b]), 1.3, None, None, mode=oracle.MODE_FIXED)
+        assert tok[b] == want["tokens"][0]
+    assert tok[[1, 2, 3, 5]].tolist() == [0, 0, 0, 0]
+    s.Close()
+
+
 # ---------------------------------------------------------------- error behaviour
 
 def test_argument_errors_panic_like_the_go_layer(rocm):
