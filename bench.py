@@ -14,7 +14,11 @@ the one the metric is quoted on).  Prints ONE JSON line.
   cpu_baseline the CPU oracle's reference-arithmetic mode timed on this box's host, one thread,
                on a bounded sample of the same workload
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C5] [--no-cpu]
+The other configurations of BASELINE.json run through the same script for their own figures (never the
+headline): --config C1 | C2 (multinomial) | C2g (greedy argmax) | C4 (speculative verify, 64 x 5 positions;
+"tokens" are verified draft positions) | C5.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C2g|C4|C5] [--no-cpu] [--no-producer]
 """
 import argparse
 import json
@@ -155,8 +159,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    gen = {"C1": synth.c1, "C2": synth.c2, "C3": synth.c3, "C5": synth.c5}[args.config]
+    gen = {"C1": synth.c1, "C2": synth.c2, "C2g": synth.c2, "C3": synth.c3, "C4": synth.c4, "C5": synth.c5}[args.config]
     w = gen()
+    if args.config in ("C2g", "C4"):
+        return main_other(args, torch, S, synth, w, dev)
     B, V = w.logits.shape
     # Several copies of the logits at different addresses, used round-robin: together they exceed the 256 MB
     # Infinity Cache, so every step streams its logits from HBM as a fresh LM-head output would be.
@@ -209,7 +215,8 @@ def main():
 
     # a step is a single launch, so the step time is the kernel's launch-to-launch duration
     ms_kernel = ms
-    kernel_name = "topk_row_kernel" if (1 <= w.top_k <= 64 and args.path == 0) else "sample_wide_kernel"
+    kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 64 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
+        if args.path == 0 else "sample_wide_kernel"
     alg_bytes = w.algorithmic_bytes()
     achieved = alg_bytes / (ms_kernel * 1e-3) / 1e9
 
@@ -235,11 +242,56 @@ def main():
                      "algorithmic_bytes_per_launch": alg_bytes,
                      "kernel_ms": ms_kernel},
     }
-    if not args.no_producer:
+    if not args.no_producer and args.config == "C3":
         out["producer"] = producer_leg(torch, dev, smp, step, B, V, args.hidden, logits_all, stream, max(5, args.steps // 10))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
+
+
+def main_other(args, torch, S, synth, w, dev):
+    """C2g (greedy argmax over the C2 logits) and C4 (speculative verify): the same JSON shape, own figures."""
+    stream = torch.cuda.current_stream().cuda_stream
+    if args.config == "C2g":
+        B, V = w.logits.shape
+        logits = torch.from_numpy(w.logits).to(dev)
+        tokens = torch.empty(B, dtype=torch.int32, device=dev)
+        smp = S.NewSampler(max_batch=B, max_vocab=V)
+        step = lambda: smp.Argmax(logits, B, V, tokens, stream=stream)
+        units, alg_bytes, kernel_name = B, B * V * 4 + 4 * B, "argmax_partial_kernel"
+        workload = f"C2 greedy: batch {B} x vocab {V}, argmax; logits resident in HBM"
+    else:
+        e = w.extra
+        B, G, V = e["target"].shape
+        t, d = torch.from_numpy(e["target"]).to(dev), torch.from_numpy(e["draft"]).to(dev)
+        dt = torch.from_numpy(e["draft_tokens"]).to(dev)
+        ua, ur = torch.from_numpy(e["u_acc"]).to(dev), torch.from_numpy(e["u_res"]).to(dev)
+        na = torch.empty(B, dtype=torch.int32, device=dev)
+        nt = torch.empty(B, dtype=torch.int32, device=dev)
+        smp = S.NewSampler(S.SamplerConfig(Temperature=w.temperature), max_batch=B, max_vocab=V)
+        step = lambda: smp.Verify(t, d, B, G, V, dt, ua, ur, na, nt, stream=stream)
+        units, alg_bytes, kernel_name = B * G, 2 * B * G * V * 4 + 4 * B * G * 2 + 4 * B * 3, "spec_stats_kernel (+ residual, pick)"
+        workload = f"C4: speculative verify, {B} sequences x {G} positions x vocab {V}, T={w.temperature}; \"tokens\" are verified draft positions"
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    smp.Status(stream)
+    achieved = alg_bytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "sampled tokens/s; achieved HBM GB/s (secondary configuration, not the headline)", "value": units / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": workload, "seed": synth.BASE_SEED},
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": alg_bytes, "kernel_ms": ms,
+                     "note": "whole step (all its launches) over the algorithmic bytes"}}))
 
 
 if __name__ == "__main__":
