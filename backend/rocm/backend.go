@@ -52,7 +52,7 @@ func cShape(shape []int) (*C.int64_t, C.int32_t) {
 
 // Backend is the reference's tensor.Backend (internal/tensor/backend.go:12-33) on device tensors: the same
 // operations, names, shape rules and panic texts as the CPU backend (internal/backend/cpu/backend.go), fp32.
-// Every operation returns a new tensor and leaves its operands untouched.  Conv2D and MaxPool2D are not built.
+// Every operation returns a new tensor and leaves its operands untouched.
 // A failed allocation or launch panics like the reference's failed NewRaw ("add: failed to create result
 // tensor: ...").
 type Backend struct{}
@@ -134,6 +134,63 @@ func (b *Backend) MatMul(x, y *Tensor) *Tensor {
 	}
 	if err := MatMul(x.Buf, x.Shape, y.Buf, y.Shape, res.Buf, nil); err != nil {
 		panic(fmt.Sprintf("matmul: %v", err))
+	}
+	return res
+}
+
+// Conv2D performs 2D convolution: input [N, C_in, H, W], kernel [C_out, C_in, K_h, K_w], zero padding.
+func (b *Backend) Conv2D(input, kernel *Tensor, stride, padding int) *Tensor {
+	if len(input.Shape) != 4 {
+		panic(fmt.Sprintf("conv2d: input must be 4D [N,C,H,W], got %dD", len(input.Shape)))
+	}
+	if len(kernel.Shape) != 4 {
+		panic(fmt.Sprintf("conv2d: kernel must be 4D [C_out,C_in,K_h,K_w], got %dD", len(kernel.Shape)))
+	}
+	if stride <= 0 || padding < 0 {
+		panic(fmt.Sprintf("conv2d: invalid stride %d or padding %d", stride, padding))
+	}
+	hOut := (input.Shape[2]+2*padding-kernel.Shape[2])/stride + 1
+	wOut := (input.Shape[3]+2*padding-kernel.Shape[3])/stride + 1
+	if hOut <= 0 || wOut <= 0 {
+		panic(fmt.Sprintf("conv2d: invalid output dimensions: out_h=%d, out_w=%d (check stride/padding)", hOut, wOut))
+	}
+	res, err := NewTensor([]int{input.Shape[0], kernel.Shape[0], hOut, wOut})
+	if err != nil {
+		panic(fmt.Sprintf("conv2d: failed to create output tensor: %v", err))
+	}
+	is, _ := cShape(input.Shape)
+	ks, _ := cShape(kernel.Shape)
+	// check() panics with the library's "conv2d: input channels ... != kernel channels ..."
+	if err := check(C.born_rocm_conv2d((*C.float)(input.Buf.ptr), is, (*C.float)(kernel.Buf.ptr), ks, C.int32_t(stride),
+		C.int32_t(padding), (*C.float)(res.Buf.ptr), nil, nil)); err != nil {
+		panic(fmt.Sprintf("conv2d: %v", err))
+	}
+	return res
+}
+
+// MaxPool2D performs 2D max pooling over [N, C, H, W] with square windows and no padding.
+func (b *Backend) MaxPool2D(input *Tensor, kernelSize, stride int) *Tensor {
+	if len(input.Shape) != 4 {
+		panic(fmt.Sprintf("maxpool2d: expected 4D input [N,C,H,W], got %dD", len(input.Shape)))
+	}
+	h, w := input.Shape[2], input.Shape[3]
+	if kernelSize <= 0 {
+		panic(fmt.Sprintf("maxpool2d: invalid kernel size %d", kernelSize))
+	}
+	if stride <= 0 {
+		panic(fmt.Sprintf("maxpool2d: invalid stride %d", stride))
+	}
+	if kernelSize > h || kernelSize > w {
+		panic(fmt.Sprintf("maxpool2d: kernel size %d too large for input %dx%d", kernelSize, h, w))
+	}
+	res, err := NewTensor([]int{input.Shape[0], input.Shape[1], (h-kernelSize)/stride + 1, (w-kernelSize)/stride + 1})
+	if err != nil {
+		panic(fmt.Sprintf("maxpool2d: failed to create output: %v", err))
+	}
+	is, _ := cShape(input.Shape)
+	if err := check(C.born_rocm_maxpool2d((*C.float)(input.Buf.ptr), is, C.int32_t(kernelSize), C.int32_t(stride),
+		(*C.float)(res.Buf.ptr), nil, nil)); err != nil {
+		panic(fmt.Sprintf("maxpool2d: %v", err))
 	}
 	return res
 }

@@ -53,6 +53,8 @@ SYMBOLS = {
     "born_rocm_mul": (C.c_int, [_vp, _vp, C.c_int32, _vp, _vp, C.c_int32, _vp, _vp]),
     "born_rocm_div": (C.c_int, [_vp, _vp, C.c_int32, _vp, _vp, C.c_int32, _vp, _vp]),
     "born_rocm_transpose": (C.c_int, [_vp, _vp, C.c_int32, _vp, _vp, _vp]),
+    "born_rocm_conv2d": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int32, C.c_int32, _vp, _vp, _vp]),
+    "born_rocm_maxpool2d": (C.c_int, [_vp, _vp, C.c_int32, C.c_int32, _vp, _vp, _vp]),
     "born_rocm_reshape": (C.c_int, [_vp, _vp, C.c_int32, _vp, C.c_int32, _vp, _vp]),
 }
 

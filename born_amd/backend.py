@@ -8,7 +8,6 @@ optimisation for uniquely owned host tensors and is not mirrored).  Programmer e
 with the reference's panic text ("add: shapes not compatible for broadcasting: ...", "matmul: shape mismatch
 ...", "transpose: duplicate axis ..."); runtime failures raise `BornRocmError`.
 
-Conv2D and MaxPool2D of that interface are not built.
 """
 import ctypes as C
 
@@ -94,6 +93,38 @@ class ROCmBackend:
             raise BackendPanic(f"matmul: shape mismatch [{m},{k}] @ [{k2},{n}]")
         out = DeviceTensor.empty((m, n))
         _check(_capi.lib().born_rocm_matmul(a.buf.ptr, b.buf.ptr, out.buf.ptr, m, k, n, k, n, n, stream))
+        return out
+
+    def Conv2D(self, input, kernel, stride, padding, stream=None):
+        if len(input.shape) != 4:
+            raise BackendPanic(f"conv2d: input must be 4D [N,C,H,W], got {len(input.shape)}D")
+        if len(kernel.shape) != 4:
+            raise BackendPanic(f"conv2d: kernel must be 4D [C_out,C_in,K_h,K_w], got {len(kernel.shape)}D")
+        N, _, H, W = input.shape
+        CO, _, KH, KW = kernel.shape
+        ho = (H + 2 * padding - KH) // stride + 1 if stride > 0 else 0
+        wo = (W + 2 * padding - KW) // stride + 1 if stride > 0 else 0
+        out = DeviceTensor.empty((N, CO, max(ho, 1), max(wo, 1)))
+        oshape = (C.c_int64 * 4)()
+        try:
+            _check(_capi.lib().born_rocm_conv2d(input.buf.ptr, _shape_arr(input.shape), kernel.buf.ptr, _shape_arr(kernel.shape),
+                                                int(stride), int(padding), out.buf.ptr, oshape, stream))
+        except SamplerPanic as e:
+            raise BackendPanic(str(e)) from None
+        out.shape = tuple(oshape[i] for i in range(4))
+        return out
+
+    def MaxPool2D(self, input, kernelSize, stride, stream=None):
+        if len(input.shape) != 4:
+            raise BackendPanic(f"maxpool2d: expected 4D input [N,C,H,W], got {len(input.shape)}D")
+        out = DeviceTensor.empty(input.shape)                        # never smaller than the result
+        oshape = (C.c_int64 * 4)()
+        try:
+            _check(_capi.lib().born_rocm_maxpool2d(input.buf.ptr, _shape_arr(input.shape), int(kernelSize), int(stride),
+                                                   out.buf.ptr, oshape, stream))
+        except SamplerPanic as e:
+            raise BackendPanic(str(e)) from None
+        out.shape = tuple(oshape[i] for i in range(4))
         return out
 
     def Reshape(self, t, new_shape, stream=None):

@@ -694,4 +694,54 @@ int born_rocm_reshape(const float *in, const int64_t *shape, int32_t ndim, const
     return BORN_ROCM_OK;
 }
 
+int born_rocm_conv2d(const float *input, const int64_t *input_shape, const float *kernel, const int64_t *kernel_shape,
+                     int32_t stride, int32_t padding, float *out, int64_t *out_shape, void *stream) {
+    if (!input || !kernel || !out || !input_shape || !kernel_shape) return fail(BORN_ROCM_ERR_ARGUMENT, "conv2d: null pointer");
+    const int64_t N = input_shape[0], C = input_shape[1], H = input_shape[2], W = input_shape[3];
+    const int64_t CO = kernel_shape[0], CK = kernel_shape[1], KH = kernel_shape[2], KW = kernel_shape[3];
+    const int64_t lim = 1 << 30;
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || CO <= 0 || KH <= 0 || KW <= 0 || N > lim || C > lim || H > lim || W > lim ||
+        CO > lim || KH > lim || KW > lim || C * KH * KW > lim)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "conv2d: invalid shape");
+    if (stride <= 0 || padding < 0) return fail(BORN_ROCM_ERR_ARGUMENT, "conv2d: invalid stride %d or padding %d", stride, padding);
+    if (C != CK)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "conv2d: input channels %lld != kernel channels %lld", (long long)C, (long long)CK);
+    const int64_t HO = (H + 2 * padding - KH) / stride + 1, WO = (W + 2 * padding - KW) / stride + 1;
+    if (H + 2 * padding - KH < 0 || W + 2 * padding - KW < 0 || HO <= 0 || WO <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "conv2d: invalid output dimensions: out_h=%lld, out_w=%lld (check stride/padding)",
+                    (long long)HO, (long long)WO);
+    if (out_shape) {
+        out_shape[0] = N;
+        out_shape[1] = CO;
+        out_shape[2] = HO;
+        out_shape[3] = WO;
+    }
+    HIP_TRY(launch_conv2d(input, kernel, out, (int)N, (int)C, (int)H, (int)W, (int)CO, (int)KH, (int)KW, (int)HO, (int)WO, stride,
+                          padding, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_maxpool2d(const float *input, const int64_t *input_shape, int32_t kernel_size, int32_t stride, float *out,
+                        int64_t *out_shape, void *stream) {
+    if (!input || !out || !input_shape) return fail(BORN_ROCM_ERR_ARGUMENT, "maxpool2d: null pointer");
+    const int64_t N = input_shape[0], C = input_shape[1], H = input_shape[2], W = input_shape[3];
+    const int64_t lim = 1 << 30;
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || N > lim || C > lim || H > lim || W > lim)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "maxpool2d: invalid shape");
+    if (kernel_size <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "maxpool2d: invalid kernel size %d", kernel_size);
+    if (stride <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "maxpool2d: invalid stride %d", stride);
+    if (kernel_size > H || kernel_size > W)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "maxpool2d: kernel size %d too large for input %lldx%lld", kernel_size, (long long)H,
+                    (long long)W);
+    const int64_t HO = (H - kernel_size) / stride + 1, WO = (W - kernel_size) / stride + 1;
+    if (out_shape) {
+        out_shape[0] = N;
+        out_shape[1] = C;
+        out_shape[2] = HO;
+        out_shape[3] = WO;
+    }
+    HIP_TRY(launch_maxpool2d(input, out, N * C, (int)H, (int)W, (int)HO, (int)WO, kernel_size, stride, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
 }  // extern "C"

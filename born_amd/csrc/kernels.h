@@ -102,6 +102,10 @@ struct TensorIndexArgs {
 };
 hipError_t launch_tensor_binary(int op, const TensorIndexArgs &t, const float *a, const float *b, float *out, hipStream_t st);
 hipError_t launch_tensor_transpose(const TensorIndexArgs &t, const float *in, float *out, hipStream_t st);
+hipError_t launch_conv2d(const float *in, const float *ker, float *out, int N, int C, int H, int W, int CO, int KH, int KW,
+                         int HO, int WO, int stride, int padding, hipStream_t st);
+hipError_t launch_maxpool2d(const float *in, float *out, long long planes, int H, int W, int HO, int WO, int ksize, int stride,
+                            hipStream_t st);
 
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st);

@@ -2,7 +2,8 @@
 //   Add / Sub / Mul / Div with NumPy-style broadcasting  (tensor.Backend, internal/tensor/backend.go:14-17;
 //     CPU form internal/backend/cpu/backend.go:32-134; shape rule internal/tensor/shape.go:83-118)
 //   Transpose by an axis permutation                      (internal/backend/cpu/backend.go:164-209)
-// All of them are bound by HBM traffic: every operand element is read once and every result written once.
+//   Conv2D, MaxPool2D                                     (internal/backend/cpu/conv2d.go, maxpool2d.go)
+// The element-wise and shape operations are bound by HBM traffic: every operand element is read once and every result written once.
 // Each result is one IEEE fp32 operation (the division correctly rounded), so results equal the CPU's bit
 // for bit.
 #include "dev_common.h"
@@ -191,6 +192,63 @@ __global__ __launch_bounds__(TOPS_BLOCK) void transpose_general_kernel(TensorInd
     }
 }
 
+// Conv2D (internal/backend/cpu/conv2d.go:35-203): input [N, C, H, W], kernel [CO, C, KH, KW], zero padding;
+// out[n, co, oh, ow] = sum over (c, kh, kw), in that order, of kernel * input, one fp32 accumulator per output,
+// product and sum each rounded (the reference's im2col + row-by-row dot product adds the terms in exactly this
+// order, the padded positions as a multiplication by 0), so results equal the CPU's bit for bit.  One output per
+// thread; neighbouring threads read neighbouring input columns and share the kernel values through the caches.
+__global__ __launch_bounds__(TOPS_BLOCK) void conv2d_kernel(const float *in, const float *ker, float *out, int N, int C,
+                                                            int H, int W, int CO, int KH, int KW, int HO, int WO, int stride,
+                                                            int padding) {
+    const long long total = (long long)N * CO * HO * WO;
+    const long long step = (long long)gridDim.x * TOPS_BLOCK;
+    for (long long i = (long long)blockIdx.x * TOPS_BLOCK + threadIdx.x; i < total; i += step) {
+        const int ow = (int)(i % WO), oh = (int)((i / WO) % HO), co = (int)((i / ((long long)WO * HO)) % CO);
+        const int n = (int)(i / ((long long)WO * HO * CO));
+        const int h0 = oh * stride - padding, w0 = ow * stride - padding;
+        const float *kp = ker + (long long)co * C * KH * KW;
+        float sum = 0.0f;
+        for (int c = 0; c < C; c++) {
+            const float *ip = in + ((long long)n * C + c) * H * W;
+            for (int kh = 0; kh < KH; kh++) {
+                const int h = h0 + kh;
+                for (int kw = 0; kw < KW; kw++) {
+                    const int w = w0 + kw;
+                    const float x = (h >= 0 && h < H && w >= 0 && w < W) ? ip[(long long)h * W + w] : 0.0f;
+                    sum += kp[(c * KH + kh) * KW + kw] * x;
+                }
+            }
+        }
+        out[i] = sum;
+    }
+}
+
+// MaxPool2D (internal/backend/cpu/maxpool2d.go:26-113): windows of kernel x kernel, no padding; the running
+// maximum starts at -1e38 and is replaced by values that compare greater, as in the reference (so a NaN never
+// wins and nothing below -1e38 is returned).
+__global__ __launch_bounds__(TOPS_BLOCK) void maxpool2d_kernel(const float *in, float *out, long long planes, int H, int W,
+                                                               int HO, int WO, int ksize, int stride) {
+    const long long total = planes * HO * WO;
+    const long long step = (long long)gridDim.x * TOPS_BLOCK;
+    for (long long i = (long long)blockIdx.x * TOPS_BLOCK + threadIdx.x; i < total; i += step) {
+        const int ow = (int)(i % WO), oh = (int)((i / WO) % HO);
+        const long long plane = i / ((long long)WO * HO);
+        const float *ip = in + plane * H * W + (long long)(oh * stride) * W + ow * stride;
+        float best = -1e38f;
+        for (int kh = 0; kh < ksize; kh++)
+            for (int kw = 0; kw < ksize; kw++) {
+                const float v = ip[(long long)kh * W + kw];
+                if (v > best) best = v;
+            }
+        out[i] = best;
+    }
+}
+
+hipError_t launch_conv2d(const float *in, const float *ker, float *out, int N, int C, int H, int W, int CO, int KH, int KW,
+                         int HO, int WO, int stride, int padding, hipStream_t st);
+hipError_t launch_maxpool2d(const float *in, float *out, long long planes, int H, int W, int HO, int WO, int ksize, int stride,
+                            hipStream_t st);
+
 static unsigned tensor_grid(long long work_items) {
     const long long want = (work_items + TOPS_BLOCK - 1) / TOPS_BLOCK;
     const long long cap = 256 * 32;                                  // a few waves of workgroups per CU, grid-stride beyond
@@ -258,6 +316,19 @@ hipError_t launch_tensor_transpose(const TensorIndexArgs &t, const float *in, fl
     } else {
         hipLaunchKernelGGL(transpose_general_kernel, dim3(tensor_grid(t.n)), dim3(TOPS_BLOCK), 0, st, t, in, out);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_conv2d(const float *in, const float *ker, float *out, int N, int C, int H, int W, int CO, int KH, int KW,
+                         int HO, int WO, int stride, int padding, hipStream_t st) {
+    hipLaunchKernelGGL(conv2d_kernel, dim3(tensor_grid((long long)N * CO * HO * WO)), dim3(TOPS_BLOCK), 0, st, in, ker, out, N, C, H,
+                       W, CO, KH, KW, HO, WO, stride, padding);
+    return hipGetLastError();
+}
+hipError_t launch_maxpool2d(const float *in, float *out, long long planes, int H, int W, int HO, int WO, int ksize, int stride,
+                            hipStream_t st) {
+    hipLaunchKernelGGL(maxpool2d_kernel, dim3(tensor_grid(planes * HO * WO)), dim3(TOPS_BLOCK), 0, st, in, out, planes, H, W, HO, WO,
+                       ksize, stride);
     return hipGetLastError();
 }
 

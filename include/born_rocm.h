@@ -214,6 +214,17 @@ int born_rocm_transpose(const float *in, const int64_t *shape, int32_t ndim, con
 int born_rocm_reshape(const float *in, const int64_t *shape, int32_t ndim, const int64_t *new_shape, int32_t new_ndim,
                       float *out, void *stream);
 
+/* born_rocm_conv2d: input [N, C, H, W] * kernel [CO, C, KH, KW], zero padding -> out [N, CO, HO, WO] with
+ * HO = (H + 2 padding - KH) / stride + 1 (WO alike) — Conv2D, internal/backend/cpu/conv2d.go:35-203.  Each output
+ * sums its C * KH * KW products in the reference's order with one fp32 accumulator, so results equal the CPU
+ * backend's bit for bit.  born_rocm_maxpool2d: windows of kernel_size x kernel_size, no padding — MaxPool2D,
+ * internal/backend/cpu/maxpool2d.go:26-113 (the running maximum starts at -1e38, as there).  input_shape /
+ * kernel_shape are 4 extents; out_shape (4 extents) may be NULL.  Same validation messages as the reference. */
+int born_rocm_conv2d(const float *input, const int64_t *input_shape, const float *kernel, const int64_t *kernel_shape,
+                     int32_t stride, int32_t padding, float *out, int64_t *out_shape, void *stream);
+int born_rocm_maxpool2d(const float *input, const int64_t *input_shape, int32_t kernel_size, int32_t stride, float *out,
+                        int64_t *out_shape, void *stream);
+
 /* Building blocks exported for parity tests (device-side evaluation of the specified fp32 exponential and of
  * the built-in uniform stream). */
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream);

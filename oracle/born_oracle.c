@@ -17,6 +17,8 @@
  *   born_oracle_binary_f32       internal/backend/cpu/backend.go:32-134, ops_float32.go:61-112,
  *                                broadcast_helpers.go:9-56, internal/tensor/shape.go:83-118
  *   born_oracle_transpose_f32    internal/backend/cpu/backend.go:164-209, ops_float32.go:115-151
+ *   born_oracle_conv2d_f32       internal/backend/cpu/conv2d.go:35-203 (im2col, dot products, rearrangement)
+ *   born_oracle_maxpool2d_f32    internal/backend/cpu/maxpool2d.go:26-113
  *   logits layout                internal/tensor/raw.go:78-105, shape.go:52-63
  * Go's math.Exp / math.Log are stood in for by glibc exp()/log() (both < 1 ulp
  * in fp64; the difference vanishes in the fp32 cast for every vector the
@@ -260,6 +262,67 @@ BORN_EXPORT int born_oracle_transpose_f32(const float *src, const int64_t *shape
         for (int d = 0; d < nd; d++) di += coords[ax[d]] * dstr[d];
         dst[di] = src[i];
     }
+    return 0;
+}
+
+/* Conv2D as the reference computes it: im2col into rows of C*KH*KW values per output position (zero where the
+ * window leaves the image, conv2d.go:167-203), then out[co, j] = sum_k kernel[co, k] * col[j, k] with one fp32
+ * accumulator, k ascending (conv2d.go:118-128), then the rearrangement to [N, CO, HO, WO] (conv2d.go:131-152).
+ * Returns 0, or -1 on shapes the reference panics on. */
+BORN_EXPORT int born_oracle_conv2d_f32(const float *in, int64_t N, int64_t C, int64_t H, int64_t W, const float *ker,
+                                       int64_t CO, int64_t CK, int64_t KH, int64_t KW, int64_t stride, int64_t padding,
+                                       float *out) {
+    if (C != CK || stride <= 0 || padding < 0 || H + 2 * padding - KH < 0 || W + 2 * padding - KW < 0) return -1;
+    int64_t HO = (H + 2 * padding - KH) / stride + 1, WO = (W + 2 * padding - KW) / stride + 1;
+    int64_t colw = C * KH * KW, colh = N * HO * WO;
+    float *col = (float *)malloc(sizeof(float) * (size_t)(colh * colw));
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)(CO * colh));
+    int64_t row = 0;
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t oh = 0; oh < HO; oh++)
+            for (int64_t ow = 0; ow < WO; ow++, row++) {
+                int64_t h0 = oh * stride - padding, w0 = ow * stride - padding, b = row * colw;
+                for (int64_t c = 0; c < C; c++)
+                    for (int64_t kh = 0; kh < KH; kh++)
+                        for (int64_t kw = 0; kw < KW; kw++) {
+                            int64_t h = h0 + kh, w = w0 + kw;
+                            col[b++] = (h >= 0 && h < H && w >= 0 && w < W) ? in[((n * C + c) * H + h) * W + w] : 0.0f;
+                        }
+            }
+    for (int64_t i = 0; i < CO; i++)
+        for (int64_t j = 0; j < colh; j++) {
+            float sum = 0.0f;
+            for (int64_t k = 0; k < colw; k++) sum += ker[i * colw + k] * col[j * colw + k];
+            tmp[i * colh + j] = sum;
+        }
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t c = 0; c < CO; c++)
+            for (int64_t h = 0; h < HO; h++)
+                for (int64_t w = 0; w < WO; w++)
+                    out[((n * CO + c) * HO + h) * WO + w] = tmp[c * colh + n * HO * WO + h * WO + w];
+    free(col);
+    free(tmp);
+    return 0;
+}
+
+/* MaxPool2D, maxpool2d.go:70-113: the running maximum starts at -1e38 and is replaced by values that compare
+ * greater.  Returns 0, or -1 on arguments the reference panics on. */
+BORN_EXPORT int born_oracle_maxpool2d_f32(const float *in, int64_t N, int64_t C, int64_t H, int64_t W, int64_t ksize,
+                                          int64_t stride, float *out) {
+    if (ksize <= 0 || stride <= 0 || ksize > H || ksize > W) return -1;
+    int64_t HO = (H - ksize) / stride + 1, WO = (W - ksize) / stride + 1;
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t c = 0; c < C; c++)
+            for (int64_t oh = 0; oh < HO; oh++)
+                for (int64_t ow = 0; ow < WO; ow++) {
+                    float best = -1e38f;
+                    for (int64_t kh = 0; kh < ksize; kh++)
+                        for (int64_t kw = 0; kw < ksize; kw++) {
+                            float v = in[((n * C + c) * H + oh * stride + kh) * W + ow * stride + kw];
+                            if (v > best) best = v;
+                        }
+                    out[((n * C + c) * HO + oh) * WO + ow] = best;
+                }
     return 0;
 }
 

@@ -56,6 +56,10 @@ def lib():
         L.born_oracle_binary_f32.argtypes = [C.c_int, f32p, i64p, C.c_int, f32p, i64p, C.c_int, f32p, i64p]
         L.born_oracle_transpose_f32.restype = C.c_int
         L.born_oracle_transpose_f32.argtypes = [f32p, i64p, C.c_int, i32p, f32p]
+        L.born_oracle_conv2d_f32.restype = C.c_int
+        L.born_oracle_conv2d_f32.argtypes = [f32p] + [C.c_int64] * 4 + [f32p] + [C.c_int64] * 6 + [f32p]
+        L.born_oracle_maxpool2d_f32.restype = C.c_int
+        L.born_oracle_maxpool2d_f32.argtypes = [f32p] + [C.c_int64] * 6 + [f32p]
         L.born_oracle_softmax_f64.restype = None
         L.born_oracle_softmax_f64.argtypes = [f32p, f64p, C.c_int64, C.c_int64, C.c_int64]
         L.born_oracle_sample.restype = C.c_int64
@@ -204,6 +208,38 @@ def transpose_ref(x, axes=None):
         raise ValueError("transpose: invalid permutation")
     order = list(range(x.ndim - 1, -1, -1)) if axes is None else list(axes)
     return out.reshape(tuple(x.shape[i] for i in order))
+
+
+def conv2d_ref(x, k, stride=1, padding=0):
+    """The reference's Conv2D: x [N,C,H,W], k [CO,C,KH,KW]; raises ValueError where the reference panics."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    if x.ndim != 4 or k.ndim != 4:
+        raise ValueError("conv2d: input and kernel must be 4D")
+    N, Cc, H, W = x.shape
+    CO, CK, KH, KW = k.shape
+    HO, WO = (H + 2 * padding - KH) // stride + 1, (W + 2 * padding - KW) // stride + 1
+    out = np.empty((N, CO, max(HO, 1), max(WO, 1)), dtype=np.float32)
+    rc = lib().born_oracle_conv2d_f32(_p(x, C.c_float), N, Cc, H, W, _p(k, C.c_float), CO, CK, KH, KW, stride, padding, _p(out, C.c_float))
+    if rc != 0:
+        raise ValueError("conv2d: invalid arguments")
+    return out.reshape(N, CO, HO, WO)
+
+
+def maxpool2d_ref(x, kernel_size, stride):
+    """The reference's MaxPool2D over [N,C,H,W]; raises ValueError where the reference panics."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if x.ndim != 4:
+        raise ValueError("maxpool2d: expected 4D input")
+    N, Cc, H, W = x.shape
+    if kernel_size <= 0 or stride <= 0 or kernel_size > H or kernel_size > W:
+        raise ValueError("maxpool2d: invalid arguments")
+    HO, WO = (H - kernel_size) // stride + 1, (W - kernel_size) // stride + 1
+    out = np.empty((N, Cc, HO, WO), dtype=np.float32)
+    rc = lib().born_oracle_maxpool2d_f32(_p(x, C.c_float), N, Cc, H, W, kernel_size, stride, _p(out, C.c_float))
+    if rc != 0:
+        raise ValueError("maxpool2d: invalid arguments")
+    return out
 
 
 def row_stats(x, T=1.0):

@@ -161,3 +161,65 @@ def test_linear_forward_as_the_reference_composes_it(oracle, be, rocm):
     assert np.all(np.abs(got - exact) <= (4 * np.sqrt(K) + 2) * 2.0 ** -24 * mag)
     ref = oracle.linear_ref(x, w, bias)
     assert np.all(np.abs(got.astype(np.float64) - ref) <= (4 * np.sqrt(K) + K + 4) * 2.0 ** -24 * mag)
+
+
+def test_conv2d_and_maxpool2d_reference_kats(be, rocm):
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_kats.json")) as f:
+        kats = json.load(f)
+    for case in kats["conv2d"]:
+        x = np.array(case["x"], dtype=np.float32).reshape(case["x_shape"])
+        k = np.array(case["k"], dtype=np.float32).reshape(case["k_shape"])
+        out = rocm.Conv2D(be.DeviceTensor.from_numpy(x), be.DeviceTensor.from_numpy(k), case["stride"], case["padding"])
+        assert list(out.Shape()) == case["shape"] and out.numpy().ravel().tolist() == case["expected"], case["source"]
+    for case in kats["maxpool2d"]:
+        x = np.array(case["x"], dtype=np.float32).reshape(case["x_shape"])
+        out = rocm.MaxPool2D(be.DeviceTensor.from_numpy(x), case["kernel"], case["stride"])
+        assert list(out.Shape()) == case["shape"], case["source"]
+        if "expected" in case:
+            assert out.numpy().ravel().tolist() == case["expected"], case["source"]
+        else:
+            assert out.numpy().ravel()[0] == case["expected_first"], case["source"]
+
+
+@pytest.mark.parametrize("cfg", [(2, 3, 7, 9, 4, 3, 2, 1, 0), (1, 2, 8, 8, 3, 3, 3, 2, 1), (3, 1, 5, 6, 2, 2, 4, 1, 2),
+                                 (1, 4, 6, 5, 5, 1, 1, 1, 0), (2, 2, 9, 7, 1, 5, 3, 3, 2), (32, 1, 28, 28, 8, 5, 5, 1, 0),
+                                 (16, 8, 12, 12, 16, 3, 3, 1, 1)])
+def test_conv2d_bit_exact(oracle, be, rocm, cfg):
+    N, C, H, W, CO, KH, KW, stride, pad = cfg
+    rng = np.random.default_rng(sum(cfg))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    k = rng.standard_normal((CO, C, KH, KW)).astype(np.float32)
+    want = oracle.conv2d_ref(x, k, stride, pad)
+    got = rocm.Conv2D(be.DeviceTensor.from_numpy(x), be.DeviceTensor.from_numpy(k), stride, pad)
+    assert got.Shape() == want.shape
+    assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32)), cfg
+
+
+@pytest.mark.parametrize("cfg", [(2, 3, 8, 8, 2, 2), (1, 2, 7, 9, 3, 1), (2, 1, 6, 5, 2, 3), (1, 1, 4, 4, 4, 1), (32, 8, 24, 24, 2, 2)])
+def test_maxpool2d_bit_exact(oracle, be, rocm, cfg):
+    N, C, H, W, ks, stride = cfg
+    rng = np.random.default_rng(sum(cfg))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    x.ravel()[::37] = np.nan                                       # never greater
+    x.ravel()[5::41] = -np.inf                                     # below the reference's floor of -1e38
+    want = oracle.maxpool2d_ref(x, ks, stride)
+    got = rocm.MaxPool2D(be.DeviceTensor.from_numpy(x), ks, stride)
+    assert got.Shape() == want.shape
+    assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32)), cfg
+
+
+def test_conv2d_and_maxpool2d_panics(be, rocm):
+    x = be.DeviceTensor.from_numpy(np.zeros((1, 2, 4, 4), np.float32))
+    k3 = be.DeviceTensor.from_numpy(np.zeros((1, 3, 2, 2), np.float32))
+    with pytest.raises(be.BackendPanic, match=r"conv2d: input channels 2 != kernel channels 3"):
+        rocm.Conv2D(x, k3, 1, 0)
+    with pytest.raises(be.BackendPanic, match=r"conv2d: input must be 4D \[N,C,H,W\], got 2D"):
+        rocm.Conv2D(be.DeviceTensor.from_numpy(np.zeros((2, 2), np.float32)), k3, 1, 0)
+    with pytest.raises(be.BackendPanic, match=r"conv2d: invalid output dimensions"):
+        rocm.Conv2D(x, be.DeviceTensor.from_numpy(np.zeros((1, 2, 5, 5), np.float32)), 1, 0)
+    with pytest.raises(be.BackendPanic, match=r"maxpool2d: kernel size 5 too large for input 4x4"):
+        rocm.MaxPool2D(x, 5, 1)
+    with pytest.raises(be.BackendPanic, match=r"maxpool2d: invalid stride 0"):
+        rocm.MaxPool2D(x, 2, 0)
+    with pytest.raises(be.BackendPanic, match=r"maxpool2d: invalid kernel size 0"):
+        rocm.MaxPool2D(x, 0, 1)

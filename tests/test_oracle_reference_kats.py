@@ -186,3 +186,53 @@ def test_binary_and_transpose_against_numpy(oracle):
         assert np.array_equal(oracle.transpose_ref(x, axes), np.transpose(x, axes)), (shape, axes)
     with pytest.raises(ValueError):
         oracle.transpose_ref(np.zeros((2, 3), np.float32), (0, 0))
+
+
+def test_conv2d_and_maxpool2d_kats(oracle):
+    for case in KATS["conv2d"]:
+        x = np.array(case["x"], dtype=np.float32).reshape(case["x_shape"])
+        k = np.array(case["k"], dtype=np.float32).reshape(case["k_shape"])
+        out = oracle.conv2d_ref(x, k, case["stride"], case["padding"])
+        assert list(out.shape) == case["shape"] and out.ravel().tolist() == case["expected"], case["source"]
+    for case in KATS["maxpool2d"]:
+        x = np.array(case["x"], dtype=np.float32).reshape(case["x_shape"])
+        out = oracle.maxpool2d_ref(x, case["kernel"], case["stride"])
+        assert list(out.shape) == case["shape"], case["source"]
+        if "expected" in case:
+            assert out.ravel().tolist() == case["expected"], case["source"]
+        else:
+            assert out.ravel()[0] == case["expected_first"], case["source"]
+
+
+def test_conv2d_and_maxpool2d_against_independent_restatements(oracle):
+    # conv2d as an explicit cross-correlation sum in fp64 over padded input (numpy), maxpool as a windowed max:
+    # a swapped kernel axis, a flipped kernel, a wrong stride or padding offset fails on asymmetric cases
+    rng = np.random.default_rng(17)
+    for (N, C, H, W, CO, KH, KW, stride, pad) in [(2, 3, 7, 9, 4, 3, 2, 1, 0), (1, 2, 8, 8, 3, 3, 3, 2, 1), (3, 1, 5, 6, 2, 2, 4, 1, 2),
+                                                  (1, 4, 6, 5, 5, 1, 1, 1, 0), (2, 2, 9, 7, 1, 5, 3, 3, 2)]:
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        k = rng.standard_normal((CO, C, KH, KW)).astype(np.float32)
+        got = oracle.conv2d_ref(x, k, stride, pad)
+        xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+        HO, WO = (H + 2 * pad - KH) // stride + 1, (W + 2 * pad - KW) // stride + 1
+        want = np.zeros((N, CO, HO, WO))
+        for oh in range(HO):
+            for ow in range(WO):
+                patch = xp[:, :, oh * stride:oh * stride + KH, ow * stride:ow * stride + KW]
+                want[:, :, oh, ow] = np.einsum("nchw,ochw->no", patch, k.astype(np.float64))
+        assert got.shape == want.shape
+        assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.max(np.abs(want))), (N, C, H, W, CO, KH, KW, stride, pad)
+    for (N, C, H, W, ks, stride) in [(2, 3, 8, 8, 2, 2), (1, 2, 7, 9, 3, 1), (2, 1, 6, 5, 2, 3), (1, 1, 4, 4, 4, 1)]:
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        got = oracle.maxpool2d_ref(x, ks, stride)
+        HO, WO = (H - ks) // stride + 1, (W - ks) // stride + 1
+        want = np.empty((N, C, HO, WO), np.float32)
+        for oh in range(HO):
+            for ow in range(WO):
+                want[:, :, oh, ow] = x[:, :, oh * stride:oh * stride + ks, ow * stride:ow * stride + ks].max(axis=(2, 3))
+        assert np.array_equal(got, want)
+    # the reference's floor of -1e38 and its treatment of NaN (never greater)
+    x = np.full((1, 1, 2, 2), -np.inf, np.float32)
+    assert oracle.maxpool2d_ref(x, 2, 1).ravel()[0] == np.float32(-1e38)
+    x = np.array([[[[np.nan, 1.0], [2.0, np.nan]]]], np.float32)
+    assert oracle.maxpool2d_ref(x, 2, 1).ravel()[0] == 2.0
