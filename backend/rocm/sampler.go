@@ -29,13 +29,14 @@ import (
 )
 
 // SamplerConfig mirrors born_sampler_config.  Zero value of a field = default
-// (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off, TopK 0 = off).
+// (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off, TopK 0 = off, MinP 0 = off).
 type SamplerConfig struct {
 	Temperature       float32
 	TopK              int
 	TopP              float32
 	RepetitionPenalty float32
 	Seed              int64
+	MinP              float32
 }
 
 // DeviceBuffer is device memory owned by the shim (Born's RawTensor is host-only,
@@ -100,6 +101,7 @@ func NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler {
 		top_p:              C.float(cfg.TopP),
 		repetition_penalty: C.float(cfg.RepetitionPenalty),
 		seed:               C.int64_t(cfg.Seed),
+		min_p:              C.float(cfg.MinP),
 	}
 	var h *C.born_sampler
 	if err := check(C.born_rocm_sampler_create(&c, C.int64_t(maxBatch), C.int64_t(maxVocab), &h)); err != nil {

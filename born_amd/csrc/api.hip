@@ -70,7 +70,17 @@ static int fill_defaults(born_sampler_config *c) {
     if (!(c->repetition_penalty > 0.0f) || !std::isfinite(c->repetition_penalty))
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: repetition_penalty must be > 0 and finite, got %g",
                     (double)c->repetition_penalty);
+    if (!(c->min_p >= 0.0f) || !(c->min_p < 1.0f))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: min_p must be in [0, 1), got %g", (double)c->min_p);
     return BORN_ROCM_OK;
+}
+
+// Distance below the row maximum beyond which a logit carries no mass: 80 (where the fixed-point masses have long
+// been zero), or the min-p bound -ln(min_p) when that is smaller.  fp64 log rounded once to fp32.
+static float mass_cutoff(const born_sampler_config &c) {
+    if (!(c.min_p > 0.0f)) return 80.0f;
+    const float d = (float)(-std::log((double)c.min_p));
+    return d < 80.0f ? d : 80.0f;
 }
 
 extern "C" {
@@ -321,6 +331,7 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     a.status = s->status;
     a.counters = s->counters;
     a.mass_shift = mass_shift(vocab);
+    a.dcut = mass_cutoff(s->cfg);
 
     hipStream_t st = (hipStream_t)stream;
     if (row_T || row_k || row_p || row_rep) {

@@ -68,8 +68,10 @@ __device__ __forceinline__ float next_below(float x) {
 
 // ---- the specified exponential and the integer mass ------------------------
 
-__device__ __forceinline__ float expneg(float d) {       // exp(-d), d >= 0; see the spec, section 6
-    if (!(d <= 80.0f)) return 0.0f;
+// exp(-d), d >= 0; see the spec, section 6.  dcut <= 80: the distance beyond which the mass is zero (80, or the
+// min-p bound -ln(min_p) when that is smaller).
+__device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
+    if (!(d <= dcut)) return 0.0f;
     float x = -d;
     float k = rintf(x * 1.44269504f);
     float r = fmaf(k, -0.693145752f, x);
@@ -84,9 +86,9 @@ __device__ __forceinline__ float expneg(float d) {       // exp(-d), d >= 0; see
     y = y + 1.0f;
     return __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
 }
-__device__ __forceinline__ float emass(float z, float m) {
+__device__ __forceinline__ float emass(float z, float m, float dcut = 80.0f) {
     float d = (z == m) ? 0.0f : m - z;
-    return expneg(d);
+    return expneg(d, dcut);
 }
 // trunc(e * 2^S): e has 24 significant bits, so e * 2^S (S <= 61) is exact in fp32
 __device__ __forceinline__ u64 qfix(float e, float scale) { return (u64)(e * scale); }

@@ -18,12 +18,16 @@ __device__ void finish_sorted(const u64 *list, int ns, const SampleArgs &a, int 
     float e[ITEMS];
     u64 cum[ITEMS];
     u64 local = 0;
+    u32 nlive = 0;
 #pragma unroll
     for (int it = 0; it < ITEMS; it++) {
         int i = tid * ITEMS + it;
         e[it] = 0.0f;
         if (i < ns) {
-            e[it] = emass(key64_z(list[i]), m);
+            const float z = key64_z(list[i]);
+            const float d = (z == m) ? 0.0f : m - z;
+            nlive += d <= a.dcut ? 1u : 0u;
+            e[it] = expneg(d, a.dcut);
             local += qfix(e[it], scale);
         }
         cum[it] = local;
@@ -35,12 +39,13 @@ __device__ void finish_sorted(const u64 *list, int ns, const SampleArgs &a, int 
     for (int it = 0; it < ITEMS; it++) cum[it] += excl;
 
     int np = ns;
+    if (a.dcut < 80.0f) np = (int)block_sum_u32<BLOCK>(nlive, scr);  // min-p: its survivors are a prefix of the rank order
     u64 Zp = Zk;
     if (a.top_p < 1.0f) {
         const u64 tp = top_p_target(a.top_p, Zk);
         u32 c = 0;
 #pragma unroll
-        for (int it = 0; it < ITEMS; it++) c += (tid * ITEMS + it < ns && cum[it] < tp) ? 1u : 0u;
+        for (int it = 0; it < ITEMS; it++) c += (tid * ITEMS + it < np && cum[it] < tp) ? 1u : 0u;
         np = (int)block_sum_u32<BLOCK>(c, scr) + 1;
         __syncthreads();
 #pragma unroll

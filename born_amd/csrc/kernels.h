@@ -48,6 +48,7 @@ struct SampleArgs {
     int *status;                  // device status word
     unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows that needed an exact (slower) refinement, [2] rows sampled without a top-k cut or by the general kernel
     int mass_shift;
+    float dcut;                   // masses are zero beyond this distance below the row maximum: min(80, -ln(min_p))
 };
 
 // Per-row configurations (device arrays of B values, each optional): a second argument of the per-row kernel

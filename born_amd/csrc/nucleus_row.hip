@@ -34,7 +34,7 @@ struct NucRow {                               // uniform per workgroup
     const float *x;
     int V;
     bool vec, penal, degenerate;
-    float T, rep, m, scale, range, sbin;
+    float T, rep, m, scale, range, sbin, dcut;
 };
 
 __device__ __forceinline__ float nuc_z(const NucRow &r, float y) {
@@ -152,6 +152,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     r.T = cfg_T;
     r.rep = cfg_rep;
     r.scale = mass_scale(a.mass_shift);
+    r.dcut = a.dcut;
     const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
     BORN_STAMP(a, row, 0);
@@ -189,7 +190,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         r.degenerate = r.m == -INFINITY;                             // nothing finite: every d is 0 by definition
         const float zmin = mn < INFINITY ? nuc_z(r, mn) : r.m;
         const float span = r.degenerate ? 0.0f : r.m - zmin;         // >= 0
-        r.range = uniform_f32(fminf(32.0f, span * 1.0001f + 1e-3f));
+        // the bins cover the logits that can carry mass: the row's span, at most 32, at most the min-p bound
+        r.range = uniform_f32(fminf(fminf(32.0f, span * 1.0001f + 1e-3f), r.dcut * 1.0001f + 1e-3f));
         r.sbin = uniform_f32((float)NUC_BINS / r.range);
     }
 
@@ -197,7 +199,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     // ---- sweep 2: integer masses by bin
     nuc_foreach(r, bm, [&](int, float y) {
         const float d = nuc_d(r, nuc_z(r, y));
-        atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d), r.scale));
+        atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
     });
     __syncthreads();
     BORN_STAMP(a, row, 3);
@@ -266,7 +268,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 if (slot >= 0) {
                     take = true;
                     key = make_key64(z, (int)c.y);
-                    qs = qfix(expneg(d), r.scale) | ((u64)slot << 62);
+                    qs = qfix(expneg(d, r.dcut), r.scale) | ((u64)slot << 62);
                 }
             }
             const u64 mk = __ballot(take);
@@ -336,7 +338,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                         const u64 key = make_key64(z, j);
                         if (pl > 0 && (key >> (64 - pl)) != pf) return;
                         const int idx = nsb - 1 - (int)((key >> (64 - pl - db)) & (u64)(nsb - 1));   // larger keys first
-                        atomicAdd(&smass[idx], qfix(expneg(d), r.scale));
+                        atomicAdd(&smass[idx], qfix(expneg(d, r.dcut), r.scale));
                         atomicAdd(&scnt[idx], 1u);
                     });
                 }
@@ -378,7 +380,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                     const int pos = atomicAdd(&s_n, 1);
                     if (pos < NUC_CAP) {
                         fkey[pos] = key;
-                        fq[pos] = qfix(expneg(d), r.scale);          // slot 0
+                        fq[pos] = qfix(expneg(d, r.dcut), r.scale);          // slot 0
                     }
                 });
             }
@@ -417,7 +419,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             if (a.probs) a.probs[row] = 0.0f;
         } else {
             a.tokens[row] = key64_id(tokkey);
-            if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m), Zp, a.mass_shift);
+            if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m, r.dcut), Zp, a.mass_shift);
         }
         if (a.nuc_len) a.nuc_len[row] = -1;                          // the nucleus listing is only produced for small top-k
         atomicAdd(&a.counters[listed ? 2 : 1], 1ull);

@@ -16,7 +16,7 @@ struct WideCtx {
     const BORN_GLOBAL float *x;
     int V;
     bool vec, has_hist, count_mode;
-    float T, rep, m, scale;
+    float T, rep, m, scale, dcut;
     const lds_u32 *bm;
     lds_u64 *mass;  // [WIDE_BINS] inclusive cumulative masses after the scan
     lds_u32 *cnt;   // [WIDE_BINS] inclusive cumulative counts (count_mode only)
@@ -162,7 +162,7 @@ __device__ __forceinline__ Found wide_resolve(const WideCtx &c, int n, int b, bo
             float d = (z == c.m) ? 0.0f : c.m - z;
             if (b < 0 || wide_bin(d) == b) {
                 in[t] = 1;
-                q[t] = qfix(expneg(d), c.scale);
+                q[t] = qfix(expneg(d, c.dcut), c.scale);
             }
         }
         lm += q[t];
@@ -212,10 +212,10 @@ __device__ __forceinline__ int wide_collect(const WideCtx &c, P pred) {
     wide_foreach(c, [&](int j, float y) {
         const float z = wide_z(c, y);
         float d = (z == c.m) ? 0.0f : c.m - z;
-        if (!c.count_mode && !(d <= 80.0f)) return;            // zero mass: invisible to mass-only selection
+        if (!c.count_mode && !(d <= c.dcut)) return;            // zero mass: invisible to mass-only selection
         u64 key = make_key64(z, j);
         if (pred(wide_bin(d), key)) {
-            if (!c.count_mode && qfix(expneg(d), c.scale) == 0) return;
+            if (!c.count_mode && qfix(expneg(d, c.dcut), c.scale) == 0) return;
             int pos = lds_add(c.s_int + 1, 1);
             if (pos < WIDE_LIST_CAP) c.list[pos] = key;
         }
@@ -253,7 +253,7 @@ __device__ __noinline__ Found wide_descend(const WideCtx &c, int b, bool by_coun
             if (wide_bin(d) != b) return;
             u64 key = make_key64(z, j);
             if (plen > 0 && (key >> (64 - plen)) != prefix) return;
-            u64 q = qfix(expneg(d), c.scale);
+            u64 q = qfix(expneg(d, c.dcut), c.scale);
             if (!c.count_mode && q == 0) return;
             int digit = (int)((key >> (64 - plen - db)) & (u64)(nsb - 1));
             int idx = nsb - 1 - digit;                             // larger keys first
@@ -333,6 +333,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     c.T = uniform_f32(a.T);
     c.rep = uniform_f32(a.rep);
     c.scale = uniform_f32(mass_scale(a.mass_shift));
+    c.dcut = a.dcut;
     c.mass = dyn;
     c.list = dyn + WIDE_BINS;
     c.cnt = (lds_u32 *)(dyn + WIDE_BINS + WIDE_LIST_CAP);
@@ -387,7 +388,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
         float d = (z == c.m) ? 0.0f : c.m - z;
         int b = wide_bin(d);
         if (c.count_mode) lds_add(c.cnt + b, 1u);
-        u64 q = qfix(expneg(d), c.scale);
+        u64 q = qfix(expneg(d, c.dcut), c.scale);
         if (q) lds_add(c.mass + b, q);
     });
     __syncthreads();
@@ -459,7 +460,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
         finish_sorted<WIDE_BLOCK, WIDE_ITEMS>((const u64 *)c.list, k, a, row, (BlockScratch *)scr);
     } else if (tid == 0) {
         a.tokens[row] = key64_id(f.key);
-        if (a.probs) a.probs[row] = prob_of(emass(key64_z(f.key), c.m), Zp, a.mass_shift);
+        if (a.probs) a.probs[row] = prob_of(emass(key64_z(f.key), c.m, c.dcut), Zp, a.mass_shift);
         if (a.nuc_len) a.nuc_len[row] = -1;              // the nucleus listing is only produced for small top-k
     }
     BORN_STAMP(a, row, 7);

@@ -27,17 +27,22 @@ __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, cons
     const float m = key64_z(list[0]);
     float e = 0.0f;
     u64 q = 0;
+    bool live = l < ns;
     if (l < ns) {
-        e = emass(key64_z(list[l]), m);
+        const float z = key64_z(list[l]);
+        const float d = (z == m) ? 0.0f : m - z;
+        live = d <= a.dcut;
+        e = expneg(d, a.dcut);
         q = qfix(e, mass_scale(a.mass_shift));
     }
     const u64 cum = wave_inclusive_scan_u62(q);
     const u64 Zk = readlane_u64(cum, WAVE - 1);
     int np = ns;
+    if (a.dcut < 80.0f) np = __popcll(__ballot(live));               // min-p: its survivors are a prefix of the rank order
     u64 Zp = Zk;
     if (a.top_p < 1.0f) {
         const u64 tp = top_p_target(a.top_p, Zk);
-        np = __popcll(__ballot(l < ns && cum < tp)) + 1;
+        np = __popcll(__ballot(l < np && cum < tp)) + 1;
         Zp = readlane_u64(cum, __builtin_amdgcn_readfirstlane(np - 1));
     }
     const u64 td = draw_target(u, Zp);

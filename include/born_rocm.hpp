@@ -26,6 +26,7 @@ struct SamplerConfig {
     float TopP = 0.0f;
     float RepetitionPenalty = 0.0f;
     int64_t Seed = 0;
+    float MinP = 0.0f;
 };
 
 class DeviceBuffer {
@@ -49,7 +50,7 @@ private:
 class Sampler {
 public:
     Sampler(const SamplerConfig &cfg, int64_t max_batch, int64_t max_vocab) {
-        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed};
+        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed, cfg.MinP};
         check(born_rocm_sampler_create(&c, max_batch, max_vocab, &h_));
     }
     Sampler(const Sampler &) = delete;

@@ -391,7 +391,7 @@ static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hle
 }
 
 /*
- * born_oracle_sample
+ * born_oracle_sample_min_p (born_oracle_sample: the same with min_p = 0)
  *   logits [B, row_stride>=V]; history [B, hist_stride] (may be NULL), hist_len
  *   [B] (NULL => hist_stride entries per row); uniforms [B].
  * outputs (any may be NULL): tokens[B], probs[B], near[B] (layer T flags: bit 0 =
@@ -402,15 +402,21 @@ static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hle
  *   nuc_ids[B, nuc_cap], nuc_probs[B, nuc_cap].
  * returns the number of out-of-range history ids met, or -1 on bad arguments.
  */
-BORN_EXPORT int64_t born_oracle_sample(
+BORN_EXPORT int64_t born_oracle_sample_min_p(
     const float *logits, int64_t B, int64_t V, int64_t row_stride,
     const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
-    const float *uniforms, float T, int32_t top_k, float top_p, float rep, int32_t mode,
+    const float *uniforms, float T, int32_t top_k, float top_p, float min_p, float rep, int32_t mode,
     int32_t *tokens, float *probs, uint8_t *near, int32_t *n_nucleus,
     int64_t nuc_cap, int32_t *nuc_ids, float *nuc_probs)
 {
     if (!logits || !uniforms || B <= 0 || V <= 0 || row_stride < V) return -1;
-    if (!(T > 0.0f) || !(top_p > 0.0f) || !(rep > 0.0f)) return -1;
+    if (!(T > 0.0f) || !(top_p > 0.0f) || !(rep > 0.0f) || !(min_p >= 0.0f) || !(min_p < 1.0f)) return -1;
+    /* min-p (spec section 2.5): a survivor stays iff m - z <= -ln(min_p).  Layer T tests the fp64 difference
+     * against the fp64 bound; layer F the fp32 difference against the bound rounded to fp32 and capped at 80
+     * (beyond which the fixed-point masses are zero anyway). */
+    const double dmin_t = min_p > 0.0f ? -log((double)min_p) : INFINITY;
+    const float dmin_f = (float)dmin_t < 80.0f ? (float)dmin_t : 80.0f;
+    const int use_min_p = min_p > 0.0f && (float)dmin_t < 80.0f;
     int64_t k = (top_k <= 0 || top_k >= V) ? V : top_k;
     int use_p = top_p < 1.0f;
     int S = born_oracle_mass_shift(V);
@@ -445,8 +451,25 @@ BORN_EXPORT int64_t born_oracle_sample(
         }
         float m = ordkey_inv((uint32_t)(keys[0] >> 32));
         float u = uniforms[b];
-        int64_t np = n, pick = n - 1;
         int is_near = 0;
+        int min_p_near = 0;      /* a survivor sits within 1e-6 of the min-p bound (layer T) */
+        if (use_min_p) {
+            /* m - z never decreases along the rank order, so the survivors are a prefix */
+            int64_t nm = 0;
+            for (int64_t i = 0; i < n; i++) {
+                float zi = ordkey_inv((uint32_t)(keys[i] >> 32));
+                if (mode == 0) {
+                    double d = (zi == m) ? 0.0 : (double)m - (double)zi;
+                    if (fabs(d - dmin_t) < 1e-6 * (dmin_t > 1.0 ? dmin_t : 1.0)) min_p_near = 1;
+                    if (d <= dmin_t) nm = i + 1;
+                } else {
+                    float d = (zi == m) ? 0.0f : m - zi;
+                    if (d <= dmin_f) nm = i + 1;
+                }
+            }
+            n = nm;
+        }
+        int64_t np = n, pick = n - 1;
         double Zp_d = 0.0;   /* nucleus normaliser as a double, for probabilities */
 
         if (mode == 0) {
@@ -486,6 +509,9 @@ BORN_EXPORT int64_t born_oracle_sample(
             }
             if (!found) pick = np - 1;
             if (cut_near) is_near |= 2;
+            /* a survivor on the min-p bound may fall either side of it: the set, its normaliser and with them
+             * the top-p cut and the draw may all differ in another correct implementation */
+            if (min_p_near) is_near |= 3;
             Zp_d = Zp;
         } else if (mode == 1) {
             uint64_t Zk = 0;
@@ -551,6 +577,18 @@ BORN_EXPORT int64_t born_oracle_sample(
     }
     free(z); free(seen); free(keys); free(e); free(q);
     return bad;
+}
+
+/* born_oracle_sample_min_p with min-p off */
+BORN_EXPORT int64_t born_oracle_sample(
+    const float *logits, int64_t B, int64_t V, int64_t row_stride,
+    const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
+    const float *uniforms, float T, int32_t top_k, float top_p, float rep, int32_t mode,
+    int32_t *tokens, float *probs, uint8_t *near, int32_t *n_nucleus,
+    int64_t nuc_cap, int32_t *nuc_ids, float *nuc_probs)
+{
+    return born_oracle_sample_min_p(logits, B, V, row_stride, history, hist_len, hist_stride, uniforms, T, top_k, top_p,
+                                    0.0f, rep, mode, tokens, probs, near, n_nucleus, nuc_cap, nuc_ids, nuc_probs);
 }
 
 /* ------------------------------------------------------------------ */

@@ -19,9 +19,9 @@ def rocm():
     return S
 
 
-def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0, max_vocab=None):
+def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0, max_vocab=None, min_p=0.0):
     B, V = x.shape
-    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=k, TopP=p, RepetitionPenalty=rep), max_batch=B,
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=k, TopP=p, RepetitionPenalty=rep, MinP=min_p), max_batch=B,
                         max_vocab=max_vocab or V)
     s.SetPath(path)
     out = rocm.sample_host(s, x, u, hist, hist_len, nucleus_cap=nuc)
@@ -32,10 +32,10 @@ def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0
 
 
 def _check_against_oracle(oracle, rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0,
-                          max_near_frac=1.0):
-    got = _run(rocm, x, u, T, k, p, rep, hist, hist_len, nuc, path)
-    fx = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED, nuc_cap=nuc)
-    tr = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_TRUTH, nuc_cap=nuc)
+                          max_near_frac=1.0, min_p=0.0):
+    got = _run(rocm, x, u, T, k, p, rep, hist, hist_len, nuc, path, min_p=min_p)
+    fx = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED, nuc_cap=nuc, min_p=min_p)
+    tr = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_TRUTH, nuc_cap=nuc, min_p=min_p)
     bad = np.nonzero(got["tokens"] != fx["tokens"])[0]
     assert bad.size == 0, f"token mismatch vs fixed-point oracle at rows {bad[:8]}: {got['tokens'][bad[:8]]} vs {fx['tokens'][bad[:8]]}"
     assert np.array_equal(got["probs"].view(np.uint32), fx["probs"].view(np.uint32)), "probabilities differ from the fixed-point oracle"
@@ -295,6 +295,63 @@ def test_general_kernel_degenerate_rows(oracle, rocm, path):
     far = rng.standard_normal((B, V), dtype=np.float32) - 200.0         # everything but one far below the maximum
     far[:, 11] = 0.0
     _check_against_oracle(oracle, rocm, far, u, 1.0, 0, 1.0, path=path)
+
+
+# ---------------------------------------------------------------- min-p
+
+@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("B,V,T,k,p,rep,H,min_p", [
+    (32, 128256, 0.7, 50, 0.9, 1.15, 512, 0.05),    # C3 shape with min-p: single-pass top-k kernel
+    (16, 32000, 1.0, 40, 1.0, 1.0, 0, 0.1),         # min-p is the only cut inside the top-k
+    (16, 32000, 1.0, 64, 1.0, 1.1, 32, 0.5),        # few survivors
+    (16, 32000, 1.0, 0, 1.0, 1.0, 0, 0.02),         # no top-k: nucleus kernel, min-p alone
+    (16, 152064, 1.2, 0, 0.95, 1.05, 2048, 0.01),   # C5 shape with min-p
+    (16, 32000, 0.9, 500, 0.9, 1.1, 64, 0.05),      # general kernel, top-k counted
+    (8, 50000, 1.0, 20000, 1.0, 1.0, 0, 0.001),     # general kernel, top-k by count descent
+    (8, 4097, 2.0, 0, 0.5, 1.0, 0, 0.2),
+    (5, 2, 1.0, 0, 1.0, 1.0, 0, 0.3),
+    (5, 1, 1.0, 0, 1.0, 1.0, 0, 0.9),
+    (8, 1000, 1.0, 10, 0.9, 1.0, 0, 1e-30),         # a bound beyond every mass: as if off
+])
+def test_min_p_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, min_p, path):
+    rng = np.random.default_rng(B * 7919 + V + int(min_p * 1000))
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.0)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
+    nuc = min(64, k) if 1 <= k <= 64 else 0
+    _, fx, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=nuc, path=path, min_p=min_p)
+    if nuc and min_p >= 0.05:
+        assert (fx["n_nucleus"] < k).any(), "the case is meant to have min-p bind"
+
+
+def test_min_p_survivor_set_and_special_rows(oracle, rocm):
+    # probabilities 1/2, 1/4, 1/8, 1/16, 1/16: the ratio to the top is 1, 1/2, 1/4, 1/8, 1/8
+    # (and a sixth entry far below, so that top_k = 5 is a real cut and the nucleus gets listed)
+    x = np.log(np.array([[0.5, 0.25, 0.125, 0.0625, 0.0625, 1e-12]] * 4, dtype=np.float64)).astype(np.float32)
+    u = np.array([0.0, 0.4, 0.8, 0.999], dtype=np.float32)
+    for min_p, n in [(0.1, 5), (0.2, 3), (0.3, 2), (0.6, 1)]:
+        got = _run(rocm, x, u, k=5, nuc=5, min_p=min_p)
+        assert (got["n_nucleus"] == n).all(), (min_p, got["n_nucleus"])
+        assert (got["tokens"] < n).all()
+        want = np.array([0.5, 0.25, 0.125, 0.0625, 0.0625][:n]) / sum([0.5, 0.25, 0.125, 0.0625, 0.0625][:n])
+        assert np.allclose(got["nuc_probs"][:, :n], want, rtol=1e-6)
+        assert (got["nuc_ids"][:, n:] == -1).all()
+    # masked rows: -inf everywhere but two entries; all -inf (every entry ties at the maximum and stays)
+    y = np.full((2, 1000), -np.inf, dtype=np.float32)
+    y[0, 17] = 1.0
+    y[0, 900] = 0.0
+    for path in (0, 1):
+        for k in (0, 8):
+            _check_against_oracle(oracle, rocm, y, np.array([0.9, 0.5], dtype=np.float32), k=k, path=path, min_p=0.5)
+
+
+def test_min_p_is_validated(rocm):
+    for bad in (-0.1, 1.0, 1.5, float("nan")):
+        with pytest.raises(rocm.SamplerPanic, match="min_p"):
+            rocm.NewSampler(rocm.SamplerConfig(MinP=bad), max_batch=1, max_vocab=16)
+    s = rocm.NewSampler(rocm.SamplerConfig(MinP=0.25), max_batch=1, max_vocab=16)
+    assert s.Config().MinP == 0.25
+    s.Close()
 
 
 def test_builtin_uniform_stream_in_sample(oracle, rocm):

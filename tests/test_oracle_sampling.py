@@ -153,7 +153,7 @@ def test_special_values(oracle):
 
 # ---------------------------------------------------------------- independent restatement in torch
 
-def _torch_sample(x, u, T, k, p, rep, hist):
+def _torch_sample(x, u, T, k, p, rep, hist, min_p=0.0):
     """Independent restatement with torch primitives (float64 probabilities)."""
     x = torch.from_numpy(x.copy())
     B, V = x.shape
@@ -167,7 +167,11 @@ def _torch_sample(x, u, T, k, p, rep, hist):
         z = row / np.float32(T)
         order = torch.from_numpy(np.lexsort((np.arange(V), -z.numpy().astype(np.float64))))  # z desc, id asc
         zs = z[order].double()
-        if 0 < k < V:
+        if min_p > 0.0:                              # probability ratio to the most likely token, on the whole row
+            full = torch.softmax(zs, dim=0)
+            keep = full / full.max() >= np.float64(np.float32(min_p))
+            zs, order = zs[keep], order[keep]
+        if 0 < k < len(zs):
             zs, order = zs[:k], order[:k]
         pr = torch.softmax(zs, dim=0)
         c = torch.cumsum(pr, 0)
@@ -199,6 +203,69 @@ def test_against_torch_restatement(oracle, T, k, p, rep):
     same = got["tokens"] == want_t
     assert np.allclose(got["probs"][same], want_p[same], rtol=1e-5)
     assert (~same).sum() <= 1
+
+
+def test_min_p_hand_vector(oracle):
+    # probabilities 1/2, 1/4, 1/8, 1/16, 1/16 => ratios to the top 1, 1/2, 1/4, 1/8, 1/8
+    pr = [0.5, 0.25, 0.125, 0.0625, 0.0625]
+    x = np.log(np.array([pr], dtype=np.float64)).astype(np.float32)
+    for mode in (oracle.MODE_TRUTH, oracle.MODE_FIXED):
+        for min_p, n in [(0.1, 5), (0.2, 3), (0.3, 2), (0.6, 1)]:
+            want = np.array(pr[:n]) / sum(pr[:n])
+            edges = np.cumsum(want)
+            for u in (0.0, 0.3, 0.55, 0.7, 0.9, 0.99):
+                r = oracle.sample(x, np.array([u], dtype=np.float32), min_p=min_p, mode=mode, nuc_cap=5)
+                assert r["n_nucleus"][0] == n
+                assert np.allclose(r["nuc_probs"][0, :n], want, rtol=1e-6) and (r["nuc_ids"][0, n:] == -1).all()
+                assert r["tokens"][0] == int(np.searchsorted(edges, u, side="right"))
+        # min-p, then top-k, then top-p on what is left: 0.2 keeps {1/2, 1/4, 1/8}; top-k 2 => {2/3, 1/3}; p = 0.6 => {1}
+        r = oracle.sample(x, np.array([0.99], dtype=np.float32), min_p=0.2, top_k=2, top_p=0.6, mode=mode, nuc_cap=5)
+        assert r["n_nucleus"][0] == 1 and r["tokens"][0] == 0 and r["probs"][0] == 1.0
+        r = oracle.sample(x, np.array([0.99], dtype=np.float32), min_p=0.2, top_k=2, top_p=0.7, mode=mode, nuc_cap=5)
+        assert r["n_nucleus"][0] == 2 and r["tokens"][0] == 1 and abs(r["probs"][0] - 1 / 3) < 1e-6
+
+
+def test_min_p_limits_and_flags(oracle):
+    rng = np.random.default_rng(21)
+    x = rng.normal(0, 2, size=(64, 500)).astype(np.float32)
+    u = rng.random(64, dtype=np.float32)
+    base = oracle.sample(x, u, temperature=0.8, top_k=20, top_p=0.9, mode=oracle.MODE_FIXED, nuc_cap=20)
+    # a bound below every ratio changes nothing; a bound just under 1 leaves the top token (and its exact ties)
+    tiny = oracle.sample(x, u, temperature=0.8, top_k=20, top_p=0.9, min_p=1e-30, mode=oracle.MODE_FIXED, nuc_cap=20)
+    for key in ("tokens", "probs", "n_nucleus", "nuc_ids", "nuc_probs"):
+        assert np.array_equal(base[key], tiny[key])
+    top = oracle.sample(x, u, temperature=0.8, min_p=0.999999, mode=oracle.MODE_TRUTH)
+    assert np.array_equal(top["tokens"], oracle.argmax_ref(x)) and np.allclose(top["probs"], 1.0)
+    # a survivor exactly on the bound is flagged: ratio 1/4 with min_p = 1/4
+    y = np.log(np.array([[0.5, 0.25, 0.125, 0.125]], dtype=np.float64)).astype(np.float32)
+    r = oracle.sample(y, np.array([0.5], dtype=np.float32), min_p=0.25, mode=oracle.MODE_TRUTH)
+    assert r["near"][0] and r["near_cut"][0]
+    # invalid values are refused
+    for bad in (-0.5, 1.0, float("nan")):
+        with pytest.raises(ValueError):
+            oracle.sample(y, np.array([0.5], dtype=np.float32), min_p=bad)
+
+
+@pytest.mark.parametrize("T,k,p,rep,min_p", [(1.0, 0, 1.0, 1.0, 0.05), (0.8, 40, 0.95, 1.1, 0.02), (0.7, 50, 0.9, 1.15, 0.1),
+                                               (1.2, 0, 0.99, 1.05, 0.01), (1.5, 0, 0.5, 0.8, 0.3)])
+def test_min_p_against_torch_restatement(oracle, T, k, p, rep, min_p):
+    rng = np.random.default_rng(17)
+    B, V, H = 48, 1000, 32
+    x = rng.normal(0, 2, size=(B, V)).astype(np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+    u = rng.random(B, dtype=np.float32)
+    want_t, want_p = _torch_sample(x, u, T, k, p, rep, hist, min_p)
+    got = oracle.sample(x, u, temperature=T, top_k=k, top_p=p, rep=rep, history=hist, mode=oracle.MODE_TRUTH, min_p=min_p)
+    ok = (got["tokens"] == want_t) | got["near"]
+    assert ok.all(), np.nonzero(~ok)
+    same = got["tokens"] == want_t
+    assert np.allclose(got["probs"][same], want_p[same], rtol=1e-5)
+    assert (~same).sum() <= 1
+    fixed = oracle.sample(x, u, temperature=T, top_k=k, top_p=p, rep=rep, history=hist, mode=oracle.MODE_FIXED, min_p=min_p)
+    diff = fixed["tokens"] != got["tokens"]
+    assert not (diff & ~got["near"]).any()
+    ok = ~got["near_cut"]
+    assert np.array_equal(fixed["n_nucleus"][ok], got["n_nucleus"][ok])
 
 
 # ---------------------------------------------------------------- layers agree, flags are honest
