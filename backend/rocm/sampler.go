@@ -29,7 +29,8 @@ import (
 )
 
 // SamplerConfig mirrors born_sampler_config.  Zero value of a field = default
-// (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off, TopK 0 = off, MinP 0 = off).
+// (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off, TopK 0 = off, MinP 0 = off, FrequencyPenalty 0 = off,
+// PresencePenalty 0 = off).
 type SamplerConfig struct {
 	Temperature       float32
 	TopK              int
@@ -37,6 +38,8 @@ type SamplerConfig struct {
 	RepetitionPenalty float32
 	Seed              int64
 	MinP              float32
+	FrequencyPenalty  float32
+	PresencePenalty   float32
 }
 
 // DeviceBuffer is device memory owned by the shim (Born's RawTensor is host-only,
@@ -102,6 +105,8 @@ func NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler {
 		repetition_penalty: C.float(cfg.RepetitionPenalty),
 		seed:               C.int64_t(cfg.Seed),
 		min_p:              C.float(cfg.MinP),
+		frequency_penalty:  C.float(cfg.FrequencyPenalty),
+		presence_penalty:   C.float(cfg.PresencePenalty),
 	}
 	var h *C.born_sampler
 	if err := check(C.born_rocm_sampler_create(&c, C.int64_t(maxBatch), C.int64_t(maxVocab), &h)); err != nil {

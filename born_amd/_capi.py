@@ -14,7 +14,8 @@ OK, ERR_ARGUMENT, ERR_HIP, ERR_UNSUPPORTED, ERR_DATA = 0, 1, 2, 3, 4
 
 class SamplerConfigC(C.Structure):
     _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("top_p", C.c_float),
-                ("repetition_penalty", C.c_float), ("seed", C.c_int64), ("min_p", C.c_float)]
+                ("repetition_penalty", C.c_float), ("seed", C.c_int64), ("min_p", C.c_float),
+                ("frequency_penalty", C.c_float), ("presence_penalty", C.c_float)]
 
 
 # every symbol include/born_rocm.h declares: name -> (restype, argtypes)

@@ -52,6 +52,8 @@ struct born_sampler {
     int *status;
     unsigned long long *counters;
     unsigned long long *lm_best;   // [max_batch] packed (value, ~column) keys of the greedy-decode LM head
+    unsigned *hist_counts;         // [max_batch][max_vocab] occurrences of each id in its row's history; all zero between
+                                   // calls; allocated when a frequency or presence penalty is first configured
     // spec-verify statistics:
     float *sp_mp, *sp_mq, *sp_mb;
     unsigned long long *sp_Zp, *sp_Zq, *sp_pd, *sp_qd, *sp_part, *sp_run, *sp_Zb;
@@ -72,8 +74,14 @@ static int fill_defaults(born_sampler_config *c) {
                     (double)c->repetition_penalty);
     if (!(c->min_p >= 0.0f) || !(c->min_p < 1.0f))
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: min_p must be in [0, 1), got %g", (double)c->min_p);
+    if (!std::isfinite(c->frequency_penalty))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: frequency_penalty must be finite, got %g", (double)c->frequency_penalty);
+    if (!std::isfinite(c->presence_penalty))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: presence_penalty must be finite, got %g", (double)c->presence_penalty);
     return BORN_ROCM_OK;
 }
+
+static bool counts_history(const born_sampler_config &c) { return c.frequency_penalty != 0.0f || c.presence_penalty != 0.0f; }
 
 // Distance below the row maximum beyond which a logit carries no mass: 80 (where the fixed-point masses have long
 // been zero), or the min-p bound -ln(min_p) when that is smaller.  fp64 log rounded once to fp32.
@@ -172,6 +180,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     alloc((void **)&s->status, sizeof(int));
     alloc((void **)&s->lm_best, rows * LM_BEST_PITCH * sizeof(unsigned long long));
     alloc((void **)&s->counters, (64 + 8 * rows) * sizeof(unsigned long long));   // [0..2] work counters; debug builds: [8..] phase stamps, [64..] per-row stamps
+    if (counts_history(c)) alloc((void **)&s->hist_counts, rows * (size_t)max_vocab * sizeof(unsigned));
     if (e != hipSuccess) {
         born_rocm_sampler_destroy(s);
         return hip_fail(e, "workspace allocation");
@@ -182,7 +191,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters, s->lm_best,
+    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters, s->lm_best, s->hist_counts,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run,
                     s->sp_mb,     s->sp_Zb};
     for (void *p : ptrs)
@@ -201,6 +210,12 @@ int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg
     born_sampler_config c = *cfg;
     int rc = fill_defaults(&c);
     if (rc) return rc;
+    if (counts_history(c) && !s->hist_counts) {
+        // the table of occurrence counts: allocated here, never inside a sampling call (which may be under graph capture)
+        const size_t bytes = (size_t)s->max_batch * (size_t)s->max_vocab * sizeof(unsigned);
+        HIP_TRY(hipMalloc((void **)&s->hist_counts, bytes));
+        HIP_TRY(hipMemset(s->hist_counts, 0, bytes));
+    }
     s->cfg = c;
     return BORN_ROCM_OK;
 }
@@ -332,8 +347,21 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     a.counters = s->counters;
     a.mass_shift = mass_shift(vocab);
     a.dcut = mass_cutoff(s->cfg);
+    a.freq = s->cfg.frequency_penalty;
+    a.pres = s->cfg.presence_penalty;
+    const bool counted = counts_history(s->cfg) && history && hist_stride > 0;
+    a.hist_counts = counted ? s->hist_counts : nullptr;
 
     hipStream_t st = (hipStream_t)stream;
+    if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
+    // The single-pass kernel relies on the penalties never raising a logit.
+    const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
+    // a failed launch must not leave the table of counts raised: remember the error, clear, then report
+    hipError_t launch_err = hipSuccess;
+#define TRY_LAUNCH(expr)                                              \
+    do {                                                              \
+        if (launch_err == hipSuccess) launch_err = (expr);            \
+    } while (0)
     if (row_T || row_k || row_p || row_rep) {
         // every kernel over the whole batch: each workgroup takes its row only if the row's configuration is its own
         RowConfigs rows;
@@ -342,20 +370,25 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.p = row_p;
         rows.rep = row_rep;
         rows.path = s->path;
-        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) HIP_TRY(launch_topk_row(a, st, &rows));
-        if (s->path != 1) HIP_TRY(launch_nucleus_row(a, st, &rows));
-        HIP_TRY(launch_sample_wide(a, st, &rows));
+        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) TRY_LAUNCH(launch_topk_row(a, st, &rows));
+        if (s->path != 1) TRY_LAUNCH(launch_nucleus_row(a, st, &rows));
+        TRY_LAUNCH(launch_sample_wide(a, st, &rows));
     } else {
-        // The single-pass kernel relies on the penalty never raising a logit (repetition_penalty >= 1).
-        const bool boosts = history && a.rep < 1.0f;
+        const bool boosts = (history && a.rep < 1.0f) || raises;   // (repetition_penalty < 1 raises the positive logits)
         if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
-            HIP_TRY(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
+            TRY_LAUNCH(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
         } else if (s->path != 1 && a.top_k == 0) {
-            HIP_TRY(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
+            TRY_LAUNCH(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
         } else {
-            HIP_TRY(launch_sample_wide(a, st));
+            TRY_LAUNCH(launch_sample_wide(a, st));
         }
     }
+#undef TRY_LAUNCH
+    if (counted) {
+        const hipError_t ce = launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st);
+        if (launch_err == hipSuccess) launch_err = ce;
+    }
+    if (launch_err != hipSuccess) return hip_fail(launch_err, "sample: kernel launch");
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;
 }

@@ -160,6 +160,28 @@ hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st) 
     return hipGetLastError();
 }
 
+// Occurrence counts of the history ids, one workgroup per row: the table is all zero before the counting launch and
+// all zero again after the clearing one, which touches exactly the entries the first one raised.
+template <bool CLEAR>
+__global__ __launch_bounds__(256) void hist_counts_kernel(const int *history, const int *hist_len, long long hist_stride, int V,
+                                                          unsigned *counts) {
+    const int row = blockIdx.x;
+    const int hlen = min((int)(hist_len ? hist_len[row] : (int)hist_stride), (int)hist_stride);
+    const int *h = history + (long long)row * hist_stride;
+    unsigned *c = counts + (long long)row * V;
+    for (int i = threadIdx.x; i < hlen; i += 256) {
+        const int t = h[i];
+        if (t < 0 || t >= V) continue;
+        if (CLEAR) c[t] = 0u; else atomicAdd(&c[t], 1u);
+    }
+}
+hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,
+                              bool clear, hipStream_t st) {
+    if (clear) hipLaunchKernelGGL(hist_counts_kernel<true>, dim3(B), dim3(256), 0, st, history, hist_len, hist_stride, V, counts);
+    else hipLaunchKernelGGL(hist_counts_kernel<false>, dim3(B), dim3(256), 0, st, history, hist_len, hist_stride, V, counts);
+    return hipGetLastError();
+}
+
 __global__ void uniforms_kernel(u64 seed, u64 step, float *u, long long n) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) u[i] = uniform_of(seed, step, (u64)i);

@@ -56,6 +56,14 @@ __device__ __forceinline__ float canon(float z) {
 }
 __device__ __forceinline__ float penalise(float x, float r) { return x > 0.0f ? x / r : x * r; }
 
+// A logit whose id the row's history holds: the repetition penalty, then (when `counts`, the row's occurrence counts by
+// id, is given) minus frequency * count, minus presence; every step rounded to fp32 on its own.
+__device__ __forceinline__ float penalise_seen(float x, float r, const unsigned *counts, int id, float freq, float pres) {
+    float y = penalise(x, r);
+    if (counts) y = __fsub_rn(__fsub_rn(y, __fmul_rn(freq, (float)counts[id])), pres);
+    return y;
+}
+
 // z from a (possibly penalised) logit: temperature then canonicalisation
 __device__ __forceinline__ float z_of(float y, float T) { return canon(T == 1.0f ? y : y / T); }
 

@@ -49,6 +49,9 @@ struct SampleArgs {
     unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows that needed an exact (slower) refinement, [2] rows sampled without a top-k cut or by the general kernel
     int mass_shift;
     float dcut;                   // masses are zero beyond this distance below the row maximum: min(80, -ln(min_p))
+    // frequency / presence penalties: how often each id occurs in its row's history, [B, V] (null: both are off)
+    const unsigned *hist_counts;
+    float freq, pres;
 };
 
 // Per-row configurations (device arrays of B values, each optional): a second argument of the per-row kernel
@@ -113,6 +116,9 @@ hipError_t launch_argmax(const float *logits, int B, int V, long long stride, in
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
                           hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
+// counts[row * V + id] += 1 for every valid id of the row's history (clear: = 0 instead, which restores an all-zero table)
+hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,
+                              bool clear, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
 hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);

@@ -35,6 +35,8 @@ struct NucRow {                               // uniform per workgroup
     int V;
     bool vec, penal, degenerate;
     float T, rep, m, scale, range, sbin, dcut;
+    const unsigned *counts;                   // occurrences of each id in the row's history (frequency / presence penalties), or null
+    float freq, pres;
 };
 
 __device__ __forceinline__ float nuc_z(const NucRow &r, float y) {
@@ -58,7 +60,7 @@ __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f)
             if (bits) {
 #pragma unroll
                 for (int t = 0; t < 4; t++)
-                    if ((bits >> t) & 1u) y[t] = penalise(y[t], r.rep);
+                    if ((bits >> t) & 1u) y[t] = penalise_seen(y[t], r.rep, r.counts, j + t, r.freq, r.pres);
             }
         }
 #pragma unroll
@@ -89,13 +91,13 @@ __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f)
         }
         for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) {
             float y = r.x[j];
-            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, r.rep);
+            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
             f(j, y);
         }
     } else {
         for (int j = tid; j < r.V; j += NUC_BLOCK) {
             float y = r.x[j];
-            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, r.rep);
+            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
             f(j, y);
         }
     }
@@ -159,7 +161,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
-    r.penal = (cfg_rep != 1.0f) && hlen > 0;
+    r.counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
+    r.freq = a.freq;
+    r.pres = a.pres;
+    r.penal = (cfg_rep != 1.0f || r.counts) && hlen > 0;
     if (r.penal)
         for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
     for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;

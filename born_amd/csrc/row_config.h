@@ -37,7 +37,8 @@ __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const Row
     if (!row_config_valid(T, top_p, rep)) {
         invalid = true;
         route = ROUTE_GENERAL;
-    } else if (rc.path != 1 && top_k >= 1 && top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && rep < 1.0f)) {
+    } else if (rc.path != 1 && top_k >= 1 && top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && rep < 1.0f) &&
+               !(a.hist_counts && (a.freq < 0.0f || a.pres < 0.0f))) {
         route = ROUTE_TOPK;
     } else if (rc.path != 1 && top_k == 0) {
         route = ROUTE_NUCLEUS;

@@ -17,6 +17,8 @@ struct WideCtx {
     int V;
     bool vec, has_hist, count_mode;
     float T, rep, m, scale, dcut;
+    const unsigned *counts;  // occurrences of each id in the row's history (frequency / presence penalties), or null
+    float freq, pres;
     const lds_u32 *bm;
     lds_u64 *mass;  // [WIDE_BINS] inclusive cumulative masses after the scan
     lds_u32 *cnt;   // [WIDE_BINS] inclusive cumulative counts (count_mode only)
@@ -56,7 +58,7 @@ __device__ __forceinline__ void wide_visit4(const WideCtx &c, const wide_f32x4 &
         if (bits) {
 #pragma unroll
             for (int t = 0; t < 4; t++)
-                if ((bits >> t) & 1u) y[t] = penalise(y[t], c.rep);
+                if ((bits >> t) & 1u) y[t] = penalise_seen(y[t], c.rep, c.counts, j + t, c.freq, c.pres);
         }
     }
 #pragma unroll
@@ -93,13 +95,13 @@ __device__ __forceinline__ void wide_foreach(const WideCtx &c, F f) {
         }
         for (int j = (n4 << 2) + tid; j < c.V; j += WIDE_BLOCK) {
             float y = c.x[j];
-            if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, c.rep);
+            if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, c.rep, c.counts, j, c.freq, c.pres);
             f(j, y);
         }
     } else {
         for (int j = tid; j < c.V; j += WIDE_BLOCK) {
             float y = c.x[j];
-            if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, c.rep);
+            if (c.has_hist && ((c.bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, c.rep, c.counts, j, c.freq, c.pres);
             f(j, y);
         }
     }
@@ -349,7 +351,10 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     BORN_STAMP(a, row, 0);
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
-    c.has_hist = (a.rep != 1.0f) && hlen > 0;
+    c.counts = a.hist_counts ? a.hist_counts + (long long)row * a.V : nullptr;
+    c.freq = a.freq;
+    c.pres = a.pres;
+    c.has_hist = (a.rep != 1.0f || c.counts) && hlen > 0;
     if (c.has_hist) {
         const int words = (V + 31) >> 5;
         for (int i = tid; i < words; i += WIDE_BLOCK) bm[i] = 0;

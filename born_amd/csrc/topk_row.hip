@@ -168,7 +168,8 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     u32 *hist = reinterpret_cast<u32 *>(pool + OFF_FB_HIST);
     u64 *list = pool + OFF_FB_LIST;
     u64 *sorted = pool + OFF_FB_SORTED;
-    const bool penal = a.rep != 1.0f && hlen > 0;
+    const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
+    const bool penal = (a.rep != 1.0f || counts) && hlen > 0;
     __syncthreads();                                                 // the proof's use of the pool is over
     if (penal) {
         for (int i = tid; i < ((V + 31) >> 5); i += ROW_BLOCK) bm[i] = 0u;
@@ -181,7 +182,7 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
     auto rank_key = [&](int j, float xv) -> u64 {
         float y = xv;
-        if (penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise(y, a.rep);
+        if (penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, a.rep, counts, j, a.freq, a.pres);
         return make_key64(z_of(y, a.T), j);
     };
     // radix descent: after each sweep the wanted key is the need-th largest inside the bucket `prefix`
@@ -289,7 +290,8 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
     // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
     // probe it at the end; a longer one probes a hash of the candidates instead.
-    const bool penal = a.rep != 1.0f && hlen > 0;
+    const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
+    const bool penal = (a.rep != 1.0f || counts) && hlen > 0;
     const bool hfast = penal && hlen <= ROW_BLOCK;
     htab[tid] = 0u;
     htab[tid + ROW_BLOCK] = 0u;
@@ -462,7 +464,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
                     slot = (slot + 1) & (ROW_HSLOTS - 1);
                 }
             }
-            if (seen) y = penalise(y, a.rep);
+            if (seen) y = penalise_seen(y, a.rep, counts, (int)(c.y & 0x7FFFFFFFu), a.freq, a.pres);
             const float z = z_of(y, a.T);
             keep = ordkey(z) > zb;
             K[tid] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;

@@ -33,17 +33,20 @@ def _check(rc):
 @dataclass
 class SamplerConfig:
     """Zero value of a field means "use the default" (Temperature 1, TopP 1 = off, RepetitionPenalty 1 = off,
-    MinP 0 = off)."""
+    MinP 0 = off, FrequencyPenalty 0 = off, PresencePenalty 0 = off)."""
     Temperature: float = 0.0
     TopK: int = 0
     TopP: float = 0.0
     RepetitionPenalty: float = 0.0
     Seed: int = 0
     MinP: float = 0.0
+    FrequencyPenalty: float = 0.0
+    PresencePenalty: float = 0.0
 
     def _c(self):
         return SamplerConfigC(float(self.Temperature), int(self.TopK), float(self.TopP),
-                              float(self.RepetitionPenalty), int(self.Seed), float(self.MinP))
+                              float(self.RepetitionPenalty), int(self.Seed), float(self.MinP),
+                              float(self.FrequencyPenalty), float(self.PresencePenalty))
 
 
 def _ptr(x):
@@ -137,7 +140,8 @@ class Sampler:
     def Config(self):
         c = SamplerConfigC()
         _check(_capi.lib().born_rocm_sampler_get_config(self._h, C.byref(c)))
-        return SamplerConfig(c.temperature, c.top_k, c.top_p, c.repetition_penalty, c.seed, c.min_p)
+        return SamplerConfig(c.temperature, c.top_k, c.top_p, c.repetition_penalty, c.seed, c.min_p,
+                             c.frequency_penalty, c.presence_penalty)
 
     def SetConfig(self, cfg):
         c = cfg._c()

@@ -48,6 +48,10 @@ typedef struct born_sampler_config {
     int64_t seed;                 /* seed of the built-in uniform stream (used only when `uniforms` is NULL) */
     float   min_p;                /* 0 => disabled ; else in (0, 1): a token stays only if its probability is at
                                      least min_p times the most likely token's (applied before top-k and top-p) */
+    float   frequency_penalty;    /* 0 => disabled ; subtracted from a token's logit once per occurrence in the history */
+    float   presence_penalty;     /* 0 => disabled ; subtracted once from the logit of every token the history holds
+                                     (both after the repetition penalty, before the temperature; finite, either sign).
+                                     A handle configured with either keeps a table of max_batch * max_vocab counters. */
 } born_sampler_config;
 
 typedef struct born_sampler born_sampler;   /* opaque: config + stream-ordered workspace + draw counter */
@@ -104,7 +108,7 @@ int born_rocm_softmax(born_sampler *s, const float *logits, int64_t batch, int64
 int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                           float *out, void *stream);
 
-/* One sampling step for `batch` rows: penalty -> temperature -> (min-p) -> top-k -> softmax -> top-p -> draw.
+/* One sampling step for `batch` rows: penalties -> temperature -> (min-p) -> top-k -> softmax -> top-p -> draw.
  * No counterpart in the reference snapshot; it consumes the `[batch, vocab]` fp32 output of the last
  * Linear (internal/nn/linear.go:78-107) where the reference's only consumers are CrossEntropy and
  * nn.Accuracy (internal/nn/cross_entropy.go:261-284).

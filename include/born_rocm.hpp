@@ -27,6 +27,8 @@ struct SamplerConfig {
     float RepetitionPenalty = 0.0f;
     int64_t Seed = 0;
     float MinP = 0.0f;
+    float FrequencyPenalty = 0.0f;
+    float PresencePenalty = 0.0f;
 };
 
 class DeviceBuffer {
@@ -50,7 +52,8 @@ private:
 class Sampler {
 public:
     Sampler(const SamplerConfig &cfg, int64_t max_batch, int64_t max_vocab) {
-        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed, cfg.MinP};
+        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed, cfg.MinP,
+                              cfg.FrequencyPenalty, cfg.PresencePenalty};
         check(born_rocm_sampler_create(&c, max_batch, max_vocab, &h_));
     }
     Sampler(const Sampler &) = delete;

@@ -364,24 +364,32 @@ static void heap_sift_down(uint64_t *h, int64_t n, int64_t i) {
     }
 }
 
-/* z_j for every j of one row: penalty (unique ids, from the original logit),
- * temperature, canonicalisation.  `seen` is a V-byte scratch (zeroed on exit).
+/* z_j for every j of one row: penalties (each id of the history once, from the original logit: the repetition
+ * penalty, then minus frequency * occurrences, minus presence, every step rounded to fp32), temperature,
+ * canonicalisation.  `count` is a V-entry scratch (zero on entry and on exit).
  * Returns the number of out-of-range history ids. */
 static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hlen,
-                     float T, float r, float *z, uint8_t *seen) {
+                     float T, float r, float freq, float pres, float *z, int32_t *count) {
     int64_t bad = 0;
+    const int additive = freq != 0.0f || pres != 0.0f;
     for (int64_t j = 0; j < V; j++) z[j] = x[j];
-    if (r != 1.0f) {
+    if (r != 1.0f || additive) {
         for (int64_t i = 0; i < hlen; i++) {
             int32_t t = hist[i];
             if (t < 0 || t >= V) { bad++; continue; }
-            if (seen[t]) continue;
-            seen[t] = 1;
-            z[t] = penalise(x[t], r);
+            count[t]++;
         }
         for (int64_t i = 0; i < hlen; i++) {
             int32_t t = hist[i];
-            if (t >= 0 && t < V) seen[t] = 0;
+            if (t < 0 || t >= V || count[t] == 0) continue;      /* count 0: a duplicate already handled */
+            float y = penalise(x[t], r);
+            if (additive) {
+                float f = freq * (float)count[t];
+                y = y - f;
+                y = y - pres;
+            }
+            z[t] = y;
+            count[t] = 0;
         }
     } else {
         for (int64_t i = 0; i < hlen; i++) if (hist[i] < 0 || hist[i] >= V) bad++;
@@ -391,7 +399,7 @@ static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hle
 }
 
 /*
- * born_oracle_sample_min_p (born_oracle_sample: the same with min_p = 0)
+ * born_oracle_sample_ex (born_oracle_sample: the same with min_p = 0 and no frequency / presence penalty)
  *   logits [B, row_stride>=V]; history [B, hist_stride] (may be NULL), hist_len
  *   [B] (NULL => hist_stride entries per row); uniforms [B].
  * outputs (any may be NULL): tokens[B], probs[B], near[B] (layer T flags: bit 0 =
@@ -402,15 +410,17 @@ static int64_t row_z(const float *x, int64_t V, const int32_t *hist, int64_t hle
  *   nuc_ids[B, nuc_cap], nuc_probs[B, nuc_cap].
  * returns the number of out-of-range history ids met, or -1 on bad arguments.
  */
-BORN_EXPORT int64_t born_oracle_sample_min_p(
+BORN_EXPORT int64_t born_oracle_sample_ex(
     const float *logits, int64_t B, int64_t V, int64_t row_stride,
     const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
-    const float *uniforms, float T, int32_t top_k, float top_p, float min_p, float rep, int32_t mode,
+    const float *uniforms, float T, int32_t top_k, float top_p, float min_p, float rep, float freq, float pres,
+    int32_t mode,
     int32_t *tokens, float *probs, uint8_t *near, int32_t *n_nucleus,
     int64_t nuc_cap, int32_t *nuc_ids, float *nuc_probs)
 {
     if (!logits || !uniforms || B <= 0 || V <= 0 || row_stride < V) return -1;
     if (!(T > 0.0f) || !(top_p > 0.0f) || !(rep > 0.0f) || !(min_p >= 0.0f) || !(min_p < 1.0f)) return -1;
+    if (!isfinite(freq) || !isfinite(pres)) return -1;
     /* min-p (spec section 2.5): a survivor stays iff m - z <= -ln(min_p).  Layer T tests the fp64 difference
      * against the fp64 bound; layer F the fp32 difference against the bound rounded to fp32 and capped at 80
      * (beyond which the fixed-point masses are zero anyway). */
@@ -422,7 +432,7 @@ BORN_EXPORT int64_t born_oracle_sample_min_p(
     int S = born_oracle_mass_shift(V);
 
     float *z = (float *)malloc(sizeof(float) * (size_t)V);
-    uint8_t *seen = (uint8_t *)calloc((size_t)V, 1);
+    int32_t *seen = (int32_t *)calloc((size_t)V, sizeof(int32_t));
     uint64_t *keys = (uint64_t *)malloc(sizeof(uint64_t) * (size_t)V);
     double *e = (double *)malloc(sizeof(double) * (size_t)k);
     uint64_t *q = (uint64_t *)malloc(sizeof(uint64_t) * (size_t)k);
@@ -431,7 +441,7 @@ BORN_EXPORT int64_t born_oracle_sample_min_p(
     for (int64_t b = 0; b < B; b++) {
         const float *x = logits + b * row_stride;
         int64_t hlen = history ? (hist_len ? hist_len[b] : hist_stride) : 0;
-        bad += row_z(x, V, history ? history + b * hist_stride : NULL, hlen, T, rep, z, seen);
+        bad += row_z(x, V, history ? history + b * hist_stride : NULL, hlen, T, rep, freq, pres, z, seen);
 
         /* rank order: the k largest 64-bit keys, descending */
         int64_t n;
@@ -579,7 +589,7 @@ BORN_EXPORT int64_t born_oracle_sample_min_p(
     return bad;
 }
 
-/* born_oracle_sample_min_p with min-p off */
+/* born_oracle_sample_ex with min-p and the frequency / presence penalties off */
 BORN_EXPORT int64_t born_oracle_sample(
     const float *logits, int64_t B, int64_t V, int64_t row_stride,
     const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
@@ -587,8 +597,8 @@ BORN_EXPORT int64_t born_oracle_sample(
     int32_t *tokens, float *probs, uint8_t *near, int32_t *n_nucleus,
     int64_t nuc_cap, int32_t *nuc_ids, float *nuc_probs)
 {
-    return born_oracle_sample_min_p(logits, B, V, row_stride, history, hist_len, hist_stride, uniforms, T, top_k, top_p,
-                                    0.0f, rep, mode, tokens, probs, near, n_nucleus, nuc_cap, nuc_ids, nuc_probs);
+    return born_oracle_sample_ex(logits, B, V, row_stride, history, hist_len, hist_stride, uniforms, T, top_k, top_p,
+                                 0.0f, rep, 0.0f, 0.0f, mode, tokens, probs, near, n_nucleus, nuc_cap, nuc_ids, nuc_probs);
 }
 
 /* ------------------------------------------------------------------ */

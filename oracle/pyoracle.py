@@ -66,10 +66,10 @@ def lib():
         L.born_oracle_sample.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, f32p,
                                          C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
                                          i32p, f32p, u8p, i32p, C.c_int64, i32p, f32p]
-        L.born_oracle_sample_min_p.restype = C.c_int64
-        L.born_oracle_sample_min_p.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, f32p,
-                                               C.c_float, C.c_int32, C.c_float, C.c_float, C.c_float, C.c_int32,
-                                               i32p, f32p, u8p, i32p, C.c_int64, i32p, f32p]
+        L.born_oracle_sample_ex.restype = C.c_int64
+        L.born_oracle_sample_ex.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, f32p,
+                                               C.c_float, C.c_int32, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int32,
+                                            i32p, f32p, u8p, i32p, C.c_int64, i32p, f32p]
         L.born_oracle_spec_verify.restype = C.c_int64
         L.born_oracle_spec_verify.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int64, i32p, f32p, f32p,
                                               C.c_float, C.c_int32, i32p, i32p, u8p]
@@ -256,7 +256,7 @@ def row_stats(x, T=1.0):
 
 
 def sample(logits, uniforms, temperature=1.0, top_k=0, top_p=1.0, rep=1.0, history=None, hist_len=None,
-           mode=MODE_TRUTH, nuc_cap=0, min_p=0.0):
+           mode=MODE_TRUTH, nuc_cap=0, min_p=0.0, freq=0.0, pres=0.0):
     """Returns dict(tokens, probs, near, n_nucleus[, nuc_ids, nuc_probs], bad_ids)."""
     x = _f32(logits)
     B, V = x.shape
@@ -278,9 +278,9 @@ def sample(logits, uniforms, temperature=1.0, top_k=0, top_p=1.0, rep=1.0, histo
     if nuc_cap > 0:
         nid = np.empty((B, nuc_cap), dtype=np.int32)
         npr = np.empty((B, nuc_cap), dtype=np.float32)
-    bad = lib().born_oracle_sample_min_p(_p(x, C.c_float), B, V, V, _p(h, C.c_int32), _p(hl, C.c_int32), hs,
+    bad = lib().born_oracle_sample_ex(_p(x, C.c_float), B, V, V, _p(h, C.c_int32), _p(hl, C.c_int32), hs,
                                    _p(u, C.c_float), float(temperature), int(top_k), float(top_p), float(min_p),
-                                   float(rep), int(mode), _p(tokens, C.c_int32), _p(probs, C.c_float), _p(near, C.c_uint8),
+                                   float(rep), float(freq), float(pres), int(mode), _p(tokens, C.c_int32), _p(probs, C.c_float), _p(near, C.c_uint8),
                                    _p(nn, C.c_int32), int(nuc_cap), _p(nid, C.c_int32), _p(npr, C.c_float))
     if bad < 0:
         raise ValueError("born_oracle_sample: bad arguments")

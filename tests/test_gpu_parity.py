@@ -19,10 +19,11 @@ def rocm():
     return S
 
 
-def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0, max_vocab=None, min_p=0.0):
+def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0, max_vocab=None, min_p=0.0,
+         freq=0.0, pres=0.0):
     B, V = x.shape
-    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=k, TopP=p, RepetitionPenalty=rep, MinP=min_p), max_batch=B,
-                        max_vocab=max_vocab or V)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=k, TopP=p, RepetitionPenalty=rep, MinP=min_p,
+                                           FrequencyPenalty=freq, PresencePenalty=pres), max_batch=B, max_vocab=max_vocab or V)
     s.SetPath(path)
     out = rocm.sample_host(s, x, u, hist, hist_len, nucleus_cap=nuc)
     out["counters"] = s.Counters()
@@ -32,10 +33,10 @@ def _run(rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0
 
 
 def _check_against_oracle(oracle, rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=None, hist_len=None, nuc=0, path=0,
-                          max_near_frac=1.0, min_p=0.0):
-    got = _run(rocm, x, u, T, k, p, rep, hist, hist_len, nuc, path, min_p=min_p)
-    fx = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED, nuc_cap=nuc, min_p=min_p)
-    tr = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_TRUTH, nuc_cap=nuc, min_p=min_p)
+                          max_near_frac=1.0, min_p=0.0, freq=0.0, pres=0.0):
+    got = _run(rocm, x, u, T, k, p, rep, hist, hist_len, nuc, path, min_p=min_p, freq=freq, pres=pres)
+    fx = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED, nuc_cap=nuc, min_p=min_p, freq=freq, pres=pres)
+    tr = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_TRUTH, nuc_cap=nuc, min_p=min_p, freq=freq, pres=pres)
     bad = np.nonzero(got["tokens"] != fx["tokens"])[0]
     assert bad.size == 0, f"token mismatch vs fixed-point oracle at rows {bad[:8]}: {got['tokens'][bad[:8]]} vs {fx['tokens'][bad[:8]]}"
     assert np.array_equal(got["probs"].view(np.uint32), fx["probs"].view(np.uint32)), "probabilities differ from the fixed-point oracle"
@@ -354,6 +355,98 @@ def test_min_p_is_validated(rocm):
     s.Close()
 
 
+# ---------------------------------------------------------------- frequency and presence penalties
+
+@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("B,V,T,k,p,rep,H,freq,pres,route", [
+    (32, 128256, 0.7, 50, 0.9, 1.15, 512, 0.3, 0.5, "topk"),     # C3 shape: single-pass kernel, history hashed
+    (16, 32000, 1.0, 40, 0.95, 1.0, 64, 0.5, 0.0, "topk"),       # frequency alone, no repetition penalty
+    (16, 32000, 1.0, 40, 0.95, 1.0, 64, 0.0, 1.5, "topk"),       # presence alone
+    (9, 8000, 0.9, 64, 0.99, 1.2, 3000, 0.2, 0.3, "topk"),       # history longer than 1024: candidates are hashed instead
+    (16, 32000, 1.0, 20, 0.9, 1.1, 128, -0.4, 0.2, "general"),   # a negative penalty raises logits: general kernel
+    (16, 32000, 1.0, 0, 1.0, 1.0, 256, 0.4, 0.4, "nucleus"),     # no top-k: three-sweep kernel
+    (16, 152064, 1.2, 0, 0.99, 1.05, 2048, 0.1, 0.6, "nucleus"), # C5 shape
+    (16, 32000, 0.9, 500, 0.9, 1.1, 64, 0.25, 0.25, "general"),
+    (8, 50000, 1.0, 20000, 0.8, 1.0, 300, 0.5, 0.5, "general"),
+    (8, 1001, 1.0, 0, 0.9, 1.0, 5000, 0.05, 1.0, "nucleus"),     # unaligned rows, history much longer than the vocabulary
+    (8, 1001, 1.0, 10, 0.9, 1.0, 5000, 0.05, 1.0, "topk"),
+])
+def test_frequency_and_presence_penalties_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, freq, pres, route, path):
+    rng = np.random.default_rng(B * 104729 + V + H)
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)        # heavy repeats of the small ids
+    x[:, :8] += np.float32(4.0)                                             # ... which are also the likely tokens
+    hist_len = rng.integers(H // 2, H + 1, size=B).astype(np.int32)
+    nuc = min(64, k) if 1 <= k <= 64 else 0
+    got, fx, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, hist_len, nuc=nuc, path=path, freq=freq, pres=pres)
+    plain = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED)
+    assert (plain["tokens"] != fx["tokens"]).any() or not np.array_equal(plain["probs"], fx["probs"]), "the penalties are meant to matter"
+    c = got["counters"]
+    if path == 0 and route == "topk":
+        assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
+    if path == 0 and route == "general" and 1 <= k <= 64:
+        assert c["general_rows"] == B
+
+
+def test_frequency_penalty_table_is_clean_between_calls(oracle, rocm):
+    # one handle, three calls with different histories and shapes: each equals a fresh evaluation by the oracle
+    rng = np.random.default_rng(77)
+    Bm, Vm = 24, 40000
+    s = rocm.NewSampler(rocm.SamplerConfig(TopK=30, TopP=0.9, RepetitionPenalty=1.1, FrequencyPenalty=0.4, PresencePenalty=0.3),
+                        max_batch=Bm, max_vocab=Vm)
+    for (B, V, H) in [(24, 40000, 700), (10, 32000, 100), (24, 40000, 1500), (5, 999, 50)]:
+        x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
+        x[:, :8] += np.float32(4.0)
+        u = rng.random(B, dtype=np.float32)
+        hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+        got = rocm.sample_host(s, x, u, hist)
+        fx = oracle.sample(x, u, 1.0, 30, 0.9, 1.1, hist, mode=oracle.MODE_FIXED, freq=0.4, pres=0.3)
+        assert np.array_equal(got["tokens"], fx["tokens"]), (B, V, H)
+        assert np.array_equal(got["probs"].view(np.uint32), fx["probs"].view(np.uint32))
+    # switching the penalties on later allocates the table then; switching them off stops using it
+    t = rocm.NewSampler(rocm.SamplerConfig(TopK=30), max_batch=5, max_vocab=999)
+    t.SetConfig(rocm.SamplerConfig(TopK=30, FrequencyPenalty=0.7))
+    got = rocm.sample_host(t, x, u, hist)
+    fx = oracle.sample(x, u, 1.0, 30, 1.0, 1.0, hist, mode=oracle.MODE_FIXED, freq=0.7)
+    assert np.array_equal(got["tokens"], fx["tokens"])
+    t.SetConfig(rocm.SamplerConfig(TopK=30))
+    got = rocm.sample_host(t, x, u, hist)
+    fx = oracle.sample(x, u, 1.0, 30, 1.0, 1.0, hist, mode=oracle.MODE_FIXED)
+    assert np.array_equal(got["tokens"], fx["tokens"])
+    # no history: the penalties have nothing to act on
+    got = rocm.sample_host(s, x, u, None)
+    fx = oracle.sample(x, u, 1.0, 30, 0.9, 1.1, None, mode=oracle.MODE_FIXED)
+    assert np.array_equal(got["tokens"], fx["tokens"])
+    for h in (s, t):
+        h.Status()
+        h.Close()
+
+
+def test_frequency_penalty_rows_the_single_pass_kernel_cannot_prove(oracle, rocm):
+    # fewer finite logits than top_k, and heavy ties: the workgroup finishes by its exact selection, which penalises
+    # every element it ranks
+    rng = np.random.default_rng(78)
+    B, V, H = 8, 5000, 400
+    x = np.full((B, V), -np.inf, dtype=np.float32)
+    x[:, :30] = rng.standard_normal((B, 30), dtype=np.float32)
+    x[4:] = np.float32(1.0)                                                # every logit ties
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, 40, size=(B, H)).astype(np.int32)
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, 0.8, 50, 0.95, 1.2, hist, nuc=50, freq=0.01, pres=0.02)
+    assert got["counters"]["fallback_rows"] > 0
+
+
+def test_frequency_and_presence_penalties_are_validated(rocm):
+    for kw in (dict(FrequencyPenalty=float("inf")), dict(PresencePenalty=float("nan"))):
+        with pytest.raises(rocm.SamplerPanic, match="penalty"):
+            rocm.NewSampler(rocm.SamplerConfig(**kw), max_batch=1, max_vocab=16)
+    s = rocm.NewSampler(rocm.SamplerConfig(FrequencyPenalty=-0.5, PresencePenalty=0.25), max_batch=1, max_vocab=16)
+    c = s.Config()
+    assert c.FrequencyPenalty == -0.5 and c.PresencePenalty == 0.25
+    s.Close()
+
+
 def test_builtin_uniform_stream_in_sample(oracle, rocm):
     rng = np.random.default_rng(9)
     B, V = 16, 6000
@@ -454,9 +547,9 @@ def test_spec_verify_bonus_draw(oracle, rocm):
 
 # ---------------------------------------------------------------- a configuration per row
 
-def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0):
+def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, **handle):
     B, V = x.shape
-    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=7, TopP=0.8, RepetitionPenalty=1.3), max_batch=B, max_vocab=V)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=7, TopP=0.8, RepetitionPenalty=1.3, **handle), max_batch=B, max_vocab=V)
     s.SetPath(path)
     dev = lambda a, dt: None if a is None else rocm.DeviceBuffer.from_numpy(np.ascontiguousarray(a, dtype=dt))
     tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
@@ -496,6 +589,32 @@ def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
         assert c["topk_rows"] > 0 and c["general_rows"] > 0                 # more than one kernel took rows
     s.Close()
     s2.Close()
+
+
+@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("freq,pres,min_p", [(0.3, 0.4, 0.0), (-0.2, 0.1, 0.0), (0.0, 0.0, 0.05), (0.2, 0.0, 0.02)])
+def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq, pres, min_p):
+    # min-p and the frequency / presence penalties stay the handle's while the other settings vary per row
+    rng = np.random.default_rng(79)
+    B, V, H = 24, 9000, 300
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    x[:, :8] += np.float32(3.0)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+    Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 300, V], B).astype(np.int32)
+    ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
+    reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
+    s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, MinP=min_p, FrequencyPenalty=freq, PresencePenalty=pres)
+    s.Status()
+    for b in range(B):
+        want = oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(ks[b]), float(ps[b]), float(reps[b]), hist[b:b + 1], None,
+                             mode=oracle.MODE_FIXED, min_p=min_p, freq=freq, pres=pres)
+        assert tok[b] == want["tokens"][0], (b, Ts[b], ks[b], ps[b], reps[b])
+        assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], b
+    if path == 0 and freq < 0:
+        assert s.Counters()["topk_rows"] == 0                            # a penalty that raises logits: never the single-pass kernel
+    s.Close()
 
 
 def test_per_row_invalid_configuration_is_reported(oracle, rocm):

@@ -153,7 +153,7 @@ def test_special_values(oracle):
 
 # ---------------------------------------------------------------- independent restatement in torch
 
-def _torch_sample(x, u, T, k, p, rep, hist, min_p=0.0):
+def _torch_sample(x, u, T, k, p, rep, hist, min_p=0.0, freq=0.0, pres=0.0):
     """Independent restatement with torch primitives (float64 probabilities)."""
     x = torch.from_numpy(x.copy())
     B, V = x.shape
@@ -164,6 +164,10 @@ def _torch_sample(x, u, T, k, p, rep, hist, min_p=0.0):
             ids = torch.unique(torch.from_numpy(hist[b].astype(np.int64)))
             sel = row[ids]
             row[ids] = torch.where(sel > 0, sel / np.float32(rep), sel * np.float32(rep))
+        if hist is not None and (freq != 0.0 or pres != 0.0):
+            counts = torch.bincount(torch.from_numpy(hist[b].astype(np.int64)), minlength=V).to(torch.float32)
+            row = row - np.float32(freq) * counts
+            row = row - np.float32(pres) * (counts > 0).to(torch.float32)
         z = row / np.float32(T)
         order = torch.from_numpy(np.lexsort((np.arange(V), -z.numpy().astype(np.float64))))  # z desc, id asc
         zs = z[order].double()
@@ -266,6 +270,67 @@ def test_min_p_against_torch_restatement(oracle, T, k, p, rep, min_p):
     assert not (diff & ~got["near"]).any()
     ok = ~got["near_cut"]
     assert np.array_equal(fixed["n_nucleus"][ok], got["n_nucleus"][ok])
+
+
+def test_frequency_and_presence_penalty_hand_vectors(oracle):
+    x = np.array([[2.0, 1.0, 0.5, -1.0]], dtype=np.float32)
+    hist = np.array([[0, 0, 1, 3]], dtype=np.int32)
+    u = np.array([0.5], dtype=np.float32)
+
+    def dist(**kw):
+        r = oracle.sample(x, u, history=hist, nuc_cap=4, mode=oracle.MODE_TRUTH, **kw)
+        out = np.zeros(4)
+        out[r["nuc_ids"][0]] = r["nuc_probs"][0]
+        return out
+
+    def softmax(y):
+        e = np.exp(np.array(y, dtype=np.float64) - max(y))
+        return e / e.sum()
+
+    # frequency: minus 0.5 per occurrence; presence: minus 0.25 once; the token never emitted keeps its logit
+    assert np.allclose(dist(freq=0.5), softmax([2.0 - 1.0, 1.0 - 0.5, 0.5, -1.0 - 0.5]), rtol=1e-6)
+    assert np.allclose(dist(pres=0.25), softmax([1.75, 0.75, 0.5, -1.25]), rtol=1e-6)
+    assert np.allclose(dist(freq=0.5, pres=0.25), softmax([0.75, 0.25, 0.5, -1.75]), rtol=1e-6)
+    # after the repetition penalty (2/1.25 = 1.6, 1/1.25 = 0.8, -1 * 1.25 = -1.25), before the temperature
+    assert np.allclose(dist(freq=0.5, pres=0.25, rep=1.25, temperature=0.5),
+                       softmax([2 * (1.6 - 1.25), 2 * (0.8 - 0.75), 2 * 0.5, 2 * (-1.25 - 0.75)]), rtol=1e-6)
+    # a negative penalty rewards repeats; ids outside the vocabulary are reported and ignored
+    assert np.allclose(dist(freq=-0.5), softmax([3.0, 1.5, 0.5, -0.5]), rtol=1e-6)
+    bad = oracle.sample(x, u, history=np.array([[0, 9, -1, 0]], dtype=np.int32), freq=0.5, nuc_cap=4)
+    assert bad["bad_ids"] == 2
+    out = np.zeros(4)
+    out[bad["nuc_ids"][0]] = bad["nuc_probs"][0]
+    assert np.allclose(out, softmax([1.0, 1.0, 0.5, -1.0]), rtol=1e-6)
+    # hist_len shortens the history: only the first two entries count
+    r = oracle.sample(x, u, history=hist, hist_len=np.array([2], dtype=np.int32), freq=0.5, nuc_cap=4)
+    out = np.zeros(4)
+    out[r["nuc_ids"][0]] = r["nuc_probs"][0]
+    assert np.allclose(out, softmax([1.0, 1.0, 0.5, -1.0]), rtol=1e-6)
+    for badv in (float("inf"), float("nan")):
+        with pytest.raises(ValueError):
+            oracle.sample(x, u, history=hist, freq=badv)
+        with pytest.raises(ValueError):
+            oracle.sample(x, u, history=hist, pres=badv)
+
+
+@pytest.mark.parametrize("T,k,p,rep,freq,pres", [(1.0, 0, 1.0, 1.0, 0.3, 0.0), (0.8, 40, 0.95, 1.1, 0.2, 0.4),
+                                                   (0.7, 50, 0.9, 1.0, 0.0, 0.6), (1.2, 0, 0.99, 1.05, -0.1, 0.2)])
+def test_frequency_and_presence_against_torch_restatement(oracle, T, k, p, rep, freq, pres):
+    rng = np.random.default_rng(19)
+    B, V, H = 48, 300, 200                       # many repeats per id
+    x = rng.normal(0, 2, size=(B, V)).astype(np.float32)
+    hist = ((rng.zipf(1.3, size=(B, H)) - 1) % V).astype(np.int32)
+    u = rng.random(B, dtype=np.float32)
+    want_t, want_p = _torch_sample(x, u, T, k, p, rep, hist, 0.0, freq, pres)
+    got = oracle.sample(x, u, temperature=T, top_k=k, top_p=p, rep=rep, history=hist, mode=oracle.MODE_TRUTH, freq=freq, pres=pres)
+    ok = (got["tokens"] == want_t) | got["near"]
+    assert ok.all(), np.nonzero(~ok)
+    same = got["tokens"] == want_t
+    assert np.allclose(got["probs"][same], want_p[same], rtol=1e-5)
+    assert (~same).sum() <= 1
+    fixed = oracle.sample(x, u, temperature=T, top_k=k, top_p=p, rep=rep, history=hist, mode=oracle.MODE_FIXED, freq=freq, pres=pres)
+    diff = fixed["tokens"] != got["tokens"]
+    assert not (diff & ~got["near"]).any()
 
 
 # ---------------------------------------------------------------- layers agree, flags are honest
