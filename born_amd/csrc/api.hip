@@ -234,7 +234,7 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (st) {
         HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s", (st & 1) ? "out-of-range history id " : "",
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s", (st & 1) ? "out-of-range history or token id " : "",
                     (st & 2) ? "out-of-range draft token " : "", (st & 8) ? "invalid per-row configuration " : "",
                     (st & 4) ? "an internal inconsistency (please report)" : "");
     }
@@ -400,6 +400,47 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
     return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, nullptr, nullptr,
                        nullptr, nullptr, tokens_out, probs_out, nucleus_len_out, nucleus_ids_out, nucleus_probs_out,
                        nucleus_cap, stream);
+}
+
+int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                             const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const int32_t *tokens,
+                             float *logprobs_out, void *stream) {
+    int rc = check_logits("token_logprobs", s, logits, batch, vocab, row_stride);
+    if (rc) return rc;
+    if (!tokens || !logprobs_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: token_logprobs: null tokens or output");
+    if (history && hist_stride <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: token_logprobs: history given with hist_stride <= 0");
+    if (!history && hist_len) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: token_logprobs: hist_len given without history");
+    if (row_stride > (int64_t)0x7FFFFFFF || hist_stride > (int64_t)0x7FFFFFFF)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: token_logprobs: stride too large");
+    SampleArgs a;
+    memset(&a, 0, sizeof(a));
+    a.logits = logits;
+    a.row_stride = row_stride;
+    a.B = (int)batch;
+    a.V = (int)vocab;
+    a.history = history;
+    a.hist_len = hist_len;
+    a.hist_stride = history ? hist_stride : 0;
+    a.T = s->cfg.temperature;
+    a.rep = s->cfg.repetition_penalty;
+    a.status = s->status;
+    a.counters = s->counters;
+    a.mass_shift = mass_shift(vocab);
+    a.dcut = 80.0f;
+    a.freq = s->cfg.frequency_penalty;
+    a.pres = s->cfg.presence_penalty;
+    const bool counted = counts_history(s->cfg) && history;
+    a.hist_counts = counted ? s->hist_counts : nullptr;
+    hipStream_t st = (hipStream_t)stream;
+    if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
+    hipError_t e = launch_token_logprobs(a, tokens, logprobs_out, st);
+    if (counted) {
+        const hipError_t ce = launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st);
+        if (e == hipSuccess) e = ce;
+    }
+    if (e != hipSuccess) return hip_fail(e, "token_logprobs: kernel launch");
+    return BORN_ROCM_OK;
 }
 
 int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,

@@ -115,6 +115,8 @@ hipError_t launch_argmax(const float *logits, int B, int V, long long stride, in
                          int *part_idx, hipStream_t st);
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
                           hipStream_t st);
+// out[row] = log_softmax(z of the row)[tokens[row]] (penalties and temperature applied, no truncation)
+hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 // counts[row * V + id] += 1 for every valid id of the row's history (clear: = 0 instead, which restores an all-zero table)
 hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,

@@ -48,10 +48,11 @@ __device__ __forceinline__ int nuc_bin(const NucRow &r, float d) {
     return d < r.range ? min((int)(d * r.sbin), NUC_BINS - 1) : NUC_BINS - 1;   // monotone in d; NaN and inf -> last bin
 }
 
-// Visits every element of the row as f(id, penalised logit); aligned rows in stages of NUC_U float4 per thread,
-// the next stage's loads in flight while this one is visited.
-template <class F>
-__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
+// Visits every element of the row with its penalised logit: aligned rows four at a time as f4(id of the first, y[4]),
+// in stages of NUC_U float4 per thread, the next stage's loads in flight while this one is visited; what is left
+// over (and every element of an unaligned row) one at a time as f1(id, y).
+template <class F4, class F1>
+__device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
         float y[4] = {q[0], q[1], q[2], q[3]};
@@ -63,8 +64,12 @@ __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f)
                     if ((bits >> t) & 1u) y[t] = penalise_seen(y[t], r.rep, r.counts, j + t, r.freq, r.pres);
             }
         }
-#pragma unroll
-        for (int t = 0; t < 4; t++) f(j + t, y[t]);
+        f4(j, y);
+    };
+    auto visit1 = [&](int j) {
+        float y = r.x[j];
+        if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
+        f1(j, y);
     };
     if (r.vec) {
         const int n4 = r.V >> 2;
@@ -89,18 +94,18 @@ __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f)
             const nuc_f32x4 q = x4[i];
             visit4(q, i << 2);
         }
-        for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) {
-            float y = r.x[j];
-            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
-            f(j, y);
-        }
+        for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) visit1(j);
     } else {
-        for (int j = tid; j < r.V; j += NUC_BLOCK) {
-            float y = r.x[j];
-            if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
-            f(j, y);
-        }
+        for (int j = tid; j < r.V; j += NUC_BLOCK) visit1(j);
     }
+}
+// Visits every element of the row as f(id, penalised logit).
+template <class F>
+__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
+    nuc_foreach4(r, bm, [&](int j, const float (&y)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) f(j + t, y[t]);
+    }, f);
 }
 
 // smallest bin whose inclusive cumulative mass reaches target
@@ -445,6 +450,117 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs 
     nucleus_row_body(a, T, p, rep);
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Log-probability of one given token per row under the softmax of the row's penalised, temperature-scaled
+// logits (no truncation): z[token] - logsumexp(z).  With temperature 1 and no history it is minus the per-row
+// loss term of the reference's CrossEntropyLoss.Forward (internal/nn/cross_entropy.go:37-90).
+//
+// One workgroup per row, ONE sweep of the row: every thread keeps a running maximum m_t and the sum of
+// exp(z - m_t) over its elements, rescaled when a group of four raises the maximum (a handful of times per
+// thread); the workgroup then combines the 1024 pairs.  Exponentials are the hardware's (relative error about
+// 1e-7), each group of four is summed in fp32 and accumulated in fp64, the combination is fp64 throughout: the
+// result is a floating-point quantity, specified by its tolerance against the fp64 value (1e-5 + 1e-6 |value|),
+// not bit for bit.
+// ---------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+__global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
+                                                                  float *__restrict__ out) {
+    extern __shared__ u64 nuc_dyn[];
+    __shared__ BlockScratch scr;
+    __shared__ double s_part[NUC_WAVES];
+    u32 *const bm = reinterpret_cast<u32 *>(nuc_dyn);                // history bitmap, one bit per id
+    const int tid = threadIdx.x, row = blockIdx.x;
+    const int V = a.V;
+
+    NucRow r;
+    r.x = a.logits + (long long)row * a.row_stride;
+    r.V = V;
+    r.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
+    r.T = a.T;
+    r.rep = a.rep;
+    r.scale = 0.0f;
+    r.dcut = 80.0f;
+    r.range = 0.0f;
+    r.sbin = 0.0f;
+    r.m = 0.0f;
+    r.degenerate = false;
+    r.counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
+    r.freq = a.freq;
+    r.pres = a.pres;
+
+    const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
+    const int *h = a.history + (long long)row * a.hist_stride;
+    r.penal = (a.rep != 1.0f || r.counts) && hlen > 0;
+    if (r.penal) {
+        for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
+        __syncthreads();
+    }
+    for (int i = tid; i < hlen; i += NUC_BLOCK) {
+        const int t = h[i];
+        if (t < 0 || t >= V) atomicOr(a.status, 1);
+        else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
+    }
+    __syncthreads();
+
+    // exp(z - m) with the conventions of the pipeline: a tie with the maximum is exactly 1 (also when both are -inf)
+    auto term = [](float z, float m) { return z == m ? 1.0f : __expf(z - m); };
+    float mt = -INFINITY;                                            // running maximum of this thread's z
+    double st = 0.0;                                                 // sum of exp(z - mt) over this thread's elements
+    auto raise = [&](float mnew) {                                   // mnew > mt
+        st *= (double)__expf(mt - mnew);                             // exp(-inf) = 0: nothing finite was seen so far
+        mt = mnew;
+    };
+    nuc_foreach4(r, bm,
+        [&](int, const float (&y)[4]) {
+            float z[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) z[t] = nuc_z(r, y[t]);
+            const float m4 = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
+            if (m4 > mt) raise(m4);
+            st += (double)((term(z[0], mt) + term(z[1], mt)) + (term(z[2], mt) + term(z[3], mt)));
+        },
+        [&](int, float y) {
+            const float z = nuc_z(r, y);
+            if (z > mt) raise(z);
+            st += (double)term(z, mt);
+        });
+
+    const float m = block_max_f32<NUC_BLOCK>(mt, &scr);
+    double part = mt == m ? st : st * exp((double)mt - (double)m);   // a thread without elements: st = 0
+    part = wave_sum_f64(part);
+    if (lane_id() == 0) s_part[wave_id()] = part;
+    __syncthreads();
+
+    if (tid == 0) {
+        double S = 0.0;
+#pragma unroll
+        for (int w = 0; w < NUC_WAVES; w++) S += s_part[w];
+        const int t = tokens[row];
+        if (t < 0 || t >= V) {
+            atomicOr(a.status, 1);
+            out[row] = __uint_as_float(0x7FC00000u);                 // not a token of this vocabulary
+        } else {
+            float y = r.x[t];
+            if (r.penal && ((bm[t >> 5] >> (t & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, t, r.freq, r.pres);
+            const float z = nuc_z(r, y);
+            const double d = z == m ? 0.0 : (double)m - (double)z;   // >= 0, +inf for a masked token
+            out[row] = (float)(-d - log(S));
+        }
+    }
+}
+
+size_t token_logprob_lds_bytes(int V) { return sizeof(u32) * (size_t)((V + 31) / 32) + 16; }
+
+hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st) {
+    hipLaunchKernelGGL(token_logprob_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), token_logprob_lds_bytes(a.V), st, a, tokens, out);
+    return hipGetLastError();
+}
+
 size_t nucleus_lds_bytes(int V) {
     return sizeof(u64) * (NUC_BINS + NUC_WAVES * NUC_WCAP + 2 * NUC_CAP) + sizeof(u32) * (size_t)((V + 31) / 32);
 }
@@ -460,6 +576,9 @@ hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConf
 hipError_t configure_nucleus() {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)token_logprob_lds_bytes((int)WIDE_MAX_VOCAB));
     if (e != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_rows_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));

@@ -191,6 +191,13 @@ class Sampler:
                                                  _ptr(temperatures), _ptr(topKs), _ptr(topPs), _ptr(penalties),
                                                  _ptr(tokens_out), _ptr(probs_out), stream))
 
+    def TokenLogprobs(self, logits, batch, vocab, history, histLen, tokens, logprobs_out, row_stride=None, hist_stride=0,
+                      stream=None):
+        """logprobs_out[b] = log_softmax(row b after the handle's penalties and temperature)[tokens[b]]; every
+        argument lives on the device."""
+        _check(_capi.lib().born_rocm_token_logprobs(self._h, _ptr(logits), batch, vocab, row_stride or vocab, _ptr(history),
+                                                    _ptr(histLen), hist_stride, _ptr(tokens), _ptr(logprobs_out), stream))
+
     def Verify(self, target, draft, batch, gamma, vocab, draftTokens, uAccept, uResidual, nAccepted_out,
                nextToken_out, stream=None):
         _check(_capi.lib().born_rocm_spec_verify(self._h, _ptr(target), _ptr(draft), batch, gamma, vocab,
@@ -241,6 +248,23 @@ def sample_host(sampler, logits, uniforms=None, history=None, hist_len=None, nuc
         out["nuc_ids"] = nuc[1].to_numpy(np.int32, (B, nucleus_cap))
         out["nuc_probs"] = nuc[2].to_numpy(np.float32, (B, nucleus_cap))
     return out
+
+
+def token_logprobs_host(sampler, logits, tokens, history=None, hist_len=None):
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    B, V = x.shape
+    d_h = d_hl = None
+    hs = 0
+    if history is not None:
+        h = np.ascontiguousarray(history, dtype=np.int32)
+        hs = h.shape[1]
+        d_h = DeviceBuffer.from_numpy(h)
+        if hist_len is not None:
+            d_hl = DeviceBuffer.from_numpy(np.ascontiguousarray(hist_len, dtype=np.int32))
+    d_out = DeviceBuffer(4 * B)
+    sampler.TokenLogprobs(DeviceBuffer.from_numpy(x), B, V, d_h, d_hl, DeviceBuffer.from_numpy(np.ascontiguousarray(tokens, dtype=np.int32)),
+                          d_out, hist_stride=hs)
+    return d_out.to_numpy(np.float32, (B,))
 
 
 def verify_host(sampler, target, draft, draft_tokens, u_acc, u_res, bonus=False):

@@ -138,6 +138,17 @@ int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, i
                           const float *temperature_rows, const int32_t *top_k_rows, const float *top_p_rows,
                           const float *repetition_penalty_rows, int32_t *tokens_out, float *probs_out, void *stream);
 
+/* Log-probability of one given token per row: logprobs_out[b] = log_softmax(z_b)[tokens[b]], z_b being row b after
+ * the handle's penalties and temperature (steps 1-3 of the sampling pipeline; no min-p / top-k / top-p truncation).
+ * With temperature 1 and no history this is minus the per-row term `-logProbs[target]` of CrossEntropyLoss.Forward,
+ * internal/nn/cross_entropy.go:37-90 (logSoftmax, :126-153): the mean of the negated outputs is that loss.  Also
+ * the log-probability reported next to a sampled token (pass tokens_out of born_rocm_sample and the same history).
+ *   tokens int32 [batch] on the device; a token outside [0, vocab) gives NaN and BORN_ROCM_ERR_DATA from
+ *   born_rocm_sampler_status (the reference panics "target index out of bounds"). */
+int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                             const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const int32_t *tokens,
+                             float *logprobs_out, void *stream);
+
 /* Speculative-decoding accept/reject with residual max(0, p - q) resampling.
  * No counterpart in the reference snapshot.
  *   target, draft  fp32 [batch, gamma, vocab] contiguous;  draft_tokens int32 [batch, gamma]

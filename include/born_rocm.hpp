@@ -96,6 +96,21 @@ public:
         check(born_rocm_sampler_status(h_, stream));
     }
 
+    // log_softmax(row b after the handle's penalties and temperature)[tokens[b]] for every row, copied to the host.
+    // With a default-configured handle and no history the negated mean is CrossEntropyLoss.Forward
+    // (internal/nn/cross_entropy.go:37-90).
+    std::vector<float> TokenLogprobs(const float *logits_dev, int64_t batch, int64_t vocab, const int32_t *history_dev,
+                                     int64_t hist_stride, const int32_t *hist_len_dev, const int32_t *tokens_dev,
+                                     void *stream = nullptr) {
+        DeviceBuffer out(4 * batch);
+        check(born_rocm_token_logprobs(h_, logits_dev, batch, vocab, vocab, history_dev, hist_len_dev, hist_stride, tokens_dev,
+                                       static_cast<float *>(out.ptr()), stream));
+        std::vector<float> lp(static_cast<size_t>(batch));
+        out.download(lp.data(), 4 * batch, stream);
+        check(born_rocm_sampler_status(h_, stream));
+        return lp;
+    }
+
     // Verify for a target of gamma + 1 positions per sequence ([batch, gamma + 1, vocab]): its last position is the
     // bonus distribution a fully accepted sequence draws its next token from (next_token is then never -1).
     void VerifyBonus(const float *target_dev, const float *draft_dev, int64_t batch, int64_t gamma, int64_t vocab,

@@ -148,6 +148,23 @@ BORN_EXPORT void born_oracle_log_softmax_f32(const float *in, float *out, int64_
     }
 }
 
+/* CrossEntropyLoss.Forward, internal/nn/cross_entropy.go:37-90 (the same arithmetic: CrossEntropyForward,
+ * internal/autodiff/ops/cross_entropy.go:231-300): per row -logSoftmax(x)[target], summed in fp32 in row order,
+ * divided by the batch size.  Returns -1 where the reference panics "target index out of bounds". */
+BORN_EXPORT int born_oracle_cross_entropy_f32(const float *in, int64_t B, int64_t V, const int32_t *targets, float *loss) {
+    if (!in || !targets || !loss || B <= 0 || V <= 0) return -1;
+    float *lp = (float *)malloc(sizeof(float) * (size_t)V);
+    float total = 0.0f;
+    for (int64_t b = 0; b < B; b++) {
+        if (targets[b] < 0 || targets[b] >= V) { free(lp); return -1; }
+        born_oracle_log_softmax_f32(in + b * V, lp, 1, V);
+        total += -lp[targets[b]];
+    }
+    free(lp);
+    *loss = total / (float)B;
+    return 0;
+}
+
 /* internal/nn/cross_entropy.go:163-170 — softmax as exp(logSoftmax) */
 BORN_EXPORT void born_oracle_softmax_via_log(const float *in, float *out, int64_t B, int64_t V) {
     born_oracle_log_softmax_f32(in, out, B, V);
@@ -586,6 +603,56 @@ BORN_EXPORT int64_t born_oracle_sample_ex(
         }
     }
     free(z); free(seen); free(keys); free(e); free(q);
+    return bad;
+}
+
+/*
+ * born_oracle_token_logprobs: out[b] = log_softmax(z_b)[tokens[b]], z_b = row b after the penalties, the temperature
+ * and canonicalisation (pipeline steps 1-3; no truncation).
+ *   mode 0  fp64: (z_t - m) - log(sum_j exp(z_j - m))
+ *   mode 1  fixed point: -(double)d_t - log((double)Z * 2^-S), d fp32, Z the integer sum of the masses
+ *   mode 2  the reference's logSoftmax arithmetic (internal/nn/cross_entropy.go:126-153) on z: fp32 running sum of
+ *           fp64 exps, lse = m + (float)log(sum), z_t - lse
+ * A row with no finite z counts every element as tied at the maximum (log-probability -log V).
+ * A token outside [0, V) yields NaN and is counted in the return value together with the out-of-range history ids;
+ * -1 on bad arguments.
+ */
+BORN_EXPORT int64_t born_oracle_token_logprobs(
+    const float *logits, int64_t B, int64_t V, int64_t row_stride,
+    const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
+    const int32_t *tokens, float T, float rep, float freq, float pres, int32_t mode, float *out)
+{
+    if (!logits || !tokens || !out || B <= 0 || V <= 0 || row_stride < V) return -1;
+    if (!(T > 0.0f) || !(rep > 0.0f) || !isfinite(freq) || !isfinite(pres)) return -1;
+    int S = born_oracle_mass_shift(V);
+    float *z = (float *)malloc(sizeof(float) * (size_t)V);
+    int32_t *count = (int32_t *)calloc((size_t)V, sizeof(int32_t));
+    int64_t bad = 0;
+    for (int64_t b = 0; b < B; b++) {
+        int64_t hlen = history ? (hist_len ? hist_len[b] : hist_stride) : 0;
+        bad += row_z(logits + b * row_stride, V, history ? history + b * hist_stride : NULL, hlen, T, rep, freq, pres, z, count);
+        int32_t t = tokens[b];
+        if (t < 0 || t >= V) { bad++; out[b] = NAN; continue; }
+        float m = z[0];
+        for (int64_t j = 1; j < V; j++) if (z[j] > m) m = z[j];
+        if (mode == 0) {
+            double s = 0.0;
+            for (int64_t j = 0; j < V; j++) s += (z[j] == m) ? 1.0 : exp((double)z[j] - (double)m);
+            double dt = (z[t] == m) ? 0.0 : (double)m - (double)z[t];
+            out[b] = (float)(-dt - log(s));
+        } else if (mode == 1) {
+            uint64_t Z = 0;
+            for (int64_t j = 0; j < V; j++) Z += qmass(z[j], m, S);
+            float dt = (z[t] == m) ? 0.0f : m - z[t];
+            out[b] = (float)(-(double)dt - log(ldexp((double)Z, -S)));
+        } else {
+            float s = 0.0f;
+            for (int64_t j = 0; j < V; j++) s += (z[j] == m) ? 1.0f : (float)exp((double)(z[j] - m));
+            float lse = m + (float)log((double)s);
+            out[b] = (z[t] == m && !isfinite(m)) ? -(float)log((double)s) : z[t] - lse;
+        }
+    }
+    free(z); free(count);
     return bad;
 }
 

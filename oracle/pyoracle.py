@@ -70,6 +70,11 @@ def lib():
         L.born_oracle_sample_ex.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, f32p,
                                                C.c_float, C.c_int32, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int32,
                                             i32p, f32p, u8p, i32p, C.c_int64, i32p, f32p]
+        L.born_oracle_token_logprobs.restype = C.c_int64
+        L.born_oracle_token_logprobs.argtypes = [f32p, C.c_int64, C.c_int64, C.c_int64, i32p, i32p, C.c_int64, i32p,
+                                                 C.c_float, C.c_float, C.c_float, C.c_float, C.c_int32, f32p]
+        L.born_oracle_cross_entropy_f32.restype = C.c_int
+        L.born_oracle_cross_entropy_f32.argtypes = [f32p, C.c_int64, C.c_int64, i32p, f32p]
         L.born_oracle_spec_verify.restype = C.c_int64
         L.born_oracle_spec_verify.argtypes = [f32p, f32p, C.c_int64, C.c_int64, C.c_int64, i32p, f32p, f32p,
                                               C.c_float, C.c_int32, i32p, i32p, u8p]
@@ -290,6 +295,37 @@ def sample(logits, uniforms, temperature=1.0, top_k=0, top_p=1.0, rep=1.0, histo
         out["nuc_ids"] = nid
         out["nuc_probs"] = npr
     return out
+
+
+def token_logprobs(logits, tokens, temperature=1.0, rep=1.0, history=None, hist_len=None, mode=MODE_TRUTH, freq=0.0, pres=0.0):
+    """log_softmax of each row (after penalties and temperature) at the row's given token; returns (values, bad ids)."""
+    x = _f32(logits)
+    B, V = x.shape
+    t = np.ascontiguousarray(tokens, dtype=np.int32)
+    assert t.shape == (B,)
+    h = hl = None
+    hs = 0
+    if history is not None:
+        h = np.ascontiguousarray(history, dtype=np.int32)
+        hs = h.shape[1]
+        if hist_len is not None:
+            hl = np.ascontiguousarray(hist_len, dtype=np.int32)
+    out = np.empty(B, dtype=np.float32)
+    bad = lib().born_oracle_token_logprobs(_p(x, C.c_float), B, V, V, _p(h, C.c_int32), _p(hl, C.c_int32), hs, _p(t, C.c_int32),
+                                           float(temperature), float(rep), float(freq), float(pres), int(mode), _p(out, C.c_float))
+    if bad < 0:
+        raise ValueError("born_oracle_token_logprobs: bad arguments")
+    return out, int(bad)
+
+
+def cross_entropy_ref(logits, targets):
+    """The reference's CrossEntropyLoss.Forward: mean over the batch of -logSoftmax(x)[target], fp32."""
+    x = _f32(logits)
+    t = np.ascontiguousarray(targets, dtype=np.int32)
+    loss = np.zeros(1, dtype=np.float32)
+    if lib().born_oracle_cross_entropy_f32(_p(x, C.c_float), x.shape[0], x.shape[1], _p(t, C.c_int32), _p(loss, C.c_float)) != 0:
+        raise ValueError("CrossEntropyLoss: target index out of bounds")
+    return float(loss[0])
 
 
 def spec_verify(target, draft, draft_tokens, u_acc, u_res, temperature=1.0, mode=MODE_TRUTH, bonus=None):

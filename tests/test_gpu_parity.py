@@ -447,6 +447,102 @@ def test_frequency_and_presence_penalties_are_validated(rocm):
     s.Close()
 
 
+# ---------------------------------------------------------------- token log-probabilities and cross-entropy
+# A floating-point quantity (one sweep, online log-sum-exp): within 1e-5 + 1e-6 |value| of the fp64 truth (and of the
+# oracle's integer-normaliser form, which is that close to the truth itself), and within 1e-4 * max(1, |x|max * 1e-2) + V * 2^-25 of the reference's fp32 arithmetic (whose sequential fp32 sum of V terms
+# is the less accurate side).
+
+@pytest.mark.parametrize("B,V,T,rep,H,freq,pres", [
+    (32, 128256, 0.7, 1.15, 512, 0.0, 0.0),       # C3 shape
+    (32, 128256, 1.0, 1.0, 0, 0.0, 0.0),          # plain log-softmax gather: the cross-entropy term
+    (16, 152064, 1.2, 1.05, 2048, 0.2, 0.3),      # C5 shape with every penalty
+    (9, 1001, 0.5, 0.8, 300, -0.1, 0.4),          # unaligned rows, boosting penalties
+    (5, 3, 1.0, 1.0, 0, 0.0, 0.0),
+    (5, 1, 2.0, 1.0, 0, 0.0, 0.0),
+])
+def test_token_logprobs_against_oracle(oracle, rocm, B, V, T, rep, H, freq, pres):
+    rng = np.random.default_rng(B * 31 + V)
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.5)).astype(np.float32)
+    tok = rng.integers(0, V, B).astype(np.int32)
+    tok[0] = int(np.argmax(x[0]))
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32) if H else None
+    if H:
+        tok[1:4] = hist[1:4, 0]                                            # penalised tokens among the queried ones
+    hist_len = rng.integers(H // 2, H + 1, size=B).astype(np.int32) if H else None
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, RepetitionPenalty=rep, FrequencyPenalty=freq, PresencePenalty=pres,
+                                           TopK=5, TopP=0.5, MinP=0.1),     # truncation settings do not enter
+                        max_batch=B, max_vocab=V)
+    got = rocm.token_logprobs_host(s, x, tok, hist, hist_len)
+    s.Status()
+    s.Close()
+    kw = dict(temperature=T, rep=rep, history=hist, hist_len=hist_len, freq=freq, pres=pres)
+    fx, _ = oracle.token_logprobs(x, tok, mode=oracle.MODE_FIXED, **kw)
+    tr, _ = oracle.token_logprobs(x, tok, mode=oracle.MODE_TRUTH, **kw)
+    rf, _ = oracle.token_logprobs(x, tok, mode=oracle.MODE_REF32, **kw)
+    assert np.all(np.abs(got.astype(np.float64) - tr) <= 1e-5 + 1e-6 * np.abs(tr))
+    assert np.all(np.abs(got.astype(np.float64) - fx) <= 1e-5 + 1e-6 * np.abs(fx))
+    # the reference sums the V exponentials sequentially in fp32: its own rounding, up to V * 2^-24 relative in the
+    # normaliser, is what separates it from the truth at large V
+    assert np.max(np.abs(got - rf)) <= 1e-4 * max(1.0, float(np.abs(x).max()) / T * 1e-2) + V * 2.0 ** -25
+    assert (got <= 0).all()
+
+
+def test_token_logprobs_match_the_sampler_and_special_rows(oracle, rocm):
+    rng = np.random.default_rng(5)
+    B, V, H = 24, 32000, 64
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.0)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, RepetitionPenalty=1.2, PresencePenalty=0.3), max_batch=B, max_vocab=V)
+    smp = rocm.sample_host(s, x, u, hist)                                   # no truncation: probs are the full softmax's
+    lp = rocm.token_logprobs_host(s, x, smp["tokens"], hist)
+    assert np.allclose(np.exp(lp.astype(np.float64)), smp["probs"], rtol=1e-5)
+    # nothing finite: every token ties; a masked token: -inf; a token outside the vocabulary: NaN and a data error
+    y = np.full((3, 1000), -np.inf, dtype=np.float32)
+    y[1, 2] = 0.0
+    y[2, :] = 1.0
+    lp = rocm.token_logprobs_host(s, y, np.array([3, 5, 999], np.int32))
+    s.Status()
+    assert abs(lp[0] + np.log(1000.0)) < 1e-6 and lp[1] == -np.inf and abs(lp[2] + np.log(1000.0)) < 1e-6
+    lp = rocm.token_logprobs_host(s, y, np.array([0, 2, 1000], np.int32))
+    assert lp[1] == 0.0 and np.isnan(lp[2])
+    with pytest.raises(rocm.BornRocmError):
+        s.Status()
+    s.Status()
+    with pytest.raises(rocm.SamplerPanic, match="null tokens"):
+        s.TokenLogprobs(rocm.DeviceBuffer(16), 1, 4, None, None, None, rocm.DeviceBuffer(4))
+    s.Close()
+
+
+def test_cross_entropy_loss_mirror(oracle, rocm):
+    import json
+    import os
+    from born_amd.loss import CrossEntropyLoss
+    from test_oracle_reference_kats import check_cross_entropy_case
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_kats.json")) as f:
+        kats = json.load(f)["cross_entropy"]
+    crit = CrossEntropyLoss(max_batch=64, max_vocab=50000)
+
+    def loss_of(x, t):
+        return crit.Forward(rocm.DeviceBuffer.from_numpy(x), x.shape, rocm.DeviceBuffer.from_numpy(t))
+
+    for case in kats:                                                       # what the reference's own tests assert
+        check_cross_entropy_case(case, loss_of)
+    rng = np.random.default_rng(6)
+    for (B, V) in [(64, 50000), (7, 10), (1, 32000)]:
+        x = (rng.standard_normal((B, V)) * 3.0).astype(np.float32)
+        t = rng.integers(0, V, B).astype(np.int32)
+        got = loss_of(x, t)
+        assert got.dtype == np.float32
+        assert abs(float(got) - oracle.cross_entropy_ref(x, t)) <= 1e-5 * max(1.0, abs(float(got)))
+    with pytest.raises(rocm.SamplerPanic, match="logits must be 2D"):
+        crit.Forward(rocm.DeviceBuffer(16), (4,), rocm.DeviceBuffer(16))
+    with pytest.raises(rocm.SamplerPanic, match="targets must have shape"):
+        crit.Forward(rocm.DeviceBuffer(32), (2, 4), rocm.DeviceBuffer(12))
+    assert crit.Parameters() == []
+    crit.Close()
+
+
 def test_builtin_uniform_stream_in_sample(oracle, rocm):
     rng = np.random.default_rng(9)
     B, V = 16, 6000

@@ -53,6 +53,82 @@ def test_log_softmax_kats(oracle):
             assert 0.0 <= loss <= case["max_loss"]
 
 
+def check_cross_entropy_case(case, loss_of):
+    """Asserts what the reference's test asserts; `loss_of(x, targets)` raises ValueError where the reference panics."""
+    import pytest
+    x = np.array(case["input"], dtype=np.float32)
+    t = np.array(case["targets"], dtype=np.int32)
+    if case.get("panics"):
+        with pytest.raises(ValueError, match="target index out of bounds"):
+            loss_of(x, t)
+        return
+    loss = float(loss_of(x, t))
+    if "expected" in case:
+        assert abs(loss - case["expected"]) < case["tol_abs"], case["source"]
+    if case.get("finite"):
+        assert math.isfinite(loss), case["source"]
+    if "min" in case:
+        assert loss >= case["min"], case["source"]
+    if "min_exclusive" in case:
+        assert loss > case["min_exclusive"], case["source"]
+    if "max" in case:
+        assert loss <= case["max"], case["source"]
+    if "equals_first_row_alone_within" in case:
+        assert abs(loss - float(loss_of(x[:1], t[:1]))) <= case["equals_first_row_alone_within"], case["source"]
+
+
+def test_cross_entropy_kats(oracle):
+    for case in KATS["cross_entropy"]:
+        check_cross_entropy_case(case, oracle.cross_entropy_ref)
+
+
+def test_cross_entropy_and_token_logprobs_against_what_the_mathematics_fixes(oracle):
+    from scipy.special import logsumexp
+    rng = np.random.default_rng(41)
+    B, V = 40, 777
+    x = (rng.standard_normal((B, V)) * 3.0).astype(np.float32)
+    t = rng.integers(0, V, B).astype(np.int32)
+    want = x.astype(np.float64)[np.arange(B), t] - logsumexp(x.astype(np.float64), axis=1)      # an independent routine
+    # the reference arithmetic: the gather of its own logSoftmax, bit for bit, and its mean
+    ref = oracle.log_softmax_ref(x)[np.arange(B), t]
+    lp2, bad = oracle.token_logprobs(x, t, mode=oracle.MODE_REF32)
+    assert bad == 0 and np.array_equal(lp2.view(np.uint32), ref.view(np.uint32))
+    total = np.float32(0.0)
+    for v in ref:
+        total = np.float32(total + np.float32(-v))
+    assert oracle.cross_entropy_ref(x, t) == float(np.float32(total / np.float32(B)))
+    assert abs(oracle.cross_entropy_ref(x, t) - float(-want.mean())) < 1e-5
+    # closed forms: uniform rows give -log V; a two-class row gives -log(1 + e^-gap)
+    assert abs(oracle.cross_entropy_ref(np.zeros((3, 50), np.float32), np.array([0, 7, 49], np.int32)) - math.log(50.0)) < 1e-6
+    assert abs(oracle.cross_entropy_ref(np.array([[0.5, -1.0]], np.float32), np.array([0], np.int32)) - math.log1p(math.exp(-1.5))) < 1e-6
+    # the three layers agree with the independent routine
+    for mode, tol in ((oracle.MODE_TRUTH, 2e-6), (oracle.MODE_FIXED, 2e-6), (oracle.MODE_REF32, 2e-5)):
+        lp, _ = oracle.token_logprobs(x, t, mode=mode)
+        assert np.max(np.abs(lp - want)) < tol, mode
+    # temperature and penalties: z is what the sampling pipeline ranks, so exp(logprob) of a sampled token is the
+    # probability the untruncated sampler reports for it
+    hist = ((rng.zipf(1.3, size=(B, 60)) - 1) % V).astype(np.int32)
+    u = rng.random(B, dtype=np.float32)
+    kw = dict(temperature=0.7, rep=1.2, history=hist, freq=0.3, pres=0.2)
+    for mode in (oracle.MODE_TRUTH, oracle.MODE_FIXED):
+        smp = oracle.sample(x, u, mode=mode, **kw)
+        lp, _ = oracle.token_logprobs(x, smp["tokens"], mode=mode, **kw)
+        assert np.allclose(np.exp(lp.astype(np.float64)), smp["probs"], rtol=2e-6)
+    # an explicit hand case: logits [2, 1, 0], history [0, 0]: rep 2 -> 1; minus 0.25 * 2 -> 0.5; minus 0.5 -> 0; T = 0.5 -> z = [0, 2, 0]
+    lp, _ = oracle.token_logprobs(np.array([[2.0, 1.0, 0.0]], np.float32), np.array([0], np.int32), temperature=0.5, rep=2.0,
+                                  history=np.array([[0, 0]], np.int32), freq=0.25, pres=0.5)
+    assert abs(lp[0] - (0.0 - math.log(2.0 + math.exp(2.0)))) < 1e-6
+    # special rows: nothing finite -> every token ties (-log V); a masked token -> -inf; a token outside the vocabulary -> NaN, counted
+    y = np.full((3, 8), -np.inf, dtype=np.float32)
+    y[1, 2] = 0.0
+    y[2, :] = 1.0
+    for mode in (oracle.MODE_TRUTH, oracle.MODE_FIXED, oracle.MODE_REF32):
+        lp, bad = oracle.token_logprobs(y, np.array([3, 5, 8], np.int32), mode=mode)
+        assert abs(lp[0] + math.log(8.0)) < 1e-6 and lp[1] == -np.inf and np.isnan(lp[2]) and bad == 1, mode
+        lp, _ = oracle.token_logprobs(y, np.array([0, 2, 0], np.int32), mode=mode)
+        assert lp[1] == 0.0 and abs(lp[2] + math.log(8.0)) < 1e-6
+
+
 def test_argmax_kats(oracle):
     for case in KATS["argmax"]:
         x = np.array(case["input"], dtype=np.float32)
