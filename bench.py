@@ -208,6 +208,10 @@ def main():
     for _ in range(args.warmup):
         step()
     ms = timed(args.steps)
+    # spread of the step time: groups of 10 back-to-back steps, each group timed on its own (outside the headline figure)
+    groups = sorted(timed(10) for _ in range(30))
+    spread = {"median": groups[len(groups) // 2], "p10": groups[len(groups) // 10], "p90": groups[(9 * len(groups)) // 10],
+              "sample": "30 groups of 10 steps, ms per step"}
     smp.Status(stream)
     counters = smp.Counters(stream)
     tok_host = tokens.cpu().numpy()
@@ -228,6 +232,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms,
+        "ms_per_step_spread": spread,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
