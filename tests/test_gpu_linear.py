@@ -277,11 +277,13 @@ def test_lm_head_argmax_tie_and_nan_rules(oracle, rocm, lin):
     s.Close()
 
 
-def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin):
-    # the decode step (LM head -> sampler, two launches) captured once into a HIP graph and replayed with new
-    # activations and uniforms in the same buffers; every replay is checked against the eager calls and the
-    # oracle, with eager work and synchronisations between the replays.  The HIP runtime is driven through
-    # ctypes (the library itself exports no graph calls).
+@pytest.mark.parametrize("extras", [{}, dict(MinP=0.02, FrequencyPenalty=0.3, PresencePenalty=0.2)])
+def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin, extras):
+    # the decode step (LM head -> sampler -> log-probability of the sampled token; with the frequency / presence
+    # penalties also the launches that raise and clear the table of counts) captured once into a HIP graph and
+    # replayed with new activations, uniforms and histories in the same buffers; every replay is checked against
+    # the eager calls and the oracle, with eager work and synchronisations between the replays.  The HIP runtime is
+    # driven through ctypes (the library itself exports no graph calls).
     import ctypes as C
     hip = C.CDLL("libamdhip64.so")
     def ok(rc):
@@ -294,12 +296,15 @@ def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin):
     hist = rocm.DeviceBuffer.from_numpy(hist_h)
     x, u = rocm.DeviceBuffer(B * K * 4), rocm.DeviceBuffer(B * 4)
     logits, tokens, probs = rocm.DeviceBuffer(B * V * 4), rocm.DeviceBuffer(B * 4), rocm.DeviceBuffer(B * 4)
+    logprobs = rocm.DeviceBuffer(B * 4)
     layer = lin.Linear(K, V, w, bias)
-    smp = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1), max_batch=B, max_vocab=V)
+    smp = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1, **extras), max_batch=B, max_vocab=V)
+    okw = dict(min_p=extras.get("MinP", 0.0), freq=extras.get("FrequencyPenalty", 0.0), pres=extras.get("PresencePenalty", 0.0))
 
     def step(stream):
         layer.Forward(x, (B, K), logits, stream=stream)
         smp.Sample(logits, B, V, hist, None, u, tokens, probs, hist_stride=32, stream=stream)
+        smp.TokenLogprobs(logits, B, V, hist, None, tokens, logprobs, hist_stride=32, stream=stream)
 
     def upload(buf, a):
         from born_amd import _capi
@@ -319,18 +324,24 @@ def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin):
     for it in range(4):
         xh = rng.standard_normal((B, K)).astype(np.float32)
         uh = rng.random(B, dtype=np.float32)
+        hist_h = ((rng.zipf(1.3, size=(B, 32)) - 1) % V).astype(np.int32)
         upload(x, xh)
         upload(u, uh)
+        upload(hist, hist_h)
         ok(hip.hipGraphLaunch(gexec, stream))
         ok(hip.hipStreamSynchronize(stream))
         got_tok, got_logits = tokens.to_numpy(np.int32, (B,)), logits.to_numpy(np.float32, (B, V))
+        got_lp = logprobs.to_numpy(np.float32, (B,))
         upload(tokens, np.full(B, -1, np.int32))
         step(None)                                                # the same step, eagerly, on the null stream
         ok(hip.hipDeviceSynchronize())
         assert np.array_equal(got_tok, tokens.to_numpy(np.int32, (B,))), it
         assert np.array_equal(got_logits, logits.to_numpy(np.float32, (B, V))), it
-        want = oracle.sample(got_logits, uh, 0.8, 40, 0.95, 1.1, hist_h, None, mode=oracle.MODE_FIXED)
+        assert np.array_equal(got_lp, logprobs.to_numpy(np.float32, (B,))), it
+        want = oracle.sample(got_logits, uh, 0.8, 40, 0.95, 1.1, hist_h, None, mode=oracle.MODE_FIXED, **okw)
         assert np.array_equal(got_tok, want["tokens"]), it
+        want_lp, _ = oracle.token_logprobs(got_logits, got_tok, temperature=0.8, rep=1.1, history=hist_h, freq=okw["freq"], pres=okw["pres"])
+        assert np.all(np.abs(got_lp - want_lp) <= 1e-5 + 1e-6 * np.abs(want_lp)), it
     ok(hip.hipGraphExecDestroy(gexec))
     ok(hip.hipGraphDestroy(graph))
     ok(hip.hipStreamDestroy(stream))
