@@ -263,6 +263,9 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 count += (u32)__popcll(mk);
             }
         });
+        // A lane that sat out the last visits (a ragged end of the row) has counted fewer appends than were made; lane 0
+        // takes part whenever any lane of its wave does, so its count is the wave's.
+        count = (u32)__builtin_amdgcn_readfirstlane((int)count);
         if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
         const int cw = (int)min(count, (u32)NUC_WCAP);
         for (int e0 = 0; e0 < cw; e0 += WAVE) {

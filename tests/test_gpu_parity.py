@@ -543,6 +543,17 @@ def test_cross_entropy_loss_mirror(oracle, rocm):
     crit.Close()
 
 
+@pytest.mark.parametrize("V", [8, 64, 100, 130, 4100])
+def test_three_sweep_kernel_rows_that_end_inside_a_wave(oracle, rocm, V):
+    # no top-k cut and a row whose last elements occupy only part of a wave: the lanes that sit out the ragged end
+    # must still see every entry the wave gathered (heavy ties make the gathered bins full)
+    rng = np.random.default_rng(V)
+    x = np.round(rng.standard_normal((6, V))).astype(np.float32)
+    u = rng.random(6, dtype=np.float32)
+    for p in (1.0, 0.9):
+        _check_against_oracle(oracle, rocm, x, u, T=5.0, k=0, p=p)
+
+
 def test_builtin_uniform_stream_in_sample(oracle, rocm):
     rng = np.random.default_rng(9)
     B, V = 16, 6000

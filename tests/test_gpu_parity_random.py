@@ -1,0 +1,126 @@
+"""Randomised parity sweep: seeded configurations drawn across the whole parameter space of the sampler (shapes,
+temperature, top-k, top-p, min-p, the three penalties, history lengths, special values in the logits, both kernel
+selections), each checked bit for bit against the fixed-point oracle and, where the truth layer does not flag the
+row, against the fp64 truth.  Complements the hand-picked cases of test_gpu_parity.py."""
+import numpy as np
+import pytest
+
+from test_gpu_parity import _check_against_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rocm():
+    from born_amd import sampler as S
+    assert S.DeviceCount() >= 1, "no HIP device visible"
+    return S
+
+
+def _draw_case(rng):
+    V = int(rng.choice([1, 2, 3, 7, 64, 65, 130, 257, 1000, 1001, 4095, 4096, 4100, 8193, 16388, 20000, 32000, 50257, 100003]))
+    B = int(rng.integers(1, 9))
+    T = float(rng.choice([0.25, 0.5, 0.7, 1.0, 1.0, 1.3, 2.0, 5.0]))
+    k = int(rng.choice([0, 0, 1, 2, 5, 40, 50, 64, 65, 100, 1000, V, V + 3]))
+    p = float(rng.choice([1.0, 1.0, 0.99, 0.95, 0.9, 0.5, 0.1, 0.01]))
+    rep = float(rng.choice([1.0, 1.0, 1.1, 1.5, 3.0, 0.8]))
+    min_p = float(rng.choice([0.0, 0.0, 0.0, 0.01, 0.05, 0.3, 0.9]))
+    freq = float(rng.choice([0.0, 0.0, 0.0, 0.1, 0.7, -0.2]))
+    pres = float(rng.choice([0.0, 0.0, 0.0, 0.2, 1.5, -0.3]))
+    H = int(rng.choice([0, 0, 1, 5, 64, 500, 1024, 1025, 3000]))
+    scale = float(rng.choice([0.1, 1.0, 2.0, 6.0]))
+    special = str(rng.choice(["none", "none", "none", "mask", "ties", "nan_inf", "few_finite", "flat"]))
+    return dict(B=B, V=V, T=T, k=k, p=p, rep=rep, min_p=min_p, freq=freq, pres=pres, H=H, scale=scale, special=special)
+
+
+def _inputs(rng, c):
+    B, V = c["B"], c["V"]
+    x = (rng.standard_normal((B, V)) * c["scale"]).astype(np.float32)
+    sp = c["special"]
+    if sp == "mask":                                   # most of the vocabulary masked out
+        m = rng.random((B, V)) < 0.9
+        x[m] = -np.inf
+    elif sp == "ties":                                 # few distinct values: heavy ties everywhere
+        x = np.round(x).astype(np.float32)
+    elif sp == "nan_inf":
+        x[rng.random((B, V)) < 0.01] = np.nan
+        x[rng.random((B, V)) < 0.002] = np.inf
+        x[rng.random((B, V)) < 0.01] = -np.inf
+    elif sp == "few_finite":                           # fewer finite logits than a typical top_k
+        keep = rng.random((B, V)) < min(1.0, 12.0 / V)
+        x[~keep] = -np.inf
+    elif sp == "flat":
+        x[:] = np.float32(0.5)
+    u = rng.random(B, dtype=np.float32)
+    if rng.random() < 0.2:
+        u[0] = 0.0
+    hist = hist_len = None
+    if c["H"]:
+        hist = ((rng.zipf(1.3, size=(B, c["H"])) - 1) % V).astype(np.int32)
+        if rng.random() < 0.5:
+            hist_len = rng.integers(0, c["H"] + 1, size=B).astype(np.int32)
+    return x, u, hist, hist_len
+
+
+@pytest.mark.parametrize("chunk", range(32))
+def test_random_configurations_against_oracle(oracle, rocm, chunk):
+    rng = np.random.default_rng(90210 + chunk)
+    for i in range(12):
+        c = _draw_case(rng)
+        x, u, hist, hist_len = _inputs(rng, c)
+        nuc = min(64, c["k"]) if 1 <= c["k"] <= 64 and c["k"] < c["V"] else 0
+        for path in (0, 1):
+            try:
+                _check_against_oracle(oracle, rocm, x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, nuc=nuc, path=path,
+                                      min_p=c["min_p"], freq=c["freq"], pres=c["pres"])
+            except Exception as e:                    # name the configuration, whatever failed
+                raise AssertionError(f"chunk {chunk} case {i} path {path}: {c}: {type(e).__name__}: {e}") from None
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_random_token_logprobs_against_oracle(oracle, rocm, chunk):
+    rng = np.random.default_rng(4711 + chunk)
+    for i in range(10):
+        c = _draw_case(rng)
+        x, _, hist, hist_len = _inputs(rng, c)
+        B, V = x.shape
+        tok = rng.integers(0, V, B).astype(np.int32)
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=c["T"], RepetitionPenalty=c["rep"], FrequencyPenalty=c["freq"],
+                                               PresencePenalty=c["pres"]), max_batch=B, max_vocab=V)
+        got = rocm.token_logprobs_host(s, x, tok, hist, hist_len)
+        s.Status()
+        s.Close()
+        want, _ = oracle.token_logprobs(x, tok, temperature=c["T"], rep=c["rep"], history=hist, hist_len=hist_len, freq=c["freq"],
+                                        pres=c["pres"], mode=oracle.MODE_TRUTH)
+        fin = np.isfinite(want)
+        assert np.array_equal(got[~fin], want[~fin]), (chunk, i, c)                      # -inf for a masked token
+        assert np.all(np.abs(got[fin].astype(np.float64) - want[fin]) <= 1e-5 + 1e-6 * np.abs(want[fin])), (chunk, i, c)
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_random_spec_verify_against_oracle(oracle, rocm, chunk):
+    rng = np.random.default_rng(1234 + chunk)
+    for i in range(6):
+        B, G = int(rng.integers(1, 7)), int(rng.integers(1, 7))
+        V = int(rng.choice([3, 64, 130, 1001, 4096, 8193, 32000, 40004]))
+        T = float(rng.choice([0.5, 1.0, 1.0, 1.7]))
+        bonus = bool(rng.random() < 0.5)
+        t = (rng.standard_normal((B, G + 1, V)) * rng.choice([0.5, 2.0])).astype(np.float32)
+        dr = (t[:, :G] + rng.choice([0.0, 0.3, 1.0]) * rng.standard_normal((B, G, V))).astype(np.float32)
+        if rng.random() < 0.3:
+            t[rng.random(t.shape) < 0.5] = -np.inf                                       # masked targets
+            t[:, :, 0] = 0.0
+        d = rng.integers(0, V, size=(B, G)).astype(np.int32)
+        ua, ur = rng.random((B, G), dtype=np.float32), rng.random(B, dtype=np.float32)
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T), max_batch=B, max_vocab=V)
+        if bonus:
+            got = rocm.verify_host(s, t, dr, d, ua, ur, bonus=True)
+            fx = oracle.spec_verify(np.ascontiguousarray(t[:, :G]), dr, d, ua, ur, temperature=T, mode=oracle.MODE_FIXED,
+                                    bonus=np.ascontiguousarray(t[:, G]))
+        else:
+            got = rocm.verify_host(s, np.ascontiguousarray(t[:, :G]), dr, d, ua, ur)
+            fx = oracle.spec_verify(np.ascontiguousarray(t[:, :G]), dr, d, ua, ur, temperature=T, mode=oracle.MODE_FIXED)
+        s.Status()
+        s.Close()
+        assert np.array_equal(got["n_accepted"], fx["n_accepted"]), (chunk, i, B, G, V, T, bonus)
+        assert np.array_equal(got["next_token"], fx["next_token"]), (chunk, i, B, G, V, T, bonus)
