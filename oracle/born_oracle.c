@@ -12,6 +12,10 @@
  *   born_oracle_softmax_via_log  internal/nn/cross_entropy.go:163-170
  *   born_oracle_argmax           internal/nn/cross_entropy.go:241-251
  *   born_oracle_exp_f32          internal/autodiff/ops/log.go:159-185
+ *   born_oracle_cross_entropy_f32  internal/nn/cross_entropy.go:37-90 (the same arithmetic:
+ *                                internal/autodiff/ops/cross_entropy.go:231-300)
+ *   born_oracle_token_logprobs   mode 2: internal/nn/cross_entropy.go:126-153 applied to the penalised,
+ *                                temperature-scaled row; modes 0 and 1: its fp64 / fixed-point forms
  *   born_oracle_matmul_f32       internal/backend/cpu/matmul.go:55-71
  *   born_oracle_linear_f32       internal/nn/linear.go:78-107
  *   born_oracle_binary_f32       internal/backend/cpu/backend.go:32-134, ops_float32.go:61-112,
@@ -25,8 +29,8 @@
  * reference's tests hold).
  *
  * What the reference does NOT contain (its snapshot predates any sampler):
- * repetition penalty, temperature, top-k, top-p, the inverse-CDF draw and the
- * speculative accept/reject step.  Their semantics are the ones frozen in
+ * repetition / frequency / presence penalties, temperature, min-p, top-k, top-p,
+ * the inverse-CDF draw and the speculative accept/reject step.  Their semantics are the ones frozen in
  * docs/SAMPLING_SPEC.md; parity with "Born's CPU sampler" for those stages is
  * therefore parity with that specification ("parity unpinned" with respect to
  * any upstream implementation).  Each of those stages is pinned in
