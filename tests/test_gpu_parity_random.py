@@ -124,3 +124,47 @@ def test_random_spec_verify_against_oracle(oracle, rocm, chunk):
         s.Close()
         assert np.array_equal(got["n_accepted"], fx["n_accepted"]), (chunk, i, B, G, V, T, bonus)
         assert np.array_equal(got["next_token"], fx["next_token"]), (chunk, i, B, G, V, T, bonus)
+
+
+@pytest.mark.parametrize("chunk", range(8))
+def test_random_row_layouts_against_oracle(oracle, rocm, chunk):
+    # rows with a pitch larger than the vocabulary and a first row that is not 16-byte aligned (the scalar code
+    # paths); what lies between the rows is NaN / +inf, so a read outside a row would show
+    rng = np.random.default_rng(777 + chunk)
+    for i in range(10):
+        c = _draw_case(rng)
+        x, u, hist, hist_len = _inputs(rng, c)
+        B, V = x.shape
+        pad, off = int(rng.choice([0, 1, 3, 4, 5, 64])), int(rng.choice([0, 1, 2, 3, 4]))
+        stride = V + pad
+        host = np.full(off + B * stride + 8, np.nan, dtype=np.float32)
+        host[1::2] = np.inf
+        for b in range(B):
+            host[off + b * stride: off + b * stride + V] = x[b]
+        d_x = rocm.DeviceBuffer.from_numpy(host)
+        d_u = rocm.DeviceBuffer.from_numpy(u)
+        d_h = rocm.DeviceBuffer.from_numpy(hist) if hist is not None else None
+        d_hl = rocm.DeviceBuffer.from_numpy(hist_len) if hist_len is not None else None
+        tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
+        fx = oracle.sample(x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, mode=oracle.MODE_FIXED, min_p=c["min_p"],
+                           freq=c["freq"], pres=c["pres"])
+        for path in (0, 1):
+            s = rocm.NewSampler(rocm.SamplerConfig(Temperature=c["T"], TopK=c["k"], TopP=c["p"], RepetitionPenalty=c["rep"], MinP=c["min_p"],
+                                                   FrequencyPenalty=c["freq"], PresencePenalty=c["pres"]), max_batch=B, max_vocab=V)
+            s.SetPath(path)
+            s.Sample(d_x.ptr + 4 * off, B, V, d_h, d_hl, d_u, tok, pr, row_stride=stride, hist_stride=0 if hist is None else hist.shape[1])
+            s.Status()
+            got_t, got_p = tok.to_numpy(np.int32, (B,)), pr.to_numpy(np.float32, (B,))
+            assert np.array_equal(got_t, fx["tokens"]), (chunk, i, path, pad, off, c)
+            assert np.array_equal(got_p.view(np.uint32), fx["probs"].view(np.uint32)), (chunk, i, path, pad, off, c)
+            # the log-probability of the sampled token reads the same layout
+            lp = rocm.DeviceBuffer(4 * B)
+            s.TokenLogprobs(d_x.ptr + 4 * off, B, V, d_h, d_hl, tok, lp, row_stride=stride, hist_stride=0 if hist is None else hist.shape[1])
+            s.Status()
+            want, _ = oracle.token_logprobs(x, got_t, temperature=c["T"], rep=c["rep"], history=hist, hist_len=hist_len, freq=c["freq"],
+                                            pres=c["pres"], mode=oracle.MODE_TRUTH)
+            got_lp = lp.to_numpy(np.float32, (B,))
+            fin = np.isfinite(want)
+            assert np.array_equal(got_lp[~fin], want[~fin]) and \
+                np.all(np.abs(got_lp[fin].astype(np.float64) - want[fin]) <= 1e-5 + 1e-6 * np.abs(want[fin])), (chunk, i, path, pad, off, c)
+            s.Close()
