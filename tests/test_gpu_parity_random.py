@@ -168,3 +168,29 @@ def test_random_row_layouts_against_oracle(oracle, rocm, chunk):
             assert np.array_equal(got_lp[~fin], want[~fin]) and \
                 np.all(np.abs(got_lp[fin].astype(np.float64) - want[fin]) <= 1e-5 + 1e-6 * np.abs(want[fin])), (chunk, i, path, pad, off, c)
             s.Close()
+
+
+@pytest.mark.parametrize("V", [262144, 393216, 393217, 400003, 524288])
+def test_large_vocabularies_against_oracle(oracle, rocm, V):
+    # around the single-pass kernel's vocabulary limit (393216) and up to the largest supported vocabulary; the handle
+    # is created larger than the call needs
+    rng = np.random.default_rng(V)
+    B = 3
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, 700)) - 1) % V).astype(np.int32)
+    for (k, p, rep, min_p, freq, pres) in [(50, 0.9, 1.15, 0.0, 0.0, 0.0), (0, 0.95, 1.1, 0.0, 0.2, 0.1), (300, 0.9, 1.0, 0.01, 0.0, 0.0),
+                                           (64, 1.0, 0.9, 0.0, 0.0, 0.0)]:
+        got = None
+        for path in (0, 1):
+            s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=k, TopP=p, RepetitionPenalty=rep, MinP=min_p, FrequencyPenalty=freq,
+                                                   PresencePenalty=pres), max_batch=B + 2, max_vocab=524288)
+            s.SetPath(path)
+            out = rocm.sample_host(s, x, u, hist)
+            s.Status()
+            s.Close()
+            if got is None:
+                got = out
+                fx = oracle.sample(x, u, 0.8, k, p, rep, hist, mode=oracle.MODE_FIXED, min_p=min_p, freq=freq, pres=pres)
+            assert np.array_equal(out["tokens"], fx["tokens"]), (V, k, p, rep, path)
+            assert np.array_equal(out["probs"].view(np.uint32), fx["probs"].view(np.uint32)), (V, k, p, rep, path)
