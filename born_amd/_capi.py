@@ -42,6 +42,8 @@ SYMBOLS = {
     "born_rocm_sample": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "born_rocm_sample_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_token_logprobs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp]),
+    "born_rocm_history_append": (C.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp]),
+    "born_rocm_gather_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp]),
     "born_rocm_spec_verify": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_spec_verify_bonus": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_expneg": (C.c_int, [_vp, _vp, _i64, _vp]),

@@ -234,8 +234,8 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (st) {
         HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s", (st & 1) ? "out-of-range history or token id " : "",
-                    (st & 2) ? "out-of-range draft token " : "", (st & 8) ? "invalid per-row configuration " : "",
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s%s", (st & 1) ? "out-of-range history or token id " : "",
+                    (st & 2) ? "out-of-range draft token " : "", (st & 8) ? "invalid per-row configuration " : "", (st & 16) ? "a full history row " : "",
                     (st & 4) ? "an internal inconsistency (please report)" : "");
     }
     return BORN_ROCM_OK;
@@ -440,6 +440,29 @@ int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch
         if (e == hipSuccess) e = ce;
     }
     if (e != hipSuccess) return hip_fail(e, "token_logprobs: kernel launch");
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_history_append(born_sampler *s, int32_t *history, int32_t *hist_len, int64_t hist_stride, const int32_t *tokens,
+                             int64_t batch, int64_t vocab, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: history_append: null handle");
+    if (!history || !hist_len || !tokens) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: history_append: null pointer");
+    if (batch <= 0 || vocab <= 0 || hist_stride <= 0 || batch > (int64_t)0x7FFFFFFF || vocab > (int64_t)0x7FFFFFFF ||
+        hist_stride > (int64_t)0x7FFFFFFF)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: history_append: batch, vocab and hist_stride must be > 0 (and fit 31 bits)");
+    HIP_TRY(launch_history_append(history, hist_len, hist_stride, tokens, (int)batch, (int)vocab, s->status, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_gather_rows(born_sampler *s, const float *table, int64_t rows, int64_t cols, int64_t row_stride, const int32_t *ids,
+                          int64_t n, float *out, int64_t out_stride, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: gather_rows: null handle");
+    if (!table || !ids || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: gather_rows: null pointer");
+    if (rows <= 0 || cols <= 0 || n <= 0 || rows > (int64_t)0x7FFFFFFF || cols > (int64_t)0x7FFFFFFF || n > (int64_t)0x7FFFFFFF)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: gather_rows: rows, cols and n must be > 0 (and fit 31 bits)");
+    if (row_stride < cols || out_stride < cols)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: gather_rows: a row stride is smaller than the row");
+    HIP_TRY(launch_gather_rows(table, (int)rows, (int)cols, row_stride, ids, (int)n, out, out_stride, s->status, (hipStream_t)stream));
     return BORN_ROCM_OK;
 }
 

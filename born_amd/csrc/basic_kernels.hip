@@ -182,6 +182,57 @@ hipError_t launch_hist_counts(const int *history, const int *hist_len, long long
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// the two small steps a decode loop needs to stay on the device: the sampled tokens join their rows' histories,
+// and become the next input rows (an embedding lookup)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void history_append_kernel(int *history, int *hist_len, long long hist_stride,
+                                                             const int *__restrict__ tokens, int B, int V, int *status) {
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    if (b >= B) return;
+    const int t = tokens[b], n = hist_len[b];
+    if (t < 0 || t >= V) {
+        atomicOr(status, 1);
+    } else if (n < 0 || n >= hist_stride) {
+        atomicOr(status, 16);
+    } else {
+        history[(long long)b * hist_stride + n] = t;
+        hist_len[b] = n + 1;
+    }
+}
+hipError_t launch_history_append(int *history, int *hist_len, long long hist_stride, const int *tokens, int B, int V, int *status,
+                                 hipStream_t st) {
+    hipLaunchKernelGGL(history_append_kernel, dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st, history, hist_len, hist_stride, tokens,
+                       B, V, status);
+    return hipGetLastError();
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ table, int rows, int cols, long long ld,
+                                                          const int *__restrict__ ids, float *__restrict__ out, long long ldo,
+                                                          int *status) {
+    const int i = blockIdx.x;
+    const int id = ids[i];
+    const bool ok = id >= 0 && id < rows;
+    if (!ok && threadIdx.x == 0) atomicOr(status, 1);
+    const float *src = table + (long long)(ok ? id : 0) * ld;
+    float *dst = out + (long long)i * ldo;
+    if (VEC) {
+        const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int j = threadIdx.x; j < (cols >> 2); j += 256)
+            reinterpret_cast<float4 *>(dst)[j] = ok ? reinterpret_cast<const float4 *>(src)[j] : zero;
+    } else {
+        for (int j = threadIdx.x; j < cols; j += 256) dst[j] = ok ? src[j] : 0.0f;
+    }
+}
+hipError_t launch_gather_rows(const float *table, int rows, int cols, long long ld, const int *ids, int n, float *out, long long ldo,
+                              int *status, hipStream_t st) {
+    const bool vec = (cols & 3) == 0 && (ld & 3) == 0 && (ldo & 3) == 0 && ((((uintptr_t)table) | ((uintptr_t)out)) & 15) == 0;
+    if (vec) hipLaunchKernelGGL(gather_rows_kernel<true>, dim3((unsigned)n), dim3(256), 0, st, table, rows, cols, ld, ids, out, ldo, status);
+    else hipLaunchKernelGGL(gather_rows_kernel<false>, dim3((unsigned)n), dim3(256), 0, st, table, rows, cols, ld, ids, out, ldo, status);
+    return hipGetLastError();
+}
+
 __global__ void uniforms_kernel(u64 seed, u64 step, float *u, long long n) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) u[i] = uniform_of(seed, step, (u64)i);

@@ -117,6 +117,12 @@ hipError_t launch_softmax(const float *logits, int B, int V, long long stride, f
                           hipStream_t st);
 // out[row] = log_softmax(z of the row)[tokens[row]] (penalties and temperature applied, no truncation)
 hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st);
+// history[b][hist_len[b]] = tokens[b]; hist_len[b] += 1 (a full row: unchanged, status bit 4; a token outside [0, V): bit 0)
+hipError_t launch_history_append(int *history, int *hist_len, long long hist_stride, const int *tokens, int B, int V, int *status,
+                                 hipStream_t st);
+// out[i][:] = table[ids[i]][:] (an id outside [0, rows): a row of zeros, status bit 0)
+hipError_t launch_gather_rows(const float *table, int rows, int cols, long long ld, const int *ids, int n, float *out, long long ldo,
+                              int *status, hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
 // counts[row * V + id] += 1 for every valid id of the row's history (clear: = 0 instead, which restores an all-zero table)
 hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,

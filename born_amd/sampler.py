@@ -198,6 +198,15 @@ class Sampler:
         _check(_capi.lib().born_rocm_token_logprobs(self._h, _ptr(logits), batch, vocab, row_stride or vocab, _ptr(history),
                                                     _ptr(histLen), hist_stride, _ptr(tokens), _ptr(logprobs_out), stream))
 
+    def HistoryAppend(self, history, histLen, hist_stride, tokens, batch, vocab, stream=None):
+        """history[b][histLen[b]] = tokens[b]; histLen[b] += 1, on the device."""
+        _check(_capi.lib().born_rocm_history_append(self._h, _ptr(history), _ptr(histLen), hist_stride, _ptr(tokens), batch, vocab, stream))
+
+    def GatherRows(self, table, rows, cols, ids, n, out, row_stride=None, out_stride=None, stream=None):
+        """out[i][:] = table[ids[i]][:] (the embedding lookup), on the device."""
+        _check(_capi.lib().born_rocm_gather_rows(self._h, _ptr(table), rows, cols, row_stride or cols, _ptr(ids), n, _ptr(out),
+                                                 out_stride or cols, stream))
+
     def Verify(self, target, draft, batch, gamma, vocab, draftTokens, uAccept, uResidual, nAccepted_out,
                nextToken_out, stream=None):
         _check(_capi.lib().born_rocm_spec_verify(self._h, _ptr(target), _ptr(draft), batch, gamma, vocab,

@@ -149,6 +149,20 @@ int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch
                              const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const int32_t *tokens,
                              float *logprobs_out, void *stream);
 
+/* The two small steps that keep a decode loop on the device (no counterpart in the reference snapshot, which has
+ * neither a generation loop nor an embedding layer):
+ *   born_rocm_history_append  history[b][hist_len[b]] = tokens[b]; hist_len[b] += 1 — the sampled tokens join the
+ *       histories the next born_rocm_sample call penalises.  A full row (hist_len[b] == hist_stride) is left as it
+ *       is, a token outside [0, vocab) is not appended; both give BORN_ROCM_ERR_DATA from born_rocm_sampler_status.
+ *   born_rocm_gather_rows     out[i][:] = table[ids[i]][:] (fp32 rows, strides in elements) — the embedding lookup
+ *       that turns the sampled tokens into the next step's input rows.  An id outside [0, rows) yields a row of
+ *       zeros and BORN_ROCM_ERR_DATA from born_rocm_sampler_status.
+ * The handle only lends its status word. */
+int born_rocm_history_append(born_sampler *s, int32_t *history, int32_t *hist_len, int64_t hist_stride, const int32_t *tokens,
+                             int64_t batch, int64_t vocab, void *stream);
+int born_rocm_gather_rows(born_sampler *s, const float *table, int64_t rows, int64_t cols, int64_t row_stride, const int32_t *ids,
+                          int64_t n, float *out, int64_t out_stride, void *stream);
+
 /* Speculative-decoding accept/reject with residual max(0, p - q) resampling.
  * No counterpart in the reference snapshot.
  *   target, draft  fp32 [batch, gamma, vocab] contiguous;  draft_tokens int32 [batch, gamma]
