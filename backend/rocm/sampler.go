@@ -219,7 +219,8 @@ func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab in
 // fp32 for Temperatures / TopPs / Penalties, int32 for TopKs; a zero DeviceBuffer means "the sampler's value for
 // every row".  Values mean what the SamplerConfig fields mean after defaults.
 type RowConfigs struct {
-	Temperatures, TopKs, TopPs, Penalties DeviceBuffer
+	Temperatures, TopKs, TopPs, Penalties             DeviceBuffer
+	MinPs, FrequencyPenalties, PresencePenalties DeviceBuffer
 }
 
 // SampleRows is Sample with a configuration per row.  A row with invalid values yields token 0 and an error
@@ -231,10 +232,19 @@ func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history Devi
 		return nil, err
 	}
 	defer out.Free()
+	// the struct holds device addresses only (C memory as far as cgo's pointer rules are concerned)
+	rc := C.born_sampler_row_configs{
+		temperature:        (*C.float)(rows.Temperatures.ptr),
+		top_k:              (*C.int32_t)(rows.TopKs.ptr),
+		top_p:              (*C.float)(rows.TopPs.ptr),
+		repetition_penalty: (*C.float)(rows.Penalties.ptr),
+		min_p:              (*C.float)(rows.MinPs.ptr),
+		frequency_penalty:  (*C.float)(rows.FrequencyPenalties.ptr),
+		presence_penalty:   (*C.float)(rows.PresencePenalties.ptr),
+	}
 	if err = check(C.born_rocm_sample_rows(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
 		C.int64_t(vocab), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
-		(*C.float)(uniforms.ptr), (*C.float)(rows.Temperatures.ptr), (*C.int32_t)(rows.TopKs.ptr),
-		(*C.float)(rows.TopPs.ptr), (*C.float)(rows.Penalties.ptr), (*C.int32_t)(out.ptr), nil, nil)); err != nil {
+		(*C.float)(uniforms.ptr), &rc, (*C.int32_t)(out.ptr), nil, nil)); err != nil {
 		return nil, err
 	}
 	tokens := make([]int32, batch)

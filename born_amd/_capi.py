@@ -18,6 +18,11 @@ class SamplerConfigC(C.Structure):
                 ("frequency_penalty", C.c_float), ("presence_penalty", C.c_float)]
 
 
+class RowConfigsC(C.Structure):
+    _fields_ = [("temperature", C.c_void_p), ("top_k", C.c_void_p), ("top_p", C.c_void_p), ("repetition_penalty", C.c_void_p),
+                ("min_p", C.c_void_p), ("frequency_penalty", C.c_void_p), ("presence_penalty", C.c_void_p)]
+
+
 # every symbol include/born_rocm.h declares: name -> (restype, argtypes)
 _vp, _i64, _i32p, _f32p = C.c_void_p, C.c_int64, C.POINTER(C.c_int32), C.POINTER(C.c_float)
 SYMBOLS = {
@@ -40,7 +45,7 @@ SYMBOLS = {
     "born_rocm_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "born_rocm_log_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "born_rocm_sample": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
-    "born_rocm_sample_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "born_rocm_sample_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_token_logprobs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp]),
     "born_rocm_history_append": (C.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp]),
     "born_rocm_gather_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp]),

@@ -307,8 +307,7 @@ int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, i
 
 static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                        const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
-                       const float *row_T, const int32_t *row_k, const float *row_p, const float *row_rep,
-                       int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
+                       const born_sampler_row_configs *per_row, int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
                        float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
     int rc = check_logits("sample", s, logits, batch, vocab, row_stride);
     if (rc) return rc;
@@ -349,12 +348,22 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     a.dcut = mass_cutoff(s->cfg);
     a.freq = s->cfg.frequency_penalty;
     a.pres = s->cfg.presence_penalty;
-    const bool counted = counts_history(s->cfg) && history && hist_stride > 0;
+    const bool any_row = per_row && (per_row->temperature || per_row->top_k || per_row->top_p || per_row->repetition_penalty ||
+                                     per_row->min_p || per_row->frequency_penalty || per_row->presence_penalty);
+    const bool counted = (counts_history(s->cfg) || (per_row && (per_row->frequency_penalty || per_row->presence_penalty))) &&
+                         history && hist_stride > 0;
+    if (counted && !s->hist_counts) {
+        // per-row penalties on a handle configured without any: the table of occurrence counts is allocated now
+        const size_t bytes = (size_t)s->max_batch * (size_t)s->max_vocab * sizeof(unsigned);
+        HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+        HIP_TRY(hipMalloc((void **)&s->hist_counts, bytes));
+        HIP_TRY(hipMemset(s->hist_counts, 0, bytes));
+    }
     a.hist_counts = counted ? s->hist_counts : nullptr;
 
     hipStream_t st = (hipStream_t)stream;
     if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
-    // The single-pass kernel relies on the penalties never raising a logit.
+    // The single-pass kernel relies on the penalties never raising a logit (per-row values are judged on the device).
     const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
     // a failed launch must not leave the table of counts raised: remember the error, clear, then report
     hipError_t launch_err = hipSuccess;
@@ -362,13 +371,16 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     do {                                                              \
         if (launch_err == hipSuccess) launch_err = (expr);            \
     } while (0)
-    if (row_T || row_k || row_p || row_rep) {
+    if (any_row) {
         // every kernel over the whole batch: each workgroup takes its row only if the row's configuration is its own
         RowConfigs rows;
-        rows.T = row_T;
-        rows.k = row_k;
-        rows.p = row_p;
-        rows.rep = row_rep;
+        rows.T = per_row->temperature;
+        rows.k = per_row->top_k;
+        rows.p = per_row->top_p;
+        rows.rep = per_row->repetition_penalty;
+        rows.min_p = per_row->min_p;
+        rows.freq = per_row->frequency_penalty;
+        rows.pres = per_row->presence_penalty;
         rows.path = s->path;
         if (s->path != 1 && vocab <= ROW_MAX_VOCAB) TRY_LAUNCH(launch_topk_row(a, st, &rows));
         if (s->path != 1) TRY_LAUNCH(launch_nucleus_row(a, st, &rows));
@@ -397,9 +409,8 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
                      const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
                      int32_t *tokens_out, float *probs_out, int32_t *nucleus_len_out, int32_t *nucleus_ids_out,
                      float *nucleus_probs_out, int64_t nucleus_cap, void *stream) {
-    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, nullptr, nullptr,
-                       nullptr, nullptr, tokens_out, probs_out, nucleus_len_out, nucleus_ids_out, nucleus_probs_out,
-                       nucleus_cap, stream);
+    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, nullptr, tokens_out,
+                       probs_out, nucleus_len_out, nucleus_ids_out, nucleus_probs_out, nucleus_cap, stream);
 }
 
 int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
@@ -468,11 +479,9 @@ int born_rocm_gather_rows(born_sampler *s, const float *table, int64_t rows, int
 
 int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
-                          const float *temperature_rows, const int32_t *top_k_rows, const float *top_p_rows,
-                          const float *repetition_penalty_rows, int32_t *tokens_out, float *probs_out, void *stream) {
-    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, temperature_rows,
-                       top_k_rows, top_p_rows, repetition_penalty_rows, tokens_out, probs_out, nullptr, nullptr, nullptr, 0,
-                       stream);
+                          const born_sampler_row_configs *rows, int32_t *tokens_out, float *probs_out, void *stream) {
+    return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, rows, tokens_out, probs_out,
+                       nullptr, nullptr, nullptr, 0, stream);
 }
 
 static int spec_verify_impl(born_sampler *s, const float *target, int64_t target_seq_stride, const float *draft,

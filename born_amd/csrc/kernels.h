@@ -59,6 +59,7 @@ struct SampleArgs {
 struct RowConfigs {
     const float *T, *p, *rep;
     const int *k;
+    const float *min_p, *freq, *pres;
     int path;                     // the handle's kernel selection (1 = always the general kernel)
 };
 

@@ -137,7 +137,11 @@ __device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, fl
 }
 
 // cfg_T, cfg_p, cfg_rep: the row's temperature, top_p and repetition penalty (the handle's, or the row's own).
-__device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep) {
+// COUNTED: a frequency or presence penalty is on (the table of occurrence counts is read for ids the history holds);
+// its own instance, so that the usual one carries none of it.
+template <bool COUNTED>
+__device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep,
+                                                 const float cfg_dcut, const float cfg_freq, const float cfg_pres) {
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over;
@@ -159,17 +163,17 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     r.T = cfg_T;
     r.rep = cfg_rep;
     r.scale = mass_scale(a.mass_shift);
-    r.dcut = a.dcut;
+    r.dcut = cfg_dcut;
     const float u = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
 
     BORN_STAMP(a, row, 0);
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
-    r.counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
-    r.freq = a.freq;
-    r.pres = a.pres;
-    r.penal = (cfg_rep != 1.0f || r.counts) && hlen > 0;
+    r.counts = COUNTED ? a.hist_counts + (long long)row * V : nullptr;
+    r.freq = COUNTED ? cfg_freq : 0.0f;
+    r.pres = COUNTED ? cfg_pres : 0.0f;
+    r.penal = (cfg_rep != 1.0f || COUNTED) && hlen > 0;
     if (r.penal)
         for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
     for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;
@@ -441,16 +445,17 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     BORN_STAMP(a, row, 7);
 }
 
+template <bool COUNTED>
 __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
-    nucleus_row_body(a, a.T, a.top_p, a.rep);
+    nucleus_row_body<COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
+template <bool COUNTED>
 __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs a, RowConfigs rc) {
-    float T, p, rep;
-    int k;
+    RowValues v;
     bool invalid;
-    if (!row_config_values(a, rc, (int)blockIdx.x, ROUTE_NUCLEUS, T, k, p, rep, invalid)) return;   // workgroup-uniform, before any barrier
-    nucleus_row_body(a, T, p, rep);
+    if (!row_config_values(a, rc, (int)blockIdx.x, ROUTE_NUCLEUS, v, invalid)) return;   // workgroup-uniform, before any barrier
+    nucleus_row_body<COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -569,22 +574,29 @@ size_t nucleus_lds_bytes(int V) {
 }
 
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
-    if (rows)
-        hipLaunchKernelGGL(nucleus_row_rows_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a, *rows);
-    else
-        hipLaunchKernelGGL(nucleus_row_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), nucleus_lds_bytes(a.V), st, a);
+    const dim3 gr((unsigned)a.B), bl(NUC_BLOCK);
+    const size_t lds = nucleus_lds_bytes(a.V);
+    if (rows) {
+        if (a.hist_counts) hipLaunchKernelGGL(nucleus_row_rows_kernel<true>, gr, bl, lds, st, a, *rows);
+        else hipLaunchKernelGGL(nucleus_row_rows_kernel<false>, gr, bl, lds, st, a, *rows);
+    } else {
+        if (a.hist_counts) hipLaunchKernelGGL(nucleus_row_kernel<true>, gr, bl, lds, st, a);
+        else hipLaunchKernelGGL(nucleus_row_kernel<false>, gr, bl, lds, st, a);
+    }
     return hipGetLastError();
 }
 
 hipError_t configure_nucleus() {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)token_logprob_lds_bytes((int)WIDE_MAX_VOCAB));
-    if (e != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(nucleus_row_rows_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB));
+    const int lds = (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB);
+    const void *kernels[] = {reinterpret_cast<const void *>(nucleus_row_kernel<false>), reinterpret_cast<const void *>(nucleus_row_kernel<true>),
+                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<false>),
+                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<true>)};
+    for (const void *k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+    }
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)token_logprob_lds_bytes((int)WIDE_MAX_VOCAB));
 }
 
 }  // namespace born

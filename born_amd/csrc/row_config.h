@@ -1,5 +1,5 @@
 // Per-row sampling configurations: when the caller passes arrays of temperature / top_k / top_p /
-// repetition_penalty (one value per row, any of them optional), the three sampling kernels are all launched
+// repetition_penalty / min_p / frequency_penalty / presence_penalty (one value per row, any of them optional), the three sampling kernels are all launched
 // over the whole batch and every workgroup first decides whether its row is its own: the single-pass kernel
 // takes 1 <= top_k <= 64 with a penalty that never raises a logit, the three-sweep kernel the rows without a
 // top-k cut, the general kernel everything else — the same rule the host applies to a uniform configuration.
@@ -11,36 +11,57 @@ namespace born {
 
 enum { ROUTE_TOPK = 0, ROUTE_NUCLEUS = 1, ROUTE_GENERAL = 2 };
 
-__device__ __forceinline__ bool row_config_valid(float T, float p, float rep) {
-    return T > 0.0f && T <= 3.402823466e+38f && p > 0.0f && p <= 1.0f && rep > 0.0f && rep <= 3.402823466e+38f;
+// Everything a row may set for itself.
+struct RowValues {
+    float T, top_p, rep, dcut, freq, pres;
+    int top_k;
+};
+
+__device__ __forceinline__ bool row_config_valid(const RowValues &v, float min_p) {
+    const float big = 3.402823466e+38f;
+    return v.T > 0.0f && v.T <= big && v.top_p > 0.0f && v.top_p <= 1.0f && v.rep > 0.0f && v.rep <= big && min_p >= 0.0f &&
+           min_p < 1.0f && fabsf(v.freq) <= big && fabsf(v.pres) <= big;
 }
 
 // Row `row`'s values (workgroup-uniform).  Returns false when another kernel owns the row.  An invalid
-// configuration (temperature or penalty not positive and finite, top_p outside (0, 1]) belongs to the general
-// kernel, which reports it through the status word (bit 3) and emits token 0.
-__device__ __forceinline__ bool row_config_values(const SampleArgs &a, const RowConfigs &rc, int row, int my_route,
-                                                  float &T, int &top_k, float &top_p, float &rep, bool &invalid) {
+// configuration (temperature or repetition penalty not positive and finite, top_p outside (0, 1], min_p outside
+// [0, 1), a frequency or presence penalty that is not finite) belongs to the general kernel, which reports it
+// through the status word (bit 3) and emits token 0.
+__device__ __forceinline__ bool row_config_values(const SampleArgs &a, const RowConfigs &rc, int row, int my_route, RowValues &v,
+                                                  bool &invalid) {
     invalid = false;
-    T = a.T;
-    top_k = a.top_k;
-    top_p = a.top_p;
-    rep = a.rep;
+    v.T = a.T;
+    v.top_k = a.top_k;
+    v.top_p = a.top_p;
+    v.rep = a.rep;
+    v.dcut = a.dcut;
+    v.freq = a.freq;
+    v.pres = a.pres;
+    float min_p = 0.0f;
     // the row is the workgroup's: the values are uniform, and are kept in scalar registers
-    if (rc.T) T = uniform_f32(rc.T[row]);
-    if (rc.p) top_p = uniform_f32(rc.p[row]);
-    if (rc.rep) rep = uniform_f32(rc.rep[row]);
+    if (rc.T) v.T = uniform_f32(rc.T[row]);
+    if (rc.p) v.top_p = uniform_f32(rc.p[row]);
+    if (rc.rep) v.rep = uniform_f32(rc.rep[row]);
+    if (rc.freq) v.freq = uniform_f32(rc.freq[row]);
+    if (rc.pres) v.pres = uniform_f32(rc.pres[row]);
     if (rc.k) {
         const int k = __builtin_amdgcn_readfirstlane(rc.k[row]);
-        top_k = (k <= 0 || k >= a.V) ? 0 : k;
+        v.top_k = (k <= 0 || k >= a.V) ? 0 : k;
+    }
+    if (rc.min_p) {
+        // the bound the host computes for a uniform configuration: min(80, -ln(min_p)), fp64 logarithm rounded once
+        min_p = uniform_f32(rc.min_p[row]);
+        v.dcut = 80.0f;
+        if (min_p > 0.0f && min_p < 1.0f) v.dcut = uniform_f32(fminf(80.0f, (float)(-log((double)min_p))));
     }
     int route;
-    if (!row_config_valid(T, top_p, rep)) {
+    if (!row_config_valid(v, min_p)) {
         invalid = true;
         route = ROUTE_GENERAL;
-    } else if (rc.path != 1 && top_k >= 1 && top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && rep < 1.0f) &&
-               !(a.hist_counts && (a.freq < 0.0f || a.pres < 0.0f))) {
+    } else if (rc.path != 1 && v.top_k >= 1 && v.top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && v.rep < 1.0f) &&
+               !(a.hist_counts && (v.freq < 0.0f || v.pres < 0.0f))) {
         route = ROUTE_TOPK;
-    } else if (rc.path != 1 && top_k == 0) {
+    } else if (rc.path != 1 && v.top_k == 0) {
         route = ROUTE_NUCLEUS;
     } else {
         route = ROUTE_GENERAL;
@@ -49,13 +70,15 @@ __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const Row
 }
 // The same, written into the kernel's own copy of the arguments.
 __device__ __forceinline__ bool row_config(SampleArgs &a, const RowConfigs &rc, int row, int my_route, bool &invalid) {
-    float T, p, rep;
-    int k;
-    const bool mine = row_config_values(a, rc, row, my_route, T, k, p, rep, invalid);
-    a.T = T;
-    a.top_k = k;
-    a.top_p = p;
-    a.rep = rep;
+    RowValues v;
+    const bool mine = row_config_values(a, rc, row, my_route, v, invalid);
+    a.T = v.T;
+    a.top_k = v.top_k;
+    a.top_p = v.top_p;
+    a.rep = v.rep;
+    a.dcut = v.dcut;
+    a.freq = v.freq;
+    a.pres = v.pres;
     return mine;
 }
 

@@ -324,6 +324,9 @@ __device__ __forceinline__ Found wide_find(const WideCtx &c, WideHeld &held, boo
 }
 
 // The general algorithm on one row (every thread of the workgroup calls it together).
+// COUNTED: a frequency or presence penalty is on (the table of occurrence counts is read for ids the history
+// holds); its own instance, so that the usual one carries none of it.
+template <bool COUNTED>
 __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds_u64 *dyn, BORN_LDS BlockScratch *scr, lds_int *s_int,
                                          lds_u64 *s_u64) {
     const int tid = threadIdx.x;
@@ -351,10 +354,10 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     BORN_STAMP(a, row, 0);
     // ---- history bitmap
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
-    c.counts = a.hist_counts ? a.hist_counts + (long long)row * a.V : nullptr;
-    c.freq = a.freq;
-    c.pres = a.pres;
-    c.has_hist = (a.rep != 1.0f || c.counts) && hlen > 0;
+    c.counts = COUNTED ? a.hist_counts + (long long)row * a.V : nullptr;
+    c.freq = COUNTED ? a.freq : 0.0f;
+    c.pres = COUNTED ? a.pres : 0.0f;
+    c.has_hist = (a.rep != 1.0f || COUNTED) && hlen > 0;
     if (c.has_hist) {
         const int words = (V + 31) >> 5;
         for (int i = tid; i < words; i += WIDE_BLOCK) bm[i] = 0;
@@ -473,15 +476,17 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
 }
 
 // One workgroup per row of the batch.
+template <bool COUNTED>
 __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a) {
     extern __shared__ u64 dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_int[8];
     __shared__ u64 s_u64[4];
-    wide_row(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
+    wide_row<COUNTED>(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own;
 // rows whose configuration is invalid end here, reported through the status word.
+template <bool COUNTED>
 __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_rows_kernel(SampleArgs a, RowConfigs rc) {
     extern __shared__ u64 dyn[];
     __shared__ BlockScratch scr;
@@ -498,23 +503,32 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_rows_kernel(SampleArgs
         }
         return;
     }
-    wide_row(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
+    wide_row<COUNTED>(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);
 }
 
 hipError_t launch(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
-    if (rows)
-        hipLaunchKernelGGL(sample_wide_rows_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a, *rows);
-    else
-        hipLaunchKernelGGL(sample_wide_kernel, dim3((unsigned)a.B), dim3(WIDE_BLOCK), wide_lds_bytes(a.V), st, a);
+    const dim3 gr((unsigned)a.B), bl(WIDE_BLOCK);
+    const size_t lds = wide_lds_bytes(a.V);
+    if (rows) {
+        if (a.hist_counts) hipLaunchKernelGGL(sample_wide_rows_kernel<true>, gr, bl, lds, st, a, *rows);
+        else hipLaunchKernelGGL(sample_wide_rows_kernel<false>, gr, bl, lds, st, a, *rows);
+    } else {
+        if (a.hist_counts) hipLaunchKernelGGL(sample_wide_kernel<true>, gr, bl, lds, st, a);
+        else hipLaunchKernelGGL(sample_wide_kernel<false>, gr, bl, lds, st, a);
+    }
     return hipGetLastError();
 }
 
 hipError_t configure() {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_wide_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)wide_lds_bytes((int)WIDE_MAX_VOCAB));
-    if (e != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(sample_wide_rows_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)wide_lds_bytes((int)WIDE_MAX_VOCAB));
+    const int lds = (int)wide_lds_bytes((int)WIDE_MAX_VOCAB);
+    const void *kernels[] = {reinterpret_cast<const void *>(sample_wide_kernel<false>), reinterpret_cast<const void *>(sample_wide_kernel<true>),
+                             reinterpret_cast<const void *>(sample_wide_rows_kernel<false>),
+                             reinterpret_cast<const void *>(sample_wide_rows_kernel<true>)};
+    for (const void *k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 }  // namespace BORN_WIDE_NS

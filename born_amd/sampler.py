@@ -183,13 +183,15 @@ class Sampler:
                                             cap, stream))
 
     def SampleRows(self, logits, batch, vocab, history, histLen, uniforms, temperatures, topKs, topPs, penalties,
-                   tokens_out, probs_out=None, row_stride=None, hist_stride=0, stream=None):
+                   tokens_out, probs_out=None, row_stride=None, hist_stride=0, stream=None, minPs=None,
+                   frequencyPenalties=None, presencePenalties=None):
         """Sample with a configuration per row: device arrays of `batch` values, each may be None (=> the
         handle's value)."""
+        rows = _capi.RowConfigsC(_ptr(temperatures), _ptr(topKs), _ptr(topPs), _ptr(penalties), _ptr(minPs),
+                                 _ptr(frequencyPenalties), _ptr(presencePenalties))
         _check(_capi.lib().born_rocm_sample_rows(self._h, _ptr(logits), batch, vocab, row_stride or vocab,
                                                  _ptr(history), _ptr(histLen), hist_stride, _ptr(uniforms),
-                                                 _ptr(temperatures), _ptr(topKs), _ptr(topPs), _ptr(penalties),
-                                                 _ptr(tokens_out), _ptr(probs_out), stream))
+                                                 C.byref(rows), _ptr(tokens_out), _ptr(probs_out), stream))
 
     def TokenLogprobs(self, logits, batch, vocab, history, histLen, tokens, logprobs_out, row_stride=None, hist_stride=0,
                       stream=None):

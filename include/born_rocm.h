@@ -126,17 +126,28 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
                      int64_t nucleus_cap, void *stream);
 
 /* The same step with a configuration per row (continuous batching: requests with different settings share a
- * batch).  temperature_rows / top_p_rows / repetition_penalty_rows fp32 [batch], top_k_rows int32 [batch], all on
- * the device, each may be NULL (=> the handle's value for every row).  Values mean what the fields of
- * born_sampler_config mean after defaults (top_k <= 0 or >= vocab: no top-k cut; top_p = 1: no top-p cut;
- * repetition_penalty = 1: none).  A row whose values are invalid (temperature or penalty not positive and finite,
- * top_p outside (0, 1]) gets token 0 and BORN_ROCM_ERR_DATA from born_rocm_sampler_status.  Every row's result
- * equals what born_rocm_sample returns for that row under a handle configured with the row's values.  No
- * counterpart in the reference snapshot. */
+ * batch).  Every member is a device array of `batch` values or NULL (=> the handle's value for every row); the
+ * values mean what the fields of born_sampler_config mean after defaults (top_k <= 0 or >= vocab: no top-k cut;
+ * top_p = 1: no top-p cut; repetition_penalty = 1, min_p = 0, frequency_penalty = 0, presence_penalty = 0: off).
+ * A row whose values are invalid (temperature or repetition penalty not positive and finite, top_p outside (0, 1],
+ * min_p outside [0, 1), a frequency or presence penalty that is not finite) gets token 0 and BORN_ROCM_ERR_DATA
+ * from born_rocm_sampler_status.  Every row's result equals what born_rocm_sample returns for that row under a
+ * handle configured with the row's values.  Per-row frequency or presence penalties use the handle's table of
+ * counters; a handle not configured with either allocates it on the first such call (which synchronises the
+ * stream, so make that call outside a graph capture).  No counterpart in the reference snapshot. */
+typedef struct born_sampler_row_configs {
+    const float   *temperature;
+    const int32_t *top_k;
+    const float   *top_p;
+    const float   *repetition_penalty;
+    const float   *min_p;
+    const float   *frequency_penalty;
+    const float   *presence_penalty;
+} born_sampler_row_configs;
+
 int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
-                          const float *temperature_rows, const int32_t *top_k_rows, const float *top_p_rows,
-                          const float *repetition_penalty_rows, int32_t *tokens_out, float *probs_out, void *stream);
+                          const born_sampler_row_configs *rows, int32_t *tokens_out, float *probs_out, void *stream);
 
 /* Log-probability of one given token per row: logprobs_out[b] = log_softmax(z_b)[tokens[b]], z_b being row b after
  * the handle's penalties and temperature (steps 1-3 of the sampling pipeline; no min-p / top-k / top-p truncation).

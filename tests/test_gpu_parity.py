@@ -654,14 +654,15 @@ def test_spec_verify_bonus_draw(oracle, rocm):
 
 # ---------------------------------------------------------------- a configuration per row
 
-def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, **handle):
+def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=None, press=None, **handle):
     B, V = x.shape
     s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=7, TopP=0.8, RepetitionPenalty=1.3, **handle), max_batch=B, max_vocab=V)
     s.SetPath(path)
     dev = lambda a, dt: None if a is None else rocm.DeviceBuffer.from_numpy(np.ascontiguousarray(a, dtype=dt))
     tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
     s.SampleRows(dev(x, np.float32), B, V, dev(hist, np.int32), None, dev(u, np.float32), dev(Ts, np.float32), dev(ks, np.int32),
-                 dev(ps, np.float32), dev(reps, np.float32), tok, pr, hist_stride=0 if hist is None else hist.shape[1])
+                 dev(ps, np.float32), dev(reps, np.float32), tok, pr, hist_stride=0 if hist is None else hist.shape[1],
+                 minPs=dev(min_ps, np.float32), frequencyPenalties=dev(freqs, np.float32), presencePenalties=dev(press, np.float32))
     return s, tok.to_numpy(np.int32, (B,)), pr.to_numpy(np.float32, (B,))
 
 
@@ -722,6 +723,55 @@ def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq
     if path == 0 and freq < 0:
         assert s.Counters()["topk_rows"] == 0                            # a penalty that raises logits: never the single-pass kernel
     s.Close()
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_per_row_min_p_and_additive_penalties(oracle, rocm, path):
+    # all seven settings per row; the handle is configured without a frequency / presence penalty, so the call itself
+    # brings the table of counts into being
+    rng = np.random.default_rng(80)
+    B, V, H = 32, 9000, 300
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    x[:, :8] += np.float32(3.0)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+    Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 300, V], B).astype(np.int32)
+    ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
+    reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
+    mps = rng.choice([0.0, 0.0, 0.01, 0.1, 0.5], B).astype(np.float32)
+    frs = rng.choice([0.0, 0.0, 0.2, 1.0, -0.3], B).astype(np.float32)
+    prs = rng.choice([0.0, 0.0, 0.4, -0.2], B).astype(np.float32)
+    s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, min_ps=mps, freqs=frs, press=prs)
+    s.Status()
+    for b in range(B):
+        want = oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(ks[b]), float(ps[b]), float(reps[b]), hist[b:b + 1], None,
+                             mode=oracle.MODE_FIXED, min_p=float(mps[b]), freq=float(frs[b]), pres=float(prs[b]))
+        assert tok[b] == want["tokens"][0], (b, Ts[b], ks[b], ps[b], reps[b], mps[b], frs[b], prs[b])
+        assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], b
+    s.Close()
+    # only the new arrays, everything else from the handle (T 0.9, top_k 7, top_p 0.8, penalty 1.3); a second call on the
+    # same handle with other histories finds the table clean
+    for rep_call in range(2):
+        hist2 = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+        s2, tok2, _ = _sample_rows(rocm, x, u, hist2, None, None, None, None, path, min_ps=mps, freqs=frs, press=prs)
+        s2.Status()
+        s2.Close()
+        for b in range(B):
+            want = oracle.sample(x[b:b + 1], u[b:b + 1], 0.9, 7, 0.8, 1.3, hist2[b:b + 1], None, mode=oracle.MODE_FIXED,
+                                 min_p=float(mps[b]), freq=float(frs[b]), pres=float(prs[b]))
+            assert tok2[b] == want["tokens"][0], (rep_call, b)
+    # invalid values of the new settings are reported like the others
+    bad_mp = mps.copy(); bad_mp[3] = 1.0; bad_mp[5] = -0.1
+    bad_fr = frs.copy(); bad_fr[7] = np.inf
+    bad_pr = prs.copy(); bad_pr[9] = np.nan
+    s3, tok3, _ = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, min_ps=bad_mp, freqs=bad_fr, press=bad_pr)
+    with pytest.raises(rocm.BornRocmError, match="invalid per-row configuration"):
+        s3.Status()
+    assert tok3[3] == 0 and tok3[5] == 0 and tok3[7] == 0 and tok3[9] == 0
+    good = [b for b in range(B) if b not in (3, 5, 7, 9)]
+    assert np.array_equal(tok3[good], tok[good])
+    s3.Close()
 
 
 def test_per_row_invalid_configuration_is_reported(oracle, rocm):

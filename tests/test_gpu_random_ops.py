@@ -147,12 +147,19 @@ def test_random_per_row_configurations(oracle, rocm, chunk, path):
         ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
         reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
         extras = [dict(), dict(MinP=0.05), dict(FrequencyPenalty=0.2, PresencePenalty=0.1)][int(rng.integers(0, 3))]
-        s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, **extras)
+        mps = frs = prs = None                                             # per-row arrays of the three, now and then
+        if rng.random() < 0.5:
+            mps = rng.choice([0.0, 0.02, 0.3], B).astype(np.float32)
+        if rng.random() < 0.5:
+            frs = rng.choice([0.0, 0.3, -0.2], B).astype(np.float32)
+            prs = rng.choice([0.0, 0.5], B).astype(np.float32)
+        s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, min_ps=mps, freqs=frs, press=prs, **extras)
         s.Status()
         s.Close()
         for b in range(B):
             want = oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(ks[b]), float(ps[b]), float(reps[b]), hist[b:b + 1], None,
-                                 mode=oracle.MODE_FIXED, min_p=extras.get("MinP", 0.0), freq=extras.get("FrequencyPenalty", 0.0),
-                                 pres=extras.get("PresencePenalty", 0.0))
+                                 mode=oracle.MODE_FIXED, min_p=extras.get("MinP", 0.0) if mps is None else float(mps[b]),
+                                 freq=extras.get("FrequencyPenalty", 0.0) if frs is None else float(frs[b]),
+                                 pres=extras.get("PresencePenalty", 0.0) if prs is None else float(prs[b]))
             assert tok[b] == want["tokens"][0], (chunk, i, b, V, H, Ts[b], ks[b], ps[b], reps[b], extras)
             assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], (chunk, i, b)
