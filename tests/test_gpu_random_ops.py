@@ -163,3 +163,51 @@ def test_random_per_row_configurations(oracle, rocm, chunk, path):
                                  pres=extras.get("PresencePenalty", 0.0) if prs is None else float(prs[b]))
             assert tok[b] == want["tokens"][0], (chunk, i, b, V, H, Ts[b], ks[b], ps[b], reps[b], extras)
             assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], (chunk, i, b)
+
+
+@pytest.mark.parametrize("chunk", range(4))
+def test_random_gemm_pitches_and_alignments(rocm, chunk):
+    # random shapes, row pitches (multiples of four and not) and base offsets, so that every load path of the GEMM
+    # (direct-to-LDS, register-staged vector, scalar) and every tile height is met; nothing outside the output's
+    # rows and columns may be written, nothing outside the operands' rows may influence the result (NaN padding)
+    from born_amd import _capi
+    rng = np.random.default_rng(31337 + chunk)
+    for i in range(10):
+        M = int(rng.choice([1, 7, 16, 24, 32, 33, 64, 100, 128, 130, 260]))
+        K = int(rng.choice([1, 5, 32, 64, 96, 128, 160, 250, 512]))
+        N = int(rng.choice([1, 3, 128, 129, 256, 300, 640, 1000]))
+        lda = K + int(rng.choice([0, 0, 1, 4, 8]))
+        ldw = K + int(rng.choice([0, 0, 3, 4, 32]))
+        ldc = N + int(rng.choice([0, 0, 1, 4]))
+        off = int(rng.choice([0, 0, 1, 2, 4]))
+        xa = np.full((M, lda), np.nan, np.float32)
+        wa = np.full((N, ldw), np.nan, np.float32)
+        xa[:, :K] = rng.standard_normal((M, K))
+        wa[:, :K] = rng.standard_normal((N, K))
+        bias = rng.standard_normal(N).astype(np.float32) if rng.random() < 0.6 else None
+        pad = np.full(off, np.nan, np.float32)
+        dx = rocm.DeviceBuffer.from_numpy(np.concatenate([pad, xa.ravel(), pad, np.zeros(1, np.float32)]))
+        dw = rocm.DeviceBuffer.from_numpy(np.concatenate([pad, wa.ravel(), pad, np.zeros(1, np.float32)]))
+        db = None if bias is None else rocm.DeviceBuffer.from_numpy(np.concatenate([pad, bias, np.zeros(1, np.float32)]))
+        sentinel = np.full(off + M * ldc + 1, -777.0, np.float32)
+        dc = rocm.DeviceBuffer.from_numpy(sentinel)
+        _capi.check(_capi.lib().born_rocm_linear(dx.ptr + 4 * off, M, K, lda, dw.ptr + 4 * off, N, ldw, None if db is None else db.ptr + 4 * off,
+                                                 dc.ptr + 4 * off, ldc, None))
+        out = dc.to_numpy(np.float32, sentinel.shape)
+        got = out[off:off + M * ldc].reshape(M, ldc)
+        tag = (chunk, i, M, K, N, lda, ldw, ldc, off, bias is not None)
+        assert np.all(out[:off] == -777.0) and out[-1] == -777.0 and np.all(got[:, N:] == -777.0), tag
+        x, w = xa[:, :K], wa[:, :K]
+        exact = x.astype(np.float64) @ w.astype(np.float64).T + (0 if bias is None else bias.astype(np.float64)[None, :])
+        assert np.all(np.abs(got[:, :N] - exact) <= _bound(x, w, bias, K)), tag
+        # the same product through matmul, b = w^T stored [K, N] with its own pitch
+        ldb = N + int(rng.choice([0, 0, 2, 4]))
+        ba = np.full((K, ldb), np.nan, np.float32)
+        ba[:, :N] = w.T
+        dbm = rocm.DeviceBuffer.from_numpy(np.concatenate([pad, ba.ravel(), np.zeros(1, np.float32)]))
+        dc2 = rocm.DeviceBuffer.from_numpy(sentinel)
+        _capi.check(_capi.lib().born_rocm_matmul(dx.ptr + 4 * off, dbm.ptr + 4 * off, dc2.ptr + 4 * off, M, K, N, lda, ldb, ldc, None))
+        out2 = dc2.to_numpy(np.float32, sentinel.shape)
+        got2 = out2[off:off + M * ldc].reshape(M, ldc)
+        assert np.all(out2[:off] == -777.0) and out2[-1] == -777.0 and np.all(got2[:, N:] == -777.0), tag
+        assert np.all(np.abs(got2[:, :N] - x.astype(np.float64) @ w.astype(np.float64).T) <= _bound(x, w, None, K)), tag
