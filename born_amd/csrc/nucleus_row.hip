@@ -51,8 +51,13 @@ __device__ __forceinline__ int nuc_bin(const NucRow &r, float d) {
 // Visits every element of the row with its penalised logit: aligned rows four at a time as f4(id of the first, y[4]),
 // in stages of NUC_U float4 per thread, the next stage's loads in flight while this one is visited; what is left
 // over (and every element of an unaligned row) one at a time as f1(id, y).
-template <class F4, class F1>
-__device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1) {
+// `pre` runs once before the first element is visited, with the first stage's loads already in flight (work that
+// must precede the visits but not the loads: building the history bitmap).
+struct NucNoPre {
+    __device__ __forceinline__ void operator()() const {}
+};
+template <class F4, class F1, class PRE = NucNoPre>
+__device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
         float y[4] = {q[0], q[1], q[2], q[3]};
@@ -79,6 +84,7 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             nuc_f32x4 va[NUC_U], vb[NUC_U];
 #pragma unroll
             for (int u = 0; u < NUC_U; u++) va[u] = x4[u * NUC_BLOCK + tid];
+            pre();
             for (int s = 0; s + 1 < nfull; s++) {
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) vb[u] = x4[((s + 1) * NUC_U + u) * NUC_BLOCK + tid];
@@ -89,6 +95,8 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             }
 #pragma unroll
             for (int u = 0; u < NUC_U; u++) visit4(va[u], (((nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+        } else {
+            pre();
         }
         for (int i = nfull * NUC_U * NUC_BLOCK + tid; i < n4; i += NUC_BLOCK) {
             const nuc_f32x4 q = x4[i];
@@ -96,6 +104,7 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
         }
         for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) visit1(j);
     } else {
+        pre();
         for (int j = tid; j < r.V; j += NUC_BLOCK) visit1(j);
     }
 }
@@ -504,17 +513,33 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     r.penal = (a.rep != 1.0f || r.counts) && hlen > 0;
-    if (r.penal) {
-        for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
-        __syncthreads();
-    }
-    for (int i = tid; i < hlen; i += NUC_BLOCK) {
-        const int t = h[i];
-        if (t < 0 || t >= V) atomicOr(a.status, 1);
-        else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
-    }
-    __syncthreads();
+    // The history bitmap is built with the row's first loads already in flight: this thread's first history entry is
+    // requested before them (loads return in order), and the barriers wait for LDS traffic only.
+    const int h0 = tid < hlen ? h[tid] : -1;
+    auto build_bitmap = [&]() {
+        if (r.penal) {
+            for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
+            lds_barrier();
+        }
+        for (int i = tid; i < hlen; i += NUC_BLOCK) {
+            const int t = i == tid ? h0 : h[i];
+            if (t < 0 || t >= V) atomicOr(a.status, 1);
+            else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
+        }
+        lds_barrier();
+    };
 
+    // z = y / T by a reciprocal and one correction step (quotient, exact remainder, update): the correctly rounded
+    // quotient but for rare last-bit cases, at a quarter of the instructions of the IEEE division the sampling
+    // kernels need for their bit-exact ranks; this kernel's result is held to a tolerance.  Infinite y bypass it.
+    const float rT = 1.0f / r.T;
+    const bool unit = r.T == 1.0f;
+    auto zof = [&](float y) {
+        if (unit) return canon(y);
+        const float q0 = y * rT;
+        const float q1 = fmaf(fmaf(-q0, r.T, y), rT, q0);
+        return canon(fabsf(y) <= 3.402823466e+38f ? q1 : q0);
+    };
     // exp(z - m) with the conventions of the pipeline: a tie with the maximum is exactly 1 (also when both are -inf)
     auto term = [](float z, float m) { return z == m ? 1.0f : __expf(z - m); };
     float mt = -INFINITY;                                            // running maximum of this thread's z
@@ -527,16 +552,17 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
         [&](int, const float (&y)[4]) {
             float z[4];
 #pragma unroll
-            for (int t = 0; t < 4; t++) z[t] = nuc_z(r, y[t]);
+            for (int t = 0; t < 4; t++) z[t] = zof(y[t]);
             const float m4 = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
             if (m4 > mt) raise(m4);
             st += (double)((term(z[0], mt) + term(z[1], mt)) + (term(z[2], mt) + term(z[3], mt)));
         },
         [&](int, float y) {
-            const float z = nuc_z(r, y);
+            const float z = zof(y);
             if (z > mt) raise(z);
             st += (double)term(z, mt);
-        });
+        },
+        build_bitmap);
 
     const float m = block_max_f32<NUC_BLOCK>(mt, &scr);
     double part = mt == m ? st : st * exp((double)mt - (double)m);   // a thread without elements: st = 0
@@ -555,7 +581,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
         } else {
             float y = r.x[t];
             if (r.penal && ((bm[t >> 5] >> (t & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, t, r.freq, r.pres);
-            const float z = nuc_z(r, y);
+            const float z = zof(y);
             const double d = z == m ? 0.0 : (double)m - (double)z;   // >= 0, +inf for a masked token
             out[row] = (float)(-d - log(S));
         }
