@@ -365,12 +365,11 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
     // The single-pass kernel relies on the penalties never raising a logit (per-row values are judged on the device).
     const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
-    // a failed launch must not leave the table of counts raised: remember the error, clear, then report
+    // a failed launch must not leave the table of counts raised: remember the first error, clear, then report
     hipError_t launch_err = hipSuccess;
-#define TRY_LAUNCH(expr)                                              \
-    do {                                                              \
-        if (launch_err == hipSuccess) launch_err = (expr);            \
-    } while (0)
+    auto keep_first = [&launch_err](hipError_t e) {
+        if (launch_err == hipSuccess) launch_err = e;
+    };
     if (any_row) {
         // every kernel over the whole batch: each workgroup takes its row only if the row's configuration is its own
         RowConfigs rows;
@@ -382,24 +381,20 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.freq = per_row->frequency_penalty;
         rows.pres = per_row->presence_penalty;
         rows.path = s->path;
-        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) TRY_LAUNCH(launch_topk_row(a, st, &rows));
-        if (s->path != 1) TRY_LAUNCH(launch_nucleus_row(a, st, &rows));
-        TRY_LAUNCH(launch_sample_wide(a, st, &rows));
+        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) keep_first(launch_topk_row(a, st, &rows));
+        if (s->path != 1) keep_first(launch_nucleus_row(a, st, &rows));
+        keep_first(launch_sample_wide(a, st, &rows));
     } else {
         const bool boosts = (history && a.rep < 1.0f) || raises;   // (repetition_penalty < 1 raises the positive logits)
         if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
-            TRY_LAUNCH(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
+            keep_first(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
         } else if (s->path != 1 && a.top_k == 0) {
-            TRY_LAUNCH(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
+            keep_first(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
         } else {
-            TRY_LAUNCH(launch_sample_wide(a, st));
+            keep_first(launch_sample_wide(a, st));
         }
     }
-#undef TRY_LAUNCH
-    if (counted) {
-        const hipError_t ce = launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st);
-        if (launch_err == hipSuccess) launch_err = ce;
-    }
+    if (counted) keep_first(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st));
     if (launch_err != hipSuccess) return hip_fail(launch_err, "sample: kernel launch");
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;
