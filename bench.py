@@ -16,9 +16,11 @@ the one the metric is quoted on).  Prints ONE JSON line.
 
 The other configurations of BASELINE.json run through the same script for their own figures (never the
 headline): --config C1 | C2 (multinomial) | C2g (greedy argmax) | C4 (speculative verify, 64 x 5 positions;
-"tokens" are verified draft positions) | C5.
+"tokens" are verified draft positions) | C5; and three sets of secondary timings at the C3 shape:
+--config C3x (the step with min-p, with the frequency / presence penalties, with per-row arrays) | LP (token
+log-probabilities) | GEN (the generation loop: embedding lookup, LM head, sampling, history append).
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C2g|C4|C5] [--no-cpu] [--no-producer]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C2g|C4|C5|C3x|LP|GEN] [--no-cpu] [--no-producer]
 """
 import argparse
 import json
@@ -159,6 +161,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.config in ("C3x", "LP", "GEN"):
+        return main_extras(args, torch, S, synth, dev)
     gen = {"C1": synth.c1, "C2": synth.c2, "C2g": synth.c2, "C3": synth.c3, "C4": synth.c4, "C5": synth.c5}[args.config]
     w = gen()
     if args.config in ("C2g", "C4"):
@@ -251,6 +255,94 @@ def main():
         out["producer"] = producer_leg(torch, dev, smp, step, B, V, args.hidden, logits_all, stream, max(5, args.steps // 10))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+def main_extras(args, torch, S, synth, dev):
+    """Secondary figures at the C3 shape (never the headline), one JSON line:
+      C3x  the sampling step with min-p, with the frequency / presence penalties, and with per-row arrays
+      LP   token log-probabilities (the cross-entropy forward term), plain and with history + penalty + temperature
+      GEN  the generation loop (embedding lookup, LM head, sampling, history append) at three shapes"""
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn, k, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(k):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / k * 1e3          # us per call
+
+    out = {"metric": "secondary figures, us per step (not the headline)", "config": {"workload": args.config, "seed": synth.BASE_SEED},
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "data": "synthetic", "dtype": "f32", "us": {}}
+    if args.config == "GEN":
+        import time
+        from born_amd import linear as L
+        from born_amd.generate import Generator
+        for (B, V, K) in [(1, 32000, 4096), (64, 32000, 4096), (256, 128256, 4096)]:
+            E = torch.randn(V, K, device=dev) * 0.02
+            W = torch.randn(V, K, device=dev) * 0.02
+            smp = S.NewSampler(S.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1, Seed=1), max_batch=B, max_vocab=V)
+            gen = Generator(E, V, K, L.Linear(K, V, W, None), smp, max_batch=B, max_len=1024)
+            prompts = [[1, 2, 3]] * B
+            gen.Generate(prompts, 8)
+            n = min(200, args.steps)
+            t0 = time.perf_counter()
+            gen.Generate(prompts, n)
+            dt = time.perf_counter() - t0
+            out["us"][f"decode step (gather + LM head + sample + append), batch {B} x vocab {V} x hidden {K}"] = dt / n * 1e6
+            smp.Close()
+            del E, W
+        print(json.dumps(out))
+        return
+    w = synth.c3()
+    B, V = w.logits.shape
+    lgs = [torch.from_numpy(w.logits).to(dev) for _ in range(max(1, args.rotate))]
+    u = torch.from_numpy(w.uniforms).to(dev)
+    h = torch.from_numpy(w.history).to(dev)
+    H = h.shape[1]
+    tok = torch.empty(B, dtype=torch.int32, device=dev)
+    pr = torch.empty(B, device=dev)
+    c = [0]
+
+    def mk(**kw):
+        return S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k, TopP=w.top_p, RepetitionPenalty=w.rep, **kw),
+                            max_batch=B, max_vocab=V)
+
+    def nxt():
+        c[0] += 1
+        return lgs[c[0] % len(lgs)]
+
+    if args.config == "C3x":
+        base, minp, fp = mk(), mk(MinP=0.05), mk(FrequencyPenalty=0.3, PresencePenalty=0.5)
+        Ts = torch.full((B,), w.temperature, device=dev)
+        ks = torch.full((B,), w.top_k, dtype=torch.int32, device=dev)
+        ps = torch.full((B,), w.top_p, device=dev)
+        rs = torch.full((B,), w.rep, device=dev)
+        cases = {
+            "C3": lambda: base.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 + min_p 0.05": lambda: minp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 with per-row arrays (same values in every row)":
+                lambda: base.SampleRows(nxt(), B, V, h, None, u, Ts, ks, ps, rs, tok, pr, hist_stride=H, stream=stream),
+        }
+    else:
+        lp = torch.empty(B, device=dev)
+        plain, full = S.NewSampler(S.SamplerConfig(), max_batch=B, max_vocab=V), mk()
+        cases = {
+            "token log-probabilities, plain (temperature 1, no history)":
+                lambda: plain.TokenLogprobs(nxt(), B, V, None, None, tok, lp, stream=stream),
+            "token log-probabilities, 512-token history + repetition penalty + T 0.7":
+                lambda: full.TokenLogprobs(nxt(), B, V, h, None, tok, lp, hist_stride=H, stream=stream),
+        }
+        tok.zero_()
+    for name, fn in cases.items():
+        out["us"][name] = timed(fn, args.steps, args.warmup)
+    out["algorithmic_bytes_per_step"] = w.algorithmic_bytes()
     print(json.dumps(out))
 
 
