@@ -221,7 +221,16 @@ func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab in
 type RowConfigs struct {
 	Temperatures, TopKs, TopPs, Penalties             DeviceBuffer
 	MinPs, FrequencyPenalties, PresencePenalties DeviceBuffer
+	// RowKinds: 0, or the OR of RowsSmallTopK / RowsNoTopK / RowsOther for the kinds of row that may occur in the call
+	// (kernels no row needs are then not launched; a row of a kind not promised yields token 0 and an error).
+	RowKinds uint32
 }
+
+const (
+	RowsSmallTopK uint32 = 1 // 1 <= top_k <= 64, no penalty that raises a logit
+	RowsNoTopK    uint32 = 2 // top_k disabled
+	RowsOther     uint32 = 4 // everything else
+)
 
 // SampleRows is Sample with a configuration per row.  A row with invalid values yields token 0 and an error
 // from the status check that follows the copy of the tokens.
@@ -241,6 +250,7 @@ func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history Devi
 		min_p:              (*C.float)(rows.MinPs.ptr),
 		frequency_penalty:  (*C.float)(rows.FrequencyPenalties.ptr),
 		presence_penalty:   (*C.float)(rows.PresencePenalties.ptr),
+		row_kinds:          C.uint32_t(rows.RowKinds),
 	}
 	if err = check(C.born_rocm_sample_rows(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
 		C.int64_t(vocab), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),

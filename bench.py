@@ -329,6 +329,8 @@ def main_extras(args, torch, S, synth, dev):
             "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 with per-row arrays (same values in every row)":
                 lambda: base.SampleRows(nxt(), B, V, h, None, u, Ts, ks, ps, rs, tok, pr, hist_stride=H, stream=stream),
+            "C3 with per-row arrays and the promise that every row has a small top-k":
+                lambda: base.SampleRows(nxt(), B, V, h, None, u, Ts, ks, ps, rs, tok, pr, hist_stride=H, stream=stream, rowKinds=1),
         }
     else:
         lp = torch.empty(B, device=dev)

@@ -20,7 +20,11 @@ class SamplerConfigC(C.Structure):
 
 class RowConfigsC(C.Structure):
     _fields_ = [("temperature", C.c_void_p), ("top_k", C.c_void_p), ("top_p", C.c_void_p), ("repetition_penalty", C.c_void_p),
-                ("min_p", C.c_void_p), ("frequency_penalty", C.c_void_p), ("presence_penalty", C.c_void_p)]
+                ("min_p", C.c_void_p), ("frequency_penalty", C.c_void_p), ("presence_penalty", C.c_void_p),
+                ("row_kinds", C.c_uint32)]
+
+
+ROWS_SMALL_TOP_K, ROWS_NO_TOP_K, ROWS_OTHER = 1, 2, 4
 
 
 # every symbol include/born_rocm.h declares: name -> (restype, argtypes)

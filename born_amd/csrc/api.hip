@@ -348,6 +348,8 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     a.dcut = mass_cutoff(s->cfg);
     a.freq = s->cfg.frequency_penalty;
     a.pres = s->cfg.presence_penalty;
+    if (per_row && (per_row->row_kinds & ~7u))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample_rows: row_kinds has unknown bits set (%u)", per_row->row_kinds);
     const bool any_row = per_row && (per_row->temperature || per_row->top_k || per_row->top_p || per_row->repetition_penalty ||
                                      per_row->min_p || per_row->frequency_penalty || per_row->presence_penalty);
     const bool counted = (counts_history(s->cfg) || (per_row && (per_row->frequency_penalty || per_row->presence_penalty))) &&
@@ -381,9 +383,15 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.freq = per_row->frequency_penalty;
         rows.pres = per_row->presence_penalty;
         rows.path = s->path;
-        if (s->path != 1 && vocab <= ROW_MAX_VOCAB) keep_first(launch_topk_row(a, st, &rows));
-        if (s->path != 1) keep_first(launch_nucleus_row(a, st, &rows));
-        keep_first(launch_sample_wide(a, st, &rows));
+        // which kernels run: all that the shape and the handle's kernel selection allow, or those the caller's promise
+        // about the kinds of row leaves (mapped through the same rules: under path 1 every row is the general kernel's)
+        const unsigned able = (s->path != 1 && vocab <= ROW_MAX_VOCAB ? 1u : 0u) | (s->path != 1 ? 2u : 0u) | 4u;
+        unsigned want = per_row->row_kinds ? (per_row->row_kinds & 7u) : 7u;
+        if (want & ~able) want |= 4u;                                // rows whose own kernel cannot run here go to the general one
+        rows.launched = want & able;
+        if (rows.launched & 1u) keep_first(launch_topk_row(a, st, &rows));
+        if (rows.launched & 2u) keep_first(launch_nucleus_row(a, st, &rows));
+        if (rows.launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
     } else {
         const bool boosts = (history && a.rep < 1.0f) || raises;   // (repetition_penalty < 1 raises the positive logits)
         if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {

@@ -61,6 +61,8 @@ struct RowConfigs {
     const int *k;
     const float *min_p, *freq, *pres;
     int path;                     // the handle's kernel selection (1 = always the general kernel)
+    unsigned launched;            // bit r set: the kernel of route r runs in this call (all three unless the caller
+                                  // promised which kinds of row occur)
 };
 
 struct SpecArgs {

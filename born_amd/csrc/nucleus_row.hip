@@ -464,6 +464,10 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs 
     RowValues v;
     bool invalid;
     if (!row_config_values(a, rc, (int)blockIdx.x, ROUTE_NUCLEUS, v, invalid)) return;   // workgroup-uniform, before any barrier
+    if (invalid) {
+        row_config_reject(a, (int)blockIdx.x);
+        return;
+    }
     nucleus_row_body<COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres);
 }
 

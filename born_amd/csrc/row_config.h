@@ -25,8 +25,8 @@ __device__ __forceinline__ bool row_config_valid(const RowValues &v, float min_p
 
 // Row `row`'s values (workgroup-uniform).  Returns false when another kernel owns the row.  An invalid
 // configuration (temperature or repetition penalty not positive and finite, top_p outside (0, 1], min_p outside
-// [0, 1), a frequency or presence penalty that is not finite) belongs to the general kernel, which reports it
-// through the status word (bit 3) and emits token 0.
+// [0, 1), a frequency or presence penalty that is not finite) belongs to the general kernel; the kernel that takes
+// an invalid row reports it through the status word (bit 3) and emits token 0 (row_config_reject).
 __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const RowConfigs &rc, int row, int my_route, RowValues &v,
                                                   bool &invalid) {
     invalid = false;
@@ -66,7 +66,22 @@ __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const Row
     } else {
         route = ROUTE_GENERAL;
     }
+    // A row whose kernel was not launched (the caller promised its kind would not occur), an invalid row when the
+    // general kernel was not launched: the launched kernel of the lowest route reports it like an invalid one.
+    if (!((rc.launched >> route) & 1u)) {
+        invalid = true;
+        route = __builtin_ctz(rc.launched);
+    }
     return route == my_route;
+}
+// What a kernel does with an invalid row of its own (every thread of the workgroup calls it, then returns).
+__device__ __forceinline__ void row_config_reject(const SampleArgs &a, int row) {
+    if (threadIdx.x == 0) {
+        atomicOr(a.status, 8);
+        a.tokens[row] = 0;
+        if (a.probs) a.probs[row] = 0.0f;
+        if (a.nuc_len) a.nuc_len[row] = -1;
+    }
 }
 // The same, written into the kernel's own copy of the arguments.
 __device__ __forceinline__ bool row_config(SampleArgs &a, const RowConfigs &rc, int row, int my_route, bool &invalid) {

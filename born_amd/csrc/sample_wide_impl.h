@@ -495,12 +495,7 @@ __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_rows_kernel(SampleArgs
     bool invalid;
     if (!row_config(a, rc, (int)blockIdx.x, ROUTE_GENERAL, invalid)) return;   // workgroup-uniform, before any barrier
     if (invalid) {
-        if (threadIdx.x == 0) {
-            atomicOr(a.status, 8);
-            a.tokens[blockIdx.x] = 0;
-            if (a.probs) a.probs[blockIdx.x] = 0.0f;
-            if (a.nuc_len) a.nuc_len[blockIdx.x] = -1;
-        }
+        row_config_reject(a, (int)blockIdx.x);
         return;
     }
     wide_row<COUNTED>(a, (int)blockIdx.x, (lds_u64 *)dyn, (BORN_LDS BlockScratch *)&scr, (lds_int *)s_int, (lds_u64 *)s_u64);

@@ -521,6 +521,10 @@ template <bool VEC>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, RowConfigs rc) {
     bool invalid;
     if (!row_config(a, rc, (int)blockIdx.x, ROUTE_TOPK, invalid)) return;   // workgroup-uniform, before any barrier
+    if (invalid) {
+        row_config_reject(a, (int)blockIdx.x);
+        return;
+    }
     topk_row_body<VEC>(a);
 }
 

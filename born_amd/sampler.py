@@ -184,11 +184,12 @@ class Sampler:
 
     def SampleRows(self, logits, batch, vocab, history, histLen, uniforms, temperatures, topKs, topPs, penalties,
                    tokens_out, probs_out=None, row_stride=None, hist_stride=0, stream=None, minPs=None,
-                   frequencyPenalties=None, presencePenalties=None):
+                   frequencyPenalties=None, presencePenalties=None, rowKinds=0):
         """Sample with a configuration per row: device arrays of `batch` values, each may be None (=> the
-        handle's value)."""
+        handle's value).  rowKinds: 0, or the OR of _capi.ROWS_* kinds of row that may occur (kernels no row needs
+        are then not launched)."""
         rows = _capi.RowConfigsC(_ptr(temperatures), _ptr(topKs), _ptr(topPs), _ptr(penalties), _ptr(minPs),
-                                 _ptr(frequencyPenalties), _ptr(presencePenalties))
+                                 _ptr(frequencyPenalties), _ptr(presencePenalties), int(rowKinds))
         _check(_capi.lib().born_rocm_sample_rows(self._h, _ptr(logits), batch, vocab, row_stride or vocab,
                                                  _ptr(history), _ptr(histLen), hist_stride, _ptr(uniforms),
                                                  C.byref(rows), _ptr(tokens_out), _ptr(probs_out), stream))

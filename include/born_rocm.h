@@ -143,7 +143,14 @@ typedef struct born_sampler_row_configs {
     const float   *min_p;
     const float   *frequency_penalty;
     const float   *presence_penalty;
+    /* Optional promise about the rows of this call, so that kernels no row needs are not launched at all (an idle
+     * launch costs about 7 us): 0 = no promise (every kernel is launched), else the OR of the kinds of row that
+     * may occur.  A row of a kind that was not promised gets token 0 and BORN_ROCM_ERR_DATA, like an invalid one. */
+    uint32_t       row_kinds;
 } born_sampler_row_configs;
+#define BORN_ROCM_ROWS_SMALL_TOP_K  1u   /* 1 <= top_k <= 64, no penalty that raises a logit, vocab <= 393216 */
+#define BORN_ROCM_ROWS_NO_TOP_K     2u   /* top_k disabled (<= 0 or >= vocab) */
+#define BORN_ROCM_ROWS_OTHER        4u   /* everything else (top_k > 64, a penalty that raises logits with a top-k cut, ...) */
 
 int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,

@@ -654,7 +654,7 @@ def test_spec_verify_bonus_draw(oracle, rocm):
 
 # ---------------------------------------------------------------- a configuration per row
 
-def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=None, press=None, **handle):
+def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=None, press=None, row_kinds=0, **handle):
     B, V = x.shape
     s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.9, TopK=7, TopP=0.8, RepetitionPenalty=1.3, **handle), max_batch=B, max_vocab=V)
     s.SetPath(path)
@@ -662,7 +662,8 @@ def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=
     tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
     s.SampleRows(dev(x, np.float32), B, V, dev(hist, np.int32), None, dev(u, np.float32), dev(Ts, np.float32), dev(ks, np.int32),
                  dev(ps, np.float32), dev(reps, np.float32), tok, pr, hist_stride=0 if hist is None else hist.shape[1],
-                 minPs=dev(min_ps, np.float32), frequencyPenalties=dev(freqs, np.float32), presencePenalties=dev(press, np.float32))
+                 minPs=dev(min_ps, np.float32), frequencyPenalties=dev(freqs, np.float32), presencePenalties=dev(press, np.float32),
+                 rowKinds=row_kinds)
     return s, tok.to_numpy(np.int32, (B,)), pr.to_numpy(np.float32, (B,))
 
 
@@ -772,6 +773,52 @@ def test_per_row_min_p_and_additive_penalties(oracle, rocm, path):
     good = [b for b in range(B) if b not in (3, 5, 7, 9)]
     assert np.array_equal(tok3[good], tok[good])
     s3.Close()
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_per_row_promised_kinds_of_row(oracle, rocm, path):
+    from born_amd import _capi
+    rng = np.random.default_rng(81)
+    B, V, H = 20, 9000, 48
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, (B, H)).astype(np.int32)
+    Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
+    ps = rng.choice([1.0, 0.9, 0.5], B).astype(np.float32)
+    reps = rng.choice([1.0, 1.15, 2.0], B).astype(np.float32)
+
+    def want(b, k):
+        return oracle.sample(x[b:b + 1], u[b:b + 1], float(Ts[b]), int(k), float(ps[b]), float(reps[b]), hist[b:b + 1], None,
+                             mode=oracle.MODE_FIXED)["tokens"][0]
+
+    # every row a small top-k, and the caller says so: only the single-pass kernel runs (under path 1 the general one)
+    ks = rng.choice([1, 5, 40, 64], B).astype(np.int32)
+    s, tok, _ = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, row_kinds=_capi.ROWS_SMALL_TOP_K)
+    s.Status()
+    assert [int(t) for t in tok] == [int(want(b, ks[b])) for b in range(B)]
+    c = s.Counters()
+    assert (c["general_rows"] == 0) if path == 0 else (c["topk_rows"] + c["fallback_rows"] == 0)
+    s.Close()
+    # two kinds promised, a third occurs in rows 3 and 11 (top_k 300), and row 7 is invalid: those rows are reported
+    ks2 = rng.choice([0, 5, 50], B).astype(np.int32)
+    ks2[3] = ks2[11] = 300
+    Tbad = Ts.copy()
+    Tbad[7] = -1.0
+    s, tok, _ = _sample_rows(rocm, x, u, hist, Tbad, ks2, ps, reps, path, row_kinds=_capi.ROWS_SMALL_TOP_K | _capi.ROWS_NO_TOP_K)
+    if path == 0:
+        with pytest.raises(rocm.BornRocmError, match="invalid per-row configuration"):
+            s.Status()
+        assert tok[3] == 0 and tok[11] == 0 and tok[7] == 0
+        good = [b for b in range(B) if b not in (3, 7, 11)]
+    else:                                                # path 1: the general kernel serves every valid row whatever was promised
+        with pytest.raises(rocm.BornRocmError, match="invalid per-row configuration"):
+            s.Status()
+        assert tok[7] == 0
+        good = [b for b in range(B) if b != 7]
+    assert [int(tok[b]) for b in good] == [int(want(b, ks2[b])) for b in good]
+    s.Close()
+    with pytest.raises(rocm.SamplerPanic, match="row_kinds"):
+        _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, row_kinds=8)
 
 
 def test_per_row_invalid_configuration_is_reported(oracle, rocm):
