@@ -73,6 +73,30 @@ public:
         return tokens;
     }
 
+    // Sample with a configuration per row: `rows` holds device arrays of `batch` values (null members: the handle's
+    // value) and, optionally, the promise of which kinds of row occur (born_sampler_row_configs::row_kinds).
+    std::vector<int32_t> SampleRows(const float *logits_dev, int64_t batch, int64_t vocab, const int32_t *history_dev,
+                                    int64_t hist_stride, const int32_t *hist_len_dev, const float *uniforms_dev,
+                                    const born_sampler_row_configs &rows, void *stream = nullptr) {
+        DeviceBuffer out(4 * batch);
+        check(born_rocm_sample_rows(h_, logits_dev, batch, vocab, vocab, history_dev, hist_len_dev, hist_stride, uniforms_dev,
+                                    &rows, static_cast<int32_t *>(out.ptr()), nullptr, stream));
+        std::vector<int32_t> tokens(static_cast<size_t>(batch));
+        out.download(tokens.data(), 4 * batch, stream);
+        check(born_rocm_sampler_status(h_, stream));
+        return tokens;
+    }
+
+    // The two device steps of a decode loop: sampled tokens join their histories; token ids become input rows.
+    void HistoryAppend(int32_t *history_dev, int32_t *hist_len_dev, int64_t hist_stride, const int32_t *tokens_dev, int64_t batch,
+                       int64_t vocab, void *stream = nullptr) {
+        check(born_rocm_history_append(h_, history_dev, hist_len_dev, hist_stride, tokens_dev, batch, vocab, stream));
+    }
+    void GatherRows(const float *table_dev, int64_t rows, int64_t cols, const int32_t *ids_dev, int64_t n, float *out_dev,
+                    void *stream = nullptr) {
+        check(born_rocm_gather_rows(h_, table_dev, rows, cols, cols, ids_dev, n, out_dev, cols, stream));
+    }
+
     std::vector<int32_t> Argmax(const float *logits_dev, int64_t batch, int64_t vocab, void *stream = nullptr) {
         DeviceBuffer out(4 * batch);
         check(born_rocm_argmax(h_, logits_dev, batch, vocab, vocab, static_cast<int32_t *>(out.ptr()), stream));
