@@ -10,6 +10,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "kernels.h"
 
@@ -179,7 +180,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     alloc((void **)&s->arg_idx, segs * sizeof(int));
     alloc((void **)&s->status, sizeof(int));
     alloc((void **)&s->lm_best, rows * LM_BEST_PITCH * sizeof(unsigned long long));
-    alloc((void **)&s->counters, (64 + 8 * rows) * sizeof(unsigned long long));   // [0..2] work counters; debug builds: [8..] phase stamps, [64..] per-row stamps
+    alloc((void **)&s->counters, (COUNTER_ROW_BASE + COUNTER_ROW_STRIDE * rows) * sizeof(unsigned long long));   // layout: dev_common.h
     if (counts_history(c)) alloc((void **)&s->hist_counts, rows * (size_t)max_vocab * sizeof(unsigned));
     if (e != hipSuccess) {
         born_rocm_sampler_destroy(s);
@@ -253,9 +254,15 @@ int born_rocm_debug_read_counters(born_sampler *s, void *stream, unsigned long l
 int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows, int64_t *fallback_rows,
                                int64_t *general_rows) {
     if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: counters: null handle");
-    unsigned long long c[4];
-    HIP_TRY(hipMemcpyAsync(c, s->counters, sizeof(c), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    // every row counts on words of its own; the totals are formed here
+    const size_t words = (size_t)COUNTER_ROW_STRIDE * (size_t)s->max_batch;
+    std::vector<unsigned long long> host(words);
+    HIP_TRY(hipMemcpyAsync(host.data(), s->counters + COUNTER_ROW_BASE, words * sizeof(unsigned long long), hipMemcpyDeviceToHost,
+                           (hipStream_t)stream));
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    unsigned long long c[3] = {0, 0, 0};
+    for (int64_t r = 0; r < s->max_batch; r++)
+        for (int w = 0; w < 3; w++) c[w] += host[(size_t)r * COUNTER_ROW_STRIDE + COUNTER_ROW_WORK + w];
     if (topk_rows) *topk_rows = (int64_t)c[0];
     if (fallback_rows) *fallback_rows = (int64_t)c[1];
     if (general_rows) *general_rows = (int64_t)c[2];

@@ -132,11 +132,20 @@ __device__ __forceinline__ float prob_of(float e, u64 Zp, int S) {
     return (float)((double)e / ldexp((double)Zp, -S));
 }
 
+// The handle's counters: [0, 64) scalars (debug builds: phase stamps), then COUNTER_ROW_STRIDE words per row:
+// eight phase stamps (debug builds) and, from COUNTER_ROW_WORK, the row's own work counters (rows settled by the
+// single-pass kernel, rows it finished by its exact selection, rows sampled by the other kernels).  A row counts on
+// words of its own: one contended word for the whole batch cost the step 0.3 us.
+// (COUNTER_ROW_BASE, COUNTER_ROW_STRIDE, COUNTER_ROW_WORK: kernels.h, shared with the host side.)
+__device__ __forceinline__ void count_row(unsigned long long *counters, int row, int which, long long by = 1) {
+    atomicAdd(&counters[COUNTER_ROW_BASE + (long long)COUNTER_ROW_STRIDE * row + COUNTER_ROW_WORK + which], (unsigned long long)by);
+}
+
 #ifdef BORN_PHASE_TIMING
 #define BORN_STAMP(args, row, slot)                                                          \
     do {                                                                                     \
         if (threadIdx.x == 0 && (row) == 0) (args).counters[8 + (slot)] = wall_clock64();    \
-        if (threadIdx.x == 0) (args).counters[64 + 8 * (row) + (slot)] = wall_clock64();     \
+        if (threadIdx.x == 0) (args).counters[COUNTER_ROW_BASE + COUNTER_ROW_STRIDE * (row) + (slot)] = wall_clock64();     \
     } while (0)
 #else
 #define BORN_STAMP(args, row, slot) do {} while (0)

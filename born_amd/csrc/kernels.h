@@ -16,6 +16,9 @@ constexpr int WIDE_LIST_CAP = 4096;        // elements the in-LDS sort can hold
 constexpr int WIDE_SUB_BINS = 2048;        // radix-descent digit = 11 bits
 constexpr int64_t WIDE_MAX_VOCAB = 524288; // history bitmap must fit LDS next to the histogram
 
+// Layout of the handle's counters (words of 8 bytes): scalars, then per row eight phase stamps and the work counters.
+constexpr int COUNTER_ROW_BASE = 64, COUNTER_ROW_STRIDE = 12, COUNTER_ROW_WORK = 8;
+
 constexpr int ARGMAX_SEG = 8192;
 constexpr int SPEC_CHUNKS = 4;              // workgroups per sequence in the residual pass of the speculative step
 
@@ -46,7 +49,7 @@ struct SampleArgs {
     int nuc_cap;
     // workspace
     int *status;                  // device status word
-    unsigned long long *counters; // [0] rows proven by the top-k kernel, [1] rows that needed an exact (slower) refinement, [2] rows sampled without a top-k cut or by the general kernel
+    unsigned long long *counters; // per row (dev_common.h, count_row): [0] settled by the single-pass kernel, [1] needed an exact (slower) refinement, [2] sampled without a top-k cut or by the general kernel
     int mass_shift;
     float dcut;                   // masses are zero beyond this distance below the row maximum: min(80, -ln(min_p))
     // frequency / presence penalties: how often each id occurs in its row's history, [B, V] (null: both are off)

@@ -448,8 +448,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             if (a.probs) a.probs[row] = prob_of(emass(key64_z(tokkey), r.m, r.dcut), Zp, a.mass_shift);
         }
         if (a.nuc_len) a.nuc_len[row] = -1;                          // the nucleus listing is only produced for small top-k
-        atomicAdd(&a.counters[listed ? 2 : 1], 1ull);
-        if (!listed) atomicAdd(&a.counters[2], 1ull);
+        count_row(a.counters, row, listed ? 2 : 1);
+        if (!listed) count_row(a.counters, row, 2);
     }
     BORN_STAMP(a, row, 7);
 }

@@ -472,7 +472,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
         if (a.nuc_len) a.nuc_len[row] = -1;              // the nucleus listing is only produced for small top-k
     }
     BORN_STAMP(a, row, 7);
-    if (tid == 0) atomicAdd(&a.counters[2], 1ull);
+    if (tid == 0) count_row(a.counters, row, 2);
 }
 
 // One workgroup per row of the batch.

@@ -249,7 +249,10 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
     __syncthreads();
     if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
-    if (tid == 0) atomicAdd(&a.counters[1], 1ull);
+    if (tid == 0) {
+        count_row(a.counters, row, 1);
+        count_row(a.counters, row, 0, -1);                           // the row was counted as settled when it started
+    }
 }
 
 template <bool VEC>
@@ -295,6 +298,9 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const bool hfast = penal && hlen <= ROW_BLOCK;
     htab[tid] = 0u;
     htab[tid + ROW_BLOCK] = 0u;
+    // Counted as settled by this kernel now, while the row's loads are in flight (taken back in the rare exact
+    // finish): an atomic at the end of the kernel is a memory round trip the launch has to wait for.
+    if (tid == 0) count_row(a.counters, row, 0);
 
     BORN_STAMP(a, row, 0);
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
@@ -509,7 +515,6 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }
     if (lane_id() == 0) atomicAdd(&a.counters[8 + 18], (u64)count);
 #endif
-    if (tid == 0) atomicAdd(&a.counters[0], 1ull);
 }
 
 template <bool VEC>
