@@ -269,6 +269,10 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ int s_n, s_valid, s_over;
     __shared__ int s_x[1 + ROW_WAVES];
 
+    // Every argument the prologue reads is requested here, in one batch with one wait: left to itself the compiler
+    // fetches them where they are first used, three dependent waits before the row's first load is issued.
+    asm volatile("" ::"s"(a.logits), "s"(a.row_stride), "s"(a.V), "s"(a.top_k), "s"(a.history), "s"(a.hist_len), "s"(a.hist_stride),
+                 "s"(a.uniforms), "s"(a.T), "s"(a.rep), "s"(a.hist_counts));
     const int tid = threadIdx.x, row = blockIdx.x;
     const int V = a.V, k = a.top_k;
     const float *x = a.logits + (long long)row * a.row_stride;
@@ -278,11 +282,15 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int nstage = (iters + ROW_U - 1) / ROW_U;
     const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;      // stages made of whole float4 blocks inside the row
 
-    // the history is requested first and used last
+    // Order of the requests: this thread's first history entry (used last, but loads return in order and it must
+    // not wait behind the row), then the row's first three stages; the LDS tables are cleared behind them.
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
-    const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
+    f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
+    if (nfull > 0) row_load_fast(va, x, 0, tid); else row_load_any<VEC>(va, x, V, 0, tid);
+    if (nfull > 1) row_load_fast(vb, x, 1, tid);                     // in flight during the search for Tw
+    if (nfull > 2) row_load_fast(vc, x, 2, tid);
 
     if (tid == 0) {
         s_n = 0;
@@ -298,15 +306,14 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const bool hfast = penal && hlen <= ROW_BLOCK;
     htab[tid] = 0u;
     htab[tid + ROW_BLOCK] = 0u;
+
+    BORN_STAMP(a, row, 0);
+    // The row's uniform is one scalar load whose result the compiler waits for on the spot: after the row's first
+    // loads have been issued, not before them.
+    const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
     // Counted as settled by this kernel now, while the row's loads are in flight (taken back in the rare exact
     // finish): an atomic at the end of the kernel is a memory round trip the launch has to wait for.
     if (tid == 0) count_row(a.counters, row, 0);
-
-    BORN_STAMP(a, row, 0);
-    f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
-    if (nfull > 0) row_load_fast(va, x, 0, tid); else row_load_any<VEC>(va, x, V, 0, tid);
-    if (nfull > 1) row_load_fast(vb, x, 1, tid);                     // in flight during the search for Tw
-    if (nfull > 2) row_load_fast(vc, x, 2, tid);
 
     // ---- Tw from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
     // need = ceil(top_k / a)-th largest of the wave results
