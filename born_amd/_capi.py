@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libborn_rocm.so")
+# the library built in-tree, unless BORN_ROCM_LIB names another build of it
+LIB_PATH = os.environ.get("BORN_ROCM_LIB") or os.path.join(_HERE, "lib", "libborn_rocm.so")
 
 OK, ERR_ARGUMENT, ERR_HIP, ERR_UNSUPPORTED, ERR_DATA = 0, 1, 2, 3, 4
 

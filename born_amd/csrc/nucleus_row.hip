@@ -517,6 +517,14 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     r.penal = (a.rep != 1.0f || r.counts) && hlen > 0;
+    // The queried token and its logit are two dependent loads: requested now, used after the sweep (at the end of the
+    // kernel they would be two memory round trips nothing overlaps).
+    int qt = -1;
+    float qy = 0.0f;
+    if (tid == 0) {
+        qt = tokens[row];
+        if (qt >= 0 && qt < V) qy = r.x[qt];
+    }
     // The history bitmap is built with the row's first loads already in flight: this thread's first history entry is
     // requested before them (loads return in order), and the barriers wait for LDS traffic only.
     const int h0 = tid < hlen ? h[tid] : -1;
@@ -578,12 +586,12 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
         double S = 0.0;
 #pragma unroll
         for (int w = 0; w < NUC_WAVES; w++) S += s_part[w];
-        const int t = tokens[row];
+        const int t = qt;
         if (t < 0 || t >= V) {
             atomicOr(a.status, 1);
             out[row] = __uint_as_float(0x7FC00000u);                 // not a token of this vocabulary
         } else {
-            float y = r.x[t];
+            float y = qy;
             if (r.penal && ((bm[t >> 5] >> (t & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, t, r.freq, r.pres);
             const float z = zof(y);
             const double d = z == m ? 0.0 : (double)m - (double)z;   // >= 0, +inf for a masked token
