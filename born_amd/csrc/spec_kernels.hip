@@ -59,6 +59,14 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
                                     (long long)(row % a.G) * V;
     const float T = a.T;
     const float scale = mass_scale(a.mass_shift);
+    // The draft token and its logit are two dependent loads: requested now, used after the reductions (at the end of
+    // the kernel they would be two memory round trips nothing overlaps).
+    int dt = -1;
+    float xdt = 0.0f;
+    if (tid == 0 && !is_bonus) {
+        dt = a.draft_tokens[row];
+        if (dt >= 0 && dt < V) xdt = x[dt];
+    }
     float m = -INFINITY;
     u64 sum = 0;
     if (RESIDENT) {
@@ -98,9 +106,8 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
         a.mb[row] = m;
         a.Zb[row] = Z;
     } else if (tid == 0) {
-        const int dt = a.draft_tokens[row];
         u64 md = 0;                                                  // mass of the draft token in this distribution
-        if (dt >= 0 && dt < V) md = qfix(emass(z_of(x[dt], T), m), scale);
+        if (dt >= 0 && dt < V) md = qfix(emass(z_of(xdt, T), m), scale);
         else atomicOr(a.status, 2);
         if (is_draft) { a.mq[row] = m; a.Zq[row] = Z; a.qd[row] = md; }
         else { a.mp[row] = m; a.Zp[row] = Z; a.pd[row] = md; }
