@@ -95,3 +95,34 @@ def test_producer_and_backend_argument_checks_need_no_gpu():
     assert L.born_rocm_reshape(p, (ctypes.c_int64 * 2)(2, 3), 2, (ctypes.c_int64 * 2)(4, 2), 2, p, None) == _capi.ERR_ARGUMENT
     assert L.born_rocm_last_error() == b"reshape: incompatible shapes: [2 3] -> [4 2] (different number of elements)"
     assert L.born_rocm_spec_verify_bonus(None, None, 0, None, 0, None, 0, 1, 1, 1, None, None, None, None, None, None) == _capi.ERR_ARGUMENT
+
+
+def test_struct_layouts_of_the_binding_match_the_header(tmp_path):
+    # the two structs that cross the boundary: sizes and member offsets as the C compiler lays them out, against the
+    # ctypes mirrors (and the C++ wrapper compiles against the same header)
+    import subprocess
+    from born_amd import _capi
+    structs = {"born_sampler_config": _capi.SamplerConfigC, "born_sampler_row_configs": _capi.RowConfigsC}
+    lines = []
+    for name, cls in structs.items():
+        lines.append(f'printf("{name} %zu\\n", sizeof({name}));')
+        for field, _ in cls._fields_:
+            lines.append(f'printf("{name}.{field} %zu\\n", offsetof({name}, {field}));')
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stddef.h>\n#include <stdio.h>\n#include "born_rocm.h"\nint main(void) {\n' + "\n".join(lines) +
+                   "\nreturn 0;\n}\n")
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = dict(line.split() for line in subprocess.check_output([str(exe)], text=True).splitlines())
+    for name, cls in structs.items():
+        assert int(got[name]) == ctypes.sizeof(cls), name
+        for field, _ in cls._fields_:
+            assert int(got[f"{name}.{field}"]) == getattr(cls, field).offset, (name, field)
+    # every member of the header's structs is mirrored (no field left out at the end)
+    hdr = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "born_rocm.h")).read(), flags=re.S)
+    for name, cls in structs.items():
+        body = re.search(r"typedef struct " + name + r" \{(.*?)\} " + name + ";", hdr, flags=re.S).group(1)
+        members = re.findall(r"(\w+)\s*;", body)
+        assert members == [f for f, _ in cls._fields_], (name, members)
+    subprocess.check_call(["g++", "-std=c++17", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), "-x", "c++",
+                           os.path.join(ROOT, "include", "born_rocm.hpp")], stderr=subprocess.DEVNULL)
