@@ -223,7 +223,7 @@ def main():
 
     # a step is a single launch, so the step time is the kernel's launch-to-launch duration
     ms_kernel = ms
-    kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 64 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
+    kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 128 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
         if args.path == 0 else "sample_wide_kernel"
     alg_bytes = w.algorithmic_bytes()
     achieved = alg_bytes / (ms_kernel * 1e-3) / 1e9

@@ -6,7 +6,7 @@
 namespace born {
 
 // The single-pass top-k kernel (one workgroup per row).
-constexpr int TOPK_MAX_K = 64;             // largest top_k it serves
+constexpr int TOPK_MAX_K = 128;            // largest top_k it serves (its last wave holds two survivors per lane)
 constexpr int ROW_MAX_VOCAB = 393216;      // largest vocabulary it takes (its history bitmap is 48 KiB of LDS)
 
 // Geometry of the general (any k, any p) kernel: one workgroup per row.

@@ -1,7 +1,7 @@
 // Per-row sampling configurations: when the caller passes arrays of temperature / top_k / top_p /
 // repetition_penalty / min_p / frequency_penalty / presence_penalty (one value per row, any of them optional), the three sampling kernels are all launched
 // over the whole batch and every workgroup first decides whether its row is its own: the single-pass kernel
-// takes 1 <= top_k <= 64 with a penalty that never raises a logit, the three-sweep kernel the rows without a
+// takes 1 <= top_k <= 128 with a penalty that never raises a logit, the three-sweep kernel the rows without a
 // top-k cut, the general kernel everything else — the same rule the host applies to a uniform configuration.
 #pragma once
 #include "dev_common.h"

@@ -1,4 +1,4 @@
-// One-launch sampler for 1 <= top_k <= 64 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
+// One-launch sampler for 1 <= top_k <= 128 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
 // of 1024 threads per row.
 //
 // The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 logits, the
@@ -46,13 +46,13 @@ static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
 static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
 
 // LDS pool (u64 words), laid out once for the proof and once for the exact selection
-constexpr int ROW_POOL = 8000;
+constexpr int ROW_POOL = 8064;
 constexpr int OFF_L = 0;                      // [ROW_WAVES][ROW_WCAP] uint2
 constexpr int OFF_C = OFF_L + ROW_WAVES * ROW_WCAP;   // [ROW_CAP] uint2
 constexpr int OFF_K = OFF_C + ROW_CAP;        // [ROW_CAP] u64
 constexpr int OFF_TAB = OFF_K + ROW_CAP;      // [ROW_SLOTS] u32
-constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [WAVE] u64
-constexpr int OFF_HTAB = OFF_SORTED + WAVE;   // [ROW_HSLOTS] u32
+constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [TOPK_MAX_K] u64
+constexpr int OFF_HTAB = OFF_SORTED + TOPK_MAX_K;   // [ROW_HSLOTS] u32
 static_assert(OFF_HTAB + ROW_HSLOTS / 2 <= ROW_POOL, "proof layout fits the pool");
 constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
 constexpr int FB_DIGIT = 11;                  // key bits per sweep
@@ -60,7 +60,8 @@ constexpr int OFF_FB_HIST = FB_BITMAP;        // [1 << FB_DIGIT] u32
 constexpr int OFF_FB_LIST = OFF_FB_HIST + (1 << FB_DIGIT) / 2;
 constexpr int FB_LIST_CAP = 768;
 constexpr int OFF_FB_SORTED = OFF_FB_LIST + FB_LIST_CAP;
-static_assert(OFF_FB_SORTED + WAVE <= ROW_POOL, "selection layout fits the pool");
+static_assert(OFF_FB_SORTED + TOPK_MAX_K <= ROW_POOL, "selection layout fits the pool");
+static_assert(TOPK_MAX_K <= 2 * WAVE, "the last wave holds at most two survivors per lane");
 static_assert(FB_LIST_CAP <= ROW_BLOCK, "one thread per gathered key");
 static_assert((long long)FB_BITMAP * 64 >= ROW_MAX_VOCAB, "one bitmap bit per id");
 
@@ -248,7 +249,7 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
         if (r < k) sorted[r] = key;
     }
     __syncthreads();
-    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
+    if (tid < WAVE) finish_sorted_by_wave(sorted, k, a, row, u_row);
     if (tid == 0) {
         count_row(a.counters, row, 1);
         count_row(a.counters, row, 0, -1);                           // the row was counted as settled when it started
@@ -318,8 +319,8 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // ---- Tw from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
     // need = ceil(top_k / a)-th largest of the wave results
     const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
-    const int aw = (k + act - 1) / act;                              // <= 64 as top_k <= 64
-    const int need = (k + aw - 1) / aw;                              // <= act
+    const int aw = min(WAVE, (k + act - 1) / act);                   // lanes of one wave
+    const int need = (k + aw - 1) / aw;                              // <= act, but for top_k > 64 on a row of one wave: no Tw then
     {
         float lm = -INFINITY;
 #pragma unroll
@@ -516,7 +517,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     }
     __syncthreads();
     BORN_STAMP(a, row, 6);
-    if (tid < WAVE) finish_sorted_wave(sorted, k, a, row, u_row);
+    if (tid < WAVE) finish_sorted_by_wave(sorted, k, a, row, u_row);
     BORN_STAMP(a, row, 7);
 #ifdef BORN_PHASE_TIMING
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }

@@ -64,4 +64,69 @@ __device__ __forceinline__ void finish_sorted_wave(const u64 *list, int ns, cons
     }
 }
 
+// The same for ns <= 128 survivors: lane l holds entries 2l and 2l + 1, so that lane order is rank order.
+__device__ __forceinline__ void finish_sorted_wave2(const u64 *list, int ns, const SampleArgs &a, int row, float u) {
+    const int l = lane_id();
+    const float m = key64_z(list[0]);
+    const float scale = mass_scale(a.mass_shift);
+    float e[2] = {0.0f, 0.0f};
+    u64 q[2] = {0ull, 0ull}, key[2] = {0ull, 0ull};
+    bool live[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int i = 2 * l + t;
+        live[t] = i < ns;
+        if (i < ns) {
+            key[t] = list[i];
+            const float z = key64_z(key[t]);
+            const float d = (z == m) ? 0.0f : m - z;
+            live[t] = d <= a.dcut;
+            e[t] = expneg(d, a.dcut);
+            q[t] = qfix(e[t], scale);
+        }
+    }
+    const u64 pair = wave_inclusive_scan_u62(q[0] + q[1]);
+    const u64 cum[2] = {pair - q[1], pair};
+    const u64 Zk = readlane_u64(pair, WAVE - 1);
+    int np = ns;
+    if (a.dcut < 80.0f) np = __popcll(__ballot(live[0])) + __popcll(__ballot(live[1]));   // min-p: a prefix of the rank order
+    u64 Zp = Zk;
+    if (a.top_p < 1.0f) {
+        const u64 tp = top_p_target(a.top_p, Zk);
+        np = __popcll(__ballot(2 * l < np && cum[0] < tp)) + __popcll(__ballot(2 * l + 1 < np && cum[1] < tp)) + 1;
+    }
+    if (np < ns || a.top_p < 1.0f) {                                 // the normaliser of the first np survivors
+        const int last = __builtin_amdgcn_readfirstlane(np - 1);
+        const u64 c0 = readlane_u64(cum[0], last >> 1), c1 = readlane_u64(cum[1], last >> 1);
+        Zp = (last & 1) ? c1 : c0;
+    }
+    const u64 td = draw_target(u, Zp);
+    const int pick = __popcll(__ballot(2 * l < np && cum[0] < td)) + __popcll(__ballot(2 * l + 1 < np && cum[1] < td));
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int i = 2 * l + t;
+        if (i == pick) {
+            a.tokens[row] = key64_id(key[t]);
+            if (a.probs) a.probs[row] = prob_of(e[t], Zp, a.mass_shift);
+        }
+        if (a.nuc_len && i < np && i < a.nuc_cap) {
+            a.nuc_ids[(long long)row * a.nuc_cap + i] = key64_id(key[t]);
+            a.nuc_probs[(long long)row * a.nuc_cap + i] = prob_of(e[t], Zp, a.mass_shift);
+        }
+    }
+    if (a.nuc_len) {
+        if (l == 0) a.nuc_len[row] = np;
+        for (int i = np + l; i < a.nuc_cap; i += WAVE) {
+            a.nuc_ids[(long long)row * a.nuc_cap + i] = -1;
+            a.nuc_probs[(long long)row * a.nuc_cap + i] = 0.0f;
+        }
+    }
+}
+
+// One survivor per lane up to a wave of them, two beyond.
+__device__ __forceinline__ void finish_sorted_by_wave(const u64 *list, int ns, const SampleArgs &a, int row, float u) {
+    if (ns <= WAVE) finish_sorted_wave(list, ns, a, row, u);
+    else finish_sorted_wave2(list, ns, a, row, u);
+}
+
 }  // namespace born
