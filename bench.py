@@ -309,9 +309,9 @@ def main_extras(args, torch, S, synth, dev):
     pr = torch.empty(B, device=dev)
     c = [0]
 
-    def mk(**kw):
-        return S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k, TopP=w.top_p, RepetitionPenalty=w.rep, **kw),
-                            max_batch=B, max_vocab=V)
+    def mk(top_k=None, **kw):
+        return S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k if top_k is None else top_k, TopP=w.top_p,
+                                            RepetitionPenalty=w.rep, **kw), max_batch=B, max_vocab=V)
 
     def nxt():
         c[0] += 1
@@ -319,12 +319,16 @@ def main_extras(args, torch, S, synth, dev):
 
     if args.config == "C3x":
         base, minp, fp = mk(), mk(MinP=0.05), mk(FrequencyPenalty=0.3, PresencePenalty=0.5)
+        k100, k128, k129 = mk(top_k=100), mk(top_k=128), mk(top_k=129)
         Ts = torch.full((B,), w.temperature, device=dev)
         ks = torch.full((B,), w.top_k, dtype=torch.int32, device=dev)
         ps = torch.full((B,), w.top_p, device=dev)
         rs = torch.full((B,), w.rep, device=dev)
         cases = {
             "C3": lambda: base.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 100": lambda: k100.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 128": lambda: k128.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 129 (the general kernel)": lambda: k129.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + min_p 0.05": lambda: minp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 with per-row arrays (same values in every row)":
