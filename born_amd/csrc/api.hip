@@ -361,26 +361,48 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
                                      per_row->min_p || per_row->frequency_penalty || per_row->presence_penalty);
     const bool counted = (counts_history(s->cfg) || (per_row && (per_row->frequency_penalty || per_row->presence_penalty))) &&
                          history && hist_stride > 0;
-    if (counted && !s->hist_counts) {
+    // The single-pass kernel relies on the penalties never raising a logit (per-row values are judged on the device).
+    const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
+    const bool boosts = (history && a.rep < 1.0f) || raises;       // (repetition_penalty < 1 raises the positive logits)
+    // which kernels run.  One configuration: the one it selects.  Per-row arrays: all that the shape and the handle's
+    // kernel selection allow, or those the caller's promise about the kinds of row leaves (mapped through the same
+    // rules: under path 1 every row is the general kernel's); each workgroup takes its row only if the row's
+    // configuration is its own.
+    unsigned launched;
+    if (any_row) {
+        const unsigned able = (s->path != 1 && vocab <= ROW_MAX_VOCAB ? 1u : 0u) | (s->path != 1 ? 2u : 0u) | 4u;
+        unsigned want = per_row->row_kinds ? (per_row->row_kinds & 7u) : 7u;
+        if (want & ~able) want |= 4u;                                // rows whose own kernel cannot run here go to the general one
+        launched = want & able;
+    } else if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
+        launched = 1u;                                               // one workgroup per row proves and finishes it
+    } else if (s->path != 1 && a.top_k == 0) {
+        launched = 2u;                                               // no top-k cut: the lean three-sweep kernel
+    } else {
+        launched = 4u;
+    }
+    // The single-pass kernel hashes the history anyway and counts the occurrences there; the other kernels read a
+    // table of counts by id that two small launches raise before them and clear after them.
+    const bool local = counted && launched == 1u && hist_stride <= TOPK_LOCAL_COUNT_HISTORY;
+    const bool table = counted && !local;
+    if (table && !s->hist_counts) {
         // per-row penalties on a handle configured without any: the table of occurrence counts is allocated now
         const size_t bytes = (size_t)s->max_batch * (size_t)s->max_vocab * sizeof(unsigned);
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
         HIP_TRY(hipMalloc((void **)&s->hist_counts, bytes));
         HIP_TRY(hipMemset(s->hist_counts, 0, bytes));
     }
-    a.hist_counts = counted ? s->hist_counts : nullptr;
+    a.hist_counts = table ? s->hist_counts : nullptr;
+    a.local_counts = local ? 1 : 0;
 
     hipStream_t st = (hipStream_t)stream;
-    if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
-    // The single-pass kernel relies on the penalties never raising a logit (per-row values are judged on the device).
-    const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
+    if (table) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
     // a failed launch must not leave the table of counts raised: remember the first error, clear, then report
     hipError_t launch_err = hipSuccess;
     auto keep_first = [&launch_err](hipError_t e) {
         if (launch_err == hipSuccess) launch_err = e;
     };
     if (any_row) {
-        // every kernel over the whole batch: each workgroup takes its row only if the row's configuration is its own
         RowConfigs rows;
         rows.T = per_row->temperature;
         rows.k = per_row->top_k;
@@ -390,26 +412,18 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.freq = per_row->frequency_penalty;
         rows.pres = per_row->presence_penalty;
         rows.path = s->path;
-        // which kernels run: all that the shape and the handle's kernel selection allow, or those the caller's promise
-        // about the kinds of row leaves (mapped through the same rules: under path 1 every row is the general kernel's)
-        const unsigned able = (s->path != 1 && vocab <= ROW_MAX_VOCAB ? 1u : 0u) | (s->path != 1 ? 2u : 0u) | 4u;
-        unsigned want = per_row->row_kinds ? (per_row->row_kinds & 7u) : 7u;
-        if (want & ~able) want |= 4u;                                // rows whose own kernel cannot run here go to the general one
-        rows.launched = want & able;
-        if (rows.launched & 1u) keep_first(launch_topk_row(a, st, &rows));
-        if (rows.launched & 2u) keep_first(launch_nucleus_row(a, st, &rows));
-        if (rows.launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
+        rows.launched = launched;
+        if (launched & 1u) keep_first(launch_topk_row(a, st, &rows));
+        if (launched & 2u) keep_first(launch_nucleus_row(a, st, &rows));
+        if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
+    } else if (launched == 1u) {
+        keep_first(launch_topk_row(a, st));
+    } else if (launched == 2u) {
+        keep_first(launch_nucleus_row(a, st));
     } else {
-        const bool boosts = (history && a.rep < 1.0f) || raises;   // (repetition_penalty < 1 raises the positive logits)
-        if (s->path != 1 && a.top_k >= 1 && a.top_k <= TOPK_MAX_K && vocab <= ROW_MAX_VOCAB && !boosts) {
-            keep_first(launch_topk_row(a, st));          // one launch: one workgroup per row proves and finishes it
-        } else if (s->path != 1 && a.top_k == 0) {
-            keep_first(launch_nucleus_row(a, st));       // no top-k cut: the lean three-sweep kernel, one launch
-        } else {
-            keep_first(launch_sample_wide(a, st));
-        }
+        keep_first(launch_sample_wide(a, st));
     }
-    if (counted) keep_first(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st));
+    if (table) keep_first(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st));
     if (launch_err != hipSuccess) return hip_fail(launch_err, "sample: kernel launch");
     if (!uniforms) s->step++;
     return BORN_ROCM_OK;

@@ -63,6 +63,12 @@ __device__ __forceinline__ float penalise_seen(float x, float r, const unsigned 
     if (counts) y = __fsub_rn(__fsub_rn(y, __fmul_rn(freq, (float)counts[id])), pres);
     return y;
 }
+// The same with the occurrence count at hand.
+__device__ __forceinline__ float penalise_counted(float x, float r, bool counted, unsigned count, float freq, float pres) {
+    float y = penalise(x, r);
+    if (counted) y = __fsub_rn(__fsub_rn(y, __fmul_rn(freq, (float)count)), pres);
+    return y;
+}
 
 // z from a (possibly penalised) logit: temperature then canonicalisation
 __device__ __forceinline__ float z_of(float y, float T) { return canon(T == 1.0f ? y : y / T); }

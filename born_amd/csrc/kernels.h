@@ -6,6 +6,7 @@
 namespace born {
 
 // The single-pass top-k kernel (one workgroup per row).
+constexpr int TOPK_LOCAL_COUNT_HISTORY = 4096;   // longest history whose occurrences it counts in LDS
 constexpr int TOPK_MAX_K = 128;            // largest top_k it serves (its last wave holds two survivors per lane)
 constexpr int ROW_MAX_VOCAB = 393216;      // largest vocabulary it takes (its history bitmap is 48 KiB of LDS)
 
@@ -55,6 +56,9 @@ struct SampleArgs {
     // frequency / presence penalties: how often each id occurs in its row's history, [B, V] (null: both are off)
     const unsigned *hist_counts;
     float freq, pres;
+    // the single-pass kernel counts the occurrences itself (in the hash of the history it builds anyway) and no
+    // table is passed: histories of at most TOPK_LOCAL_COUNT_HISTORY tokens
+    int local_counts;
 };
 
 // Per-row configurations (device arrays of B values, each optional): a second argument of the per-row kernel

@@ -59,7 +59,7 @@ __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const Row
         invalid = true;
         route = ROUTE_GENERAL;
     } else if (rc.path != 1 && v.top_k >= 1 && v.top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && v.rep < 1.0f) &&
-               !(a.hist_counts && (v.freq < 0.0f || v.pres < 0.0f))) {
+               !((a.hist_counts || a.local_counts) && (v.freq < 0.0f || v.pres < 0.0f))) {
         route = ROUTE_TOPK;
     } else if (rc.path != 1 && v.top_k == 0) {
         route = ROUTE_NUCLEUS;

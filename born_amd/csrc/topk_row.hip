@@ -40,6 +40,18 @@ constexpr int ROW_MARGIN = 16;                // candidates kept beyond top_k
 constexpr int ROW_HSLOTS = 2048;              // slots of the history hash (at most ROW_BLOCK tokens: load factor <= 0.5)
 __device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 __device__ __forceinline__ u32 row_hhash(u32 id) { return (id * 2654435761u) >> (32 - 11); }
+// A slot of a history hash: id + 1 in the low bits, the number of occurrences above them (kept only when the
+// frequency / presence penalties are counted by the kernel itself).
+constexpr int HSLOT_ID_BITS = 19;
+constexpr u32 HSLOT_ID_MASK = (1u << HSLOT_ID_BITS) - 1u;
+static_assert(ROW_MAX_VOCAB < (int)HSLOT_ID_MASK, "id + 1 fits the low bits of a slot");
+static_assert(TOPK_LOCAL_COUNT_HISTORY < (1 << (32 - HSLOT_ID_BITS)), "an occurrence count fits the high bits of a slot");
+constexpr int FB_HSLOTS = 2 * TOPK_LOCAL_COUNT_HISTORY;   // slots of the exact selection's history hash (load factor <= 0.5)
+__device__ __forceinline__ u32 fb_hhash(u32 id) { return (id * 2654435761u) >> (32 - 13); }
+static_assert(FB_HSLOTS == (1 << 13), "fb_hhash produces 13 bits");
+// The id + 1 of a slot; slots hold nothing else unless the kernel counts (LOCAL).
+template <bool LOCAL>
+__device__ __forceinline__ u32 hslot_id(u32 e) { return LOCAL ? (e & HSLOT_ID_MASK) : e; }
 static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS == 2 * ROW_BLOCK, "row_hhash produces 11 bits; two slots per thread to clear");
 static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
 static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
@@ -64,6 +76,7 @@ static_assert(OFF_FB_SORTED + TOPK_MAX_K <= ROW_POOL, "selection layout fits the
 static_assert(TOPK_MAX_K <= 2 * WAVE, "the last wave holds at most two survivors per lane");
 static_assert(FB_LIST_CAP <= ROW_BLOCK, "one thread per gathered key");
 static_assert((long long)FB_BITMAP * 64 >= ROW_MAX_VOCAB, "one bitmap bit per id");
+static_assert(FB_HSLOTS / 2 <= FB_BITMAP, "the history hash takes the bitmap's place");
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -161,7 +174,7 @@ __device__ __forceinline__ void row_foreach(const float *x, int V, int tid, F f)
 
 // Exact selection of the row's top_k rank keys for any input (every thread of the workgroup calls it).
 // pool: the workgroup's LDS pool; s_n, s_x: two shared ints.
-template <bool VEC>
+template <bool VEC, bool LOCAL>
 __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, const float *x, int hlen, const int *h, float u_row,
                                                  u64 *pool, int *s_n, int *s_x) {
     const int tid = threadIdx.x, V = a.V, k = a.top_k;
@@ -170,9 +183,26 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     u64 *list = pool + OFF_FB_LIST;
     u64 *sorted = pool + OFF_FB_SORTED;
     const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
-    const bool penal = (a.rep != 1.0f || counts) && hlen > 0;
+    constexpr bool local = LOCAL;                                    // occurrences are counted here, in a hash of the history
+    const bool counted = counts || local;
+    const bool penal = (a.rep != 1.0f || counted) && hlen > 0;
     __syncthreads();                                                 // the proof's use of the pool is over
-    if (penal) {
+    if (penal && local) {
+        for (int i = tid; i < FB_HSLOTS; i += ROW_BLOCK) bm[i] = 0u;
+        __syncthreads();
+        for (int i = tid; i < min(hlen, TOPK_LOCAL_COUNT_HISTORY); i += ROW_BLOCK) {   // at most half the slots get taken
+            const int t = h[i];
+            if (t < 0 || t >= V) continue;
+            u32 slot = fb_hhash((u32)t);
+            for (;;) {
+                const u32 old = atomicCAS(&bm[slot], 0u, (u32)t + 1u);
+                if (old == 0u || (old & HSLOT_ID_MASK) == (u32)t + 1u) break;
+                slot = (slot + 1) & (FB_HSLOTS - 1);
+            }
+            atomicAdd(&bm[slot], 1u << HSLOT_ID_BITS);
+        }
+        __syncthreads();
+    } else if (penal) {
         for (int i = tid; i < ((V + 31) >> 5); i += ROW_BLOCK) bm[i] = 0u;
         __syncthreads();
         for (int i = tid; i < hlen; i += ROW_BLOCK) {
@@ -183,7 +213,20 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
     auto rank_key = [&](int j, float xv) -> u64 {
         float y = xv;
-        if (penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, a.rep, counts, j, a.freq, a.pres);
+        if (penal && local) {
+            u32 slot = fb_hhash((u32)j);
+            for (;;) {
+                const u32 e = bm[slot];
+                if (e == 0u) break;
+                if ((e & HSLOT_ID_MASK) == (u32)j + 1u) {
+                    y = penalise_counted(y, a.rep, true, e >> HSLOT_ID_BITS, a.freq, a.pres);
+                    break;
+                }
+                slot = (slot + 1) & (FB_HSLOTS - 1);
+            }
+        } else if (penal && ((bm[j >> 5] >> (j & 31)) & 1u)) {
+            y = penalise_seen(y, a.rep, counts, j, a.freq, a.pres);
+        }
         return make_key64(z_of(y, a.T), j);
     };
     // radix descent: after each sweep the wanted key is the need-th largest inside the bucket `prefix`
@@ -256,7 +299,8 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
 }
 
-template <bool VEC>
+// LOCAL: the frequency / presence penalties are on and the kernel counts the occurrences itself (SampleArgs::local_counts).
+template <bool VEC, bool LOCAL>
 __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ u64 pool[ROW_POOL];
     uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= Tw
@@ -303,8 +347,11 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
     // probe it at the end; a longer one probes a hash of the candidates instead.
     const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
-    const bool penal = (a.rep != 1.0f || counts) && hlen > 0;
+    constexpr bool local = LOCAL;                                    // occurrences are counted here, not read from a table
+    const bool counted = counts || local;
+    const bool penal = (a.rep != 1.0f || counted) && hlen > 0;
     const bool hfast = penal && hlen <= ROW_BLOCK;
+    u32 *const ccnt = htab;                                          // a long history: occurrences by candidate (the hash is unused then)
     htab[tid] = 0u;
     htab[tid + ROW_BLOCK] = 0u;
 
@@ -338,9 +385,10 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             u32 slot = row_hhash((u32)h0);
             for (;;) {
                 const u32 old = atomicCAS(&htab[slot], 0u, (u32)h0 + 1u);
-                if (old == 0u || old == (u32)h0 + 1u) break;        // inserted, or a duplicate of an earlier occurrence
+                if (old == 0u || hslot_id<LOCAL>(old) == (u32)h0 + 1u) break;   // inserted, or a duplicate of an earlier occurrence
                 slot = (slot + 1) & (ROW_HSLOTS - 1);
             }
+            if (local) atomicAdd(&htab[slot], 1u << HSLOT_ID_BITS);
         }
     }
     const u32 twkey = row_pick(s_wthr, need);
@@ -449,6 +497,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
                 if (e == 0u) break;
                 if ((C[e - 1].y & 0x7FFFFFFFu) == (u32)tk) {
                     atomicOr(&C[e - 1].y, 0x80000000u);
+                    if (local) atomicAdd(&ccnt[e - 1], 1u);
                     break;
                 }
                 slot = (slot + 1) & (ROW_SLOTS - 1);
@@ -467,18 +516,25 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             const uint2 c = C[tid];
             float y = __uint_as_float(c.x);
             bool seen = (c.y & 0x80000000u) != 0u;
+            u32 occ = 0u;
             if (hfast) {                                             // is the candidate's id in the hashed history?
                 u32 slot = row_hhash(c.y);
                 for (;;) {
                     const u32 e = htab[slot];
-                    if (e == 0u || e == c.y + 1u) {
+                    if (e == 0u || hslot_id<LOCAL>(e) == c.y + 1u) {
                         seen = e != 0u;
+                        if (local) occ = e >> HSLOT_ID_BITS;
                         break;
                     }
                     slot = (slot + 1) & (ROW_HSLOTS - 1);
                 }
+            } else if (local) {
+                occ = ccnt[tid];
             }
-            if (seen) y = penalise_seen(y, a.rep, counts, (int)(c.y & 0x7FFFFFFFu), a.freq, a.pres);
+            if (seen) {
+                if (counts) occ = counts[c.y & 0x7FFFFFFFu];
+                y = penalise_counted(y, a.rep, counted, occ, a.freq, a.pres);
+            }
             const float z = z_of(y, a.T);
             keep = ordkey(z) > zb;
             K[tid] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
@@ -490,7 +546,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     BORN_STAMP(a, row, 5);
     ok = ok && s_valid >= k;
     if (!ok) {                                                       // wave-uniform, workgroup-uniform
-        row_select_exact<VEC>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
+        row_select_exact<VEC, LOCAL>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
         return;
     }
 
@@ -525,12 +581,12 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 #endif
 }
 
-template <bool VEC>
+template <bool VEC, bool LOCAL>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
-    topk_row_body<VEC>(a);
+    topk_row_body<VEC, LOCAL>(a);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
-template <bool VEC>
+template <bool VEC, bool LOCAL>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, RowConfigs rc) {
     bool invalid;
     if (!row_config(a, rc, (int)blockIdx.x, ROUTE_TOPK, invalid)) return;   // workgroup-uniform, before any barrier
@@ -538,21 +594,24 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, 
         row_config_reject(a, (int)blockIdx.x);
         return;
     }
-    topk_row_body<VEC>(a);
+    topk_row_body<VEC, LOCAL>(a);
+}
+
+template <bool VEC, bool LOCAL>
+static void launch_topk_row_as(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
+    const dim3 gr((unsigned)a.B), bl(ROW_BLOCK);
+    if (rows)
+        hipLaunchKernelGGL((topk_row_rows_kernel<VEC, LOCAL>), gr, bl, 0, st, a, *rows);
+    else
+        hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL>), gr, bl, 0, st, a);
 }
 
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
     const bool vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
-    const dim3 gr((unsigned)a.B), bl(ROW_BLOCK);
-    if (rows) {
-        if (vec)
-            hipLaunchKernelGGL(topk_row_rows_kernel<true>, gr, bl, 0, st, a, *rows);
-        else
-            hipLaunchKernelGGL(topk_row_rows_kernel<false>, gr, bl, 0, st, a, *rows);
-    } else if (vec) {
-        hipLaunchKernelGGL(topk_row_kernel<true>, gr, bl, 0, st, a);
+    if (vec) {
+        if (a.local_counts) launch_topk_row_as<true, true>(a, st, rows); else launch_topk_row_as<true, false>(a, st, rows);
     } else {
-        hipLaunchKernelGGL(topk_row_kernel<false>, gr, bl, 0, st, a);
+        if (a.local_counts) launch_topk_row_as<false, true>(a, st, rows); else launch_topk_row_as<false, false>(a, st, rows);
     }
     return hipGetLastError();
 }

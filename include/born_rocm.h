@@ -133,8 +133,9 @@ int born_rocm_sample(born_sampler *s, const float *logits, int64_t batch, int64_
  * min_p outside [0, 1), a frequency or presence penalty that is not finite) gets token 0 and BORN_ROCM_ERR_DATA
  * from born_rocm_sampler_status.  Every row's result equals what born_rocm_sample returns for that row under a
  * handle configured with the row's values.  Per-row frequency or presence penalties use the handle's table of
- * counters; a handle not configured with either allocates it on the first such call (which synchronises the
- * stream, so make that call outside a graph capture).  No counterpart in the reference snapshot. */
+ * counters (unless row_kinds promises small top-k rows only and hist_stride <= 4096: that kernel counts by itself);
+ * a handle not configured with either allocates it on the first such call (which synchronises the stream, so make
+ * that call outside a graph capture).  No counterpart in the reference snapshot. */
 typedef struct born_sampler_row_configs {
     const float   *temperature;
     const int32_t *top_k;

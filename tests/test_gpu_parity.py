@@ -376,6 +376,10 @@ def test_min_p_is_validated(rocm):
     (8, 50000, 1.0, 20000, 0.8, 1.0, 300, 0.5, 0.5, "general"),
     (8, 1001, 1.0, 0, 0.9, 1.0, 5000, 0.05, 1.0, "nucleus"),     # unaligned rows, history much longer than the vocabulary
     (8, 1001, 1.0, 10, 0.9, 1.0, 5000, 0.05, 1.0, "topk"),
+    (12, 50257, 0.8, 100, 0.95, 1.1, 4096, 0.02, 0.4, "topk"),    # the longest history counted inside the kernel
+    (12, 50257, 0.8, 100, 0.95, 1.1, 4097, 0.02, 0.4, "topk"),    # one more: the table of counts
+    (16, 32000, 1.0, 40, 0.95, 1.0, 1024, 0.5, 0.1, "topk"),      # the longest history hashed whole
+    (16, 32000, 1.0, 40, 0.95, 1.0, 1025, 0.5, 0.1, "topk"),
 ])
 def test_frequency_and_presence_penalties_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, freq, pres, route, path):
     rng = np.random.default_rng(B * 104729 + V + H)
@@ -429,16 +433,19 @@ def test_frequency_penalty_table_is_clean_between_calls(oracle, rocm):
         h.Close()
 
 
-def test_frequency_penalty_rows_the_single_pass_kernel_cannot_prove(oracle, rocm):
+@pytest.mark.parametrize("H", [400, 3000, 4096, 5000])
+def test_frequency_penalty_rows_the_single_pass_kernel_cannot_prove(oracle, rocm, H):
     # fewer finite logits than top_k, and heavy ties: the workgroup finishes by its exact selection, which penalises
-    # every element it ranks
-    rng = np.random.default_rng(78)
-    B, V, H = 8, 5000, 400
+    # every element it ranks (occurrences counted in its own hash of the history up to 4096 tokens, read from the
+    # handle's table beyond)
+    rng = np.random.default_rng(78 + H)
+    B, V = 8, 5000
     x = np.full((B, V), -np.inf, dtype=np.float32)
     x[:, :30] = rng.standard_normal((B, 30), dtype=np.float32)
     x[4:] = np.float32(1.0)                                                # every logit ties
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, 40, size=(B, H)).astype(np.int32)
+    hist[1::2] = rng.integers(0, V, size=(B // 2, H)).astype(np.int32)    # many distinct ids in every other row
     got, _, _ = _check_against_oracle(oracle, rocm, x, u, 0.8, 50, 0.95, 1.2, hist, nuc=50, freq=0.01, pres=0.02)
     assert got["counters"]["fallback_rows"] > 0
 

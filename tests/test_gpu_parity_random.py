@@ -27,7 +27,7 @@ def _draw_case(rng):
     min_p = float(rng.choice([0.0, 0.0, 0.0, 0.01, 0.05, 0.3, 0.9]))
     freq = float(rng.choice([0.0, 0.0, 0.0, 0.1, 0.7, -0.2]))
     pres = float(rng.choice([0.0, 0.0, 0.0, 0.2, 1.5, -0.3]))
-    H = int(rng.choice([0, 0, 1, 5, 64, 500, 1024, 1025, 3000]))
+    H = int(rng.choice([0, 0, 1, 5, 64, 500, 1024, 1025, 3000, 4096, 4097, 6000]))
     scale = float(rng.choice([0.1, 1.0, 2.0, 6.0]))
     special = str(rng.choice(["none", "none", "none", "mask", "ties", "nan_inf", "few_finite", "flat"]))
     return dict(B=B, V=V, T=T, k=k, p=p, rep=rep, min_p=min_p, freq=freq, pres=pres, H=H, scale=scale, special=special)
