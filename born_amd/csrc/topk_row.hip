@@ -23,6 +23,10 @@
 // keys are unique), 11 bits per sweep of the row, until the top_k keys and the rest of the last
 // bucket fit a list; then the same rank sort and last wave.  The sweeps re-read the row from the
 // caches.
+// Frequency / presence penalties need the number of occurrences of a candidate in the history.  For
+// histories of at most TOPK_LOCAL_COUNT_HISTORY tokens the LOCAL instances count them where the
+// history is hashed anyway (the count rides in the high bits of the slot); otherwise the counts
+// come from a table by id that the caller's launches raise and clear around this one.
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
