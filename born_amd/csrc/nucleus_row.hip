@@ -275,6 +275,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             const bool pass = (!(y < lo0) && !(y > hi0)) || (!(y < lo1) && !(y > hi1)) || (!(y < lo2) && !(y > hi2));
             const u64 mk = __ballot(pass);
             if (mk) {                                                // wave-uniform
+                // A lane that sat out earlier visits (the row's last whole float4 blocks end inside the wave, its ragged
+                // tail starts again at lane 0) has missed their appends; lane 0 takes part whenever any lane of its wave
+                // does, so its count is the wave's.
+                count = (u32)__builtin_amdgcn_readfirstlane((int)count);
                 if (pass) {
                     const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
                     if (pos < (u32)NUC_WCAP) list[pos] = make_uint2(__float_as_uint(y), (u32)j);

@@ -556,6 +556,63 @@ def test_cross_entropy_loss_mirror(oracle, rocm):
     crit.Close()
 
 
+@pytest.mark.parametrize("V,pad", [(7, 5), (7, 1), (6, 2), (4102, 2), (4103, 1), (8198, 2)])
+def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pad):
+    # 16-byte aligned rows whose length is not a multiple of four, with the whole float4 blocks ending at lane 0 or 1 of a
+    # wave: the ragged tail restarts at lane 0, next to lanes that sat out the last block.  Few distinct values, so that
+    # the wanted bins take entries from both parts.
+    rng = np.random.default_rng(V * 31 + pad)
+    B, H = 6, 40
+    x = np.round(rng.standard_normal((B, V)) * 0.6).astype(np.float32)
+    x[0, :] = np.float32(0.25)
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+    stride = V + pad
+    assert stride % 4 == 0
+    host = np.full(B * stride + 8, np.nan, dtype=np.float32)
+    for b in range(B):
+        host[b * stride: b * stride + V] = x[b]
+    for (T, p, rep, min_p, freq) in [(5.0, 0.9, 1.0, 0.05, 0.1), (1.0, 0.9, 1.2, 0.0, 0.0), (0.7, 1.0, 1.0, 0.0, 0.0)]:
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=0, TopP=p, RepetitionPenalty=rep, MinP=min_p, FrequencyPenalty=freq),
+                            max_batch=B, max_vocab=V)
+        d_x, d_u, d_h = rocm.DeviceBuffer.from_numpy(host), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer.from_numpy(hist)
+        tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
+        s.Sample(d_x, B, V, d_h, None, d_u, tok, pr, row_stride=stride, hist_stride=H)
+        s.Status()
+        fx = oracle.sample(x, u, T, 0, p, rep, hist, None, mode=oracle.MODE_FIXED, min_p=min_p, freq=freq)
+        assert np.array_equal(tok.to_numpy(np.int32, (B,)), fx["tokens"]), (T, p, rep, min_p, freq)
+        assert np.array_equal(pr.to_numpy(np.float32, (B,)).view(np.uint32), fx["probs"].view(np.uint32))
+        assert s.Counters()["general_rows"] == B
+        s.Close()
+
+
+def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
+    # the case a wide seeded sweep of test_random_row_layouts_against_oracle found (its chunk 1096, third case)
+    import test_gpu_parity_random as R
+    rng = np.random.default_rng(777 + 1096)
+    for _ in range(3):
+        c = R._draw_case(rng)
+        x, u, hist, hist_len = R._inputs(rng, c)
+        rng.choice([0, 1, 3, 4, 5, 64]), rng.choice([0, 1, 2, 3, 4])     # that test's padding and offset draws
+    assert c["V"] == 7 and c["k"] >= c["V"]
+    B, V = x.shape
+    stride = V + 5
+    host = np.full(B * stride + 8, np.nan, dtype=np.float32)
+    host[1::2] = np.inf
+    for b in range(B):
+        host[b * stride: b * stride + V] = x[b]
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=c["T"], TopK=c["k"], TopP=c["p"], RepetitionPenalty=c["rep"], MinP=c["min_p"],
+                                           FrequencyPenalty=c["freq"], PresencePenalty=c["pres"]), max_batch=B, max_vocab=V)
+    d_x, d_u, d_h = rocm.DeviceBuffer.from_numpy(host), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer.from_numpy(hist)
+    tok = rocm.DeviceBuffer(4 * B)
+    s.Sample(d_x, B, V, d_h, None, d_u, tok, None, row_stride=stride, hist_stride=hist.shape[1])
+    s.Status()
+    fx = oracle.sample(x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, mode=oracle.MODE_FIXED, min_p=c["min_p"], freq=c["freq"],
+                       pres=c["pres"])
+    assert np.array_equal(tok.to_numpy(np.int32, (B,)), fx["tokens"])
+    s.Close()
+
+
 @pytest.mark.parametrize("V", [8, 64, 100, 130, 4100])
 def test_three_sweep_kernel_rows_that_end_inside_a_wave(oracle, rocm, V):
     # no top-k cut and a row whose last elements occupy only part of a wave: the lanes that sit out the ragged end
