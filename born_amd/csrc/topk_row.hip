@@ -4,19 +4,21 @@
 // The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 logits, the
 // loads of one stage in flight while the stage before it is examined.
 //
-//   Tw  From the first stage alone: every wave takes the a-th largest of its lane maxima, and the
-//       w-th largest of the wave results has >= w * a >= top_k logits of that stage at or above
-//       it.  So the row's top_k-th largest logit is >= Tw, and only logits >= Tw matter.
-//   L   Every logit >= Tw of the whole row (the first stage included) is appended, exact value
-//       and id, to the list of the wave that met it (ballot + lane rank, no atomics): one
-//       compare per logit in the common case.
-//   T2  Same counting argument over the lists: >= top_k + 16 candidates reach T2 >= Tw.  The
-//       candidates >= T2 (about 2 top_k) are compacted into C.
-//   Any logit outside C is below T2, and so is its z after a penalty (repetition_penalty >= 1
-//   only lowers a logit) and the monotone division by the temperature.  The ids in C are hashed
-//   and probed with the history; the row is proven if top_k candidates end up with z strictly
-//   above that bound.  A rank sort orders them and one wave computes the integer CDF, the top-p
-//   cut and the draw.
+//   T   A threshold that the row's top_k-th largest logit is known to reach.  First from the first stage alone:
+//       every wave takes the a-th largest of its lane maxima, and the w-th largest of the wave results has
+//       >= w * a >= top_k logits of that stage at or above it.
+//   L   Every logit >= T met from then on is appended, exact value and id, to the list of the wave that met it
+//       (ballot + lane rank, no atomics): one compare per logit in the common case.
+//   T'  Every three stages, with the next stages' loads in flight, the lists' entries are binned by key distance
+//       above T (one LDS atomic each); the highest bin boundary with >= top_k + 16 entries at or above it becomes
+//       the new T and every wave drops its entries below it.  The lists so end the pass with little more than
+//       top_k + 16 entries between them, and nothing has to be thinned out after the last load.
+//   Any logit outside the lists is below T, and so is its z after a penalty (repetition_penalty >= 1
+//   only lowers a logit) and the monotone division by the temperature.  Every wave turns its own entries into rank
+//   keys (probing its hash of the history) and appends them to one array; the row is proven if top_k candidates
+//   end up with z strictly above that bound.  A rank sort orders them and one wave computes the integer CDF, the
+//   top-p cut and the draw.  (A history longer than the workgroup is not hashed: the candidates' ids are, and the
+//   history probes them.)
 // Rows that cannot be proven (fewer than top_k finite logits, heavy ties, list overflow, penalised
 // tokens dropping below the bound) are finished by the same workgroup with an exact selection that
 // works for any input: a radix descent over the 64-bit rank keys (z descending, id ascending; the
@@ -38,9 +40,9 @@ constexpr int ROW_BLOCK = 1024;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
 constexpr int ROW_U = 4;                      // 128-bit loads per thread and stage
 constexpr int ROW_WCAP = 256;                 // list entries per wave
-constexpr int ROW_CAP = 512;                  // candidates >= T2 the tail can hold
+constexpr int ROW_CAP = 512;                  // candidates the tail can hold
 constexpr int ROW_SLOTS = 1024;               // hash slots (load factor <= 0.5)
-constexpr int ROW_MARGIN = 16;                // candidates kept beyond top_k
+constexpr int ROW_MARGIN = 16;                // entries a raised threshold keeps beyond top_k
 constexpr int ROW_HSLOTS = 2048;              // slots of the history hash (at most ROW_BLOCK tokens: load factor <= 0.5)
 __device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 __device__ __forceinline__ u32 row_hhash(u32 id) { return (id * 2654435761u) >> (32 - 11); }
@@ -303,20 +305,120 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
 }
 
+// Block indices clamped into the row: a stage that reaches past the row's end (or lies wholly beyond it) re-reads the
+// row's last block instead of branching around its loads, so that the loads of later stages can stay in flight.  The
+// row starts 16-byte aligned and its pitch is a multiple of four floats (VEC), so the last block lies inside the pitch.
+__device__ __forceinline__ void row_load_clamped(f32x4 (&v)[ROW_U], const float *x, int n4, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++) {
+        const int i4 = min((stage * ROW_U + u) * ROW_BLOCK + tid, n4 - 1);
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i4);
+    }
+}
+// row_filter for a stage that may reach past the row's end: elements at or beyond V count as -inf.
+__device__ __forceinline__ void row_filter_masked(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid, int V) {
+    f32x4 m[ROW_U];
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) m[u][c] = (((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c < V) ? v[u][c] : -INFINITY;
+    row_filter(m, tw, list, count, stage, tid);
+}
+
+constexpr int ROW_TBINS = 256;                // bins of the threshold histogram (four per lane)
+static_assert(ROW_TBINS == 4 * WAVE && ROW_TBINS <= ROW_BLOCK, "one 128-bit read per lane covers the bins");
+
+// Raises the threshold in the middle of the pass (every thread of the workgroup calls it, between two stages; global
+// loads stay in flight).  The lists hold every logit >= the threshold among the stages seen so far.  All of their
+// entries are binned by key distance above the threshold; the highest bin boundary with at least `want` entries at
+// or above it is a lower bound of the row's want-th largest logit, so it becomes the new threshold and every wave
+// drops the entries below it from its own list.  The bin width follows the largest key listed one round earlier
+// (`smax`: waves must agree on it, so it cannot be this round's); later, larger keys share the top bin.
+//   H: this round's bins (all zero on entry); Hclear: the next round's bins, zeroed here (with three sets in rotation
+//   they were last read two rounds ago, before the previous round's barrier);
+//   Mnext: where this round's largest key is published for the next round.
+__device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, int want, u32 smax, u32 *H, u32 *Hclear, u32 *Mnext,
+                                            int *s_over, int tid) {
+    const int l = lane_id();
+    if (count > (u32)ROW_WCAP && l == 0) *s_over = 1;
+    const int cw = (int)min(count, (u32)ROW_WCAP);
+    const u32 range = smax > twkey ? smax - twkey : 0u;
+    const int sh = max(0, 24 - (int)__clz(range));                   // (range >> sh) < ROW_TBINS
+    u32 mx = 0u;
+    for (int e = l; e < cw; e += WAVE) {
+        const u32 key = ordkey(__uint_as_float(list[e].x));
+        mx = max(mx, key);
+        if (key >= twkey) atomicAdd(&H[min((key - twkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
+    }
+    mx = wave_max_u32(mx);
+    if (l == 0 && mx) atomicMax(Mnext, mx);
+    if (tid < ROW_TBINS) Hclear[tid] = 0u;
+    lds_barrier();
+    const uint4 h = reinterpret_cast<const uint4 *>(H)[WAVE - 1 - l];   // lane 0 holds the four highest bins
+    const u32 s4 = h.x + h.y + h.z + h.w;
+    const u32 incl = wave_inclusive_scan_u32(s4);                    // entries in this lane's bins and all higher ones
+    const u32 total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
+    if (total < (u32)want) return;                                   // wave-uniform, the same in every wave
+    const int L = __ffsll((long long)__ballot(incl >= (u32)want)) - 1;   // the lane whose bins hold the crossing
+    const u32 excl = (u32)__builtin_amdgcn_readlane((int)(incl - s4), L);
+    const u32 hw = (u32)__builtin_amdgcn_readlane((int)h.w, L), hz = (u32)__builtin_amdgcn_readlane((int)h.z, L);
+    const u32 hy = (u32)__builtin_amdgcn_readlane((int)h.y, L);
+    const u32 need = (u32)want - excl;                               // >= 1
+    int bin = 4 * (WAVE - 1 - L) + 3;
+    u32 c = hw;
+    if (c < need) { bin--; c += hz; if (c < need) { bin--; c += hy; if (c < need) bin--; } }
+    const u32 nk = twkey + ((u32)bin << sh);                         // at most the key of an entry of that bin: no overflow
+    if (nk <= twkey) return;
+    // in-place compaction of the wave's own list: every read is issued before the first write
+    uint2 ent[ROW_WCAP / WAVE];
+    bool keep[ROW_WCAP / WAVE];
+#pragma unroll
+    for (int r = 0; r < ROW_WCAP / WAVE; r++) {
+        const int e = l + r * WAVE;
+        keep[r] = false;
+        if (e < cw) {
+            ent[r] = list[e];
+            keep[r] = ordkey(__uint_as_float(ent[r].x)) >= nk;
+        }
+    }
+    u32 kept = 0u;
+#pragma unroll
+    for (int r = 0; r < ROW_WCAP / WAVE; r++) {
+        if (r * WAVE < cw) {                                         // wave-uniform
+            const u64 m = __ballot(keep[r]);
+            if (keep[r]) list[kept + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u))] = ent[r];
+            kept += (u32)__popcll(m);
+        }
+    }
+    count = kept;
+    twkey = nk;
+}
+
 // LOCAL: the frequency / presence penalties are on and the kernel counts the occurrences itself (SampleArgs::local_counts).
 template <bool VEC, bool LOCAL>
 __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ u64 pool[ROW_POOL];
-    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= Tw
-    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);       // candidates >= T2; .y bit 31 = id occurs in the history
-    u64 *const K = pool + OFF_K;                                     // their rank keys, 0 = dropped
+    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= the threshold
+    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);       // long histories: the candidates; .y bit 31 = id occurs in the history
+    u64 *const K = pool + OFF_K;                                     // the candidates' rank keys
     u32 *const tab = reinterpret_cast<u32 *>(pool + OFF_TAB);
+    u32 *const Khi = tab;                                            // the candidates' z alone, once the hash of their ids has served
     u64 *const sorted = pool + OFF_SORTED;
     u32 *const htab = reinterpret_cast<u32 *>(pool + OFF_HTAB);
-    __shared__ int s_rank[ROW_BLOCK];
-    __shared__ u32 s_wthr[ROW_WAVES], s_wthr2[ROW_WAVES];
-    __shared__ int s_n, s_valid, s_over;
+    __shared__ u32 s_wthr[ROW_WAVES], s_wmax[ROW_WAVES];
+    __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
+    __shared__ u32 s_max[2];
+    __shared__ int s_n, s_valid, s_over, s_next;
     __shared__ int s_x[1 + ROW_WAVES];
+#ifdef BORN_PHASE_TIMING
+    // debug builds: the phase stamps stay in registers until the row is finished (a store per stamp would make every
+    // phase wait for the previous stamp's store)
+    u64 stamp_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const u64 cyc0_ = __builtin_readcyclecounter();
+#define ROW_STAMP(slot) stamp_[slot] = wall_clock64()
+#else
+#define ROW_STAMP(slot) do {} while (0)
+#endif
 
     // Every argument the prologue reads is requested here, in one batch with one wait: left to itself the compiler
     // fetches them where they are first used, three dependent waits before the row's first load is issued.
@@ -329,7 +431,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int n4 = (V + 3) >> 2;
     const int iters = (n4 + ROW_BLOCK - 1) / ROW_BLOCK;             // float4 blocks per thread
     const int nstage = (iters + ROW_U - 1) / ROW_U;
-    const int nfull = VEC ? (V >> 2) / (ROW_U * ROW_BLOCK) : 0;      // stages made of whole float4 blocks inside the row
+    const int nfull = (V >> 2) / (ROW_U * ROW_BLOCK);                // stages made of whole float4 blocks inside the row
 
     // Order of the requests: this thread's first history entry (used last, but loads return in order and it must
     // not wait behind the row), then the row's first three stages; the LDS tables are cleared behind them.
@@ -337,17 +439,25 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
-    if (nfull > 0) row_load_fast(va, x, 0, tid); else row_load_any<VEC>(va, x, V, 0, tid);
-    if (nfull > 1) row_load_fast(vb, x, 1, tid);                     // in flight during the search for Tw
-    if (nfull > 2) row_load_fast(vc, x, 2, tid);
+    if (VEC) {
+        row_load_clamped(va, x, n4, 0, tid);
+        row_load_clamped(vb, x, n4, 1, tid);                         // in flight during the search for the first threshold
+        row_load_clamped(vc, x, n4, 2, tid);
+    } else {
+        row_load_any<false>(va, x, V, 0, tid);
+    }
 
     if (tid == 0) {
         s_n = 0;
         s_valid = 0;
         s_over = 0;
+        s_next = 0;
+        s_max[0] = 0u;
+        s_max[1] = 0u;
     }
     tab[tid] = 0u;
     static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
+    if (tid < ROW_TBINS) s_bins[0][tid] = 0u;                        // every round clears the bins of the next
     // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
     // probe it at the end; a longer one probes a hash of the candidates instead.
     const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
@@ -358,8 +468,9 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     u32 *const ccnt = htab;                                          // a long history: occurrences by candidate (the hash is unused then)
     htab[tid] = 0u;
     htab[tid + ROW_BLOCK] = 0u;
+    if (tid < TOPK_MAX_K) sorted[tid] = 0ull;
 
-    BORN_STAMP(a, row, 0);
+    ROW_STAMP(0);
     // The row's uniform is one scalar load whose result the compiler waits for on the spot: after the row's first
     // loads have been issued, not before them.
     const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
@@ -367,19 +478,32 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // finish): an atomic at the end of the kernel is a memory round trip the launch has to wait for.
     if (tid == 0) count_row(a.counters, row, 0);
 
-    // ---- Tw from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per wave and the
-    // need = ceil(top_k / a)-th largest of the wave results
+    // ---- the first threshold, from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per
+    // wave and the need = ceil(top_k / a)-th largest of the wave results
     const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
     const int aw = min(WAVE, (k + act - 1) / act);                   // lanes of one wave
-    const int need = (k + aw - 1) / aw;                              // <= act, but for top_k > 64 on a row of one wave: no Tw then
+    const int need = (k + aw - 1) / aw;                              // <= act, but for top_k > 64 on a row of one wave: no threshold then
     {
         float lm = -INFINITY;
+        if (nfull > 0) {
 #pragma unroll
-        for (int u = 0; u < ROW_U; u++)
+            for (int u = 0; u < ROW_U; u++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
-        const u32 wk = wave_kth_largest_bound(ordkey(lm), aw, 14);
-        if (lane_id() == 0) s_wthr[wave_id()] = wk;
+                for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
+        } else {                                                     // the row ends inside the first stage
+#pragma unroll
+            for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if ((u * ROW_BLOCK + tid) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
+        }
+        const u32 lk = ordkey(lm);
+        const u32 wk = wave_kth_largest_bound(lk, aw, 14);
+        const u32 wm = wave_max_u32(lk);
+        if (lane_id() == 0) {
+            s_wthr[wave_id()] = wk;
+            s_wmax[wave_id()] = wm;
+        }
     }
     lds_barrier();
     if (hfast && tid < hlen) {
@@ -395,106 +519,107 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             if (local) atomicAdd(&htab[slot], 1u << HSLOT_ID_BITS);
         }
     }
-    const u32 twkey = row_pick(s_wthr, need);
+    u32 twkey = row_pick(s_wthr, need);
+    const u32 max0 = wave_max_u32(lane_id() < ROW_WAVES ? s_wmax[lane_id()] : 0u);   // the largest key of the first stage
     // at or below the key of -inf: fewer than top_k finite logits in the first stage (or a vocabulary too small
-    // for the counting argument); nothing is listed and the row goes to the general kernel
+    // for the counting argument); nothing is listed and the row goes to the exact selection
     const bool have_tw = twkey > ordkey(-INFINITY);
-    const float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
+    float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
+    const int want = k + ROW_MARGIN;                                 // entries a raised threshold keeps at least
 
-    // ---- the pass over the row
+    // ---- the pass over the row.  Every three stages the threshold is raised from what the lists hold by then, so
+    // that they end the pass with little more than `want` entries between them.
     uint2 *list = L + wave_id() * ROW_WCAP;
     u32 count = 0;
-    {
+    int round = 0;
+    auto tighten = [&]() {
+        if (have_tw) {                                               // workgroup-uniform
+            const u32 smax = max(max0, s_max[round & 1]);
+            row_tighten(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+            tw = ordkey_inv(twkey);
+            round++;
+        }
+    };
+    // A history that fits the workgroup was hashed above and the candidates probe it; otherwise the candidates' ids are
+    // hashed and the history probes them.
+    const bool fast = !penal || hfast;
+    // A logit outside the lists has a key of at most twkey - 1 (twkey > the key of -inf, so that is the key of a float
+    // or of -inf), and so has its z: a penalty only lowers a logit and the division by the temperature is monotone.
+    // The row is proven if top_k candidates have z strictly above that bound.
+    u32 zb = 0u;
+    if (VEC) {
+        // at the loop head va, vb, vc = stages s, s + 1, s + 2 are requested: two stages stay in flight while one
+        // is examined.  The stages of the loop lie wholly inside the row; the last three (the last of which may reach
+        // past its end) are examined without new requests.
         int s = 0;
-        if (nfull > 2) {
-            // at the loop head va, vb, vc = stages s, s + 1, s + 2 are requested: two stages stay in flight
-            // while one is examined
-            while (s + 5 < nfull) {
-                row_filter(va, tw, list, count, s, tid);
-                row_load_fast(va, x, s + 3, tid);
-                row_filter(vb, tw, list, count, s + 1, tid);
-                row_load_fast(vb, x, s + 4, tid);
-                row_filter(vc, tw, list, count, s + 2, tid);
-                row_load_fast(vc, x, s + 5, tid);
-                s += 3;
-            }
-            const int r = nfull - s;                                 // 3, 4 or 5 whole stages remain
+        while (s + 3 < nstage) {
             row_filter(va, tw, list, count, s, tid);
-            if (r > 3) row_load_fast(va, x, s + 3, tid);
+            row_load_clamped(va, x, n4, s + 3, tid);
             row_filter(vb, tw, list, count, s + 1, tid);
-            if (r > 4) row_load_fast(vb, x, s + 4, tid);
+            row_load_clamped(vb, x, n4, s + 4, tid);
             row_filter(vc, tw, list, count, s + 2, tid);
-            if (r > 3) row_filter(va, tw, list, count, s + 3, tid);
-            if (r > 4) row_filter(vb, tw, list, count, s + 4, tid);
-            s = nfull;
-        } else {
-            row_filter(va, tw, list, count, 0, tid);                 // the first stage, whole or ragged
-            if (nfull > 1) row_filter(vb, tw, list, count, 1, tid);
-            s = nfull > 1 ? 2 : 1;
+            row_load_clamped(vc, x, n4, s + 5, tid);
+            s += 3;
+            tighten();
         }
-        for (; s < nstage; s++) {
-            row_load_any<VEC>(va, x, V, s, tid);
+        if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T)); // the threshold is final
+        auto last_stages = [&](const f32x4 (&v)[ROW_U], int st) {
+            if (st >= nstage) return;                                // wave-uniform
+            if (st < nfull) row_filter(v, tw, list, count, st, tid); else row_filter_masked(v, tw, list, count, st, tid, V);
+        };
+        last_stages(va, s);
+        last_stages(vb, s + 1);
+        last_stages(vc, s + 2);
+    } else {
+        // rows that 128-bit loads cannot take: one stage at a time, then one raise of the threshold
+        row_filter(va, tw, list, count, 0, tid);
+        for (int s = 1; s < nstage; s++) {
+            row_load_any<false>(va, x, V, s, tid);
             row_filter(va, tw, list, count, s, tid);
         }
+        tighten();
+        if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));
     }
     if (count > (u32)ROW_WCAP && lane_id() == 0) s_over = 1;
     const int cw = (int)min(count, (u32)ROW_WCAP);
+    ROW_STAMP(1);
+#ifdef BORN_PHASE_TIMING
+    __shared__ u64 s_wend[ROW_WAVES];
+    if (lane_id() == 0) s_wend[wave_id()] = stamp_[1];
+#endif
 
-    BORN_STAMP(a, row, 1);
-    // ---- T2 over the lists: a2 lanes per wave, need2-th largest of the wave results.  A wave with fewer than
-    // a2 lanes holding a candidate reports 0.
-    const int want = k + ROW_MARGIN;
-    const int a2 = (want + ROW_WAVES - 1) / ROW_WAVES;
-    const int need2 = (want + a2 - 1) / a2;
+    // ---- C: every wave moves its entries into one array (one LDS atomic per wave reserves the range).  What follows
+    // is the work of as many threads as there are candidates, so most waves only pass the barriers: an instruction
+    // that all sixteen waves execute costs the compute unit sixteen issue slots.
     {
-        u32 best = 0u;
-        for (int e = lane_id(); e < cw; e += WAVE) best = max(best, ordkey(__uint_as_float(list[e].x)));
-        const int lanes = __popcll(__ballot(best != 0u));            // every entry is >= tw
-        const u32 wk = lanes >= a2 ? wave_kth_largest_bound(best, a2, 14, twkey) : 0u;
-        if (lane_id() == 0) s_wthr2[wave_id()] = wk;
-    }
-    __syncthreads();
-    const u32 t2key = max(twkey, row_pick(s_wthr2, need2));         // at least top_k logits reach it either way
-
-    // ---- C: compact the list entries >= T2 (a wave reserves its range with one LDS atomic)
-    {
-        int cnt = 0;
-        for (int e = lane_id(); e < cw; e += WAVE) cnt += ordkey(__uint_as_float(list[e].x)) >= t2key ? 1 : 0;
-        const u32 incl = wave_inclusive_scan_u32((u32)cnt);
-        const u32 total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
-        u32 base = 0;
-        if (lane_id() == 0 && total) base = (u32)atomicAdd(&s_n, (int)total);
+        u32 base = 0u;
+        if (lane_id() == 0 && cw) base = (u32)atomicAdd(&s_n, cw);
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
-        u32 pos = base + incl - (u32)cnt;
         for (int e = lane_id(); e < cw; e += WAVE) {
-            const uint2 c = list[e];
-            if (ordkey(__uint_as_float(c.x)) >= t2key) {
-                if (pos < (u32)ROW_CAP) {
-                    C[pos] = c;
-                    if (penal && !hfast) {                           // a long history probes a hash of the candidate ids
-                        u32 slot = row_hash(c.y);
-                        while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
-                    }
+            const u32 pos = base + (u32)e;
+            if (pos < (u32)ROW_CAP) {
+                const uint2 c = list[e];
+                C[pos] = c;
+                if (!fast) {                                         // a long history probes a hash of the candidate ids
+                    u32 slot = row_hash(c.y);
+                    while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
                 }
-                pos++;
             }
         }
     }
     __syncthreads();
-    BORN_STAMP(a, row, 2);
+    ROW_STAMP(2);
     const int n = s_n;
     bool ok = have_tw && !s_over && n >= k && n <= ROW_CAP;
-
-    BORN_STAMP(a, row, 3);
-    if (!hfast) {
-        // long (or unpenalised) history: report ids out of range, flag the candidates that were already emitted
+    if (!fast) {
+        // report ids out of range, flag the candidates that were already emitted
         for (int i = tid; i < hlen; i += ROW_BLOCK) {
             const int tk = (i == tid) ? h0 : h[i];
             if (tk < 0 || tk >= V) {
                 atomicOr(a.status, 1);
                 continue;
             }
-            if (!(ok && penal)) continue;
+            if (!ok) continue;
             u32 slot = row_hash((u32)tk);
             for (;;) {
                 const u32 e = tab[slot];
@@ -509,78 +634,90 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         }
         __syncthreads();
     }
-    BORN_STAMP(a, row, 4);
-
-    // ---- exact z; the row is proven if top_k candidates stay strictly above the bound.  A logit outside C has
-    // a key of at most T2 - 1 (T2 > the key of -inf, so that is the key of a float or of -inf).
-    if (ok) {
-        const u32 zb = ordkey(z_of(ordkey_inv(t2key - 1u), a.T));
-        bool keep = false;
-        if (tid < n) {
-            const uint2 c = C[tid];
-            float y = __uint_as_float(c.x);
-            bool seen = (c.y & 0x80000000u) != 0u;
-            u32 occ = 0u;
-            if (hfast) {                                             // is the candidate's id in the hashed history?
-                u32 slot = row_hhash(c.y);
-                for (;;) {
-                    const u32 e = htab[slot];
-                    if (e == 0u || hslot_id<LOCAL>(e) == c.y + 1u) {
-                        seen = e != 0u;
-                        if (local) occ = e >> HSLOT_ID_BITS;
-                        break;
-                    }
-                    slot = (slot + 1) & (ROW_HSLOTS - 1);
+    // ---- exact z and rank key of every candidate, one thread each
+    if (ok && tid < n) {
+        const uint2 c = C[tid];
+        float y = __uint_as_float(c.x);
+        bool seen = (c.y & 0x80000000u) != 0u;
+        u32 occ = 0u;
+        if (hfast) {                                                 // is the candidate's id in the hashed history?
+            u32 slot = row_hhash(c.y);
+            for (;;) {
+                const u32 en = htab[slot];
+                if (en == 0u || hslot_id<LOCAL>(en) == c.y + 1u) {
+                    seen = en != 0u;
+                    if (local) occ = en >> HSLOT_ID_BITS;
+                    break;
                 }
-            } else if (local) {
-                occ = ccnt[tid];
+                slot = (slot + 1) & (ROW_HSLOTS - 1);
             }
-            if (seen) {
-                if (counts) occ = counts[c.y & 0x7FFFFFFFu];
-                y = penalise_counted(y, a.rep, counted, occ, a.freq, a.pres);
-            }
-            const float z = z_of(y, a.T);
-            keep = ordkey(z) > zb;
-            K[tid] = keep ? make_key64(z, (int)(c.y & 0x7FFFFFFFu)) : 0ull;
+        } else if (local) {
+            occ = ccnt[tid];
         }
-        const int nk = __popcll(__ballot(keep));                     // one uniform add per wave
-        if (lane_id() == 0 && nk) atomicAdd(&s_valid, nk);
+        if (seen) {
+            if (counts) occ = counts[c.y & 0x7FFFFFFFu];
+            y = penalise_counted(y, a.rep, counted, occ, a.freq, a.pres);
+        }
+        const float z = z_of(y, a.T);
+        K[tid] = make_key64(z, (int)(c.y & 0x7FFFFFFFu));
+        Khi[tid] = ordkey(z);
+        const int nk = __popcll(__ballot(ordkey(z) > zb));           // the active lanes of this wave
+        if (nk && lane_id() == 0) atomicAdd(&s_valid, nk);           // (lane 0 is active whenever a lane of its wave is)
     }
+    if (ok && tid >= n && tid < ((n + 31) & ~31)) Khi[tid] = 0u;     // the rank sort reads z in groups of 32: below any real one
     __syncthreads();
-    BORN_STAMP(a, row, 5);
+    ROW_STAMP(3);
     ok = ok && s_valid >= k;
     if (!ok) {                                                       // wave-uniform, workgroup-uniform
         row_select_exact<VEC, LOCAL>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
         return;
     }
 
-    // ---- rank sort: every key counts the keys above it (keys are unique); the comparisons of one key are
-    // split over ROW_BLOCK / np threads
-    {
-        const int np = next_pow2(n), parts = ROW_BLOCK / np;         // n <= ROW_CAP < ROW_BLOCK: parts >= 2
-        const int e = tid & (np - 1), part = tid / np;
-        const int len = (n + parts - 1) / parts;
-        int r = 0;
-        if (e < n) {
-            const u64 key = K[e];
-            const int j1 = min(n, (part + 1) * len);
-#pragma unroll 8
-            for (int j = part * len; j < j1; j++) r += K[j] > key ? 1 : 0;
+    // ---- rank sort: every candidate counts the candidates with a larger z (32-bit compares; 64-bit ones run at a
+    // quarter of the rate) and the top_k take their place in rank order.  Candidates with equal z would count the same
+    // and leave the next place empty (`sorted` starts as zeros, no key is zero): the first wave then repeats the count
+    // with the whole keys (z descending, id ascending; unique).  Equal z across the cut shows as nobody counting
+    // exactly top_k.
+    if (tid < n) {
+        const u32 khi = Khi[tid];
+        const uint4 *K4 = reinterpret_cast<const uint4 *>(Khi);      // wave-uniform addresses: four z per read,
+        int r = 0;                                                   // eight reads in flight
+        for (int q = 0; q < ((n + 31) >> 5) * 8; q += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) v[t] = K4[q + t];
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                r += (v[t].x > khi ? 1 : 0) + (v[t].y > khi ? 1 : 0) + (v[t].z > khi ? 1 : 0) + (v[t].w > khi ? 1 : 0);
         }
-        s_rank[tid] = r;
-        __syncthreads();
-        if (tid < n && K[tid] != 0ull) {
-            int rr = 0;
-            for (int q = 0; q < parts; q++) rr += s_rank[q * np + tid];
-            if (rr < k) sorted[rr] = K[tid];
-        }
+        if (r < k) sorted[r] = K[tid];
+        else if (r == k) s_next = 1;
     }
     __syncthreads();
-    BORN_STAMP(a, row, 6);
-    if (tid < WAVE) finish_sorted_by_wave(sorted, k, a, row, u_row);
-    BORN_STAMP(a, row, 7);
+    ROW_STAMP(6);
+    if (tid >= WAVE) return;                                         // the first wave alone goes on
+    {
+        bool hole = false;
+        for (int i = tid; i < k; i += WAVE) hole |= sorted[i] == 0ull;
+        if (__ballot(hole) != 0ull || (n > k && s_next == 0)) {      // wave-uniform
+            for (int c = tid; c < n; c += WAVE) {
+                const u64 key = K[c];
+                int r = 0;
+                for (int j = 0; j < n; j++) r += K[j] > key ? 1 : 0;
+                if (r < k) sorted[r] = key;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+    finish_sorted_by_wave(sorted, k, a, row, u_row);
+    ROW_STAMP(7);
 #ifdef BORN_PHASE_TIMING
-    if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)s_valid; }
+    for (int w = 0; w < ROW_WAVES; w++) stamp_[5] = max(stamp_[5], s_wend[w]);   // the last wave to end its pass
+    if (tid == 0)
+        for (int i = 0; i < 8; i++) a.counters[COUNTER_ROW_BASE + COUNTER_ROW_STRIDE * row + i] = stamp_[i];
+    if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)round; a.counters[8 + 19] = __builtin_readcyclecounter() - cyc0_; a.counters[8 + 20] = stamp_[7] - stamp_[0]; }
     if (lane_id() == 0) atomicAdd(&a.counters[8 + 18], (u64)count);
 #endif
 }
