@@ -36,9 +36,12 @@
 
 namespace born {
 
-constexpr int ROW_BLOCK = 1024;
+#ifndef BORN_ROW_BLOCK
+#define BORN_ROW_BLOCK 1024
+#endif
+constexpr int ROW_BLOCK = BORN_ROW_BLOCK;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
-constexpr int ROW_U = 4;                      // 128-bit loads per thread and stage
+constexpr int ROW_U = 4096 / ROW_BLOCK;       // 128-bit loads per thread and stage: a stage is 16384 logits
 constexpr int ROW_WCAP = 256;                 // list entries per wave
 constexpr int ROW_CAP = 512;                  // candidates the tail can hold
 constexpr int ROW_SLOTS = 1024;               // hash slots (load factor <= 0.5)
@@ -58,13 +61,13 @@ static_assert(FB_HSLOTS == (1 << 13), "fb_hhash produces 13 bits");
 // The id + 1 of a slot; slots hold nothing else unless the kernel counts (LOCAL).
 template <bool LOCAL>
 __device__ __forceinline__ u32 hslot_id(u32 e) { return LOCAL ? (e & HSLOT_ID_MASK) : e; }
-static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS == 2 * ROW_BLOCK, "row_hhash produces 11 bits; two slots per thread to clear");
+static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS >= 2 * ROW_BLOCK, "row_hhash produces 11 bits; load factor <= 0.5");
 static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
 static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
 static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
 
 // LDS pool (u64 words), laid out once for the proof and once for the exact selection
-constexpr int ROW_POOL = 8064;
+constexpr int ROW_POOL = 8064 + (ROW_BLOCK < 1024 ? 2048 : 0);   // (a smaller workgroup pads its pool so that a compute unit holds one)
 constexpr int OFF_L = 0;                      // [ROW_WAVES][ROW_WCAP] uint2
 constexpr int OFF_C = OFF_L + ROW_WAVES * ROW_WCAP;   // [ROW_CAP] uint2
 constexpr int OFF_K = OFF_C + ROW_CAP;        // [ROW_CAP] u64
@@ -73,10 +76,10 @@ constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [TOPK_MAX_K] u64
 constexpr int OFF_HTAB = OFF_SORTED + TOPK_MAX_K;   // [ROW_HSLOTS] u32
 static_assert(OFF_HTAB + ROW_HSLOTS / 2 <= ROW_POOL, "proof layout fits the pool");
 constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
-constexpr int FB_DIGIT = 11;                  // key bits per sweep
+constexpr int FB_DIGIT = ROW_BLOCK >= 1024 ? 11 : 10;   // key bits per sweep: two digits per thread
 constexpr int OFF_FB_HIST = FB_BITMAP;        // [1 << FB_DIGIT] u32
 constexpr int OFF_FB_LIST = OFF_FB_HIST + (1 << FB_DIGIT) / 2;
-constexpr int FB_LIST_CAP = 768;
+constexpr int FB_LIST_CAP = ROW_BLOCK >= 1024 ? 768 : 512;
 constexpr int OFF_FB_SORTED = OFF_FB_LIST + FB_LIST_CAP;
 static_assert(OFF_FB_SORTED + TOPK_MAX_K <= ROW_POOL, "selection layout fits the pool");
 static_assert(TOPK_MAX_K <= 2 * WAVE, "the last wave holds at most two survivors per lane");
@@ -455,8 +458,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         s_max[0] = 0u;
         s_max[1] = 0u;
     }
-    tab[tid] = 0u;
-    static_assert(ROW_SLOTS == ROW_BLOCK, "one hash slot per thread to clear");
+    for (int i = tid; i < ROW_SLOTS; i += ROW_BLOCK) tab[i] = 0u;
     if (tid < ROW_TBINS) s_bins[0][tid] = 0u;                        // every round clears the bins of the next
     // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
     // probe it at the end; a longer one probes a hash of the candidates instead.
@@ -466,8 +468,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const bool penal = (a.rep != 1.0f || counted) && hlen > 0;
     const bool hfast = penal && hlen <= ROW_BLOCK;
     u32 *const ccnt = htab;                                          // a long history: occurrences by candidate (the hash is unused then)
-    htab[tid] = 0u;
-    htab[tid + ROW_BLOCK] = 0u;
+    for (int i = tid; i < ROW_HSLOTS; i += ROW_BLOCK) htab[i] = 0u;
     if (tid < TOPK_MAX_K) sorted[tid] = 0ull;
 
     ROW_STAMP(0);
