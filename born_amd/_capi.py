@@ -50,6 +50,7 @@ SYMBOLS = {
     "born_rocm_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "born_rocm_log_softmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "born_rocm_sample": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "born_rocm_sample_static": (C.c_int, [C.POINTER(SamplerConfigC), _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_sample_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_token_logprobs": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _vp]),
     "born_rocm_history_append": (C.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp]),

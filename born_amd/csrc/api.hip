@@ -47,6 +47,7 @@ struct born_sampler {
     int S_max;                     // argmax segments per row at max_vocab
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // see born_rocm_sampler_set_path
+    bool fixed_workspace;          // the workspace may not grow (born_rocm_sample_static: nothing is allocated, ever)
     // device workspace
     float *arg_val;                // argmax partials [max_batch][S_max]
     int *arg_idx;
@@ -68,8 +69,8 @@ static int fill_defaults(born_sampler_config *c) {
     if (c->top_k < 0) c->top_k = 0;
     if (!(c->temperature > 0.0f) || !std::isfinite(c->temperature))
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: temperature must be > 0 and finite, got %g", (double)c->temperature);
-    if (!(c->top_p > 0.0f) || std::isnan(c->top_p))
-        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: top_p must be > 0, got %g", (double)c->top_p);
+    if (!(c->top_p > 0.0f) || !(c->top_p <= 1.0f))
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: top_p must be in (0, 1], got %g", (double)c->top_p);
     if (!(c->repetition_penalty > 0.0f) || !std::isfinite(c->repetition_penalty))
         return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: repetition_penalty must be > 0 and finite, got %g",
                     (double)c->repetition_penalty);
@@ -386,7 +387,17 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     const bool local = counted && launched == 1u && hist_stride <= TOPK_LOCAL_COUNT_HISTORY;
     const bool table = counted && !local;
     if (table && !s->hist_counts) {
-        // per-row penalties on a handle configured without any: the table of occurrence counts is allocated now
+        // per-row penalties on a handle configured without any: the table of occurrence counts is allocated now,
+        // which a stream under capture (or a caller that must not allocate) cannot take
+        if (s->fixed_workspace)
+            return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample: frequency / presence penalties over a history of more than %d "
+                        "tokens (or outside the single-pass kernel) need a table of counts, which this entry point cannot allocate",
+                        TOPK_LOCAL_COUNT_HISTORY);
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &capturing));
+        if (capturing != hipStreamCaptureStatusNone)
+            return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample: the table of occurrence counts would be allocated inside a stream "
+                        "capture; configure the handle with a frequency or presence penalty (born_rocm_sampler_set_config) beforehand");
         const size_t bytes = (size_t)s->max_batch * (size_t)s->max_vocab * sizeof(unsigned);
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
         HIP_TRY(hipMalloc((void **)&s->hist_counts, bytes));
@@ -505,6 +516,73 @@ int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, i
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
                           const born_sampler_row_configs *rows, int32_t *tokens_out, float *probs_out, void *stream) {
     return sample_impl(s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, rows, tokens_out, probs_out,
+                       nullptr, nullptr, nullptr, 0, stream);
+}
+
+// ---- a sampling step for callers that cannot allocate ------------------------------------------------------------
+// The sampling kernels' workspace (a status word and the per-row work counters) normally belongs to a handle, whose
+// creation allocates it.  born_rocm_sample_static takes no handle: its workspace is this array, part of the library's
+// image on every device it runs on.  In host code the array's name is a stand-in, not a device address: the address on
+// the current device is asked for once per device and kept.
+constexpr int64_t STATIC_MAX_BATCH = 4096;
+constexpr size_t STATIC_COUNTER_WORDS = (size_t)COUNTER_ROW_BASE + (size_t)COUNTER_ROW_STRIDE * (size_t)STATIC_MAX_BATCH;
+static __device__ __align__(256) unsigned long long scratch[STATIC_COUNTER_WORDS + 32];   // counters, then the status word
+constexpr int STATIC_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static unsigned long long *g_scratch_ptr[STATIC_MAX_DEVICES];   // per device: each holds its own copy at its own address
+
+static int static_scratch(unsigned long long **out) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample_static: device ordinal %d is beyond the %d this entry point keeps an address for",
+                    dev, STATIC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        unsigned long long *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(BORN_ROCM_ERR_HIP, "sampler: sample_static: the workspace has no address on device %d", dev);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return BORN_ROCM_OK;
+}
+
+int born_rocm_sample_static(const born_sampler_config *cfg, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                            const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                            int32_t *tokens_out, float *probs_out, int32_t *status_out, void *stream) {
+    if (!uniforms)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: sample_static: uniforms must be given (the built-in stream counts its draws in a handle)");
+    if (batch > STATIC_MAX_BATCH)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample_static: batch %lld exceeds the %lld rows its fixed workspace holds",
+                    (long long)batch, (long long)STATIC_MAX_BATCH);
+    if (vocab > WIDE_MAX_VOCAB)
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: sample_static: vocab %lld exceeds the supported %lld", (long long)vocab,
+                    (long long)WIDE_MAX_VOCAB);
+    born_sampler_config c;
+    if (cfg) c = *cfg; else memset(&c, 0, sizeof(c));
+    int rc = fill_defaults(&c);
+    if (rc) return rc;
+    std::call_once(g_cfg_once, [] {
+        g_cfg_err = configure_kernels();
+        if (g_cfg_err == hipSuccess) g_cfg_err = configure_nucleus();
+    });
+    if (g_cfg_err != hipSuccess) return hip_fail(g_cfg_err, "configure_kernels");
+    unsigned long long *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    // A handle on the stack that owns nothing: its workspace is the fixed array (through the address kept for this
+    // device).  The counters only ever accumulate and the status word is only ever OR-ed into, so nothing in the array
+    // has to start a call at zero; a caller that wants the status passes a word of its own (zeroed by the caller).
+    born_sampler s;
+    memset(&s, 0, sizeof(s));
+    s.cfg = c;
+    s.max_batch = batch > 0 ? batch : 1;
+    s.max_vocab = vocab > 0 ? vocab : 1;
+    s.fixed_workspace = true;
+    s.counters = ws;
+    s.status = status_out ? status_out : reinterpret_cast<int *>(ws + STATIC_COUNTER_WORDS);
+    return sample_impl(&s, logits, batch, vocab, row_stride, history, hist_len, hist_stride, uniforms, nullptr, tokens_out, probs_out,
                        nullptr, nullptr, nullptr, 0, stream);
 }
 

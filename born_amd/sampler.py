@@ -115,6 +115,17 @@ def DeviceName(device=0):
     return buf.value.decode()
 
 
+def SampleStatic(cfg, logits, batch, vocab, history, histLen, uniforms, tokens_out, probs_out=None, status_out=None,
+                 row_stride=None, hist_stride=0, stream=None):
+    """Sample without a handle and without any allocation (born_rocm_sample_static): the kernels' workspace is a
+    fixed array inside the library, good for at most 4096 rows.  Results equal Sampler.Sample under the same
+    configuration.  `status_out`: an int32 device word the status bits are OR-ed into (the caller zeroes it), or None."""
+    c = (cfg or SamplerConfig())._c()
+    _check(_capi.lib().born_rocm_sample_static(C.byref(c), _ptr(logits), batch, vocab, row_stride or vocab, _ptr(history),
+                                               _ptr(histLen), hist_stride, _ptr(uniforms), _ptr(tokens_out), _ptr(probs_out),
+                                               _ptr(status_out), stream))
+
+
 class Sampler:
     """One handle = one stream at a time.  Outputs stay on the device; `Sample`/`Verify` return after
     enqueueing, and the `*_host` helpers copy the (tiny) results back and synchronise."""

@@ -157,6 +157,26 @@ int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, i
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
                           const born_sampler_row_configs *rows, int32_t *tokens_out, float *probs_out, void *stream);
 
+/* born_rocm_sample for callers that cannot allocate device memory at any time: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference and takes no handle (creating
+ * one allocates): the kernels' workspace (the per-row work counters and a status word) is a fixed array inside the
+ * library, one copy per device, sized for at most 4096 rows; a larger batch is BORN_ROCM_ERR_UNSUPPORTED.  The call
+ * allocates and frees nothing and returns after enqueueing, like born_rocm_sample, and every row's token and
+ * probability equal what born_rocm_sample returns under a handle configured with *cfg.
+ *   cfg        as for born_rocm_sampler_create (NULL: all defaults)
+ *   uniforms   required (the built-in uniform stream counts its draws in a handle)
+ *   status_out int32 device word or NULL: the bits born_rocm_sampler_status reports (1 = a history id outside the
+ *              vocabulary) are OR-ed into it; the caller zeroes and reads it
+ * Not served (BORN_ROCM_ERR_UNSUPPORTED): frequency / presence penalties where the kernel cannot count the
+ * occurrences itself (histories beyond 4096 tokens, top_k outside 1..128); nucleus listings and per-row
+ * configurations have no static form.  All calls on one device share that device's array: calls that overlap on one
+ * device (two streams, two threads) race on it.  The first call on a device looks up the array's address; make that
+ * call outside a graph capture. */
+int born_rocm_sample_static(const born_sampler_config *cfg, const float *logits, int64_t batch, int64_t vocab,
+                            int64_t row_stride, const int32_t *history, const int32_t *hist_len, int64_t hist_stride,
+                            const float *uniforms, int32_t *tokens_out, float *probs_out, int32_t *status_out,
+                            void *stream);
+
 /* Log-probability of one given token per row: logprobs_out[b] = log_softmax(z_b)[tokens[b]], z_b being row b after
  * the handle's penalties and temperature (steps 1-3 of the sampling pipeline; no min-p / top-k / top-p truncation).
  * With temperature 1 and no history this is minus the per-row term `-logProbs[target]` of CrossEntropyLoss.Forward,

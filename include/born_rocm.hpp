@@ -73,6 +73,18 @@ public:
         return tokens;
     }
 
+    // The same step for callers that cannot allocate (born_rocm_sample_static): no handle, every buffer the caller's,
+    // at most 4096 rows; `status_dev` (optional) is an int32 device word the status bits are OR-ed into.
+    static void SampleStatic(const SamplerConfig &cfg, const float *logits_dev, int64_t batch, int64_t vocab,
+                             const int32_t *history_dev, int64_t hist_stride, const int32_t *hist_len_dev,
+                             const float *uniforms_dev, int32_t *tokens_dev, float *probs_dev = nullptr,
+                             int32_t *status_dev = nullptr, void *stream = nullptr) {
+        born_sampler_config c{cfg.Temperature, cfg.TopK, cfg.TopP, cfg.RepetitionPenalty, cfg.Seed, cfg.MinP,
+                              cfg.FrequencyPenalty, cfg.PresencePenalty};
+        check(born_rocm_sample_static(&c, logits_dev, batch, vocab, vocab, history_dev, hist_len_dev, hist_stride, uniforms_dev,
+                                      tokens_dev, probs_dev, status_dev, stream));
+    }
+
     // Sample with a configuration per row: `rows` holds device arrays of `batch` values (null members: the handle's
     // value) and, optionally, the promise of which kinds of row occur (born_sampler_row_configs::row_kinds).
     std::vector<int32_t> SampleRows(const float *logits_dev, int64_t batch, int64_t vocab, const int32_t *history_dev,
