@@ -57,6 +57,7 @@ SYMBOLS = {
     "born_rocm_gather_rows": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp]),
     "born_rocm_spec_verify": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "born_rocm_spec_verify_bonus": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "born_rocm_exp": (C.c_int, [_vp, _vp, _i64, _vp]),
     "born_rocm_expneg": (C.c_int, [_vp, _vp, _i64, _vp]),
     "born_rocm_uniforms": (C.c_int, [_i64, _i64, _vp, _i64, _vp]),
     "born_rocm_linear": (C.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _vp]),

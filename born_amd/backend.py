@@ -85,6 +85,12 @@ class ROCmBackend:
     def Div(self, a, b, stream=None):
         return self._binary(_capi.lib().born_rocm_div, a, b, stream)
 
+    def Exp(self, a, stream=None):
+        """Element-wise float32(exp(float64(x))): ops.Exp, internal/autodiff/ops/log.go:159-185."""
+        out = DeviceTensor.empty(a.shape)
+        _check(_capi.lib().born_rocm_exp(a.buf.ptr, out.buf.ptr, a.NumElements(), stream))
+        return out
+
     def MatMul(self, a, b, stream=None):
         if len(a.shape) != 2 or len(b.shape) != 2:
             raise BackendPanic(f"matmul: only 2D tensors supported, got {len(a.shape)}D and {len(b.shape)}D")

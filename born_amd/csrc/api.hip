@@ -670,6 +670,15 @@ int born_rocm_spec_verify_bonus(born_sampler *s, const float *target, int64_t ta
                             draft_tokens, u_accept, u_residual, n_accepted_out, next_token_out, stream);
 }
 
+int born_rocm_exp(const float *x, float *out, int64_t n, void *stream) {
+    if (!x || !out) return fail(BORN_ROCM_ERR_ARGUMENT, "exp: null pointer");
+    if (n < 0) return fail(BORN_ROCM_ERR_ARGUMENT, "exp: negative element count %lld", (long long)n);
+    if (n > ((int64_t)1 << 40)) return fail(BORN_ROCM_ERR_UNSUPPORTED, "exp: %lld elements exceed the supported 2^40", (long long)n);
+    if (n == 0) return BORN_ROCM_OK;
+    HIP_TRY(launch_exp(x, out, n, (hipStream_t)stream));
+    return BORN_ROCM_OK;
+}
+
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream) {
     if (!d_in || !e_out || n <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: expneg: null pointer or n <= 0");
     HIP_TRY(launch_expneg(d_in, e_out, n, (hipStream_t)stream));

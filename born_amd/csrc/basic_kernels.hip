@@ -160,6 +160,36 @@ hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st) 
     return hipGetLastError();
 }
 
+// Element-wise exponential with the reference's arithmetic (ops.Exp, internal/autodiff/ops/log.go:159-185):
+// float32(exp(float64(x))), the fp64 exponential rounded once to fp32.  One flat pass: 128-bit non-temporal loads and
+// stores where the buffers allow them (both 16-byte aligned), four elements per thread; a scalar tail.
+typedef float exp_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float exp_ref32(float x) { return (float)exp((double)x); }
+template <bool VEC>
+__global__ __launch_bounds__(256) void exp_kernel(const float *__restrict__ x, float *__restrict__ out, long long n) {
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (VEC) {
+        const long long n4 = n >> 2;
+        if (t < n4) {
+            const exp_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const exp_f32x4 *>(x) + t);
+            exp_f32x4 r;
+#pragma unroll
+            for (int c = 0; c < 4; c++) r[c] = exp_ref32(v[c]);
+            __builtin_nontemporal_store(r, reinterpret_cast<exp_f32x4 *>(out) + t);
+        }
+        if (t < (n & 3)) out[(n4 << 2) + t] = exp_ref32(x[(n4 << 2) + t]);
+    } else {
+        for (long long i = t * 4; i < min(n, t * 4 + 4); i++) out[i] = exp_ref32(x[i]);
+    }
+}
+hipError_t launch_exp(const float *x, float *out, long long n, hipStream_t st) {
+    const bool vec = ((((uintptr_t)x) | ((uintptr_t)out)) & 15) == 0;
+    const unsigned blocks = (unsigned)(((n + 3) / 4 + 255) / 256);
+    if (vec) hipLaunchKernelGGL(exp_kernel<true>, dim3(blocks), dim3(256), 0, st, x, out, n);
+    else hipLaunchKernelGGL(exp_kernel<false>, dim3(blocks), dim3(256), 0, st, x, out, n);
+    return hipGetLastError();
+}
+
 // Occurrence counts of the history ids, one workgroup per row: the table is all zero before the counting launch and
 // all zero again after the clearing one, which touches exactly the entries the first one raised.
 template <bool CLEAR>

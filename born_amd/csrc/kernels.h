@@ -134,6 +134,8 @@ hipError_t launch_history_append(int *history, int *hist_len, long long hist_str
 hipError_t launch_gather_rows(const float *table, int rows, int cols, long long ld, const int *ids, int n, float *out, long long ldo,
                               int *status, hipStream_t st);
 hipError_t launch_expneg(const float *d, float *e, long long n, hipStream_t st);
+// out[i] = float32(exp(float64(x[i])))
+hipError_t launch_exp(const float *x, float *out, long long n, hipStream_t st);
 // counts[row * V + id] += 1 for every valid id of the row's history (clear: = 0 instead, which restores an all-zero table)
 hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,
                               bool clear, hipStream_t st);

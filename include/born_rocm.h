@@ -295,6 +295,11 @@ int born_rocm_conv2d(const float *input, const int64_t *input_shape, const float
 int born_rocm_maxpool2d(const float *input, const int64_t *input_shape, int32_t kernel_size, int32_t stride, float *out,
                         int64_t *out_shape, void *stream);
 
+/* Element-wise exponential, out[i] = float32(exp(float64(x[i]))) — ops.Exp, internal/autodiff/ops/log.go:159-185
+ * (a helper without a backward operation; its fp32 branch).  x and out are device arrays of n fp32 values (any shape,
+ * flat); they may be the same buffer.  n = 0 is a no-op. */
+int born_rocm_exp(const float *x, float *out, int64_t n, void *stream);
+
 /* Building blocks exported for parity tests (device-side evaluation of the specified fp32 exponential and of
  * the built-in uniform stream). */
 int born_rocm_expneg(const float *d_in, float *e_out, int64_t n, void *stream);

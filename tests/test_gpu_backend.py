@@ -223,3 +223,44 @@ def test_conv2d_and_maxpool2d_panics(be, rocm):
         rocm.MaxPool2D(x, 2, 0)
     with pytest.raises(be.BackendPanic, match=r"maxpool2d: invalid kernel size 0"):
         rocm.MaxPool2D(x, 0, 1)
+
+
+def test_exp_reference_kat_and_oracle(oracle, be, rocm):
+    """born_rocm_exp against the reference's own vector (TestExp, internal/autodiff/ops/ops_test.go:778-791, 1e-6) and
+    against the oracle's restatement of ops.Exp (fp64 exponential rounded once to fp32).  The device's fp64 exponential
+    and the host's may differ in their last fp64 bit, which shows in fp32 only where the fp64 value sits on an fp32
+    rounding boundary: the bar is equality to within one fp32 unit in the last place, and bit equality on all but a
+    stated handful of elements."""
+    import json
+    import os
+    kats = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))["exp"]
+    for case in kats:
+        x = np.array(case["input"], dtype=np.float32)
+        got = rocm.Exp(be.DeviceTensor.from_numpy(x)).numpy()
+        want = np.array([1.0, np.e, np.e * np.e])
+        assert np.max(np.abs(got - want)) <= case["tol_abs"], case["source"]
+    rng = np.random.default_rng(5)
+    for n in (1, 3, 4, 5, 1023, 4096, 262147):                        # ragged tails and whole 128-bit groups
+        x = (rng.standard_normal(n) * 20.0).astype(np.float32)
+        got = rocm.Exp(be.DeviceTensor.from_numpy(x)).numpy()
+        want = oracle.exp_ref(x)
+        same = got.view(np.uint32) == want.view(np.uint32)
+        assert same.mean() >= 1.0 - 1e-5, (n, int((~same).sum()))
+        assert np.all(np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64)) <= 1)
+    # special values: signed zeros, infinities, NaN, overflow, results that are subnormal or underflow to zero
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 88.72, 88.73, 89.0, -87.4, -100.0, -103.9, -104.0, -200.0, 1e-10], dtype=np.float32)
+    got = rocm.Exp(be.DeviceTensor.from_numpy(x)).numpy()
+    want = oracle.exp_ref(x)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.all(np.abs(got[ok].view(np.int32).astype(np.int64) - want[ok].view(np.int32).astype(np.int64)) <= 1), (got, want)
+    assert got[0] == 1.0 and got[1] == 1.0 and np.isinf(got[2]) and got[3] == 0.0 and np.isinf(got[7]) and got[12] == 0.0
+    # an unaligned view takes the scalar route and gives the same values
+    base = be.DeviceTensor.from_numpy(np.concatenate([[0.0], x[~np.isnan(x)]]).astype(np.float32))
+    from born_amd import _capi
+    from born_amd.sampler import DeviceBuffer
+    m = int((~np.isnan(x)).sum())
+    out = DeviceBuffer(4 * (m + 1))
+    assert _capi.lib().born_rocm_exp(base.buf.ptr + 4, out.ptr + 4, m, None) == 0
+    got2 = out.to_numpy(np.float32, (m + 1,))[1:]
+    assert np.array_equal(got2.view(np.uint32), got[~np.isnan(x)].view(np.uint32))
