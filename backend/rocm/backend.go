@@ -9,6 +9,8 @@ import "C"
 
 import (
 	"fmt"
+	"runtime"
+	"strings"
 	"unsafe"
 )
 
@@ -20,6 +22,34 @@ import (
 type Tensor struct {
 	Buf   DeviceBuffer
 	Shape []int
+}
+
+// Device is the value a device-aware tensor.Device enum would carry for this backend; the reference's enum
+// (internal/tensor/raw.go:14-20: CPU, CUDA, Vulkan, Metal, WebGPU) has no ROCm member, so the package defines its own
+// until one is added there (INTEGRATION.md shows the one-line change).
+type Device int
+
+// ROCm is the only device of this backend.
+const ROCm Device = 5 // the value that follows WebGPU in the reference's enum
+
+func (d Device) String() string {
+	if d == ROCm {
+		return "ROCm"
+	}
+	return "Unknown"
+}
+
+// Device reports where the tensor's memory lives (the reference's RawTensor.Device, internal/tensor/raw.go:139-141).
+func (t *Tensor) Device() Device { return ROCm }
+
+// Free releases the tensor's device memory now instead of waiting for the garbage collector; the tensor must not be
+// used afterwards.  Calling it twice is harmless.
+func (t *Tensor) Free() {
+	if t.Buf.ptr != nil {
+		_ = t.Buf.Free()
+		t.Buf = DeviceBuffer{}
+		runtime.SetFinalizer(t, nil)
+	}
 }
 
 func numElements(shape []int) int {
@@ -36,7 +66,10 @@ func NewTensor(shape []int) (*Tensor, error) {
 	if err != nil {
 		return nil, err
 	}
-	return &Tensor{Buf: buf, Shape: append([]int(nil), shape...)}, nil
+	t := &Tensor{Buf: buf, Shape: append([]int(nil), shape...)}
+	// every operation of the backend returns a new tensor: without this a chain of operations would leak device memory
+	runtime.SetFinalizer(t, func(t *Tensor) { t.Free() })
+	return t, nil
 }
 
 func cShape(shape []int) (*C.int64_t, C.int32_t) {
@@ -63,6 +96,9 @@ func New() *Backend { return &Backend{} }
 // Name returns the backend name.
 func (b *Backend) Name() string { return "ROCm" }
 
+// Device returns the compute device type (tensor.Backend.Device, internal/tensor/backend.go:32).
+func (b *Backend) Device() Device { return ROCm }
+
 type binaryFn func(a *C.float, as *C.int64_t, an C.int32_t, b *C.float, bs *C.int64_t, bn C.int32_t, out *C.float,
 	stream unsafe.Pointer) C.int
 
@@ -74,8 +110,8 @@ func (b *Backend) binary(op string, fn binaryFn, x, y *Tensor) *Tensor {
 		nd = len(y.Shape)
 	}
 	out := make([]C.int64_t, nd+1)
-	if rc := C.born_rocm_broadcast_shape(xs, xn, ys, yn, &out[0]); rc != C.BORN_ROCM_OK {
-		panic(fmt.Sprintf("%s: %s", op, lastError()[len("broadcast: "):]))
+	if rc, msg := callMsg(func() C.int { return C.born_rocm_broadcast_shape(xs, xn, ys, yn, &out[0]) }); rc != C.BORN_ROCM_OK {
+		panic(fmt.Sprintf("%s: %s", op, strings.TrimPrefix(msg, "broadcast: ")))
 	}
 	shape := make([]int, nd)
 	for i := range shape {
@@ -85,7 +121,9 @@ func (b *Backend) binary(op string, fn binaryFn, x, y *Tensor) *Tensor {
 	if err != nil {
 		panic(fmt.Sprintf("%s: failed to create result tensor: %v", op, err))
 	}
-	if err := check(fn((*C.float)(x.Buf.ptr), xs, xn, (*C.float)(y.Buf.ptr), ys, yn, (*C.float)(res.Buf.ptr), nil)); err != nil {
+	if err := call(func() C.int {
+		return fn((*C.float)(x.Buf.ptr), xs, xn, (*C.float)(y.Buf.ptr), ys, yn, (*C.float)(res.Buf.ptr), nil)
+	}); err != nil {
 		panic(fmt.Sprintf("%s: %v", op, err))
 	}
 	return res
@@ -160,9 +198,9 @@ func (b *Backend) Conv2D(input, kernel *Tensor, stride, padding int) *Tensor {
 	}
 	is, _ := cShape(input.Shape)
 	ks, _ := cShape(kernel.Shape)
-	// check() panics with the library's "conv2d: input channels ... != kernel channels ..."
-	if err := check(C.born_rocm_conv2d((*C.float)(input.Buf.ptr), is, (*C.float)(kernel.Buf.ptr), ks, C.int32_t(stride),
-		C.int32_t(padding), (*C.float)(res.Buf.ptr), nil, nil)); err != nil {
+	// call() panics with the library's "conv2d: input channels ... != kernel channels ..."
+	if err := call(func() C.int { return C.born_rocm_conv2d((*C.float)(input.Buf.ptr), is, (*C.float)(kernel.Buf.ptr), ks, C.int32_t(stride),
+		C.int32_t(padding), (*C.float)(res.Buf.ptr), nil, nil) }); err != nil {
 		panic(fmt.Sprintf("conv2d: %v", err))
 	}
 	return res
@@ -188,8 +226,8 @@ func (b *Backend) MaxPool2D(input *Tensor, kernelSize, stride int) *Tensor {
 		panic(fmt.Sprintf("maxpool2d: failed to create output: %v", err))
 	}
 	is, _ := cShape(input.Shape)
-	if err := check(C.born_rocm_maxpool2d((*C.float)(input.Buf.ptr), is, C.int32_t(kernelSize), C.int32_t(stride),
-		(*C.float)(res.Buf.ptr), nil, nil)); err != nil {
+	if err := call(func() C.int { return C.born_rocm_maxpool2d((*C.float)(input.Buf.ptr), is, C.int32_t(kernelSize), C.int32_t(stride),
+		(*C.float)(res.Buf.ptr), nil, nil) }); err != nil {
 		panic(fmt.Sprintf("maxpool2d: %v", err))
 	}
 	return res
@@ -203,7 +241,7 @@ func (b *Backend) Reshape(t *Tensor, newShape []int) *Tensor {
 	}
 	ts, tn := cShape(t.Shape)
 	ns, nn := cShape(newShape)
-	if err := check(C.born_rocm_reshape((*C.float)(t.Buf.ptr), ts, tn, ns, nn, (*C.float)(res.Buf.ptr), nil)); err != nil {
+	if err := call(func() C.int { return C.born_rocm_reshape((*C.float)(t.Buf.ptr), ts, tn, ns, nn, (*C.float)(res.Buf.ptr), nil) }); err != nil {
 		panic(fmt.Sprintf("reshape: %v", err))
 	}
 	return res
@@ -236,8 +274,8 @@ func (b *Backend) Transpose(t *Tensor, axes ...int) *Tensor {
 		panic(fmt.Sprintf("transpose: %v", err))
 	}
 	ts, tn := cShape(t.Shape)
-	// check() panics with the library's "transpose: invalid axis ..." / "transpose: duplicate axis ..."
-	if err := check(C.born_rocm_transpose((*C.float)(t.Buf.ptr), ts, tn, &cax[0], (*C.float)(res.Buf.ptr), nil)); err != nil {
+	// call() panics with the library's "transpose: invalid axis ..." / "transpose: duplicate axis ..."
+	if err := call(func() C.int { return C.born_rocm_transpose((*C.float)(t.Buf.ptr), ts, tn, &cax[0], (*C.float)(res.Buf.ptr), nil) }); err != nil {
 		panic(fmt.Sprintf("transpose: %v", err))
 	}
 	return res

@@ -53,14 +53,14 @@ func NewGenerator(embedding DeviceBuffer, vocab, hidden int, head *Linear, sampl
 
 // HistoryAppend writes each row's sampled token behind the row's history on the device.
 func (s *Sampler) HistoryAppend(history, histLen DeviceBuffer, histStride int, tokens DeviceBuffer, batch, vocab int, stream unsafe.Pointer) error {
-	return check(C.born_rocm_history_append(s.h, (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
-		(*C.int32_t)(tokens.ptr), C.int64_t(batch), C.int64_t(vocab), stream))
+	return call(func() C.int { return C.born_rocm_history_append(s.h, (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
+		(*C.int32_t)(tokens.ptr), C.int64_t(batch), C.int64_t(vocab), stream) })
 }
 
 // GatherRows is the embedding lookup out[i][:] = table[ids[i]][:] on the device.
 func (s *Sampler) GatherRows(table DeviceBuffer, rows, cols int, ids DeviceBuffer, n int, out DeviceBuffer, stream unsafe.Pointer) error {
-	return check(C.born_rocm_gather_rows(s.h, (*C.float)(table.ptr), C.int64_t(rows), C.int64_t(cols), C.int64_t(cols),
-		(*C.int32_t)(ids.ptr), C.int64_t(n), (*C.float)(out.ptr), C.int64_t(cols), stream))
+	return call(func() C.int { return C.born_rocm_gather_rows(s.h, (*C.float)(table.ptr), C.int64_t(rows), C.int64_t(cols), C.int64_t(cols),
+		(*C.int32_t)(ids.ptr), C.int64_t(n), (*C.float)(out.ptr), C.int64_t(cols), stream) })
 }
 
 // Step enqueues one decode step for rows [0, batch): four launches, no synchronisation.
@@ -71,9 +71,9 @@ func (g *Generator) Step(batch int, stream unsafe.Pointer) error {
 	if err := g.head.Forward(g.hid, []int{batch, g.hidden}, g.logits, stream); err != nil {
 		return err
 	}
-	if err := check(C.born_rocm_sample(g.sampler.h, (*C.float)(g.logits.ptr), C.int64_t(batch), C.int64_t(g.vocab), C.int64_t(g.vocab),
+	if err := call(func() C.int { return C.born_rocm_sample(g.sampler.h, (*C.float)(g.logits.ptr), C.int64_t(batch), C.int64_t(g.vocab), C.int64_t(g.vocab),
 		(*C.int32_t)(g.hist.ptr), (*C.int32_t)(g.histLen.ptr), C.int64_t(g.maxLen), nil, (*C.int32_t)(g.current.ptr), nil, nil, nil,
-		nil, 0, stream)); err != nil {
+		nil, 0, stream) }); err != nil {
 		return err
 	}
 	return g.sampler.HistoryAppend(g.hist, g.histLen, g.maxLen, g.current, batch, g.vocab, stream)
@@ -114,7 +114,7 @@ func (g *Generator) Generate(prompts [][]int32, steps int) ([][]int32, error) {
 	if err := g.hist.Download(unsafe.Pointer(&hist[0]), int64(4*len(hist))); err != nil {
 		return nil, err
 	}
-	if err := check(C.born_rocm_sampler_status(g.sampler.h, nil)); err != nil {
+	if err := call(func() C.int { return C.born_rocm_sampler_status(g.sampler.h, nil) }); err != nil {
 		return nil, err
 	}
 	out := make([][]int32, batch)

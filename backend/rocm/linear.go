@@ -86,9 +86,9 @@ func (l *Linear) Forward(input DeviceBuffer, shape []int, out DeviceBuffer, stre
 	if out.bytes < int64(batch)*int64(l.outFeatures)*4 {
 		panic("Linear.Forward: output buffer too small")
 	}
-	return check(C.born_rocm_linear((*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
+	return call(func() C.int { return C.born_rocm_linear((*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
 		C.int64_t(l.inFeatures), (*C.float)(l.weight.ptr), C.int64_t(l.outFeatures), C.int64_t(l.inFeatures),
-		(*C.float)(l.bias.ptr), (*C.float)(out.ptr), C.int64_t(l.outFeatures), stream))
+		(*C.float)(l.bias.ptr), (*C.float)(out.ptr), C.int64_t(l.outFeatures), stream) })
 }
 
 // ForwardArgmax is greedy decoding fused into the layer: tokens[b] = argmax_j Forward(input)[b][j] with the
@@ -107,9 +107,9 @@ func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]i
 		return nil, err
 	}
 	defer out.Free()
-	if err = check(C.born_rocm_linear_argmax(s.h, (*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
+	if err = call(func() C.int { return C.born_rocm_linear_argmax(s.h, (*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
 		C.int64_t(l.inFeatures), (*C.float)(l.weight.ptr), C.int64_t(l.outFeatures), C.int64_t(l.inFeatures),
-		(*C.float)(l.bias.ptr), (*C.int32_t)(out.ptr), nil)); err != nil {
+		(*C.float)(l.bias.ptr), (*C.int32_t)(out.ptr), nil) }); err != nil {
 		return nil, err
 	}
 	tokens := make([]int32, batch)
@@ -129,6 +129,6 @@ func MatMul(a DeviceBuffer, aShape []int, b DeviceBuffer, bShape []int, c Device
 	if k != kAlt {
 		panic(fmt.Sprintf("matmul: shape mismatch [%d,%d] @ [%d,%d]", m, k, kAlt, n))
 	}
-	return check(C.born_rocm_matmul((*C.float)(a.ptr), (*C.float)(b.ptr), (*C.float)(c.ptr), C.int64_t(m),
-		C.int64_t(k), C.int64_t(n), C.int64_t(k), C.int64_t(n), C.int64_t(n), stream))
+	return call(func() C.int { return C.born_rocm_matmul((*C.float)(a.ptr), (*C.float)(b.ptr), (*C.float)(c.ptr), C.int64_t(m),
+		C.int64_t(k), C.int64_t(n), C.int64_t(k), C.int64_t(n), C.int64_t(n), stream) })
 }

@@ -32,9 +32,9 @@ func NewCrossEntropyLoss(maxBatch, maxClasses int) *CrossEntropyLoss {
 // every buffer lives on the device.
 func (s *Sampler) TokenLogprobs(logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
 	histLen, tokens, out DeviceBuffer, stream unsafe.Pointer) error {
-	return check(C.born_rocm_token_logprobs(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
+	return call(func() C.int { return C.born_rocm_token_logprobs(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
 		C.int64_t(vocab), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
-		(*C.int32_t)(tokens.ptr), (*C.float)(out.ptr), stream))
+		(*C.int32_t)(tokens.ptr), (*C.float)(out.ptr), stream) })
 }
 
 // Forward returns the mean cross-entropy of logits [batch, classes] (fp32, device) against targets [batch]
@@ -59,7 +59,7 @@ func (c *CrossEntropyLoss) Forward(logits DeviceBuffer, shape []int, targets Dev
 	if err = out.Download(unsafe.Pointer(&lp[0]), int64(4*batch)); err != nil {
 		return 0, err
 	}
-	if err = check(C.born_rocm_sampler_status(c.s.h, nil)); err != nil {
+	if err = call(func() C.int { return C.born_rocm_sampler_status(c.s.h, nil) }); err != nil {
 		if strings.Contains(err.Error(), "device reported") {
 			panic("CrossEntropyLoss: target index out of bounds")
 		}

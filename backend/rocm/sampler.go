@@ -60,39 +60,54 @@ type SamplerBackend interface {
 type Sampler struct {
 	h                  *C.born_sampler
 	maxBatch, maxVocab int
+	out                DeviceBuffer // 2 * maxBatch int32 on the device: the results of a step, allocated once with the handle
 }
 
+// The library keeps its last error message per OS thread, and a goroutine may move to another thread between two
+// cgo calls: every call whose failure is turned into a message runs with its goroutine pinned to the thread.
 func lastError() string { return C.GoString(C.born_rocm_last_error()) }
 
-// check turns a status code into the reference's error convention.
-func check(rc C.int) error {
+// callMsg runs one C call and returns its status with the message that belongs to it ("" on success).
+func callMsg(f func() C.int) (C.int, string) {
+	runtime.LockOSThread()
+	defer runtime.UnlockOSThread()
+	rc := f()
+	if rc == C.BORN_ROCM_OK {
+		return rc, ""
+	}
+	return rc, lastError()
+}
+
+// call turns a status code into the reference's error convention.
+func call(f func() C.int) error {
+	rc, msg := callMsg(f)
 	switch rc {
 	case C.BORN_ROCM_OK:
 		return nil
 	case C.BORN_ROCM_ERR_ARGUMENT:
-		panic(lastError()) // programmer error: "sampler: ..."
+		panic(msg) // programmer error: "sampler: ..."
 	default:
-		return errors.New(lastError())
+		return errors.New(msg)
 	}
 }
 
 // Alloc returns device memory; Upload/Download copy through the shim (synchronous for pageable memory).
 func Alloc(bytes int64) (DeviceBuffer, error) {
 	var p unsafe.Pointer
-	if err := check(C.born_rocm_alloc(C.int64_t(bytes), &p)); err != nil {
+	if err := call(func() C.int { return C.born_rocm_alloc(C.int64_t(bytes), &p) }); err != nil {
 		return DeviceBuffer{}, err
 	}
 	return DeviceBuffer{ptr: p, bytes: bytes}, nil
 }
 
-func (b DeviceBuffer) Free() error { return check(C.born_rocm_free(b.ptr)) }
+func (b DeviceBuffer) Free() error { return call(func() C.int { return C.born_rocm_free(b.ptr) }) }
 
 func (b DeviceBuffer) Upload(src unsafe.Pointer, bytes int64) error {
-	return check(C.born_rocm_h2d(b.ptr, src, C.int64_t(bytes), nil))
+	return call(func() C.int { return C.born_rocm_h2d(b.ptr, src, C.int64_t(bytes), nil) })
 }
 
 func (b DeviceBuffer) Download(dst unsafe.Pointer, bytes int64) error {
-	return check(C.born_rocm_d2h(dst, b.ptr, C.int64_t(bytes), nil))
+	return call(func() C.int { return C.born_rocm_d2h(dst, b.ptr, C.int64_t(bytes), nil) })
 }
 
 // NewSampler fills defaults for zero fields and panics on invalid ones, like NewAdam
@@ -109,10 +124,15 @@ func NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler {
 		presence_penalty:   C.float(cfg.PresencePenalty),
 	}
 	var h *C.born_sampler
-	if err := check(C.born_rocm_sampler_create(&c, C.int64_t(maxBatch), C.int64_t(maxVocab), &h)); err != nil {
+	if err := call(func() C.int { return C.born_rocm_sampler_create(&c, C.int64_t(maxBatch), C.int64_t(maxVocab), &h) }); err != nil {
 		panic("sampler: " + err.Error())
 	}
-	s := &Sampler{h: h, maxBatch: maxBatch, maxVocab: maxVocab}
+	out, err := Alloc(int64(8 * maxBatch))
+	if err != nil {
+		C.born_rocm_sampler_destroy(h)
+		panic("sampler: " + err.Error())
+	}
+	s := &Sampler{h: h, maxBatch: maxBatch, maxVocab: maxVocab, out: out}
 	runtime.SetFinalizer(s, func(s *Sampler) { s.Close() })
 	return s
 }
@@ -121,7 +141,49 @@ func (s *Sampler) Close() {
 	if s.h != nil {
 		C.born_rocm_sampler_destroy(s.h)
 		s.h = nil
+		_ = s.out.Free()
+		s.out = DeviceBuffer{}
 	}
+}
+
+// results returns the handle's own device buffer for the int32 results of a step (no allocation per call: an
+// allocation synchronises the device, which a decode loop cannot afford).
+func (s *Sampler) results(batch int) DeviceBuffer {
+	if batch > s.maxBatch {
+		panic("sampler: batch exceeds the handle's maxBatch")
+	}
+	return s.out
+}
+
+// NewSampler makes *Backend a SamplerBackend: code that holds a tensor backend discovers the capability by type
+// assertion, `sb, ok := any(backend).(rocm.SamplerBackend)`, as nn.ReLU discovers ReLUBackend
+// (internal/nn/activation.go:41-52).
+func (b *Backend) NewSampler(cfg SamplerConfig, maxBatch, maxVocab int) *Sampler {
+	return NewSampler(cfg, maxBatch, maxVocab)
+}
+
+var _ SamplerBackend = (*Backend)(nil)
+
+// SampleStatic is Sample for callers that cannot allocate device memory at all (born_rocm_sample_static): no handle,
+// every buffer the caller's (tokens int32 [batch] on the device, probs and status optional), at most 4096 rows,
+// explicit uniforms.  It enqueues and returns; the results are valid once the stream is synchronised.
+func SampleStatic(cfg SamplerConfig, logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
+	histLen, uniforms, tokens, probs, status DeviceBuffer, stream unsafe.Pointer) error {
+	c := C.born_sampler_config{
+		temperature:        C.float(cfg.Temperature),
+		top_k:              C.int32_t(cfg.TopK),
+		top_p:              C.float(cfg.TopP),
+		repetition_penalty: C.float(cfg.RepetitionPenalty),
+		seed:               C.int64_t(cfg.Seed),
+		min_p:              C.float(cfg.MinP),
+		frequency_penalty:  C.float(cfg.FrequencyPenalty),
+		presence_penalty:   C.float(cfg.PresencePenalty),
+	}
+	return call(func() C.int {
+		return C.born_rocm_sample_static(&c, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
+			(*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride), (*C.float)(uniforms.ptr),
+			(*C.int32_t)(tokens.ptr), (*C.float)(probs.ptr), (*C.int32_t)(status.ptr), stream)
+	})
 }
 
 // Sample draws one token per row from device-resident fp32 logits [batch, vocab].
@@ -133,32 +195,24 @@ func (s *Sampler) Sample(logits DeviceBuffer, batch, vocab int, history DeviceBu
 	if batch <= 0 || vocab <= 0 {
 		panic("sampler: Sample: batch and vocab must be > 0")
 	}
-	out, err := Alloc(int64(4 * batch))
-	if err != nil {
-		return nil, err
-	}
-	defer out.Free()
-	if err = check(C.born_rocm_sample(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
+	out := s.results(batch)
+	if err = call(func() C.int { return C.born_rocm_sample(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
 		(*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride), (*C.float)(uniforms.ptr),
-		(*C.int32_t)(out.ptr), nil, nil, nil, nil, 0, nil)); err != nil {
+		(*C.int32_t)(out.ptr), nil, nil, nil, nil, 0, nil) }); err != nil {
 		return nil, err
 	}
 	tokens = make([]int32, batch)
 	if err = out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil { // synchronises the stream
 		return nil, err
 	}
-	return tokens, check(C.born_rocm_sampler_status(s.h, nil))
+	return tokens, call(func() C.int { return C.born_rocm_sampler_status(s.h, nil) })
 }
 
 // Argmax is the greedy decode: reference argmax per row (internal/nn/cross_entropy.go:241-251).
 func (s *Sampler) Argmax(logits DeviceBuffer, batch, vocab int) ([]int32, error) {
-	out, err := Alloc(int64(4 * batch))
-	if err != nil {
-		return nil, err
-	}
-	defer out.Free()
-	if err = check(C.born_rocm_argmax(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
-		(*C.int32_t)(out.ptr), nil)); err != nil {
+	out := s.results(batch)
+	if err := call(func() C.int { return C.born_rocm_argmax(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
+		(*C.int32_t)(out.ptr), nil) }); err != nil {
 		return nil, err
 	}
 	tokens := make([]int32, batch)
@@ -170,23 +224,19 @@ func (s *Sampler) Argmax(logits DeviceBuffer, batch, vocab int) ([]int32, error)
 // token of sequence b was accepted.
 func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
 	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
-	out, err := Alloc(int64(8 * batch))
-	if err != nil {
-		return nil, nil, err
-	}
-	defer out.Free()
+	out := s.results(batch)
 	na := (*C.int32_t)(out.ptr)
 	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
-	if err = check(C.born_rocm_spec_verify(s.h, (*C.float)(target.ptr), (*C.float)(draft.ptr), C.int64_t(batch),
+	if err = call(func() C.int { return C.born_rocm_spec_verify(s.h, (*C.float)(target.ptr), (*C.float)(draft.ptr), C.int64_t(batch),
 		C.int64_t(gamma), C.int64_t(vocab), (*C.int32_t)(draftTokens.ptr), (*C.float)(uAccept.ptr),
-		(*C.float)(uResidual.ptr), na, nt, nil)); err != nil {
+		(*C.float)(uResidual.ptr), na, nt, nil) }); err != nil {
 		return nil, nil, err
 	}
 	both := make([]int32, 2*batch)
 	if err = out.Download(unsafe.Pointer(&both[0]), int64(8*batch)); err != nil {
 		return nil, nil, err
 	}
-	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
+	return both[:batch], both[batch:], call(func() C.int { return C.born_rocm_sampler_status(s.h, nil) })
 }
 
 // VerifyBonus is Verify for a target that scored gamma+1 positions: `target` is [batch, gamma+1, vocab] and its
@@ -194,25 +244,21 @@ func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, dr
 // token from it (nextToken is never -1).
 func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
 	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
-	out, err := Alloc(int64(8 * batch))
-	if err != nil {
-		return nil, nil, err
-	}
-	defer out.Free()
+	out := s.results(batch)
 	na := (*C.int32_t)(out.ptr)
 	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
 	seq := C.int64_t((gamma + 1) * vocab)
 	bonus := (*C.float)(unsafe.Add(target.ptr, 4*gamma*vocab))
-	if err = check(C.born_rocm_spec_verify_bonus(s.h, (*C.float)(target.ptr), seq, (*C.float)(draft.ptr),
+	if err = call(func() C.int { return C.born_rocm_spec_verify_bonus(s.h, (*C.float)(target.ptr), seq, (*C.float)(draft.ptr),
 		C.int64_t(gamma*vocab), bonus, seq, C.int64_t(batch), C.int64_t(gamma), C.int64_t(vocab),
-		(*C.int32_t)(draftTokens.ptr), (*C.float)(uAccept.ptr), (*C.float)(uResidual.ptr), na, nt, nil)); err != nil {
+		(*C.int32_t)(draftTokens.ptr), (*C.float)(uAccept.ptr), (*C.float)(uResidual.ptr), na, nt, nil) }); err != nil {
 		return nil, nil, err
 	}
 	both := make([]int32, 2*batch)
 	if err = out.Download(unsafe.Pointer(&both[0]), int64(8*batch)); err != nil {
 		return nil, nil, err
 	}
-	return both[:batch], both[batch:], check(C.born_rocm_sampler_status(s.h, nil))
+	return both[:batch], both[batch:], call(func() C.int { return C.born_rocm_sampler_status(s.h, nil) })
 }
 
 // RowConfigs carries a configuration per row of a batch (continuous batching): device arrays of `batch` values,
@@ -236,11 +282,8 @@ const (
 // from the status check that follows the copy of the tokens.
 func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
 	histLen, uniforms DeviceBuffer, rows RowConfigs) ([]int32, error) {
-	out, err := Alloc(int64(4 * batch))
-	if err != nil {
-		return nil, err
-	}
-	defer out.Free()
+	out := s.results(batch)
+	var err error
 	// the struct holds device addresses only (C memory as far as cgo's pointer rules are concerned)
 	rc := C.born_sampler_row_configs{
 		temperature:        (*C.float)(rows.Temperatures.ptr),
@@ -252,14 +295,14 @@ func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history Devi
 		presence_penalty:   (*C.float)(rows.PresencePenalties.ptr),
 		row_kinds:          C.uint32_t(rows.RowKinds),
 	}
-	if err = check(C.born_rocm_sample_rows(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
+	if err = call(func() C.int { return C.born_rocm_sample_rows(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab),
 		C.int64_t(vocab), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
-		(*C.float)(uniforms.ptr), &rc, (*C.int32_t)(out.ptr), nil, nil)); err != nil {
+		(*C.float)(uniforms.ptr), &rc, (*C.int32_t)(out.ptr), nil, nil) }); err != nil {
 		return nil, err
 	}
 	tokens := make([]int32, batch)
 	if err = out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil {
 		return nil, err
 	}
-	return tokens, check(C.born_rocm_sampler_status(s.h, nil))
+	return tokens, call(func() C.int { return C.born_rocm_sampler_status(s.h, nil) })
 }
