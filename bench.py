@@ -201,11 +201,29 @@ def main():
 
     counter = [0]
 
+    # One sampling step = one call of born_rocm_sample (the same C entry point Sampler.Sample makes, the same
+    # arguments).  The calls are bound once, pointers and sizes already converted, so that the host side of a step is
+    # the C call alone: with the Python wrapper's per-call conversions the host lags behind a 27 us kernel at the start
+    # of a timed region, and that lag would be charged to the steps.
+    from born_amd import _capi
+    import functools
+    lib = _capi.lib()
+
+    def bind(lg):
+        return functools.partial(lib.born_rocm_sample, smp._h, lg.data_ptr(), B, V, V, None if history is None else history.data_ptr(),
+                                 None, H, uniforms.data_ptr(), tokens.data_ptr(), probs.data_ptr(), None, None, None, 0, stream)
+
+    calls = [bind(lg) for lg in logits_all]
+    smp.Sample(logits, B, V, history, None, uniforms, tokens, probs, hist_stride=H, stream=stream)   # the wrapper once: checks every argument
+
     def step(lg=None):
         if lg is None:
-            lg = logits_all[counter[0] % nrot]
+            rc = calls[counter[0] % nrot]()
             counter[0] += 1
-        smp.Sample(lg, B, V, history, None, uniforms, tokens, probs, hist_stride=H, stream=stream)
+        else:
+            rc = bind(lg)()
+        if rc:
+            _capi.check(rc)
 
     def timed(k):
         torch.cuda.synchronize()
@@ -249,7 +267,7 @@ def main():
     # read back above confirm it: rows settled by the single-pass kernel, by its exact selection, by the other two
     kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 128 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
         if args.path == 0 else "sample_wide_kernel"
-    launches = args.steps + args.warmup + 300 + (0 if producer is None else producer["iters"] + 1)
+    launches = 1 + args.steps + args.warmup + 300 + (0 if producer is None else producer["iters"] + 1)
     if kernel_name == "topk_row_kernel":
         confirmed = counters["topk_rows"] + counters["fallback_rows"] == B * launches and counters["general_rows"] == 0
     else:

@@ -1025,6 +1025,9 @@ def test_config_c5_slice_and_full_size_properties(oracle, rocm):
     assert np.array_equal(part["probs"].view(np.uint32), fx["probs"].view(np.uint32))
     diff = part["tokens"] != tr["tokens"]
     assert not (diff & ~tr["near"]).any()
+    # CDF steps are about 1e-5 wide on these flat rows, so the 1e-6 criterion flags many rows by itself; what is held
+    # to a bound is the number of tokens that actually differ from the fp64 layer (a draw within ~3e-7 of a step)
+    assert int(diff.sum()) <= 2, f"{int(diff.sum())} of 24 tokens differ from the fp64 layer"
     assert np.allclose(part["probs"][~diff], tr["probs"][~diff], rtol=1e-5)
     print(f"C5 slice: {int(tr['near'].sum())} of 24 rows flagged near a CDF step, {int(diff.sum())} tokens differ from the truth layer")
     s.Status()
