@@ -99,7 +99,7 @@ def cpu_baseline(w, seconds=12.0):
     return out
 
 
-def producer_leg(torch, dev, smp, sample_step, B, V, hidden, logits_all, stream, iters):
+def producer_leg(torch, dev, smp, sample_step, B, V, hidden, logits_all, stream, iters, fused_args=None):
     """The logits producer in front of the sampler: x[B, hidden] @ W[V, hidden]^T + b on the fp32 matrix cores
     (born_rocm_linear), written into the buffers the sampling step reads.  Random-init weights of the LM-head
     shape; reported beside the headline metric, never part of it."""
@@ -137,7 +137,29 @@ def producer_leg(torch, dev, smp, sample_step, B, V, hidden, logits_all, stream,
     ms_both = timed(both, iters)
     flops = 2.0 * B * hidden * V
     tf = flops / (ms_head * 1e-3) / 1e12
-    return {"kernel": "gemm_f32_dma_kernel", "workload": f"LM head: [{B}, {hidden}] @ [{V}, {hidden}]^T + bias, fp32 in / fp32 accumulate / fp32 out",
+    fused = None
+    if fused_args is not None:
+        # the same head with the sampling step in its epilogue (born_rocm_linear_sample): the logits are never written
+        history, H, uniforms, tokens, probs = fused_args
+        tok_ref = tokens.clone()                                     # tokens of the unfused pair on `scratch`
+
+        def fused_step():
+            L.ForwardSample(smp, layer, x, (B, hidden), history, None, uniforms, tokens, probs, hist_stride=H, stream=stream)
+
+        fused_step()
+        torch.cuda.synchronize()
+        got = tokens.cpu().numpy()
+        settled = got >= 0
+        agree = bool((got[settled] == tok_ref.cpu().numpy()[settled]).all())
+        if not settled.all():
+            try:
+                smp.Status(stream)
+            except Exception:
+                pass
+        ms_fused = timed(fused_step, iters)
+        fused = {"ms": ms_fused, "rows_settled": int(settled.sum()), "rows": int(B), "tokens_equal_the_unfused_pair": agree,
+                 "logits_bytes_not_written": int(B) * int(V) * 4}
+    return {"fused_head_and_sampling": fused, "kernel": "gemm_f32_dma_kernel", "workload": f"LM head: [{B}, {hidden}] @ [{V}, {hidden}]^T + bias, fp32 in / fp32 accumulate / fp32 out",
             "ms": ms_head, "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                                         "frac": tf / MFMA_FP32_PEAK_TFLOPS},
             "weight_stream_GBs": V * hidden * 4 / (ms_head * 1e-3) / 1e9,
@@ -239,7 +261,8 @@ def main():
     # steps below then run on a device that is already at its working clocks, as in a serving loop.
     producer = None
     if not args.no_producer and args.config == "C3":
-        producer = producer_leg(torch, dev, smp, step, B, V, args.hidden, logits_all, stream, max(5, args.steps // 10))
+        producer = producer_leg(torch, dev, smp, step, B, V, args.hidden, logits_all, stream, max(5, args.steps // 10),
+                                fused_args=(history, H, uniforms, tokens, probs))
 
     if args.copy_probe:
         dst = torch.empty_like(logits_all[0])
@@ -267,7 +290,7 @@ def main():
     # read back above confirm it: rows settled by the single-pass kernel, by its exact selection, by the other two
     kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 128 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
         if args.path == 0 else "sample_wide_kernel"
-    launches = 1 + args.steps + args.warmup + 300 + (0 if producer is None else producer["iters"] + 1)
+    launches = 1 + args.steps + args.warmup + 300 + (0 if producer is None else 2 * (producer["iters"] + 1))   # the chained and the fused steps of the LM-head leg count too
     if kernel_name == "topk_row_kernel":
         confirmed = counters["topk_rows"] + counters["fallback_rows"] == B * launches and counters["general_rows"] == 0
     else:

@@ -63,6 +63,7 @@ SYMBOLS = {
     "born_rocm_linear": (C.c_int, [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i64, _vp]),
     "born_rocm_matmul": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp]),
     "born_rocm_linear_argmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),
+    "born_rocm_linear_sample": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "born_rocm_broadcast_shape": (C.c_int, [_vp, C.c_int32, _vp, C.c_int32, _vp]),
     "born_rocm_add": (C.c_int, [_vp, _vp, C.c_int32, _vp, _vp, C.c_int32, _vp, _vp]),
     "born_rocm_sub": (C.c_int, [_vp, _vp, C.c_int32, _vp, _vp, C.c_int32, _vp, _vp]),

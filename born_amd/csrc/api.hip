@@ -54,6 +54,11 @@ struct born_sampler {
     int *status;
     unsigned long long *counters;
     unsigned long long *lm_best;   // [max_batch] packed (value, ~column) keys of the greedy-decode LM head
+    // sampling fused into the LM head (allocated by the first born_rocm_linear_sample call):
+    float *lm_samp;                // [max_batch][LM_SAMPLE_MAX] logits at a strided sample of the columns
+    float *lm_thr;                 // [max_batch] thresholds
+    unsigned *lm_cnt;              // [max_batch] candidate counters, LM_CAND_PITCH words apart
+    uint2 *lm_cand;                // [max_batch][LM_CAND_CAP] candidates
     unsigned *hist_counts;         // [max_batch][max_vocab] occurrences of each id in its row's history; all zero between
                                    // calls; allocated when a frequency or presence penalty is first configured
     // spec-verify statistics:
@@ -193,7 +198,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
 
 int born_rocm_sampler_destroy(born_sampler *s) {
     if (!s) return BORN_ROCM_OK;
-    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters, s->lm_best, s->hist_counts,
+    void *ptrs[] = {s->arg_val, s->arg_idx, s->status, s->counters, s->lm_best, s->hist_counts, s->lm_samp, s->lm_thr, s->lm_cnt, s->lm_cand,
                     s->sp_mp,     s->sp_mq,        s->sp_Zp, s->sp_Zq,     s->sp_pd,   s->sp_qd, s->sp_part, s->sp_run,
                     s->sp_mb,     s->sp_Zb};
     for (void *p : ptrs)
@@ -236,8 +241,9 @@ int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (st) {
         HIP_TRY(hipMemsetAsync(s->status, 0, sizeof(int), (hipStream_t)stream));
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s%s", (st & 1) ? "out-of-range history or token id " : "",
+        return fail(BORN_ROCM_ERR_DATA, "sampler: device reported %s%s%s%s%s%s", (st & 1) ? "out-of-range history or token id " : "",
                     (st & 2) ? "out-of-range draft token " : "", (st & 8) ? "invalid per-row configuration " : "", (st & 16) ? "a full history row " : "",
+                    (st & 32) ? "a row the fused LM-head sampling could not settle (token -1: run linear + sample for the call) " : "",
                     (st & 4) ? "an internal inconsistency (please report)" : "");
     }
     return BORN_ROCM_OK;
@@ -693,7 +699,7 @@ int born_rocm_uniforms(int64_t seed, int64_t step, float *u_out, int64_t n, void
 // `best` / `tokens` set: the greedy-decode epilogue (c unused); otherwise the product is stored to c.
 static int gemm_entry(const char *what, const float *a, const float *b, const float *bias, float *c, int64_t m,
                       int64_t k, int64_t n, int64_t lda, int64_t ldb, int64_t ldc, bool bt, void *stream,
-                      unsigned long long *best = nullptr, int32_t *tokens = nullptr) {
+                      unsigned long long *best = nullptr, int32_t *tokens = nullptr, int bm = 0) {
     if (!a || !b || (!c && !best)) return fail(BORN_ROCM_ERR_ARGUMENT, "%s: null pointer", what);
     const int64_t lim = 0x7FFFFFFF;
     if (m <= 0 || k <= 0 || n <= 0 || m > lim - 256 || k > lim - 64 || n > lim - 256)
@@ -705,6 +711,7 @@ static int gemm_entry(const char *what, const float *a, const float *b, const fl
     memset(&g, 0, sizeof g);
     g.best = best;
     g.tokens = tokens;
+    g.bm = bm;
     g.a = a;
     g.b = b;
     g.bias = bias;
@@ -741,6 +748,105 @@ int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int6
                     (long long)s->max_batch);
     return gemm_entry("linear_argmax", x, weight, bias, nullptr, batch, in_features, out_features, x_stride, w_stride,
                       out_features, true, stream, s->lm_best, tokens_out);
+}
+
+// LM head and sampling step in one call: x[batch, in] @ weight[out, in]^T + bias is never written.  Four launches:
+// the same product over a strided sample of at most 1024 weight rows (a small GEMM into the handle's workspace), the
+// per-row thresholds from it, the full product whose epilogue lists the logits at or above each row's threshold, and
+// the sampling step over the lists.
+int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
+                            const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
+                            const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                            int32_t *tokens_out, float *probs_out, void *stream) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: null handle");
+    if (!x || !weight || !tokens_out) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: null pointer");
+    if (batch <= 0 || in_features <= 0 || out_features <= 0)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: batch, in_features and out_features must be > 0");
+    if (batch > s->max_batch || out_features > s->max_vocab)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: shape [%lld, %lld] exceeds the handle's [%lld, %lld]", (long long)batch,
+                    (long long)out_features, (long long)s->max_batch, (long long)s->max_vocab);
+    if (x_stride < in_features || w_stride < in_features)
+        return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: a row pitch is smaller than the row");
+    if (history && hist_stride <= 0) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: history given with hist_stride <= 0");
+    if (!history && hist_len) return fail(BORN_ROCM_ERR_ARGUMENT, "linear_sample: hist_len given without history");
+    const int64_t lim = 0x7FFFFFFF;
+    if (hist_stride > lim || in_features > lim - 64 || out_features > lim - 256 || batch > lim - 256 ||
+        w_stride * (int64_t)((out_features + LM_SAMPLE_MAX - 1) / LM_SAMPLE_MAX) > ((int64_t)1 << 40))
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: shape too large");
+    const int top_k = (s->cfg.top_k <= 0 || s->cfg.top_k >= out_features) ? 0 : s->cfg.top_k;
+    if (top_k < 1 || top_k > TOPK_MAX_K || out_features > ROW_MAX_VOCAB || (history && s->cfg.repetition_penalty < 1.0f) ||
+        counts_history(s->cfg))
+        return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: the fused step serves 1 <= top_k <= %d over at most %d columns with a repetition "
+                    "penalty >= 1 and no frequency / presence penalty; use born_rocm_linear + born_rocm_sample", TOPK_MAX_K, ROW_MAX_VOCAB);
+    hipStream_t st = (hipStream_t)stream;
+    if (!s->lm_cand) {
+        if (s->fixed_workspace) return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: this handle cannot allocate its workspace");
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing(st, &capturing));
+        if (capturing != hipStreamCaptureStatusNone)
+            return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: the first call on a handle allocates its workspace; make it outside a stream capture");
+        const size_t rows = (size_t)s->max_batch;
+        HIP_TRY(hipMalloc((void **)&s->lm_samp, rows * LM_SAMPLE_MAX * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&s->lm_thr, rows * sizeof(float)));
+        HIP_TRY(hipMalloc((void **)&s->lm_cnt, rows * LM_CAND_PITCH * sizeof(unsigned)));
+        HIP_TRY(hipMalloc((void **)&s->lm_cand, rows * LM_CAND_CAP * sizeof(uint2)));
+    }
+    // 1. the product over every sstep-th weight row (no bias: the threshold kernel adds it)
+    const int64_t sstep = (out_features + LM_SAMPLE_MAX - 1) / LM_SAMPLE_MAX;
+    const int64_t nsamp = (out_features + sstep - 1) / sstep;
+    // (at most 1024 columns: tiles of 32 rows, so that more than a handful of workgroups share the narrow product)
+    int rc = gemm_entry("linear_sample", x, weight, nullptr, s->lm_samp, batch, in_features, nsamp, x_stride, sstep * w_stride,
+                        LM_SAMPLE_MAX, true, stream, nullptr, nullptr, batch > 32 ? 32 : 0);
+    if (rc) return rc;
+    // 2. thresholds: the kth largest sampled logit of a row, reached by about kth * sstep of all its logits: the aim is
+    // LM_CAND_TARGET candidates, and never fewer than the top_k + 16 the finish wants to see
+    int64_t kth = (LM_CAND_TARGET + sstep - 1) / sstep;
+    if (kth < 4) kth = 4;
+    if (kth * sstep < 4 * (int64_t)(top_k + 16)) kth = (4 * (int64_t)(top_k + 16) + sstep - 1) / sstep;
+    HIP_TRY(launch_lm_threshold(s->lm_samp, LM_SAMPLE_MAX, (int)batch, (int)nsamp, bias, (int)sstep, (int)kth, s->lm_thr, s->lm_cnt, st));
+    // 3. the full product, candidates listed by the epilogue
+    GemmArgs g;
+    memset(&g, 0, sizeof g);
+    g.a = x;
+    g.b = weight;
+    g.bias = bias;
+    g.M = (int)batch;
+    g.N = (int)out_features;
+    g.K = (int)in_features;
+    g.lda = x_stride;
+    g.ldb = w_stride;
+    g.ldc = out_features;
+    g.vec_a = ((uintptr_t)x & 15) == 0 && (x_stride & 3) == 0;
+    g.vec_b = ((uintptr_t)weight & 15) == 0 && (w_stride & 3) == 0;
+    g.thr = s->lm_thr;
+    g.cand_cnt = s->lm_cnt;
+    g.cand = s->lm_cand;
+    g.cand_cap = LM_CAND_CAP;
+    HIP_TRY(launch_gemm_f32(g, true, st));
+    // 4. the sampling step over the lists
+    SampleArgs a;
+    memset(&a, 0, sizeof(a));
+    a.B = (int)batch;
+    a.V = (int)out_features;
+    a.history = history;
+    a.hist_len = hist_len;
+    a.hist_stride = history ? hist_stride : 0;
+    a.uniforms = uniforms;
+    a.seed = (unsigned long long)s->cfg.seed;
+    a.step = s->step;
+    a.T = s->cfg.temperature;
+    a.top_p = s->cfg.top_p;
+    a.rep = s->cfg.repetition_penalty;
+    a.top_k = top_k;
+    a.tokens = tokens_out;
+    a.probs = probs_out;
+    a.status = s->status;
+    a.counters = s->counters;
+    a.mass_shift = mass_shift(out_features);
+    a.dcut = mass_cutoff(s->cfg);
+    HIP_TRY(launch_cand_rows(a, s->lm_thr, s->lm_cnt, s->lm_cand, LM_CAND_CAP, st));
+    if (!uniforms) s->step++;
+    return BORN_ROCM_OK;
 }
 
 }  // extern "C"

@@ -102,8 +102,18 @@ struct GemmArgs {
     bool vec_a, vec_b;            // 128-bit loads are legal (base 16-byte aligned, pitch a multiple of 4)
     unsigned long long *best;     // non-null: keep only each row's largest result as a packed key (c unused), keys LM_BEST_PITCH words apart ..
     int *tokens;                  // .. and write its column here
+    // non-null: keep only the results >= thr[row], appended as (value bits, column) to the row's list (c unused)
+    const float *thr;             // [M]
+    unsigned *cand_cnt;           // [M] counters LM_CAND_PITCH words apart, zero when the launch starts; may end above cand_cap
+    uint2 *cand;                  // [M][cand_cap]
+    int cand_cap;
+    int bm;                       // 0: tile height chosen from M; else 16, 32, 64 or 128 (a narrow product wants more, lower tiles)
 };
 constexpr int LM_BEST_PITCH = 16;
+constexpr int LM_CAND_PITCH = 32;          // u32 words between the candidate counters of consecutive rows (a 128-byte line each)
+constexpr int LM_CAND_CAP = 4096;          // candidates a row's list holds
+constexpr int LM_SAMPLE_MAX = 1024;        // columns of the strided sample the thresholds come from
+constexpr int LM_CAND_TARGET = 1536;       // candidates per row the thresholds aim at (the count varies by about a third around it)
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st);
 
 // Index map of an element-wise or shape operation over a (collapsed) result of nd dimensions: shape[d] and,
@@ -141,6 +151,14 @@ hipError_t launch_hist_counts(const int *history, const int *hist_len, long long
                               bool clear, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
+// Sampling fused into the LM head, in three steps around the GEMM that lists the candidates:
+//   thr[row] = the kth largest of samp[row][0..nsamp) + bias[j * sstep] (-inf if there are fewer); cand_cnt[row] = 0
+hipError_t launch_lm_threshold(const float *samp, long long ld, int B, int nsamp, const float *bias, int sstep, int kth, float *thr,
+                               unsigned *cand_cnt, hipStream_t st);
+//   the sampling step over each row's listed candidates (every logit >= thr[row]); a row it cannot settle gets token -1
+//   and status bit 5
+hipError_t launch_cand_rows(const SampleArgs &a, const float *thr, const unsigned *cand_cnt, const uint2 *cand, int cand_cap,
+                            hipStream_t st);
 hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
 hipError_t configure_nucleus();

@@ -93,6 +93,16 @@ __device__ __forceinline__ u64 gemm_shfl_xor_u64(u64 x, int o) {
     return ((u64)hi << 32) | lo;
 }
 
+// EPI 2 (sampling fused into the LM head): every result at or above its row's threshold is appended, value and
+// column, to the row's candidate list (one global atomic per candidate: a few per row and tile); the logits are
+// never written.  A NaN is never listed.  The counter may run past the list's capacity: the reader sees that.
+__device__ __forceinline__ void gemm_offer_candidate(const GemmArgs &g, int row, int col, float v, float thr) {
+    if (v >= thr) {
+        const unsigned pos = atomicAdd(&g.cand_cnt[(long long)row * LM_CAND_PITCH], 1u);
+        if (pos < (unsigned)g.cand_cap) g.cand[(long long)row * g.cand_cap + pos] = make_uint2(__float_as_uint(v), (unsigned)col);
+    }
+}
+
 // 32 x 32 blocks: accumulator v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4, column r of its block
 template <int EPI, int IB, int JB>
 __device__ __forceinline__ void gemm_finish32(const GemmArgs &g, const f32x16 (&acc)[IB][JB], int m0, int n0, int wm,
@@ -114,6 +124,56 @@ __device__ __forceinline__ void gemm_finish32(const GemmArgs &g, const f32x16 (&
                     }
                 }
             }
+        }
+    } else if (EPI == 2) {
+        // A candidate's place in its row's list costs a global atomic, and one per candidate where it is met would make
+        // the wave wait for a memory round trip some forty times.  The wave stages its candidates in LDS instead
+        // (ballot + lane rank, no atomics) and then asks for all their places at once.
+        constexpr int STAGE = 192;                                   // a 64 x 64 block of C yields about 70
+        __shared__ uint2 st_vc[GEMM_THREADS / WAVE][STAGE];
+        __shared__ int st_row[GEMM_THREADS / WAVE][STAGE];
+        uint2 *const vc = st_vc[threadIdx.x >> 6];
+        int *const rw = st_row[threadIdx.x >> 6];
+        u32 count = 0;                                               // wave-uniform
+        float bias[JB];
+#pragma unroll
+        for (int j = 0; j < JB; j++) {
+            const int col = n0 + (wn * JB + j) * 32 + r;
+            bias[j] = (g.bias && col < g.N) ? g.bias[col] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < IB; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + (wm * IB + i) * 32 + (v >> 2) * 8 + h * 4 + (v & 3);
+                const float thr = row < g.M ? g.thr[row] : INFINITY;
+#pragma unroll
+                for (int j = 0; j < JB; j++) {
+                    const int col = n0 + (wn * JB + j) * 32 + r;
+                    const float sum = acc[i][j][v];
+                    const float val = g.bias ? sum + bias[j] : sum;
+                    const bool pass = col < g.N && val >= thr;       // a NaN never passes; rows past the batch have thr = +inf
+                    const u64 m = __ballot(pass);
+                    if (m) {                                         // wave-uniform
+                        if (pass) {
+                            const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+                            if (pos < (u32)STAGE) {
+                                vc[pos] = make_uint2(__float_as_uint(val), (unsigned)col);
+                                rw[pos] = row;
+                            } else {
+                                gemm_offer_candidate(g, row, col, val, thr);   // the stage is full: straight to the list
+                            }
+                        }
+                        count += (u32)__popcll(m);
+                    }
+                }
+            }
+        }
+        const int staged = (int)min(count, (u32)STAGE);
+        for (int e = (int)(threadIdx.x & (WAVE - 1)); e < staged; e += WAVE) {   // (the wave's own LDS writes are visible to it in order)
+            const int row = rw[e];
+            const unsigned pos = atomicAdd(&g.cand_cnt[(long long)row * LM_CAND_PITCH], 1u);
+            if (pos < (unsigned)g.cand_cap) g.cand[(long long)row * g.cand_cap + pos] = vc[e];
         }
     } else {
         float bias[JB];
@@ -156,6 +216,18 @@ __device__ __forceinline__ void gemm_finish16(const GemmArgs &g, const f32x4 (&a
             for (int v = 0; v < 4; v++) {
                 const int row = m0 + 4 * q16 + v;
                 if (row < g.M) g.c[(long long)row * g.ldc + col] = g.bias ? acc16[jb][v] + bias : acc16[jb][v];
+            }
+        }
+    } else if (EPI == 2) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = m0 + 4 * q16 + v;
+            if (row >= g.M) continue;
+            const float thr = g.thr[row];
+#pragma unroll
+            for (int jb = 0; jb < 2; jb++) {
+                const int col = n0 + wn * 32 + jb * 16 + j16;
+                if (col < g.N) gemm_offer_candidate(g, row, col, g.bias ? acc16[jb][v] + g.bias[col] : acc16[jb][v], thr);
             }
         }
     } else {
@@ -523,12 +595,88 @@ __global__ void argmax_keys_token_kernel(u64 *best, int *tokens, int n) {
     }
 }
 
+// Thresholds of the candidate epilogue.  samp[row][j] (+ bias[j * sstep]) are the row's logits at a strided sample of
+// at most LM_SAMPLE_MAX columns; the kth largest of them becomes thr[row]: about kth * sstep logits of the whole row
+// reach it, which is what the epilogue will list.  It is a heuristic only: what is listed is decided by the full
+// product, and the row's finish proves that nothing outside the list can matter.  An exact radix select over the
+// order keys, eight bits per pass; every wave reads the digit counts and reaches the same digit.  The launch also puts
+// the row's candidate counter back to zero.  Fewer than kth samples that are numbers: -inf (every logit is listed).
+constexpr int THR_BLOCK = 1024;
+__global__ __launch_bounds__(THR_BLOCK) void lm_threshold_kernel(const float *samp, long long ld, int nsamp, const float *bias, int sstep,
+                                                                 int kth, float *thr, unsigned *cand_cnt) {
+    __shared__ __attribute__((aligned(16))) u32 hist[4][256];
+    const int tid = threadIdx.x, row = blockIdx.x, l = lane_id();
+    for (int i = tid; i < 4 * 256; i += THR_BLOCK) (&hist[0][0])[i] = 0u;
+    constexpr int PER = LM_SAMPLE_MAX / THR_BLOCK;
+    u32 key[PER];
+#pragma unroll
+    for (int t = 0; t < PER; t++) {
+        const int j = t * THR_BLOCK + tid;
+        key[t] = 0u;                                                 // below every number's key: a NaN, or no sample
+        if (j < nsamp) {
+            float v = samp[(long long)row * ld + j];
+            if (bias) v = v + bias[(long long)j * sstep];
+            if (v == v) key[t] = ordkey(v);
+        }
+    }
+    if (tid == 0) cand_cnt[(long long)row * LM_CAND_PITCH] = 0u;
+    __syncthreads();
+    u32 prefix = 0u;
+    int need = kth;
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+        const int shift = 24 - 8 * pass;
+#pragma unroll
+        for (int t = 0; t < PER; t++)
+            if (t * THR_BLOCK + tid < nsamp && (pass == 0 || (key[t] >> (shift + 8)) == prefix)) atomicAdd(&hist[pass][(key[t] >> shift) & 255u], 1u);
+        __syncthreads();
+        // the largest digit D with (keys of this prefix in digits >= D) >= need; lane 0 holds the four highest digits
+        const uint4 h4 = reinterpret_cast<const uint4 *>(hist[pass])[WAVE - 1 - l];
+        const u32 s4 = h4.x + h4.y + h4.z + h4.w;
+        const u32 incl = wave_inclusive_scan_u32(s4);
+        const u64 reach = __ballot(incl >= (u32)need);
+        if (reach == 0ull) {                                         // fewer than kth samples in all: wave-uniform, the same in every wave
+            prefix = 0u;
+            break;
+        }
+        const int L = __ffsll((long long)reach) - 1;
+        u32 above = (u32)__builtin_amdgcn_readlane((int)(incl - s4), L);   // keys in the digits of the lanes before L
+        const u32 hw = (u32)__builtin_amdgcn_readlane((int)h4.w, L), hz = (u32)__builtin_amdgcn_readlane((int)h4.z, L);
+        const u32 hy = (u32)__builtin_amdgcn_readlane((int)h4.y, L);
+        int D = 4 * (WAVE - 1 - L) + 3;
+        if (above + hw < (u32)need) {
+            above += hw;
+            D--;
+            if (above + hz < (u32)need) {
+                above += hz;
+                D--;
+                if (above + hy < (u32)need) {
+                    above += hy;
+                    D--;
+                }
+            }
+        }
+        need -= (int)above;
+        prefix = (prefix << 8) | (u32)D;
+    }
+    if (tid == 0) thr[row] = prefix ? ordkey_inv(prefix) : -INFINITY;
+}
+hipError_t launch_lm_threshold(const float *samp, long long ld, int B, int nsamp, const float *bias, int sstep, int kth, float *thr,
+                               unsigned *cand_cnt, hipStream_t st) {
+    if (nsamp <= 0 || nsamp > LM_SAMPLE_MAX || kth <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(lm_threshold_kernel, dim3((unsigned)B), dim3(THR_BLOCK), 0, st, samp, ld, nsamp, bias, sstep, kth, thr, cand_cnt);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
-    const int bm = g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
+    const int bm = g.bm ? g.bm : g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
-    if (g.best) {                                                    // argmax epilogue: W[N,K] form only
+    if (g.cand) {                                                    // candidate epilogue: W[N,K] form only
+        if (!b_transposed || !g.thr || !g.cand_cnt || g.cand_cap <= 0) return hipErrorInvalidValue;
+        launch_gemm_nt<2>(g, bm, grid, fast, st);
+    } else if (g.best) {                                             // argmax epilogue: W[N,K] form only
         if (!b_transposed || !g.tokens) return hipErrorInvalidValue;
         launch_gemm_nt<1>(g, bm, grid, fast, st);
         hipLaunchKernelGGL(argmax_keys_token_kernel, dim3((unsigned)((g.M + 255) / 256)), dim3(256), 0, st, g.best, g.tokens, g.M);

@@ -723,6 +723,188 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 #endif
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The sampling step over a list of candidates instead of the row itself (sampling fused into the LM head: the GEMM's
+// epilogue lists every logit >= thr[row] of a row, value and column, and writes no logits).  The list takes the place
+// of the pass over the row: its entries go to the waves' lists 1024 at a time, the threshold is raised after each
+// round, and the finish is the single-pass kernel's (candidates gathered in one array, exact z, rank sort, one wave
+// for the integer CDF, the top-p cut and the draw).  Everything outside the list is below thr[row], so the same
+// proof applies.  What this kernel cannot settle (a list that overflowed, fewer than top_k candidates above the
+// bound, a history longer than the workgroup with a penalty) it reports: token -1, status bit 5; the caller runs
+// the unfused pair for those calls.
+// ---------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const float *thr, const unsigned *cand_cnt, const uint2 *cand, int cap) {
+    __shared__ u64 pool[ROW_POOL];
+    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);
+    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);
+    u64 *const K = pool + OFF_K;
+    u32 *const Khi = reinterpret_cast<u32 *>(pool + OFF_TAB);
+    u64 *const sorted = pool + OFF_SORTED;
+    u32 *const htab = reinterpret_cast<u32 *>(pool + OFF_HTAB);
+    __shared__ u32 s_wmax[ROW_WAVES];
+    __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
+    __shared__ u32 s_max[2];
+    __shared__ int s_n, s_valid, s_over, s_next;
+
+    const int tid = threadIdx.x, row = blockIdx.x;
+    const int V = a.V, k = a.top_k;
+    const unsigned cnt = cand_cnt[(long long)row * LM_CAND_PITCH];
+    const uint2 *mine = cand + (long long)row * cap;
+    const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
+    const int *h = a.history + (long long)row * a.hist_stride;
+    const int h0 = (tid < hlen) ? h[tid] : -1;
+    const bool penal = a.rep != 1.0f && hlen > 0;
+    const float u_row = a.uniforms ? a.uniforms[row] : uniform_of(a.seed, a.step, (u64)row);
+    if (tid == 0) {
+        s_n = 0;
+        s_valid = 0;
+        s_over = 0;
+        s_next = 0;
+        s_max[0] = 0u;
+        s_max[1] = 0u;
+    }
+    for (int i = tid; i < ROW_SLOTS; i += ROW_BLOCK) Khi[i] = 0u;
+    for (int i = tid; i < ROW_HSLOTS; i += ROW_BLOCK) htab[i] = 0u;
+    if (tid < ROW_TBINS) s_bins[0][tid] = 0u;
+    if (tid < TOPK_MAX_K) sorted[tid] = 0ull;
+    // ids of the history outside the vocabulary are reported whatever becomes of the row
+    for (int i = tid; i < hlen; i += ROW_BLOCK) {
+        const int t = i == tid ? h0 : h[i];
+        if (t < 0 || t >= V) atomicOr(a.status, 1);
+    }
+    auto unsettled = [&]() {                                         // workgroup-uniform
+        if (tid == 0) {
+            a.tokens[row] = -1;
+            if (a.probs) a.probs[row] = 0.0f;
+            atomicOr(a.status, 32);
+            count_row(a.counters, row, 1);
+        }
+    };
+    const float t0 = thr[row];
+    if (cnt > (unsigned)cap || cnt < (unsigned)k || (penal && hlen > ROW_BLOCK) || t0 != t0) {
+        unsettled();
+        return;
+    }
+    // the largest candidate (the bins of the threshold's histogram span from the threshold to it)
+    u32 mx = 0u;
+    for (unsigned e = tid; e < cnt; e += ROW_BLOCK) mx = max(mx, ordkey(__uint_as_float(mine[e].x)));
+    mx = wave_max_u32(mx);
+    if (lane_id() == 0) s_wmax[wave_id()] = mx;
+    __syncthreads();
+    if (penal && tid < hlen && h0 >= 0 && h0 < V) {                  // the history's hash, probed by the candidates
+        u32 slot = row_hhash((u32)h0);
+        for (;;) {
+            const u32 old = atomicCAS(&htab[slot], 0u, (u32)h0 + 1u);
+            if (old == 0u || old == (u32)h0 + 1u) break;
+            slot = (slot + 1) & (ROW_HSLOTS - 1);
+        }
+    }
+    const u32 max0 = wave_max_u32(lane_id() < ROW_WAVES ? s_wmax[lane_id()] : 0u);
+    u32 twkey = ordkey(t0);                                          // every logit outside the list has a smaller key
+    const int want = k + ROW_MARGIN;
+    uint2 *list = L + wave_id() * ROW_WCAP;
+    u32 count = 0;
+    int round = 0;
+    for (unsigned base = 0; base < cnt; base += ROW_BLOCK) {         // workgroup-uniform
+        const unsigned e = base + tid;
+        uint2 c = make_uint2(0u, 0u);
+        bool pass = false;
+        if (e < cnt) {
+            c = mine[e];
+            pass = ordkey(__uint_as_float(c.x)) >= twkey && c.y < (u32)V;
+        }
+        const u64 m = __ballot(pass);
+        if (pass) {
+            const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+            if (pos < (u32)ROW_WCAP) list[pos] = c;
+        }
+        count += (u32)__popcll(m);
+        const u32 smax = max(max0, s_max[round & 1]);
+        row_tighten(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+        round++;
+    }
+    if (count > (u32)ROW_WCAP && lane_id() == 0) s_over = 1;
+    const int cw = (int)min(count, (u32)ROW_WCAP);
+    const u32 zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));       // bound of z for everything outside the lists
+    {
+        u32 base = 0u;
+        if (lane_id() == 0 && cw) base = (u32)atomicAdd(&s_n, cw);
+        base = (u32)__builtin_amdgcn_readfirstlane((int)base);
+        for (int e = lane_id(); e < cw; e += WAVE)
+            if (base + (u32)e < (u32)ROW_CAP) C[base + e] = list[e];
+    }
+    __syncthreads();
+    const int n = s_n;
+    bool ok = !s_over && n >= k && n <= ROW_CAP;
+    if (ok && tid < n) {                                             // exact z and rank key of every candidate
+        const uint2 c = C[tid];
+        float y = __uint_as_float(c.x);
+        if (penal) {
+            u32 slot = row_hhash(c.y);
+            for (;;) {
+                const u32 en = htab[slot];
+                if (en == 0u) break;
+                if (en == c.y + 1u) {
+                    y = penalise(y, a.rep);
+                    break;
+                }
+                slot = (slot + 1) & (ROW_HSLOTS - 1);
+            }
+        }
+        const float z = z_of(y, a.T);
+        K[tid] = make_key64(z, (int)c.y);
+        Khi[tid] = ordkey(z);
+        const int nk = __popcll(__ballot(ordkey(z) > zb));
+        if (nk && lane_id() == 0) atomicAdd(&s_valid, nk);
+    }
+    __syncthreads();
+    ok = ok && s_valid >= k;
+    if (!ok) {
+        unsettled();
+        return;
+    }
+    if (tid < n) {                                                   // rank sort on z, as in the single-pass kernel
+        const u32 khi = Khi[tid];
+        const uint4 *K4 = reinterpret_cast<const uint4 *>(Khi);
+        int r = 0;
+        for (int q = 0; q < ((n + 31) >> 5) * 8; q += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) v[t] = K4[q + t];
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                r += (v[t].x > khi ? 1 : 0) + (v[t].y > khi ? 1 : 0) + (v[t].z > khi ? 1 : 0) + (v[t].w > khi ? 1 : 0);
+        }
+        if (r < k) sorted[r] = K[tid];
+        else if (r == k) s_next = 1;
+    }
+    __syncthreads();
+    if (tid >= WAVE) return;
+    {
+        bool hole = false;
+        for (int i = tid; i < k; i += WAVE) hole |= sorted[i] == 0ull;
+        if (__ballot(hole) != 0ull || (n > k && s_next == 0)) {      // equal z among the candidates: whole keys decide
+            for (int c = tid; c < n; c += WAVE) {
+                const u64 key = K[c];
+                int r = 0;
+                for (int j = 0; j < n; j++) r += K[j] > key ? 1 : 0;
+                if (r < k) sorted[r] = key;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+    finish_sorted_by_wave(sorted, k, a, row, u_row);
+    if (tid == 0) count_row(a.counters, row, 0);
+}
+
+hipError_t launch_cand_rows(const SampleArgs &a, const float *thr, const unsigned *cand_cnt, const uint2 *cand, int cand_cap,
+                            hipStream_t st) {
+    hipLaunchKernelGGL(cand_row_kernel, dim3((unsigned)a.B), dim3(ROW_BLOCK), 0, st, a, thr, cand_cnt, cand, cand_cap);
+    return hipGetLastError();
+}
+
 template <bool VEC, bool LOCAL>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
     topk_row_body<VEC, LOCAL>(a);

@@ -83,6 +83,44 @@ def ForwardArgmax(sampler, layer, input, input_shape, tokens_out, stream=None):
     return tokens_out
 
 
+def ForwardSample(sampler, layer, input, input_shape, history, histLen, uniforms, tokens_out, probs_out=None, hist_stride=0,
+                  stream=None):
+    """The LM head and the sampling step in one call (born_rocm_linear_sample): tokens_out[b] is what sampler.Sample
+    draws from layer.Forward(input)[b], the logits never written.  A row the fused step cannot settle gets token -1
+    (sampler.Status() then reports it); ForwardSampleHost shows the fallback."""
+    if len(input_shape) != 2:
+        raise LinearPanic(f"Linear.Forward: expected 2D input [batch, features], got shape {list(input_shape)}")
+    batch, feat = int(input_shape[0]), int(input_shape[1])
+    if feat != layer.inFeatures:
+        raise LinearPanic(f"Linear.Forward: expected input with {layer.inFeatures} features, got {feat}")
+    _check(_capi.lib().born_rocm_linear_sample(sampler._h, _ptr(input), batch, layer.inFeatures, layer.inFeatures, _ptr(layer.weight),
+                                               layer.outFeatures, layer.inFeatures, _ptr(layer.bias), _ptr(history), _ptr(histLen),
+                                               hist_stride, _ptr(uniforms), _ptr(tokens_out), _ptr(probs_out), stream))
+    return tokens_out
+
+
+def ForwardSampleHost(sampler, layer, input, input_shape, history, histLen, uniforms, hist_stride=0):
+    """ForwardSample with the tokens and probabilities copied back, and the fallback a caller owes the rows the fused
+    step could not settle: the whole call is repeated as Forward + Sample over materialised logits.  Returns
+    (tokens, probs, fell_back)."""
+    batch = int(input_shape[0])
+    tok, pr = DeviceBuffer(4 * batch), DeviceBuffer(4 * batch)
+    ForwardSample(sampler, layer, input, input_shape, history, histLen, uniforms, tok, pr, hist_stride)
+    tokens = tok.to_numpy(np.int32, (batch,))
+    fell_back = bool((tokens < 0).any())
+    if fell_back:
+        try:
+            sampler.Status()                                         # clears the "could not settle" report
+        except _capi.BornRocmError as e:
+            if e.code != _capi.ERR_DATA:
+                raise
+        logits = DeviceBuffer(4 * batch * layer.outFeatures)
+        layer.Forward(input, input_shape, logits)
+        sampler.Sample(logits, batch, layer.outFeatures, history, histLen, uniforms, tok, pr, hist_stride=hist_stride)
+        tokens = tok.to_numpy(np.int32, (batch,))
+    return tokens, pr.to_numpy(np.float32, (batch,)), fell_back
+
+
 def NewLinear(in_features, out_features, seed=None, stream=None):
     """Xavier/Glorot-uniform weights in [-sqrt(6/(in+out)), +sqrt(6/(in+out))], zero bias, both uploaded to the
     device.  The reference draws from the process-global unseeded generator; a seed can be given here."""

@@ -253,6 +253,23 @@ int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int6
                             const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
                             int32_t *tokens_out, void *stream);
 
+/* The LM head and the sampling step in one call: tokens_out[b] is what born_rocm_sample draws from the logits
+ * born_rocm_linear would produce, bit for bit, and those [batch, out_features] logits are never written to memory —
+ * Linear.Forward (internal/nn/linear.go:78-107) with the reference's only logits consumers replaced by a sampler that
+ * lives in the GEMM's epilogue.  The handle's configuration must be one the single-pass sampler serves: 1 <= top_k <=
+ * 128, out_features <= 393216, repetition penalty >= 1, no frequency / presence penalty (else
+ * BORN_ROCM_ERR_UNSUPPORTED).  How: the product over a strided sample of at most 1024 weight rows gives every row a
+ * threshold that about 1500 of its logits reach; the full product's epilogue lists the logits at or above
+ * it (value and column); the sampling step runs over the list and proves that nothing outside it can belong to the
+ * row's top_k.  A row it cannot settle (a list of more than 4096, fewer than top_k candidates above the bound, a
+ * history of more than 1024 tokens with a penalty) gets token -1 and born_rocm_sampler_status returns
+ * BORN_ROCM_ERR_DATA: the caller then runs born_rocm_linear + born_rocm_sample for that call.  The first call on a
+ * handle allocates 48 KiB of workspace per row of max_batch (outside a stream capture). */
+int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
+                            const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
+                            const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
+                            int32_t *tokens_out, float *probs_out, void *stream);
+
 /* The element-wise and shape operations of tensor.Backend (internal/tensor/backend.go:12-33) on fp32 device
  * memory.  Operands are row-major and contiguous; shapes are given as arrays of `ndim` extents (0 <= ndim <= 8,
  * every extent > 0).  `out` is contiguous in the result's shape and must not overlap an operand.

@@ -347,3 +347,92 @@ def test_lm_head_and_sampling_step_replay_from_a_hip_graph(oracle, rocm, lin, ex
     ok(hip.hipStreamDestroy(stream))
     smp.Status()
     smp.Close()
+
+
+def _fused_vs_unfused(rocm, lin, x, w, bias, cfg, hist=None, expect_settled=True):
+    """Tokens and probabilities of born_rocm_linear_sample against born_rocm_linear + born_rocm_sample on the same
+    operands: the candidates the epilogue lists are the values the plain GEMM would write, so the two must agree bit
+    for bit.  Returns what the fused call gave."""
+    M, K = x.shape
+    N = w.shape[0]
+    rng = np.random.default_rng(M + 3 * N)
+    u = rng.random(M, dtype=np.float32)
+    s = rocm.NewSampler(cfg, max_batch=M, max_vocab=N)
+    layer = lin.Linear(K, N, rocm.DeviceBuffer.from_numpy(w), None if bias is None else rocm.DeviceBuffer.from_numpy(bias))
+    dx, du = rocm.DeviceBuffer.from_numpy(x), rocm.DeviceBuffer.from_numpy(u)
+    dh = None if hist is None else rocm.DeviceBuffer.from_numpy(hist)
+    H = 0 if hist is None else hist.shape[1]
+    logits = rocm.DeviceBuffer(M * N * 4)
+    layer.Forward(dx, (M, K), logits)
+    tok_ref, pr_ref = rocm.DeviceBuffer(4 * M), rocm.DeviceBuffer(4 * M)
+    s.Sample(logits, M, N, dh, None, du, tok_ref, pr_ref, hist_stride=H)
+    s.Status()
+    tok, pr = rocm.DeviceBuffer(4 * M), rocm.DeviceBuffer(4 * M)
+    lin.ForwardSample(s, layer, dx, (M, K), dh, None, du, tok, pr, hist_stride=H)
+    got, gp = tok.to_numpy(np.int32, (M,)), pr.to_numpy(np.float32, (M,))
+    want, wp = tok_ref.to_numpy(np.int32, (M,)), pr_ref.to_numpy(np.float32, (M,))
+    settled = got >= 0
+    if expect_settled:
+        s.Status()
+        assert settled.all(), np.nonzero(~settled)[0][:8]
+    assert np.array_equal(got[settled], want[settled])
+    assert np.array_equal(gp[settled].view(np.uint32), wp[settled].view(np.uint32))
+    # the host-side wrapper owes the caller the unsettled rows: it repeats the call unfused
+    t2, p2, fell_back = lin.ForwardSampleHost(s, layer, dx, (M, K), dh, None, du, hist_stride=H)
+    assert fell_back == (not settled.all())
+    assert np.array_equal(t2, want) and np.array_equal(p2.view(np.uint32), wp.view(np.uint32))
+    s.Close()
+    return got, settled
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 300), (5, 1000, 777), (16, 128, 2600), (17, 96, 1320), (48, 64, 4096), (65, 32, 5000),
+                                   (130, 257, 9000), (256, 512, 33000), (12, 4096, 32000)])
+def test_lm_head_sampling_fused_equals_linear_then_sample(rocm, lin, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(M * 31 + K * 7 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * (1.5 / np.sqrt(K))).astype(np.float32)
+    bias = (0.3 * rng.standard_normal(N)).astype(np.float32)
+    hist = rng.integers(0, N, size=(M, 40)).astype(np.int32)
+    cfg = rocm.SamplerConfig(Temperature=0.7, TopK=min(50, N - 1), TopP=0.9, RepetitionPenalty=1.15)
+    for b in (bias, None):
+        _fused_vs_unfused(rocm, lin, x, w, b, cfg, hist)
+    _fused_vs_unfused(rocm, lin, x, w, bias, rocm.SamplerConfig(Temperature=1.0, TopK=min(128, N - 1)), None)
+
+
+def test_lm_head_sampling_fused_penalised_favourites_and_unsettled_rows(rocm, lin):
+    """Histories that hold the very tokens a row favours (the penalty moves candidates across the cut), then rows the
+    fused step must hand back: every logit equal (the list overflows) and a history longer than the workgroup."""
+    M, K, N = 24, 128, 6000
+    rng = np.random.default_rng(99)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * (2.0 / np.sqrt(K))).astype(np.float32)
+    logits = x.astype(np.float64) @ w.astype(np.float64).T
+    hist = np.argsort(-logits, axis=1)[:, :60].astype(np.int32)      # the sixty largest of every row
+    cfg = rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.3)
+    _fused_vs_unfused(rocm, lin, x, w, None, cfg, hist, expect_settled=False)
+    # all logits equal: every column reaches the threshold
+    got, settled = _fused_vs_unfused(rocm, lin, np.zeros((3, K), np.float32), w, None, rocm.SamplerConfig(TopK=5), None, expect_settled=False)
+    assert not settled.any()
+    long_hist = rng.integers(0, N, size=(M, 1500)).astype(np.int32)
+    got, settled = _fused_vs_unfused(rocm, lin, x, w, None, cfg, long_hist, expect_settled=False)
+    assert not settled.any()
+
+
+def test_lm_head_sampling_fused_argument_errors(rocm, lin):
+    from born_amd import _capi
+    M, K, N = 4, 64, 500
+    x = rocm.DeviceBuffer.from_numpy(np.zeros((M, K), np.float32))
+    layer = lin.Linear(K, N, rocm.DeviceBuffer.from_numpy(np.zeros((N, K), np.float32)), None)
+    u = rocm.DeviceBuffer.from_numpy(np.zeros(M, np.float32))
+    tok = rocm.DeviceBuffer(4 * M)
+    for cfg in (rocm.SamplerConfig(TopP=0.9), rocm.SamplerConfig(TopK=200), rocm.SamplerConfig(TopK=5, FrequencyPenalty=0.5)):
+        s = rocm.NewSampler(cfg, max_batch=M, max_vocab=N)
+        with pytest.raises(_capi.BornRocmError) as e:
+            lin.ForwardSample(s, layer, x, (M, K), None, None, u, tok)
+        assert e.value.code == _capi.ERR_UNSUPPORTED
+        s.Close()
+    s = rocm.NewSampler(rocm.SamplerConfig(TopK=5), max_batch=M, max_vocab=N)
+    with pytest.raises(rocm.SamplerPanic):
+        lin.ForwardSample(s, layer, x, (M + 1, K), None, None, u, tok)        # beyond the handle's batch
+    s.Close()
