@@ -119,6 +119,56 @@ func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]i
 	return tokens, nil
 }
 
+// ForwardSample is the layer and the sampling step in one call (born_rocm_linear_sample): tokens[b] is what
+// s.Sample draws from Forward(input)[b], and the [batch, out_features] logits are never written.  The sampler's
+// configuration must be one the single-pass kernel serves (1 <= TopK <= 128, RepetitionPenalty >= 1, no frequency or
+// presence penalty).  A row the fused step cannot settle comes back as -1; the whole call is then repeated over
+// materialised logits (Forward + Sample), so the caller always gets the tokens of the unfused pair.
+func (l *Linear) ForwardSample(s *Sampler, input DeviceBuffer, shape []int, history DeviceBuffer, histStride int,
+	histLen, uniforms DeviceBuffer) ([]int32, error) {
+	if len(shape) != 2 {
+		panic(fmt.Sprintf("Linear.Forward: expected 2D input [batch, features], got shape %v", shape))
+	}
+	if shape[1] != l.inFeatures {
+		panic(fmt.Sprintf("Linear.Forward: expected input with %d features, got %d", l.inFeatures, shape[1]))
+	}
+	batch := shape[0]
+	out := s.results(batch)
+	if err := call(func() C.int {
+		return C.born_rocm_linear_sample(s.h, (*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
+			C.int64_t(l.inFeatures), (*C.float)(l.weight.ptr), C.int64_t(l.outFeatures), C.int64_t(l.inFeatures),
+			(*C.float)(l.bias.ptr), (*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride),
+			(*C.float)(uniforms.ptr), (*C.int32_t)(out.ptr), nil, nil)
+	}); err != nil {
+		return nil, err
+	}
+	tokens := make([]int32, batch)
+	if err := out.Download(unsafe.Pointer(&tokens[0]), int64(4*batch)); err != nil { // synchronises the stream
+		return nil, err
+	}
+	settled := true
+	for _, t := range tokens {
+		if t < 0 {
+			settled = false
+			break
+		}
+	}
+	status := call(func() C.int { return C.born_rocm_sampler_status(s.h, nil) })
+	if settled {
+		return tokens, status
+	}
+	// the status only repeated what the tokens said; the rows are settled over materialised logits
+	logits, err := Alloc(int64(4 * batch * l.outFeatures))
+	if err != nil {
+		return nil, err
+	}
+	defer logits.Free()
+	if err := l.Forward(input, shape, logits, nil); err != nil {
+		return nil, err
+	}
+	return s.Sample(logits, batch, l.outFeatures, history, histStride, histLen, uniforms)
+}
+
 // MatMul computes c[m,n] = a[m,k] @ b[k,n] (tensor.Backend.MatMul, internal/tensor/backend.go:20; the CPU
 // form and its panics: internal/backend/cpu/matmul.go:13-50).  aShape and bShape are the 2-D shapes.
 func MatMul(a DeviceBuffer, aShape []int, b DeviceBuffer, bShape []int, c DeviceBuffer, stream unsafe.Pointer) error {

@@ -161,6 +161,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over;
     __shared__ u64 s_win, s_mass;
+    __shared__ u32 s_wcount[NUC_WAVES];
 
     u64 *const mass = nuc_dyn;                                                   // [NUC_BINS] masses, then cumulative
     uint2 *const stage = reinterpret_cast<uint2 *>(nuc_dyn + NUC_BINS);          // [NUC_WAVES][NUC_WCAP] (logit bits, id)
@@ -270,25 +271,26 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         nuc_range(r, w1, lo1, hi1);
         nuc_range(r, w2, lo2, hi2);
         uint2 *list = stage + wave_id() * NUC_WCAP;
-        u32 count = 0;
+        // The wave's running count of staged entries lives in LDS, not in a register of every lane: the row visitor
+        // lets different lanes of a wave sit out different visits (the row's last whole float4 blocks end inside a
+        // wave, its ragged tail starts again at lane 0), and a lane that missed an append must not reuse a position.
+        // Whichever lane appends first in a visit advances the count; LDS operations of one wave complete in order.
+        volatile u32 *const wcount = &s_wcount[wave_id()];         // (volatile: another lane's store must be re-read)
+        if (lane_id() == 0) *wcount = 0u;                            // (this wave's own earlier LDS operations precede it)
         nuc_foreach(r, bm, [&](int j, float y) {
             const bool pass = (!(y < lo0) && !(y > hi0)) || (!(y < lo1) && !(y > hi1)) || (!(y < lo2) && !(y > hi2));
             const u64 mk = __ballot(pass);
-            if (mk) {                                                // wave-uniform
-                // A lane that sat out earlier visits (the row's last whole float4 blocks end inside the wave, its ragged
-                // tail starts again at lane 0) has missed their appends; lane 0 takes part whenever any lane of its wave
-                // does, so its count is the wave's.
-                count = (u32)__builtin_amdgcn_readfirstlane((int)count);
+            if (mk) {                                                // uniform over the lanes that take part in this visit
+                const u32 base = *wcount;
                 if (pass) {
-                    const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                    const u32 rank = __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                    const u32 pos = base + rank;
                     if (pos < (u32)NUC_WCAP) list[pos] = make_uint2(__float_as_uint(y), (u32)j);
+                    if (rank == 0u) *wcount = base + (u32)__popcll(mk);
                 }
-                count += (u32)__popcll(mk);
             }
         });
-        // A lane that sat out the last visits (a ragged end of the row) has counted fewer appends than were made; lane 0
-        // takes part whenever any lane of its wave does, so its count is the wave's.
-        count = (u32)__builtin_amdgcn_readfirstlane((int)count);
+        const u32 count = *wcount;
         if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
         const int cw = (int)min(count, (u32)NUC_WCAP);
         for (int e0 = 0; e0 < cw; e0 += WAVE) {

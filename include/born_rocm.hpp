@@ -185,6 +185,18 @@ public:
                                         std::to_string(features));
         check(born_rocm_linear(input_dev, batch, in_, in_, w_, out_, in_, b_, out_dev, out_, stream));
     }
+    // The layer and the sampling step in one call (born_rocm_linear_sample): tokens_dev[b] is what the sampler draws
+    // from Forward(input)[b], the logits never written; a row the fused step cannot settle gets token -1 (the caller
+    // then runs Forward + Sampler::Sample for the call).
+    void ForwardSample(const Sampler &sampler, const float *input_dev, int64_t batch, int64_t features, const int32_t *history_dev,
+                       int64_t hist_stride, const int32_t *hist_len_dev, const float *uniforms_dev, int32_t *tokens_dev,
+                       float *probs_dev = nullptr, void *stream = nullptr) const {
+        if (features != in_)
+            throw std::invalid_argument("Linear.Forward: expected input with " + std::to_string(in_) + " features, got " +
+                                        std::to_string(features));
+        check(born_rocm_linear_sample(sampler.handle(), input_dev, batch, in_, in_, w_, out_, in_, b_, history_dev, hist_len_dev,
+                                      hist_stride, uniforms_dev, tokens_dev, probs_dev, stream));
+    }
 
 private:
     int64_t in_, out_;

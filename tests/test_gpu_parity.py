@@ -586,6 +586,33 @@ def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pa
         s.Close()
 
 
+@pytest.mark.parametrize("pad_extra", [0, 4])
+def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra):
+    # every vocabulary size modulo 256 (so: every way the row's last whole 128-bit blocks and its ragged tail can fall
+    # on the lanes of a wave), at two row pitches; few distinct values, so that the wanted bins take entries from all
+    # parts of the row and a lost or duplicated staged entry changes the result
+    B, H = 3, 24
+    for V in range(4096, 4096 + 256):
+        rng = np.random.default_rng(V * 7 + pad_extra)
+        x = np.round(rng.standard_normal((B, V)) * 0.6).astype(np.float32)
+        u = rng.random(B, dtype=np.float32)
+        hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+        stride = ((V + 3) & ~3) + pad_extra
+        host = np.full(B * stride + 8, np.nan, dtype=np.float32)
+        for b in range(B):
+            host[b * stride: b * stride + V] = x[b]
+        T, p, rep = (1.0, 0.9, 1.2) if V % 2 else (0.7, 1.0, 1.0)
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=0, TopP=p, RepetitionPenalty=rep), max_batch=B, max_vocab=V)
+        d_x, d_u, d_h = rocm.DeviceBuffer.from_numpy(host), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer.from_numpy(hist)
+        tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
+        s.Sample(d_x, B, V, d_h, None, d_u, tok, pr, row_stride=stride, hist_stride=H)
+        s.Status()
+        fx = oracle.sample(x, u, T, 0, p, rep, hist, None, mode=oracle.MODE_FIXED)
+        assert np.array_equal(tok.to_numpy(np.int32, (B,)), fx["tokens"]), (V, pad_extra)
+        assert np.array_equal(pr.to_numpy(np.float32, (B,)).view(np.uint32), fx["probs"].view(np.uint32)), (V, pad_extra)
+        s.Close()
+
+
 def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
     # the case a wide seeded sweep of test_random_row_layouts_against_oracle found (its chunk 1096, third case)
     import test_gpu_parity_random as R
