@@ -10,7 +10,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libborn_rocm.so")
-SOURCES = ["api.hip", "basic_kernels.hip", "topk_row.hip", "nucleus_row.hip", "sample_wide.hip", "spec_kernels.hip", "linear.hip", "tensor_ops.hip"]
+SOURCES = ["api.hip", "basic_kernels.hip", "topk_row.hip", "nucleus_row.hip", "sample_wide.hip", "spec_kernels.hip", "linear.hip", "tensor_ops.hip",
+           "division.cpp"]          # .cpp: host code only
 
 # -ffp-contract=off and correctly rounded fp32 division: every floating-point step of the
 # fixed-point pipeline must be a single IEEE rounding, identical on host and device.
@@ -20,6 +21,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+HOST_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-Wall"]
 
 
 def hipcc():
@@ -34,8 +36,11 @@ def build(verbose=False):
     objs = []
     procs = []
     for src in SOURCES:
-        obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
-        cmd = [hipcc()] + FLAGS + os.environ.get("BORN_EXTRA_HIPCC_FLAGS", "").split() + ["-c", os.path.join(CSRC, src), "-o", obj]
+        obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + ".o")
+        if src.endswith(".cpp"):
+            cmd = [hipcc()] + HOST_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        else:
+            cmd = [hipcc()] + FLAGS + os.environ.get("BORN_EXTRA_HIPCC_FLAGS", "").split() + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

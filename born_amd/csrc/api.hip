@@ -48,6 +48,7 @@ struct born_sampler {
     unsigned long long step;       // draws made with the built-in uniform stream
     int path;                      // see born_rocm_sampler_set_path
     bool fixed_workspace;          // the workspace may not grow (born_rocm_sample_static: nothing is allocated, ever)
+    float div_T, div_rcp;          // the last temperature whose division shortcut was looked up, and the answer (kernels.h, rcp_T)
     // device workspace
     float *arg_val;                // argmax partials [max_batch][S_max]
     int *arg_idx;
@@ -436,6 +437,13 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
     } else if (launched == 1u) {
         keep_first(launch_topk_row(a, st));
     } else if (launched == 2u) {
+        if (a.T != 1.0f) {                                           // (host arithmetic only: nothing is launched or waited for)
+            if (s->div_T != a.T) {
+                s->div_rcp = division_shortcut_reciprocal(a.T);
+                s->div_T = a.T;
+            }
+            a.rcp_T = s->div_rcp;
+        }
         keep_first(launch_nucleus_row(a, st));
     } else {
         keep_first(launch_sample_wide(a, st));

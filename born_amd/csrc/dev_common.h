@@ -48,11 +48,11 @@ __device__ __forceinline__ int key64_id(u64 k) { return (int)(0xFFFFFFFFu - (u32
 __device__ __forceinline__ float key64_z(u64 k) { return ordkey_inv((u32)(k >> 32)); }
 
 // NaN -> -inf, +inf -> FLT_MAX, -0 -> +0
+// (selects, not early returns: the early returns compiled to three nested branches per logit)
 __device__ __forceinline__ float canon(float z) {
-    if (z != z) return -INFINITY;
-    if (z > 3.402823466e+38f) return 3.402823466e+38f;
-    if (z == 0.0f) return 0.0f;
-    return z;
+    z = (z != z) ? -INFINITY : z;
+    z = (z > 3.402823466e+38f) ? 3.402823466e+38f : z;
+    return (z == 0.0f) ? 0.0f : z;
 }
 __device__ __forceinline__ float penalise(float x, float r) { return x > 0.0f ? x / r : x * r; }
 
@@ -85,8 +85,8 @@ __device__ __forceinline__ float next_below(float x) {
 // exp(-d), d >= 0; see the spec, section 6.  dcut <= 80: the distance beyond which the mass is zero (80, or the
 // min-p bound -ln(min_p) when that is smaller).
 __device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
-    if (!(d <= dcut)) return 0.0f;
-    float x = -d;
+    const bool in = d <= dcut;                                    // false for NaN too
+    float x = in ? -d : 0.0f;                                     // (a select at each end instead of a branch around the polynomial)
     float k = rintf(x * 1.44269504f);
     float r = fmaf(k, -0.693145752f, x);
     r = fmaf(k, -1.42860677e-06f, r);
@@ -98,7 +98,8 @@ __device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
     float r2 = r * r;
     y = fmaf(y, r2, r);
     y = y + 1.0f;
-    return __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
+    const float e = __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
+    return in ? e : 0.0f;
 }
 __device__ __forceinline__ float emass(float z, float m, float dcut = 80.0f) {
     float d = (z == m) ? 0.0f : m - z;

@@ -59,7 +59,13 @@ struct SampleArgs {
     // the single-pass kernel counts the occurrences itself (in the hash of the history it builds anyway) and no
     // table is passed: histories of at most TOPK_LOCAL_COUNT_HISTORY tokens
     int local_counts;
+    // RN(1 / T) when the three-instruction division shortcut equals the correctly rounded y / T for every y it is
+    // applied to (division.cpp decides, on the host), else 0: the kernels then divide
+    float rcp_T;
 };
+
+// division.cpp
+float division_shortcut_reciprocal(float T);
 
 // Per-row configurations (device arrays of B values, each optional): a second argument of the per-row kernel
 // instances only, so that the uniform instances keep their argument block (and register allocation) as it is.

@@ -20,12 +20,15 @@
 
 namespace born {
 
-constexpr int NUC_BLOCK = 1024;
+#ifndef BORN_NUC_BLOCK
+#define BORN_NUC_BLOCK 1024
+#endif
+constexpr int NUC_BLOCK = BORN_NUC_BLOCK;
 constexpr int NUC_WAVES = NUC_BLOCK / WAVE;
 constexpr int NUC_U = 4;                      // 128-bit loads per thread and stage
 constexpr int NUC_BINS = 4096;
-constexpr int NUC_WCAP = 160;                 // staged entries per wave
-constexpr int NUC_CAP = 1024;                 // gathered entries (one per thread)
+constexpr int NUC_WCAP = NUC_BLOCK == 1024 ? 160 : 256;   // staged entries per wave
+constexpr int NUC_CAP = NUC_BLOCK;            // gathered entries (one per thread)
 constexpr int NUC_PER = NUC_BINS / NUC_BLOCK; // bins per thread in the scan
 
 typedef float nuc_f32x4 __attribute__((ext_vector_type(4)));
@@ -34,7 +37,7 @@ struct NucRow {                               // uniform per workgroup
     const float *x;
     int V;
     bool vec, penal, degenerate;
-    float T, rep, m, scale, range, sbin, dcut;
+    float T, rcp, rep, m, scale, range, sbin, dcut;        // rcp: RN(1 / T) where the division shortcut is exact, else 0
     const unsigned *counts;                   // occurrences of each id in the row's history (frequency / presence penalties), or null
     float freq, pres;
 };
@@ -45,7 +48,17 @@ __device__ __forceinline__ float nuc_z(const NucRow &r, float y) {
 }
 __device__ __forceinline__ float nuc_d(const NucRow &r, float z) { return r.degenerate ? 0.0f : r.m - z; }
 __device__ __forceinline__ int nuc_bin(const NucRow &r, float d) {
-    return d < r.range ? min((int)(d * r.sbin), NUC_BINS - 1) : NUC_BINS - 1;   // monotone in d; NaN and inf -> last bin
+    return (int)fminf(d * r.sbin, (float)(NUC_BINS - 1));          // monotone in d; NaN, inf and all beyond the span -> last bin
+}
+// z for a logit of ordinary magnitude by the division shortcut (r.rcp != 0): equal to nuc_z for 2^-100 <= |y| < 2^100,
+// which `ordinary` tests; the result is finite and not zero, so it is its own canonical form.
+__device__ __forceinline__ bool nuc_ordinary(float y) {
+    return ((__float_as_uint(y) & 0x7FFFFFFFu) - (27u << 23)) < (200u << 23);
+}
+__device__ __forceinline__ float nuc_z_shortcut(const NucRow &r, float y) {
+    const float q = __fmul_rn(y, r.rcp);
+    const float e = __fmaf_rn(-q, r.T, y);
+    return __fmaf_rn(e, r.rcp, q);
 }
 
 // Visits every element of the row with its penalised logit: aligned rows four at a time as f4(id of the first, y[4]),
@@ -156,7 +169,8 @@ __device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, fl
 // its own instance, so that the usual one carries none of it.
 template <bool COUNTED>
 __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep,
-                                                 const float cfg_dcut, const float cfg_freq, const float cfg_pres) {
+                                                 const float cfg_dcut, const float cfg_freq, const float cfg_pres,
+                                                 const float cfg_rcp) {
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over;
@@ -177,6 +191,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     r.V = V;
     r.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
     r.T = cfg_T;
+    r.rcp = cfg_rcp;
     r.rep = cfg_rep;
     r.scale = mass_scale(a.mass_shift);
     r.dcut = cfg_dcut;
@@ -227,10 +242,19 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 
     BORN_STAMP(a, row, 2);
     // ---- sweep 2: integer masses by bin
-    nuc_foreach(r, bm, [&](int, float y) {
-        const float d = nuc_d(r, nuc_z(r, y));
-        atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-    });
+    if (r.rcp != 0.0f && !r.degenerate) {
+        nuc_foreach(r, bm, [&](int, float y) {
+            float z = nuc_z_shortcut(r, y);
+            if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
+            const float d = r.m - z;
+            atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
+        });
+    } else {
+        nuc_foreach(r, bm, [&](int, float y) {
+            const float d = nuc_d(r, nuc_z(r, y));
+            atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
+        });
+    }
     __syncthreads();
     BORN_STAMP(a, row, 3);
     u64 Zk;
@@ -270,27 +294,50 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         nuc_range(r, w0, lo0, hi0);
         nuc_range(r, w1, lo1, hi1);
         nuc_range(r, w2, lo2, hi2);
+        // The three value ranges as disjoint intervals in ascending order, overlapping ones merged (the draw's two bins
+        // are neighbours, and often the cut's bin is one of them): most rows test one or two intervals per logit.
+        // An unused interval is (+inf, -inf), which only a NaN passes (as it passes a real one: classified below).
+        if (lo1 < lo0) { float t = lo0; lo0 = lo1; lo1 = t; t = hi0; hi0 = hi1; hi1 = t; }
+        if (lo2 < lo1) { float t = lo1; lo1 = lo2; lo2 = t; t = hi1; hi1 = hi2; hi2 = t; }
+        if (lo1 < lo0) { float t = lo0; lo0 = lo1; lo1 = t; t = hi0; hi0 = hi1; hi1 = t; }
+        int nint = 3;
+        if (!(lo1 > hi0)) { hi0 = fmaxf(hi0, hi1); lo1 = lo2; hi1 = hi2; lo2 = INFINITY; hi2 = -INFINITY; nint--; }
+        if (nint == 3 ? !(lo2 > hi1) : !(lo1 > hi0)) {
+            if (nint == 3) { hi1 = fmaxf(hi1, hi2); lo2 = INFINITY; hi2 = -INFINITY; }
+            else { hi0 = fmaxf(hi0, hi1); lo1 = INFINITY; hi1 = -INFINITY; }
+            nint--;
+        }
         uint2 *list = stage + wave_id() * NUC_WCAP;
         // The wave's running count of staged entries lives in LDS, not in a register of every lane: the row visitor
         // lets different lanes of a wave sit out different visits (the row's last whole float4 blocks end inside a
         // wave, its ragged tail starts again at lane 0), and a lane that missed an append must not reuse a position.
         // Whichever lane appends first in a visit advances the count; LDS operations of one wave complete in order.
-        volatile u32 *const wcount = &s_wcount[wave_id()];         // (volatile: another lane's store must be re-read)
-        if (lane_id() == 0) *wcount = 0u;                            // (this wave's own earlier LDS operations precede it)
-        nuc_foreach(r, bm, [&](int j, float y) {
-            const bool pass = (!(y < lo0) && !(y > hi0)) || (!(y < lo1) && !(y > hi1)) || (!(y < lo2) && !(y > hi2));
+        const int wid = wave_id();
+        // (relaxed atomic accesses: re-read at every visit as a volatile would be, but they keep the LDS address space,
+        // where a volatile access became a flat one that waits for the row's loads in flight)
+        u32 *const wcount = &s_wcount[wid];
+        if (lane_id() == 0) __hip_atomic_store(wcount, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        auto append = [&](bool pass, float y, int j) {
             const u64 mk = __ballot(pass);
             if (mk) {                                                // uniform over the lanes that take part in this visit
-                const u32 base = *wcount;
+                const u32 base = __hip_atomic_load(wcount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
                 if (pass) {
                     const u32 rank = __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
                     const u32 pos = base + rank;
                     if (pos < (u32)NUC_WCAP) list[pos] = make_uint2(__float_as_uint(y), (u32)j);
-                    if (rank == 0u) *wcount = base + (u32)__popcll(mk);
+                    if (rank == 0u) __hip_atomic_store(wcount, base + (u32)__popcll(mk), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
                 }
             }
-        });
-        const u32 count = *wcount;
+        };
+        // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
+        if (nint == 1) {
+            nuc_foreach(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+        } else {
+            nuc_foreach(r, bm, [&](int j, float y) {
+                append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
+            });
+        }
+        const u32 count = __hip_atomic_load(wcount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
         if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
         const int cw = (int)min(count, (u32)NUC_WCAP);
         for (int e0 = 0; e0 < cw; e0 += WAVE) {
@@ -350,7 +397,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     u64 Zp = Zk, tokkey = 0ull;
     u64 *const smass = reinterpret_cast<u64 *>(stage);               // [2048] sub-histogram of masses
     u32 *const scnt = reinterpret_cast<u32 *>(fkey);                 // [2048] and of counts
-    static_assert(NUC_WAVES * NUC_WCAP >= 2048 && NUC_CAP * 2 >= 2048, "the sub-histograms fit the list storage");
+    static_assert(NUC_WAVES * NUC_WCAP >= 2048 && NUC_CAP * 4 >= 2048, "the sub-histograms fit the list storage");
     for (int phase = cut ? 0 : 1; phase < 2; phase++) {
         const u64 target = phase == 0 ? tp : draw_target(u, Zp);
         const int b = phase == 0 ? w0 : nuc_first_reaching(cum, target);
@@ -467,8 +514,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 }
 
 template <bool COUNTED>
-__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_kernel(SampleArgs a) {
-    nucleus_row_body<COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres);
+__global__ __launch_bounds__(NUC_BLOCK, 4) void nucleus_row_kernel(SampleArgs a) {
+    nucleus_row_body<COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres, a.rcp_T);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
 template <bool COUNTED>
@@ -480,7 +527,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs 
         row_config_reject(a, (int)blockIdx.x);
         return;
     }
-    nucleus_row_body<COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres);
+    nucleus_row_body<COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres, 0.0f);   // (a row's own temperature: no shortcut)
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -225,6 +225,63 @@ def test_topk_kernel_ties_and_special_values(oracle, rocm, path):
     _check_against_oracle(oracle, rocm, x, u, 1.0, 40, 0.95, nuc=64, path=path)
 
 
+def _shaped_rows(kind, B, V, rng):
+    """Rows whose large values sit where a threshold that tightens while the row streams is most easily
+    wrong: late in the row, in a narrow band, in huge ranges, or tied across the cut."""
+    i = np.arange(V, dtype=np.float64)
+    if kind == "ascending":                 # every later stage beats everything before it
+        x = np.tile(i / V * 20 - 10, (B, 1)) + rng.standard_normal((B, V)) * 1e-3
+    elif kind == "descending":              # the first stage already holds the whole answer
+        x = np.tile(10 - i / V * 20, (B, 1)) + rng.standard_normal((B, V)) * 1e-3
+    elif kind == "late_step":               # the answer lies wholly in the last tenth of the row
+        x = rng.standard_normal((B, V))
+        x[:, V - V // 10:] += 30
+    elif kind == "late_few":                # a handful of winners at the very end, nothing close to them
+        x = rng.standard_normal((B, V))
+        x[:, -37:] += 12
+    elif kind == "cauchy":                  # a range of 1e6 and more between neighbours in order
+        x = rng.standard_cauchy((B, V)) * 3
+    elif kind == "narrow":                  # the whole row within a few hundred ulps
+        x = 5.0 + rng.integers(0, 300, size=(B, V)) * 2.0 ** -21
+    elif kind == "few_values":              # a dozen distinct values: ties across every cut
+        x = rng.integers(0, 12, size=(B, V)) * 0.37 - 2
+    elif kind == "negative_huge":           # large negative magnitudes: order keys far from the float's own order
+        x = -np.abs(rng.standard_normal((B, V))) * 1e30
+    elif kind == "rising_blocks":           # each block of 4096 a little higher than the last one
+        x = rng.standard_normal((B, V)) + (np.arange(V) // 4096) * 0.5
+    else:
+        raise ValueError(kind)
+    return x.astype(np.float32)
+
+
+@pytest.mark.parametrize("kind", ["ascending", "descending", "late_step", "late_few", "cauchy", "narrow", "few_values",
+                                  "negative_huge", "rising_blocks"])
+@pytest.mark.parametrize("V,pad", [(49152, 0), (49153, 3), (65537, 0), (128256, 0), (151937, 7), (393216, 0)])
+def test_topk_kernel_rows_that_stress_the_streamed_threshold(oracle, rocm, kind, V, pad):
+    """The single-pass kernel raises its threshold while the row streams. Whatever the shape of the row, the
+    result is the oracle's, bit for bit: either the single pass proves its candidate set or the row falls back."""
+    rng = np.random.default_rng([len(kind), ord(kind[0]), ord(kind[-1]), V])
+    B, H = 6, 96
+    x = _shaped_rows(kind, B, V, rng)
+    u = rng.random(B, dtype=np.float32)
+    top = np.argsort(-x, axis=1, kind="stable")[:, :H // 2].astype(np.int32)      # half the history penalises the winners
+    hist = np.concatenate([top, rng.integers(0, V, size=(B, H - H // 2)).astype(np.int32)], axis=1)
+    for k, p, rep in [(50, 0.9, 1.3), (128, 1.0, 1.0), (1, 1.0, 2.0)]:
+        want = oracle.sample(x, u, 0.7, k, p, rep, hist if rep != 1.0 else None, mode=oracle.MODE_FIXED, nuc_cap=min(k, 64))
+        s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.7, TopK=k, TopP=p, RepetitionPenalty=rep), max_batch=B, max_vocab=V)
+        xp = np.full((B, V + pad), 1e38, np.float32)                                  # padding must never be read as data
+        xp[:, :V] = x
+        d_x, d_u, d_t, d_p = rocm.DeviceBuffer.from_numpy(xp), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
+        d_h = rocm.DeviceBuffer.from_numpy(hist) if rep != 1.0 else None
+        s.Sample(d_x, B, V, d_h, None, d_u, d_t, probs_out=d_p, row_stride=V + pad, hist_stride=H if rep != 1.0 else 0)
+        s.Status()
+        c = s.Counters()
+        s.Close()
+        assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
+        assert np.array_equal(d_t.to_numpy(np.int32, (B,)), want["tokens"]), (kind, V, k)
+        assert np.array_equal(d_p.to_numpy(np.float32, (B,)).view(np.uint32), want["probs"].view(np.uint32)), (kind, V, k)
+
+
 @pytest.mark.parametrize("path", TOPK_PATHS)
 def test_topk_and_general_kernels_agree(oracle, rocm, path):
     rng = np.random.default_rng(7)
@@ -611,6 +668,28 @@ def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra):
         assert np.array_equal(tok.to_numpy(np.int32, (B,)), fx["tokens"]), (V, pad_extra)
         assert np.array_equal(pr.to_numpy(np.float32, (B,)).view(np.uint32), fx["probs"].view(np.uint32)), (V, pad_extra)
         s.Close()
+
+
+@pytest.mark.parametrize("T", [0.7, 1.2, 0.35, 1.9999999, 1.0])
+def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, rocm, T):
+    """Without a top-k cut every logit is divided by the temperature. For most temperatures the kernel replaces the
+    division by a multiplication and two fused multiply-adds that give the same quotient for logits of ordinary
+    magnitude (1.9999999 is a temperature it must divide by); zeros, denormals, tiny and huge values, infinities
+    and NaNs take the division itself. All of them, mixed into ordinary rows: bit-exact against the oracle."""
+    rng = np.random.default_rng(int(T * 1e6))
+    B, V = 12, 20011
+    x = (rng.standard_normal((B, V)) * 2.5).astype(np.float32)
+    odd = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 3e-31, -3e-31, 7.9e-31, 2 ** -100, -(2 ** -100), 2 ** -101, 1.2e30, -1.2e30,
+                    2 ** 100, 2 ** 99, -(2 ** 100), 3e38, -3e38, np.inf, -np.inf, np.nan], dtype=np.float32)
+    for b in range(1, B):
+        at = rng.choice(V, size=40 * b, replace=False)
+        x[b, at] = rng.choice(odd if b % 3 else odd[:17], size=at.size)        # (rows b % 3 == 0: no infinities, no huge values)
+    x[5, :] = rng.choice(np.array([0.0, -0.0, 1e-45, 2 ** -101, 3e-31], dtype=np.float32), size=V)   # nothing of ordinary magnitude
+    u = rng.random(B, dtype=np.float32)
+    hist = rng.integers(0, V, size=(B, 64)).astype(np.int32)
+    for p, rep, min_p in [(0.9, 1.0, 0.0), (1.0, 1.3, 0.0), (0.97, 1.1, 0.02)]:
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, 0, p, rep, hist if rep != 1.0 else None, min_p=min_p)
+        assert got["counters"]["general_rows"] == B and got["counters"]["topk_rows"] == 0
 
 
 def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
