@@ -229,7 +229,7 @@ int born_rocm_sampler_set_config(born_sampler *s, const born_sampler_config *cfg
 }
 
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path) {
-    if (!s || path < 0 || path > 1) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
+    if (!s || path < 0 || path > 2) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_path: null handle or unknown path");
     s->path = path;
     return BORN_ROCM_OK;
 }
@@ -432,7 +432,7 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.path = s->path;
         rows.launched = launched;
         if (launched & 1u) keep_first(launch_topk_row(a, st, &rows));
-        if (launched & 2u) keep_first(launch_nucleus_row(a, st, &rows));
+        if (launched & 2u) keep_first(launch_nucleus_row(a, st, &rows, s->path == 2));
         if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
     } else if (launched == 1u) {
         keep_first(launch_topk_row(a, st));
@@ -444,7 +444,7 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
             }
             a.rcp_T = s->div_rcp;
         }
-        keep_first(launch_nucleus_row(a, st));
+        keep_first(launch_nucleus_row(a, st, nullptr, s->path == 2));
     } else {
         keep_first(launch_sample_wide(a, st));
     }

@@ -20,16 +20,22 @@
 
 namespace born {
 
-#ifndef BORN_NUC_BLOCK
-#define BORN_NUC_BLOCK 1024
-#endif
-constexpr int NUC_BLOCK = BORN_NUC_BLOCK;
-constexpr int NUC_WAVES = NUC_BLOCK / WAVE;
+// Threads per row: 1024 (one workgroup per CU: the shortest time per row, for batches that leave CUs idle anyway) or
+// 512 (two workgroups per CU: one row's sweeps that wait for memory overlap the other's sweep that computes; for
+// batches of more rows than the device has CUs). The geometry below follows from it.
 constexpr int NUC_U = 4;                      // 128-bit loads per thread and stage
 constexpr int NUC_BINS = 4096;
-constexpr int NUC_WCAP = NUC_BLOCK == 1024 ? 160 : 256;   // staged entries per wave
-constexpr int NUC_CAP = NUC_BLOCK;            // gathered entries (one per thread)
-constexpr int NUC_PER = NUC_BINS / NUC_BLOCK; // bins per thread in the scan
+template <int BLOCK>
+struct NucGeom {
+    static_assert(BLOCK == 512 || BLOCK == 1024, "threads per row");
+    static constexpr int WAVES = BLOCK / WAVE;
+    static constexpr int WCAP = BLOCK == 1024 ? 160 : 256;       // staged entries per wave
+    static constexpr int CAP = BLOCK;                             // gathered entries (one per thread)
+    static constexpr int PER = NUC_BINS / BLOCK;                  // bins per thread in the scan
+    static constexpr int SUB = 2048 / BLOCK;                      // sub-bins per thread in a radix-descent scan
+    static_assert(WAVES * WCAP >= 2048 && CAP * 4 >= 2048, "the sub-histograms fit the list storage");
+};
+constexpr int NUC_BLOCK_MAX = 1024;
 
 typedef float nuc_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -75,7 +81,7 @@ template <bool NT>
 __device__ __forceinline__ nuc_f32x4 nuc_load4(const nuc_f32x4 *p) {
     return NT ? __builtin_nontemporal_load(p) : *p;
 }
-template <bool NT = false, class F4, class F1, class PRE = NucNoPre>
+template <int NUC_BLOCK, bool NT = false, class F4, class F1, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
@@ -128,9 +134,9 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     }
 }
 // Visits every element of the row as f(id, penalised logit).
-template <class F>
+template <int NUC_BLOCK, class F>
 __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
-    nuc_foreach4(r, bm, [&](int j, const float (&y)[4]) {
+    nuc_foreach4<NUC_BLOCK>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
     }, f);
@@ -167,10 +173,12 @@ __device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, fl
 // cfg_T, cfg_p, cfg_rep: the row's temperature, top_p and repetition penalty (the handle's, or the row's own).
 // COUNTED: a frequency or presence penalty is on (the table of occurrence counts is read for ids the history holds);
 // its own instance, so that the usual one carries none of it.
-template <bool COUNTED>
+template <int NUC_BLOCK, bool COUNTED>
 __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep,
                                                  const float cfg_dcut, const float cfg_freq, const float cfg_pres,
                                                  const float cfg_rcp) {
+    constexpr int NUC_WAVES = NucGeom<NUC_BLOCK>::WAVES, NUC_WCAP = NucGeom<NUC_BLOCK>::WCAP, NUC_CAP = NucGeom<NUC_BLOCK>::CAP,
+                  NUC_PER = NucGeom<NUC_BLOCK>::PER, NUC_SUB = NucGeom<NUC_BLOCK>::SUB;
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over;
@@ -225,7 +233,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     // ---- sweep 1: maximum and smallest finite penalised logit
     {
         float mx = -INFINITY, mn = INFINITY;
-        nuc_foreach(r, bm, [&](int, float y) {
+        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
             mx = fmaxf(mx, y);
             mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
         });
@@ -243,14 +251,14 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     BORN_STAMP(a, row, 2);
     // ---- sweep 2: integer masses by bin
     if (r.rcp != 0.0f && !r.degenerate) {
-        nuc_foreach(r, bm, [&](int, float y) {
+        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         });
     } else {
-        nuc_foreach(r, bm, [&](int, float y) {
+        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         });
@@ -331,9 +339,9 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         };
         // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
         if (nint == 1) {
-            nuc_foreach(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+            nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
         } else {
-            nuc_foreach(r, bm, [&](int j, float y) {
+            nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) {
                 append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
             });
         }
@@ -397,7 +405,6 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     u64 Zp = Zk, tokkey = 0ull;
     u64 *const smass = reinterpret_cast<u64 *>(stage);               // [2048] sub-histogram of masses
     u32 *const scnt = reinterpret_cast<u32 *>(fkey);                 // [2048] and of counts
-    static_assert(NUC_WAVES * NUC_WCAP >= 2048 && NUC_CAP * 4 >= 2048, "the sub-histograms fit the list storage");
     for (int phase = cut ? 0 : 1; phase < 2; phase++) {
         const u64 target = phase == 0 ? tp : draw_target(u, Zp);
         const int b = phase == 0 ? w0 : nuc_first_reaching(cum, target);
@@ -416,7 +423,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 {
                     const u64 pf = prefix;
                     const int pl = plen;
-                    nuc_foreach(r, bm, [&](int j, float y) {
+                    nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) {
                         const float z = nuc_z(r, y);
                         const float d = nuc_d(r, z);
                         if (nuc_bin(r, d) != b) return;
@@ -429,13 +436,21 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 }
                 __syncthreads();
                 {
-                    // inclusive scan over nsb <= 2048 sub-bins, two per thread
-                    const int i0 = 2 * tid, i1 = i0 + 1;
-                    const u64 c0 = i0 < nsb ? smass[i0] : 0ull, c1 = i1 < nsb ? smass[i1] : 0ull;
+                    // inclusive scan over nsb <= 2048 sub-bins, NUC_SUB consecutive ones per thread
+                    u64 c[NUC_SUB], sum = 0ull;
+#pragma unroll
+                    for (int t = 0; t < NUC_SUB; t++) {
+                        const int i = NUC_SUB * tid + t;
+                        sum += i < nsb ? smass[i] : 0ull;
+                        c[t] = sum;
+                    }
                     u64 tot;
-                    const u64 excl = block_inclusive_scan_u64<NUC_BLOCK>(c0 + c1, &scr, &tot) - (c0 + c1);
-                    if (i0 < nsb) smass[i0] = excl + c0;
-                    if (i1 < nsb) smass[i1] = excl + c0 + c1;
+                    const u64 excl = block_inclusive_scan_u64<NUC_BLOCK>(sum, &scr, &tot) - sum;
+#pragma unroll
+                    for (int t = 0; t < NUC_SUB; t++) {
+                        const int i = NUC_SUB * tid + t;
+                        if (i < nsb) smass[i] = excl + c[t];
+                    }
                 }
                 __syncthreads();
                 int lo = 0, hi = nsb - 1;                            // first sub-bin at which base + cumulative reaches target
@@ -456,7 +471,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             {
                 const u64 pf = prefix;
                 const int pl = plen;
-                nuc_foreach(r, bm, [&](int j, float y) {
+                nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) {
                     const float z = nuc_z(r, y);
                     const float d = nuc_d(r, z);
                     if (nuc_bin(r, d) != b) return;
@@ -513,13 +528,14 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     BORN_STAMP(a, row, 7);
 }
 
-template <bool COUNTED>
-__global__ __launch_bounds__(NUC_BLOCK, 4) void nucleus_row_kernel(SampleArgs a) {
-    nucleus_row_body<COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres, a.rcp_T);
+// (at most 128 registers either way: 512 threads are launched two workgroups to a CU)
+template <int BLOCK, bool COUNTED>
+__global__ __launch_bounds__(BLOCK, 4) void nucleus_row_kernel(SampleArgs a) {
+    nucleus_row_body<BLOCK, COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres, a.rcp_T);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
-template <bool COUNTED>
-__global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs a, RowConfigs rc) {
+template <int BLOCK, bool COUNTED>
+__global__ __launch_bounds__(BLOCK, 4) void nucleus_row_rows_kernel(SampleArgs a, RowConfigs rc) {
     RowValues v;
     bool invalid;
     if (!row_config_values(a, rc, (int)blockIdx.x, ROUTE_NUCLEUS, v, invalid)) return;   // workgroup-uniform, before any barrier
@@ -527,7 +543,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void nucleus_row_rows_kernel(SampleArgs 
         row_config_reject(a, (int)blockIdx.x);
         return;
     }
-    nucleus_row_body<COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres, 0.0f);   // (a row's own temperature: no shortcut)
+    nucleus_row_body<BLOCK, COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres, 0.0f);   // (a row's own temperature: no shortcut)
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -548,8 +564,9 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
-__global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
+__global__ __launch_bounds__(NUC_BLOCK_MAX) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
                                                                   float *__restrict__ out) {
+    constexpr int NUC_BLOCK = NUC_BLOCK_MAX, NUC_WAVES = NUC_BLOCK / WAVE;
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ double s_part[NUC_WAVES];
@@ -619,7 +636,7 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
         st *= (double)__expf(mt - mnew);                             // exp(-inf) = 0: nothing finite was seen so far
         mt = mnew;
     };
-    nuc_foreach4<true>(r, bm,
+    nuc_foreach4<NUC_BLOCK, true>(r, bm,
         [&](int, const float (&y)[4]) {
             float z[4];
 #pragma unroll
@@ -662,34 +679,67 @@ __global__ __launch_bounds__(NUC_BLOCK) void token_logprob_kernel(SampleArgs a, 
 size_t token_logprob_lds_bytes(int V) { return sizeof(u32) * (size_t)((V + 31) / 32) + 16; }
 
 hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st) {
-    hipLaunchKernelGGL(token_logprob_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK), token_logprob_lds_bytes(a.V), st, a, tokens, out);
+    hipLaunchKernelGGL(token_logprob_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK_MAX), token_logprob_lds_bytes(a.V), st, a, tokens, out);
     return hipGetLastError();
 }
 
-size_t nucleus_lds_bytes(int V) {
-    return sizeof(u64) * (NUC_BINS + NUC_WAVES * NUC_WCAP + 2 * NUC_CAP) + sizeof(u32) * (size_t)((V + 31) / 32);
+template <int BLOCK>
+static size_t nucleus_lds_bytes_of(int V) {
+    typedef NucGeom<BLOCK> G;
+    return sizeof(u64) * (NUC_BINS + G::WAVES * G::WCAP + 2 * G::CAP) + sizeof(u32) * (size_t)((V + 31) / 32);
+}
+size_t nucleus_lds_bytes(int V) { return nucleus_lds_bytes_of<1024>(V); }
+
+constexpr size_t LDS_PER_CU = 160 * 1024;
+
+// CUs of the current device (asked once per device)
+static int cu_count() {
+    static int known[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (known[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        known[dev] = n;
+    }
+    return known[dev];
 }
 
-hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
-    const dim3 gr((unsigned)a.B), bl(NUC_BLOCK);
-    const size_t lds = nucleus_lds_bytes(a.V);
+template <int BLOCK>
+static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
+    const dim3 gr((unsigned)a.B), bl(BLOCK);
+    const size_t lds = nucleus_lds_bytes_of<BLOCK>(a.V);
     if (rows) {
-        if (a.hist_counts) hipLaunchKernelGGL(nucleus_row_rows_kernel<true>, gr, bl, lds, st, a, *rows);
-        else hipLaunchKernelGGL(nucleus_row_rows_kernel<false>, gr, bl, lds, st, a, *rows);
+        if (a.hist_counts) hipLaunchKernelGGL((nucleus_row_rows_kernel<BLOCK, true>), gr, bl, lds, st, a, *rows);
+        else hipLaunchKernelGGL((nucleus_row_rows_kernel<BLOCK, false>), gr, bl, lds, st, a, *rows);
     } else {
-        if (a.hist_counts) hipLaunchKernelGGL(nucleus_row_kernel<true>, gr, bl, lds, st, a);
-        else hipLaunchKernelGGL(nucleus_row_kernel<false>, gr, bl, lds, st, a);
+        if (a.hist_counts) hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, true>), gr, bl, lds, st, a);
+        else hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, false>), gr, bl, lds, st, a);
     }
+}
+
+hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows, bool two_per_cu) {
+    // More rows than CUs, and two rows' LDS fit one CU: 512 threads per row, two rows to a CU at a time.
+    if ((two_per_cu || a.B > cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU) launch_nucleus_of<512>(a, st, rows);
+    else launch_nucleus_of<1024>(a, st, rows);
     return hipGetLastError();
 }
 
 hipError_t configure_nucleus() {
     const int lds = (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB);
-    const void *kernels[] = {reinterpret_cast<const void *>(nucleus_row_kernel<false>), reinterpret_cast<const void *>(nucleus_row_kernel<true>),
-                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<false>),
-                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<true>)};
+    const void *kernels[] = {reinterpret_cast<const void *>(nucleus_row_kernel<1024, false>), reinterpret_cast<const void *>(nucleus_row_kernel<1024, true>),
+                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<1024, false>),
+                             reinterpret_cast<const void *>(nucleus_row_rows_kernel<1024, true>)};
     for (const void *k : kernels) {
         const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+    }
+    const int lds512 = (int)(LDS_PER_CU / 2);
+    const void *half[] = {reinterpret_cast<const void *>(nucleus_row_kernel<512, false>), reinterpret_cast<const void *>(nucleus_row_kernel<512, true>),
+                          reinterpret_cast<const void *>(nucleus_row_rows_kernel<512, false>),
+                          reinterpret_cast<const void *>(nucleus_row_rows_kernel<512, true>)};
+    for (const void *k : half) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds512);
         if (e != hipSuccess) return e;
     }
     return hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

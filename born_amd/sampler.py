@@ -159,7 +159,8 @@ class Sampler:
         _check(_capi.lib().born_rocm_sampler_set_config(self._h, C.byref(c)))
 
     def SetPath(self, path):
-        """Diagnostics: 0 = kernel chosen from TopK, 1 = always the general kernel."""
+        """Diagnostics: 0 = kernel chosen from TopK, 1 = always the general kernel, 2 = as 0 with 512 threads per row in
+        the kernel for TopK 0 whatever the batch (by default: for batches of more rows than the device has CUs)."""
         _check(_capi.lib().born_rocm_sampler_set_path(self._h, int(path)))
 
     def Status(self, stream=None):

@@ -315,7 +315,7 @@ def test_kernel_selection_by_shape(oracle, rocm):
 # ---------------------------------------------------------------- sampling: kernel without a top-k cut (path 0, top_k 0)
 # and the general kernel (path 0 for top_k > 128, path 1 for everything)
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("B,V,T,k,p,rep,H", [
     (64, 32000, 1.0, 0, 1.0, 1.0, 0),            # C2 multinomial shape
     (16, 152064, 1.2, 0, 0.99, 1.05, 2048),      # C5 shape, 16 rows
@@ -336,14 +336,14 @@ def test_general_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path
     assert got["counters"]["general_rows"] == B
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_general_kernel_degenerate_rows(oracle, rocm, path):
     rng = np.random.default_rng(8)
     B, V = 12, 30000
     u = rng.random(B, dtype=np.float32)
     x = np.zeros((B, V), np.float32)                                    # every logit equal: radix descent on ids
     got, _, _ = _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 1.0, path=path)
-    if path == 0:
+    if path != 1:
         assert got["counters"]["fallback_rows"] == B                    # ... taken by the kernel without a top-k cut
     _check_against_oracle(oracle, rocm, x, u, 1.0, 0, 0.5, path=path)
     _check_against_oracle(oracle, rocm, x, u, 1.0, 9000, 0.9, path=path)
@@ -363,7 +363,7 @@ def test_general_kernel_degenerate_rows(oracle, rocm, path):
 
 # ---------------------------------------------------------------- min-p
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("B,V,T,k,p,rep,H,min_p", [
     (32, 128256, 0.7, 50, 0.9, 1.15, 512, 0.05),    # C3 shape with min-p: single-pass top-k kernel
     (16, 32000, 1.0, 40, 1.0, 1.0, 0, 0.1),         # min-p is the only cut inside the top-k
@@ -420,7 +420,7 @@ def test_min_p_is_validated(rocm):
 
 # ---------------------------------------------------------------- frequency and presence penalties
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("B,V,T,k,p,rep,H,freq,pres,route", [
     (32, 128256, 0.7, 50, 0.9, 1.15, 512, 0.3, 0.5, "topk"),     # C3 shape: single-pass kernel, history hashed
     (16, 32000, 1.0, 40, 0.95, 1.0, 64, 0.5, 0.0, "topk"),       # frequency alone, no repetition penalty
@@ -450,9 +450,9 @@ def test_frequency_and_presence_penalties_against_oracle(oracle, rocm, B, V, T, 
     plain = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED)
     assert (plain["tokens"] != fx["tokens"]).any() or not np.array_equal(plain["probs"], fx["probs"]), "the penalties are meant to matter"
     c = got["counters"]
-    if path == 0 and route == "topk":
+    if path != 1 and route == "topk":
         assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
-    if path == 0 and route == "general" and 1 <= k <= 128:
+    if path != 1 and route == "general" and 1 <= k <= 128:
         assert c["general_rows"] == B
 
 
@@ -613,8 +613,13 @@ def test_cross_entropy_loss_mirror(oracle, rocm):
     crit.Close()
 
 
+# path 2: the three-sweep kernel with 512 threads per row (what batches of more rows than CUs get), path 0: 1024
+NUCLEUS_PATHS = [0, 2]
+
+
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
 @pytest.mark.parametrize("V,pad", [(7, 5), (7, 1), (6, 2), (4102, 2), (4103, 1), (8198, 2)])
-def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pad):
+def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pad, path):
     # 16-byte aligned rows whose length is not a multiple of four, with the whole float4 blocks ending at lane 0 or 1 of a
     # wave: the ragged tail restarts at lane 0, next to lanes that sat out the last block.  Few distinct values, so that
     # the wanted bins take entries from both parts.
@@ -632,6 +637,7 @@ def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pa
     for (T, p, rep, min_p, freq) in [(5.0, 0.9, 1.0, 0.05, 0.1), (1.0, 0.9, 1.2, 0.0, 0.0), (0.7, 1.0, 1.0, 0.0, 0.0)]:
         s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=0, TopP=p, RepetitionPenalty=rep, MinP=min_p, FrequencyPenalty=freq),
                             max_batch=B, max_vocab=V)
+        s.SetPath(path)
         d_x, d_u, d_h = rocm.DeviceBuffer.from_numpy(host), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer.from_numpy(hist)
         tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
         s.Sample(d_x, B, V, d_h, None, d_u, tok, pr, row_stride=stride, hist_stride=H)
@@ -643,8 +649,9 @@ def test_three_sweep_kernel_ragged_tail_after_a_partial_wave(oracle, rocm, V, pa
         s.Close()
 
 
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
 @pytest.mark.parametrize("pad_extra", [0, 4])
-def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra):
+def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra, path):
     # every vocabulary size modulo 256 (so: every way the row's last whole 128-bit blocks and its ragged tail can fall
     # on the lanes of a wave), at two row pitches; few distinct values, so that the wanted bins take entries from all
     # parts of the row and a lost or duplicated staged entry changes the result
@@ -660,6 +667,7 @@ def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra):
             host[b * stride: b * stride + V] = x[b]
         T, p, rep = (1.0, 0.9, 1.2) if V % 2 else (0.7, 1.0, 1.0)
         s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, TopK=0, TopP=p, RepetitionPenalty=rep), max_batch=B, max_vocab=V)
+        s.SetPath(path)
         d_x, d_u, d_h = rocm.DeviceBuffer.from_numpy(host), rocm.DeviceBuffer.from_numpy(u), rocm.DeviceBuffer.from_numpy(hist)
         tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
         s.Sample(d_x, B, V, d_h, None, d_u, tok, pr, row_stride=stride, hist_stride=H)
@@ -670,8 +678,9 @@ def test_three_sweep_kernel_every_row_length_residue(oracle, rocm, pad_extra):
         s.Close()
 
 
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
 @pytest.mark.parametrize("T", [0.7, 1.2, 0.35, 1.9999999, 1.0])
-def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, rocm, T):
+def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, rocm, T, path):
     """Without a top-k cut every logit is divided by the temperature. For most temperatures the kernel replaces the
     division by a multiplication and two fused multiply-adds that give the same quotient for logits of ordinary
     magnitude (1.9999999 is a temperature it must divide by); zeros, denormals, tiny and huge values, infinities
@@ -688,7 +697,7 @@ def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, roc
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, size=(B, 64)).astype(np.int32)
     for p, rep, min_p in [(0.9, 1.0, 0.0), (1.0, 1.3, 0.0), (0.97, 1.1, 0.02)]:
-        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, 0, p, rep, hist if rep != 1.0 else None, min_p=min_p)
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, 0, p, rep, hist if rep != 1.0 else None, min_p=min_p, path=path)
         assert got["counters"]["general_rows"] == B and got["counters"]["topk_rows"] == 0
 
 
@@ -719,15 +728,16 @@ def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
     s.Close()
 
 
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
 @pytest.mark.parametrize("V", [8, 64, 100, 130, 4100])
-def test_three_sweep_kernel_rows_that_end_inside_a_wave(oracle, rocm, V):
+def test_three_sweep_kernel_rows_that_end_inside_a_wave(oracle, rocm, V, path):
     # no top-k cut and a row whose last elements occupy only part of a wave: the lanes that sit out the ragged end
     # must still see every entry the wave gathered (heavy ties make the gathered bins full)
     rng = np.random.default_rng(V)
     x = np.round(rng.standard_normal((6, V))).astype(np.float32)
     u = rng.random(6, dtype=np.float32)
     for p in (1.0, 0.9):
-        _check_against_oracle(oracle, rocm, x, u, T=5.0, k=0, p=p)
+        _check_against_oracle(oracle, rocm, x, u, T=5.0, k=0, p=p, path=path)
 
 
 def test_builtin_uniform_stream_in_sample(oracle, rocm):
@@ -843,7 +853,7 @@ def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=
     return s, tok.to_numpy(np.int32, (B,)), pr.to_numpy(np.float32, (B,))
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
     # one batch, every row its own settings, covering the three kernels' territories (top-k <= 128, no top-k cut,
     # top-k > 64, a boosting penalty < 1); each row must equal the oracle under that row's settings
@@ -869,14 +879,14 @@ def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
     for b in range(B):
         want = oracle.sample(x[b:b + 1], u[b:b + 1], 0.9, int(ks[b]), 0.8, 1.3, hist[b:b + 1], None, mode=oracle.MODE_FIXED)
         assert tok2[b] == want["tokens"][0], b
-    if path == 0:
+    if path != 1:
         c = s.Counters()
         assert c["topk_rows"] > 0 and c["general_rows"] > 0                 # more than one kernel took rows
     s.Close()
     s2.Close()
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("freq,pres,min_p", [(0.3, 0.4, 0.0), (-0.2, 0.1, 0.0), (0.0, 0.0, 0.05), (0.2, 0.0, 0.02)])
 def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq, pres, min_p):
     # min-p and the frequency / presence penalties stay the handle's while the other settings vary per row
@@ -897,12 +907,12 @@ def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq
                              mode=oracle.MODE_FIXED, min_p=min_p, freq=freq, pres=pres)
         assert tok[b] == want["tokens"][0], (b, Ts[b], ks[b], ps[b], reps[b])
         assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], b
-    if path == 0 and freq < 0:
+    if path != 1 and freq < 0:
         assert s.Counters()["topk_rows"] == 0                            # a penalty that raises logits: never the single-pass kernel
     s.Close()
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_per_row_min_p_and_additive_penalties(oracle, rocm, path):
     # all seven settings per row; the handle is configured without a frequency / presence penalty, so the call itself
     # brings the table of counts into being
@@ -951,7 +961,7 @@ def test_per_row_min_p_and_additive_penalties(oracle, rocm, path):
     s3.Close()
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_per_row_promised_kinds_of_row(oracle, rocm, path):
     from born_amd import _capi
     rng = np.random.default_rng(81)
@@ -973,7 +983,7 @@ def test_per_row_promised_kinds_of_row(oracle, rocm, path):
     s.Status()
     assert [int(t) for t in tok] == [int(want(b, ks[b])) for b in range(B)]
     c = s.Counters()
-    assert (c["general_rows"] == 0) if path == 0 else (c["topk_rows"] + c["fallback_rows"] == 0)
+    assert (c["general_rows"] == 0) if path != 1 else (c["topk_rows"] + c["fallback_rows"] == 0)
     s.Close()
     # two kinds promised, a third occurs in rows 3 and 11 (top_k 300), and row 7 is invalid: those rows are reported
     ks2 = rng.choice([0, 5, 50], B).astype(np.int32)
@@ -981,7 +991,7 @@ def test_per_row_promised_kinds_of_row(oracle, rocm, path):
     Tbad = Ts.copy()
     Tbad[7] = -1.0
     s, tok, _ = _sample_rows(rocm, x, u, hist, Tbad, ks2, ps, reps, path, row_kinds=_capi.ROWS_SMALL_TOP_K | _capi.ROWS_NO_TOP_K)
-    if path == 0:
+    if path != 1:
         with pytest.raises(rocm.BornRocmError, match="invalid per-row configuration"):
             s.Status()
         assert tok[3] == 0 and tok[11] == 0 and tok[7] == 0

@@ -71,7 +71,7 @@ def test_random_configurations_against_oracle(oracle, rocm, chunk):
         nuc = 0                                        # the nucleus is listed for top_k <= 4096
         if 1 <= c["k"] < c["V"] and c["k"] <= 4096:
             nuc = int(rng.choice([c["k"], max(1, c["k"] // 3), c["k"] + 5]))
-        for path in (0, 1):
+        for path in (0, 1, 2):
             try:
                 _check_against_oracle(oracle, rocm, x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, nuc=nuc, path=path,
                                       min_p=c["min_p"], freq=c["freq"], pres=c["pres"])
@@ -150,7 +150,7 @@ def test_random_row_layouts_against_oracle(oracle, rocm, chunk):
         tok, pr = rocm.DeviceBuffer(4 * B), rocm.DeviceBuffer(4 * B)
         fx = oracle.sample(x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, mode=oracle.MODE_FIXED, min_p=c["min_p"],
                            freq=c["freq"], pres=c["pres"])
-        for path in (0, 1):
+        for path in (0, 1, 2):
             s = rocm.NewSampler(rocm.SamplerConfig(Temperature=c["T"], TopK=c["k"], TopP=c["p"], RepetitionPenalty=c["rep"], MinP=c["min_p"],
                                                    FrequencyPenalty=c["freq"], PresencePenalty=c["pres"]), max_batch=B, max_vocab=V)
             s.SetPath(path)
@@ -184,7 +184,7 @@ def test_large_vocabularies_against_oracle(oracle, rocm, V):
     for (k, p, rep, min_p, freq, pres) in [(50, 0.9, 1.15, 0.0, 0.0, 0.0), (0, 0.95, 1.1, 0.0, 0.2, 0.1), (300, 0.9, 1.0, 0.01, 0.0, 0.0),
                                            (64, 1.0, 0.9, 0.0, 0.0, 0.0)]:
         got = None
-        for path in (0, 1):
+        for path in (0, 1, 2):
             s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=k, TopP=p, RepetitionPenalty=rep, MinP=min_p, FrequencyPenalty=freq,
                                                    PresencePenalty=pres), max_batch=B + 2, max_vocab=524288)
             s.SetPath(path)

@@ -130,7 +130,7 @@ def test_random_argmax_and_softmax_rows(oracle, rocm, chunk):
         s.Close()
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("chunk", range(4))
 def test_random_per_row_configurations(oracle, rocm, chunk, path):
     from test_gpu_parity import _sample_rows
