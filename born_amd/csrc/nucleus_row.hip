@@ -23,12 +23,12 @@ namespace born {
 // Threads per row: 1024 (one workgroup per CU: the shortest time per row, for batches that leave CUs idle anyway) or
 // 512 (two workgroups per CU: one row's sweeps that wait for memory overlap the other's sweep that computes; for
 // batches of more rows than the device has CUs). The geometry below follows from it.
-constexpr int NUC_U = 4;                      // 128-bit loads per thread and stage
 constexpr int NUC_BINS = 4096;
 template <int BLOCK>
 struct NucGeom {
     static_assert(BLOCK == 512 || BLOCK == 1024, "threads per row");
     static constexpr int WAVES = BLOCK / WAVE;
+    static constexpr int U = 4;                                   // 128-bit loads per thread and stage (more in flight measured slower)
     static constexpr int WCAP = BLOCK == 1024 ? 160 : 256;       // staged entries per wave
     static constexpr int CAP = BLOCK;                             // gathered entries (one per thread)
     static constexpr int PER = NUC_BINS / BLOCK;                  // bins per thread in the scan
@@ -103,6 +103,7 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     };
     if (r.vec) {
         const int n4 = r.V >> 2;
+        constexpr int NUC_U = NucGeom<NUC_BLOCK>::U;
         const int nfull = n4 / (NUC_U * NUC_BLOCK);
         const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
         if (nfull > 0) {
@@ -134,9 +135,9 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     }
 }
 // Visits every element of the row as f(id, penalised logit).
-template <int NUC_BLOCK, class F>
+template <int NUC_BLOCK, bool NT = false, class F>
 __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
-    nuc_foreach4<NUC_BLOCK>(r, bm, [&](int j, const float (&y)[4]) {
+    nuc_foreach4<NUC_BLOCK, NT>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
     }, f);
@@ -339,9 +340,9 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         };
         // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
         if (nint == 1) {
-            nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+            nuc_foreach<NUC_BLOCK, true>(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
         } else {
-            nuc_foreach<NUC_BLOCK>(r, bm, [&](int j, float y) {
+            nuc_foreach<NUC_BLOCK, true>(r, bm, [&](int j, float y) {
                 append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
             });
         }
