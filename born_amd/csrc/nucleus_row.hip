@@ -68,7 +68,7 @@ __device__ __forceinline__ float nuc_z_shortcut(const NucRow &r, float y) {
 }
 
 // Visits every element of the row with its penalised logit: aligned rows four at a time as f4(id of the first, y[4]),
-// in stages of NUC_U float4 per thread, the next stage's loads in flight while this one is visited; what is left
+// in stages of U float4 per thread (the last stage may be partial), the next stage's loads in flight while this one is visited; what is left
 // over (and every element of an unaligned row) one at a time as f1(id, y).
 // `pre` runs once before the first element is visited, with the first stage's loads already in flight (work that
 // must precede the visits but not the loads: building the history bitmap).
@@ -104,29 +104,31 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     if (r.vec) {
         const int n4 = r.V >> 2;
         constexpr int NUC_U = NucGeom<NUC_BLOCK>::U;
-        const int nfull = n4 / (NUC_U * NUC_BLOCK);
+        const int nst = (n4 + NUC_U * NUC_BLOCK - 1) / (NUC_U * NUC_BLOCK);      // stages, the last one whole or partial
         const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
-        if (nfull > 0) {
+        if (nst > 0) {
+            // Loads are unconditional, of a block index clamped to the row's last block (a load under a condition makes
+            // the compiler wait for every load in flight); only the visits of the last stage ask whether the block exists.
             nuc_f32x4 va[NUC_U], vb[NUC_U];
+            const int lastb = n4 - 1;
 #pragma unroll
-            for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + u * NUC_BLOCK + tid);
+            for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + tid, lastb));
             pre();
-            for (int s = 0; s + 1 < nfull; s++) {
+            for (int s = 0; s + 1 < nst; s++) {
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + ((s + 1) * NUC_U + u) * NUC_BLOCK + tid);
+                for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + min(((s + 1) * NUC_U + u) * NUC_BLOCK + tid, lastb));
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
             }
 #pragma unroll
-            for (int u = 0; u < NUC_U; u++) visit4(va[u], (((nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+            for (int u = 0; u < NUC_U; u++) {
+                const int i = ((nst - 1) * NUC_U + u) * NUC_BLOCK + tid;
+                if (i < n4) visit4(va[u], i << 2);
+            }
         } else {
             pre();
-        }
-        for (int i = nfull * NUC_U * NUC_BLOCK + tid; i < n4; i += NUC_BLOCK) {
-            const nuc_f32x4 q = nuc_load4<NT>(x4 + i);
-            visit4(q, i << 2);
         }
         for (int j = (n4 << 2) + tid; j < r.V; j += NUC_BLOCK) visit1(j);
     } else {
