@@ -14,6 +14,7 @@
 //            first entry in rank order whose cumulative mass reaches a target is found with an LDS max.
 // A wanted bin too full for the lists (heavy ties, masked rows) is refined in place by a radix descent over
 // the rank keys of that bin, 11 bits per sweep.
+#include <type_traits>
 #include "dev_common.h"
 #include "kernels.h"
 #include "row_config.h"
@@ -43,6 +44,8 @@ struct NucRow {                               // uniform per workgroup
     const float *x;
     int V;
     bool vec, penal, degenerate;
+    bool masked = false;                      // the visitor replaces every seen logit by `skip`; the seen ids are visited apart
+    float skip = 0.0f;
     float T, rcp, rep, m, scale, range, sbin, dcut;        // rcp: RN(1 / T) where the division shortcut is exact, else 0
     const unsigned *counts;                   // occurrences of each id in the row's history (frequency / presence penalties), or null
     float freq, pres;
@@ -87,18 +90,34 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
         float y[4] = {q[0], q[1], q[2], q[3]};
         if (r.penal) {
-            const u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
-            if (bits) {
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    if ((bits >> t) & 1u) y[t] = penalise_seen(y[t], r.rep, r.counts, j + t, r.freq, r.pres);
+            // One seen element per turn, the lowest first: with a long history nearly every wave has some lane with a seen
+            // id among its four, but a lane rarely holds two, so the wave computes one penalty per visit, not four.
+            u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
+            if (r.masked) {
+                if (bits) {
+                    y[0] = (bits & 1u) ? r.skip : y[0];
+                    y[1] = (bits & 2u) ? r.skip : y[1];
+                    y[2] = (bits & 4u) ? r.skip : y[2];
+                    y[3] = (bits & 8u) ? r.skip : y[3];
+                }
+                bits = 0u;
+            }
+            while (bits) {
+                const u32 low = bits & (0u - bits);
+                const float v = low == 1u ? y[0] : low == 2u ? y[1] : low == 4u ? y[2] : y[3];
+                const float pv = penalise_seen(v, r.rep, r.counts, j + (31 - __clz(low)), r.freq, r.pres);
+                y[0] = low == 1u ? pv : y[0];
+                y[1] = low == 2u ? pv : y[1];
+                y[2] = low == 4u ? pv : y[2];
+                y[3] = low == 8u ? pv : y[3];
+                bits ^= low;
             }
         }
         f4(j, y);
     };
     auto visit1 = [&](int j) {
         float y = r.x[j];
-        if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
+        if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = r.masked ? r.skip : penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
         f1(j, y);
     };
     if (r.vec) {
@@ -184,7 +203,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                   NUC_PER = NucGeom<NUC_BLOCK>::PER, NUC_SUB = NucGeom<NUC_BLOCK>::SUB;
     extern __shared__ u64 nuc_dyn[];
     __shared__ BlockScratch scr;
-    __shared__ int s_n, s_over;
+    __shared__ int s_n, s_over, s_nseen;
     __shared__ u64 s_win, s_mass;
     __shared__ u32 s_wcount[NUC_WAVES];
 
@@ -223,20 +242,63 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         s_n = 0;
         s_over = 0;
         s_win = 0ull;
+        s_nseen = 0;
     }
     __syncthreads();
+    // The ids the history holds, each once (whoever sets an id's bit first lists it): at most NUC_SEEN per thread, kept
+    // in registers with their penalised logits for the whole kernel. The sweeps then see a constant in place of a seen
+    // logit (chosen per sweep so that it contributes nothing) and visit the seen ids apart, every lane busy; applying the
+    // penalty inside the sweep costs a whole wave the penalty arithmetic whenever one of its lanes holds a seen id, which
+    // with a long history is nearly always. A history too long for the registers keeps the penalty inside the sweeps.
+    constexpr int NUC_SEEN = 4;
+    u32 *const seen_list = reinterpret_cast<u32 *>(fkey);            // [NUC_SEEN * NUC_BLOCK], free until the gather classifies
+    static_assert(NUC_SEEN * NUC_BLOCK * sizeof(u32) <= 2 * NUC_CAP * sizeof(u64), "the list of seen ids fits the gathered entries' storage");
+    const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
     for (int i = tid; i < hlen; i += NUC_BLOCK) {
         const int t = h[i];
         if (t < 0 || t >= V) atomicOr(a.status, 1);
-        else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
+        else if (r.penal) {
+            const u32 bit = 1u << (t & 31);
+            const u32 old = atomicOr(&bm[t >> 5], bit);
+            if (list_seen && !(old & bit)) seen_list[atomicAdd(&s_nseen, 1)] = (u32)t;
+        }
     }
     __syncthreads();
+    int seen_id[NUC_SEEN];
+    float seen_y[NUC_SEEN];
+    r.masked = list_seen;
+    r.skip = -INFINITY;                                              // sweep 1: neither the maximum nor the smallest finite value
+    {
+        const int nseen = list_seen ? s_nseen : 0;
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++) {
+            const int i = tid + k * NUC_BLOCK;
+            seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
+        }
+        float raw[NUC_SEEN];
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++) raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++)
+            seen_y[k] = seen_id[k] >= 0 ? penalise_seen(raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
+    }
+    // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
+    auto sweep = [&](auto nt, auto f) {
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value>(r, bm, f);
+        if (r.masked) {
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++)
+                if (seen_id[k] >= 0) f(seen_id[k], seen_y[k]);
+        }
+    };
+    typedef std::integral_constant<bool, false> Cached;             // the row is read again: ordinary loads
+    typedef std::integral_constant<bool, true> Streamed;             // the row's last sweep: non-temporal loads
 
     BORN_STAMP(a, row, 1);
     // ---- sweep 1: maximum and smallest finite penalised logit
     {
         float mx = -INFINITY, mn = INFINITY;
-        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             mx = fmaxf(mx, y);
             mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
         });
@@ -249,19 +311,24 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         // the bins cover the logits that can carry mass: the row's span, at most 32, at most the min-p bound
         r.range = uniform_f32(fminf(fminf(32.0f, span * 1.0001f + 1e-3f), r.dcut * 1.0001f + 1e-3f));
         r.sbin = uniform_f32((float)NUC_BINS / r.range);
+        // sweeps 2 and 3: a value 200 below the maximum in z (no mass; outside every wanted range unless the last bin,
+        // which takes everything beyond the span, is wanted: the gather then lists the constant once per seen id, with no
+        // mass and ranked last, next to the id's real entry). A maximum that leaves no such value: penalties inside the sweeps.
+        if (r.masked && fabsf(r.m) < 1e6f) r.skip = uniform_f32((r.m - 200.0f) * r.T);
+        else r.masked = false;
     }
 
     BORN_STAMP(a, row, 2);
     // ---- sweep 2: integer masses by bin
     if (r.rcp != 0.0f && !r.degenerate) {
-        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         });
     } else {
-        nuc_foreach<NUC_BLOCK>(r, bm, [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         });
@@ -342,9 +409,9 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         };
         // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
         if (nint == 1) {
-            nuc_foreach<NUC_BLOCK, true>(r, bm, [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+            sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
         } else {
-            nuc_foreach<NUC_BLOCK, true>(r, bm, [&](int j, float y) {
+            sweep(Streamed(), [&](int j, float y) {
                 append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
             });
         }
@@ -405,6 +472,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     // mass reaches a target.  A bin that is listed is resolved from `mine`; any other bin (the lists overflowed:
     // heavy ties, masked rows; or the draw's bin was not the predicted one) by a radix descent over the rank
     // keys of that bin, 11 bits per sweep, until its bucket fits the list.
+    r.masked = false;                                                // (the sweeps of a radix descent apply the penalties themselves)
     u64 Zp = Zk, tokkey = 0ull;
     u64 *const smass = reinterpret_cast<u64 *>(stage);               // [2048] sub-histogram of masses
     u32 *const scnt = reinterpret_cast<u32 *>(fkey);                 // [2048] and of counts

@@ -701,6 +701,31 @@ def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, roc
         assert got["counters"]["general_rows"] == B and got["counters"]["topk_rows"] == 0
 
 
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
+@pytest.mark.parametrize("V,H,scale", [(50, 40, 1.0), (300, 900, 1.0), (5000, 2048, 1.0), (6000, 2100, 1.0), (6000, 4200, 1.0),
+                                       (5000, 600, 3e6), (4099, 4096, 1.0)])
+def test_three_sweep_kernel_seen_ids_visited_apart(oracle, rocm, V, H, scale, path):
+    """With penalties on, the kernel lists the ids of the history once each, keeps their penalised logits in registers
+    (up to four per thread: 2048 ids at 512 threads per row, 4096 at 1024) and shows the sweeps a constant in their
+    place; longer histories, and rows whose maximum is too large for such a constant, keep the penalty inside the
+    sweeps. Both ways, with repeated ids, with draws from the very end of the rank order (where the constant's own
+    bin is the wanted one) and with the counted penalties: bit-exact against the oracle."""
+    rng = np.random.default_rng(V * 13 + H)
+    B = 8
+    x = (rng.standard_normal((B, V)) * scale).astype(np.float32)
+    hist = ((rng.zipf(1.3, size=(B, H)) - 1) % V).astype(np.int32)
+    hist[:, ::3] = rng.integers(0, V, size=hist[:, ::3].shape)
+    hl = rng.integers(max(1, H - 3), H + 1, size=B).astype(np.int32)
+    u = rng.random(B, dtype=np.float32)
+    u[0] = np.float32(1.0) - np.float32(2.0 ** -24)        # the last element in rank order
+    u[1] = np.float32(0.99999)
+    u[2] = 0.0
+    for (T, p, rep, freq, pres) in [(3.0, 1.0, 1.3, 0.0, 0.0), (1.2, 0.999, 1.05, 0.0, 0.0), (2.0, 1.0, 1.0, 0.3, 0.2),
+                                    (0.8, 0.9, 2.0, 0.1, 0.0)]:
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T * scale, 0, p, rep, hist, hl, path=path, freq=freq, pres=pres)
+        assert got["counters"]["general_rows"] == B
+
+
 def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
     # the case a wide seeded sweep of test_random_row_layouts_against_oracle found (its chunk 1096, third case)
     import test_gpu_parity_random as R
