@@ -254,13 +254,39 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     u32 *const seen_list = reinterpret_cast<u32 *>(fkey);            // [NUC_SEEN * NUC_BLOCK], free until the gather classifies
     static_assert(NUC_SEEN * NUC_BLOCK * sizeof(u32) <= 2 * NUC_CAP * sizeof(u64), "the list of seen ids fits the gathered entries' storage");
     const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
-    for (int i = tid; i < hlen; i += NUC_BLOCK) {
-        const int t = h[i];
-        if (t < 0 || t >= V) atomicOr(a.status, 1);
-        else if (r.penal) {
-            const u32 bit = 1u << (t & 31);
-            const u32 old = atomicOr(&bm[t >> 5], bit);
-            if (list_seen && !(old & bit)) seen_list[atomicAdd(&s_nseen, 1)] = (u32)t;
+    if (list_seen) {
+        int hv[NUC_SEEN];                                            // (all of the thread's history loads in flight together)
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++) {
+            const int i = tid + k * NUC_BLOCK;
+            hv[k] = i < hlen ? h[i] : -2;
+        }
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++) {
+            const int t = hv[k];
+            bool first = false;
+            if (t >= 0 && t < V) {
+                const u32 bit = 1u << (t & 31);
+                const u32 old = atomicOr(&bm[t >> 5], bit);
+                first = !(old & bit);
+            } else if (t != -2) {
+                atomicOr(a.status, 1);
+            }
+            // one addition to the list's length per wave
+            const u64 mk = __ballot(first);
+            if (mk) {
+                const u32 rank = __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                int base = 0;
+                if (first && rank == 0u) base = atomicAdd(&s_nseen, __popcll(mk));
+                base = __builtin_amdgcn_readlane(base, __builtin_ctzll(mk));
+                if (first) seen_list[base + (int)rank] = (u32)t;
+            }
+        }
+    } else {
+        for (int i = tid; i < hlen; i += NUC_BLOCK) {
+            const int t = h[i];
+            if (t < 0 || t >= V) atomicOr(a.status, 1);
+            else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
         }
     }
     __syncthreads();
