@@ -265,7 +265,7 @@ int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int6
  * row's top_k.  A row it cannot settle (a list of more than 4096, fewer than top_k candidates above the bound, a
  * history of more than 1024 tokens with a penalty) gets token -1 and born_rocm_sampler_status returns
  * BORN_ROCM_ERR_DATA: the caller then runs born_rocm_linear + born_rocm_sample for that call.  The first call on a
- * handle allocates 48 KiB of workspace per row of max_batch (outside a stream capture). */
+ * handle allocates about 36 KiB of workspace per row of max_batch (outside a stream capture). */
 int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
                             const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
                             const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,
