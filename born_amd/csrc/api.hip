@@ -618,7 +618,13 @@ static int spec_verify_impl(born_sampler *s, const float *target, int64_t target
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: spec_verify: batch * gamma too large");
     const int64_t rows = batch * gamma;
     if (rows > s->spec_rows) {
-        // grow the per-position statistics (stream-ordered use only; the old buffers are idle once synchronised)
+        // grow the per-position statistics (stream-ordered use only; the old buffers are idle once synchronised);
+        // not inside a stream capture, which a synchronisation or an allocation would invalidate
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &capturing));
+        if (capturing != hipStreamCaptureStatusNone)
+            return fail(BORN_ROCM_ERR_UNSUPPORTED, "sampler: spec_verify: the per-position statistics would grow to %lld rows inside a "
+                        "stream capture; make one call of this size before capturing", (long long)rows);
         HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
         void **ps[] = {(void **)&s->sp_mp, (void **)&s->sp_mq, (void **)&s->sp_Zp, (void **)&s->sp_Zq, (void **)&s->sp_pd,
                        (void **)&s->sp_qd, (void **)&s->sp_part, (void **)&s->sp_run, (void **)&s->sp_mb, (void **)&s->sp_Zb};

@@ -207,7 +207,9 @@ int born_rocm_gather_rows(born_sampler *s, const float *table, int64_t rows, int
  * No counterpart in the reference snapshot.
  *   target, draft  fp32 [batch, gamma, vocab] contiguous;  draft_tokens int32 [batch, gamma]
  *   u_accept fp32 [batch, gamma];  u_residual fp32 [batch]
- *   n_accepted_out int32 [batch];  next_token_out int32 [batch] (-1 when every draft token was accepted) */
+ *   n_accepted_out int32 [batch];  next_token_out int32 [batch] (-1 when every draft token was accepted)
+ * The first call with a larger batch * gamma than any before it grows the handle's per-position statistics: it
+ * synchronises the stream and allocates, and is refused (BORN_ROCM_ERR_UNSUPPORTED) inside a stream capture. */
 int born_rocm_spec_verify(born_sampler *s, const float *target, const float *draft, int64_t batch,
                           int64_t gamma, int64_t vocab, const int32_t *draft_tokens, const float *u_accept,
                           const float *u_residual, int32_t *n_accepted_out, int32_t *next_token_out,

@@ -436,3 +436,63 @@ def test_lm_head_sampling_fused_argument_errors(rocm, lin):
     with pytest.raises(rocm.SamplerPanic):
         lin.ForwardSample(s, layer, x, (M + 1, K), None, None, u, tok)        # beyond the handle's batch
     s.Close()
+
+
+def test_calls_that_would_allocate_are_refused_inside_a_capture_and_leave_it_valid(oracle, rocm, lin):
+    # Three calls allocate on first use: per-row frequency penalties on a handle configured without any, a speculative
+    # step larger than any before it, the first fused LM-head sampling call.  Inside a stream capture each is refused
+    # with BORN_ROCM_ERR_UNSUPPORTED before it touches the stream, so the capture goes on: an ordinary sampling step
+    # recorded after the refusals replays correctly.
+    import ctypes as C
+    from born_amd import _capi
+    hip = C.CDLL("libamdhip64.so")
+    def ok(rc):
+        assert rc == 0, f"HIP error {rc}"
+    rng = np.random.default_rng(405)
+    B, K, V, G = 4, 128, 8000, 3
+    xh = rng.standard_normal((B, V)).astype(np.float32)
+    uh = rng.random(B, dtype=np.float32)
+    hist_h = rng.integers(0, V, (B, 16)).astype(np.int32)
+    logits, u, hist = rocm.DeviceBuffer.from_numpy(xh), rocm.DeviceBuffer.from_numpy(uh), rocm.DeviceBuffer.from_numpy(hist_h)
+    tokens, probs = rocm.DeviceBuffer(B * 4), rocm.DeviceBuffer(B * 4)
+    freqs = rocm.DeviceBuffer.from_numpy(np.full(B, 0.2, np.float32))
+    w = rocm.DeviceBuffer.from_numpy((rng.standard_normal((V, K)) * 0.1).astype(np.float32))
+    layer = lin.Linear(K, V, w, None)
+    xin = rocm.DeviceBuffer.from_numpy(rng.standard_normal((B, K)).astype(np.float32))
+    tgt = rocm.DeviceBuffer.from_numpy(rng.standard_normal((B, G, V)).astype(np.float32))
+    dtok = rocm.DeviceBuffer.from_numpy(rng.integers(0, V, (B, G)).astype(np.int32))
+    ua = rocm.DeviceBuffer.from_numpy(rng.random((B, G), dtype=np.float32))
+    nacc, nxt = rocm.DeviceBuffer(B * 4), rocm.DeviceBuffer(B * 4)
+    smp = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1), max_batch=B, max_vocab=V)
+
+    stream = C.c_void_p()
+    ok(hip.hipStreamCreate(C.byref(stream)))
+    smp.Sample(logits, B, V, hist, None, u, tokens, probs, hist_stride=16, stream=stream)       # warm-up outside the capture
+    ok(hip.hipStreamSynchronize(stream))
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    ok(hip.hipStreamBeginCapture(stream, 0))
+    for call in (lambda: smp.SampleRows(logits, B, V, hist, None, u, None, None, None, None, tokens, probs, hist_stride=16, stream=stream,
+                                        frequencyPenalties=freqs),
+                 lambda: smp.Verify(tgt, tgt, B, G, V, dtok, ua, u, nacc, nxt, stream=stream),
+                 lambda: lin.ForwardSample(smp, layer, xin, (B, K), hist, None, u, tokens, probs, hist_stride=16, stream=stream)):
+        with pytest.raises(_capi.BornRocmError) as e:
+            call()
+        assert e.value.code == _capi.ERR_UNSUPPORTED and "capture" in str(e.value)
+    smp.Sample(logits, B, V, hist, None, u, tokens, probs, hist_stride=16, stream=stream)
+    ok(hip.hipStreamEndCapture(stream, C.byref(graph)))
+    ok(hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)))
+    want = oracle.sample(xh, uh, 0.8, 40, 0.95, 1.1, hist_h, None, mode=oracle.MODE_FIXED)
+    for it in range(2):
+        _capi.check(_capi.lib().born_rocm_h2d(tokens.ptr, np.full(B, -1, np.int32).ctypes.data, 4 * B, None))
+        ok(hip.hipDeviceSynchronize())
+        ok(hip.hipGraphLaunch(gexec, stream))
+        ok(hip.hipStreamSynchronize(stream))
+        assert np.array_equal(tokens.to_numpy(np.int32, (B,)), want["tokens"]), it
+    ok(hip.hipGraphExecDestroy(gexec))
+    ok(hip.hipGraphDestroy(graph))
+    ok(hip.hipStreamDestroy(stream))
+    # outside a capture the same calls allocate and work
+    smp.Verify(tgt, tgt, B, G, V, dtok, ua, u, nacc, nxt)
+    assert nacc.to_numpy(np.int32, (B,)).tolist() == [G] * B                                # identical models accept everything
+    smp.Status()
+    smp.Close()
