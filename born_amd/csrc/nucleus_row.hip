@@ -193,14 +193,15 @@ __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f)
     }, f);
 }
 
-// smallest bin whose inclusive cumulative mass reaches target
+// smallest bin whose inclusive cumulative mass reaches target (the last bin if none does); called by whole waves.
+// Two rounds of 64 lanes: which run of 64 bins, then which bin of the run (a binary search is twelve dependent LDS reads).
+static_assert(NUC_BINS == WAVE * WAVE, "two rounds of one wave cover the bins");
 __device__ __forceinline__ int nuc_first_reaching(const u64 *cum, u64 target) {
-    int lo = 0, hi = NUC_BINS - 1;
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (cum[mid] >= target) hi = mid; else lo = mid + 1;
-    }
-    return lo;
+    const int l = lane_id();
+    const u64 runs = __ballot(cum[l * WAVE + WAVE - 1] >= target);
+    const int c = runs ? __builtin_ctzll(runs) : WAVE - 1;
+    const u64 bins = __ballot(cum[c * WAVE + l] >= target);
+    return c * WAVE + (bins ? __builtin_ctzll(bins) : WAVE - 1);
 }
 
 // Range of penalised logits that can fall into bin w, widened so that it can only over-select.
@@ -230,7 +231,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                                                  const float cfg_rcp) {
     constexpr int NUC_WAVES = NucGeom<NUC_BLOCK>::WAVES, NUC_WCAP = NucGeom<NUC_BLOCK>::WCAP, NUC_CAP = NucGeom<NUC_BLOCK>::CAP,
                   NUC_PER = NucGeom<NUC_BLOCK>::PER, NUC_SUB = NucGeom<NUC_BLOCK>::SUB;
-    extern __shared__ u64 nuc_dyn[];
+    extern __shared__ __align__(16) u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over, s_nseen;
     __shared__ u64 s_win, s_mass;
@@ -508,6 +509,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     BORN_STAMP(a, row, 5);
     const bool listed = !s_over && s_n <= NUC_CAP;                   // the wanted bins fit the lists
     const int n = listed ? s_n : 0;
+    const int n4 = (n + 3) & ~3;                                     // the list padded to whole groups of four ..
+    if (tid >= n && tid < n4) {
+        fkey[tid] = 0ull;                                            // .. with entries of no slot and no mass
+        fq[tid] = 3ull << 62;
+    }
     __syncthreads();
 
     // ---- cumulative mass of every listed entry within its bin, in rank order
@@ -516,9 +522,15 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     if (tid < n) {
         mykey = fkey[tid];
         myslot = (int)(fq[tid] >> 62);
-        for (int j = 0; j < n; j++) {
-            const u64 kj = fkey[j], qj = fq[j];
-            if ((int)(qj >> 62) == myslot && kj >= mykey) mine += qj & 0x3FFFFFFFFFFFFFFFull;
+        // four entries a turn, their eight words read with four 128-bit LDS loads before any is used (one dependent
+        // read per entry made this loop wait for LDS: a few hundred entries took longer than a sweep of the row)
+        const ulonglong2 *k2 = reinterpret_cast<const ulonglong2 *>(fkey), *q2 = reinterpret_cast<const ulonglong2 *>(fq);
+        for (int j = 0; j < n4; j += 4) {
+            const ulonglong2 ka = k2[j >> 1], kb = k2[(j >> 1) + 1], qa = q2[j >> 1], qb = q2[(j >> 1) + 1];
+            const u64 ks[4] = {ka.x, ka.y, kb.x, kb.y}, qs[4] = {qa.x, qa.y, qb.x, qb.y};
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                if ((int)(qs[t] >> 62) == myslot && ks[t] >= mykey) mine += qs[t] & 0x3FFFFFFFFFFFFFFFull;
         }
     }
     __syncthreads();                                                 // the lists may be overwritten from here on
@@ -693,7 +705,7 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
 __global__ __launch_bounds__(NUC_BLOCK_MAX) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
                                                                   float *__restrict__ out) {
     constexpr int NUC_BLOCK = NUC_BLOCK_MAX, NUC_WAVES = NUC_BLOCK / WAVE;
-    extern __shared__ u64 nuc_dyn[];
+    extern __shared__ __align__(16) u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ double s_part[NUC_WAVES];
     u32 *const bm = reinterpret_cast<u32 *>(nuc_dyn);                // history bitmap, one bit per id
