@@ -376,7 +376,14 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 
     BORN_STAMP(a, row, 2);
     // ---- sweep 2: integer masses by bin
-    if (r.rcp != 0.0f && !r.degenerate) {
+    if (r.T == 1.0f && !r.degenerate) {
+        sweep(Cached(), [&](int, float y) {
+            float z = y;                                             // a logit of ordinary magnitude is its own canonical form
+            if (!nuc_ordinary(y)) z = canon(y);
+            const float d = r.m - z;
+            atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
+        });
+    } else if (r.rcp != 0.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
