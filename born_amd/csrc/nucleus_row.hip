@@ -185,12 +185,12 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     }
 }
 // Visits every element of the row as f(id, penalised logit).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, class F>
-__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f) {
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, class F, class PRE = NucNoPre>
+__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f, PRE pre = PRE()) {
     nuc_foreach4<NUC_BLOCK, NT, AHEAD>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
-    }, f);
+    }, f, pre);
 }
 
 // smallest bin whose inclusive cumulative mass reaches target (the last bin if none does); called by whole waves.
@@ -265,82 +265,86 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     r.freq = COUNTED ? cfg_freq : 0.0f;
     r.pres = COUNTED ? cfg_pres : 0.0f;
     r.penal = (cfg_rep != 1.0f || COUNTED) && hlen > 0;
-    if (r.penal)
-        for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
-    for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;
-    if (tid == 0) {
-        s_n = 0;
-        s_over = 0;
-        s_win = 0ull;
-        s_nseen = 0;
-    }
-    __syncthreads();
-    // The ids the history holds, each once (whoever sets an id's bit first lists it): at most NUC_SEEN per thread, kept
-    // in registers with their penalised logits for the whole kernel. The sweeps then see a constant in place of a seen
-    // logit (chosen per sweep so that it contributes nothing) and visit the seen ids apart, every lane busy; applying the
-    // penalty inside the sweep costs a whole wave the penalty arithmetic whenever one of its lanes holds a seen id, which
-    // with a long history is nearly always. A history too long for the registers keeps the penalty inside the sweeps.
     constexpr int NUC_SEEN = 4;
     u32 *const seen_list = reinterpret_cast<u32 *>(fkey);            // [NUC_SEEN * NUC_BLOCK], free until the gather classifies
     static_assert(NUC_SEEN * NUC_BLOCK * sizeof(u32) <= 2 * NUC_CAP * sizeof(u64), "the list of seen ids fits the gathered entries' storage");
     const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
-    if (list_seen) {
-        int hv[NUC_SEEN];                                            // (all of the thread's history loads in flight together)
-#pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++) {
-            const int i = tid + k * NUC_BLOCK;
-            hv[k] = i < hlen ? h[i] : -2;
-        }
-#pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++) {
-            const int t = hv[k];
-            bool first = false;
-            if (t >= 0 && t < V) {
-                const u32 bit = 1u << (t & 31);
-                const u32 old = atomicOr(&bm[t >> 5], bit);
-                first = !(old & bit);
-            } else if (t != -2) {
-                atomicOr(a.status, 1);
-            }
-            // one addition to the list's length per wave
-            const u64 mk = __ballot(first);
-            if (mk) {
-                const u32 rank = __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
-                int base = 0;
-                if (first && rank == 0u) base = atomicAdd(&s_nseen, __popcll(mk));
-                base = __builtin_amdgcn_readlane(base, __builtin_ctzll(mk));
-                if (first) seen_list[base + (int)rank] = (u32)t;
-            }
-        }
-    } else {
-        for (int i = tid; i < hlen; i += NUC_BLOCK) {
-            const int t = h[i];
-            if (t < 0 || t >= V) atomicOr(a.status, 1);
-            else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
-        }
-    }
-    __syncthreads();
     int seen_id[NUC_SEEN];
     float seen_y[NUC_SEEN];
     r.masked = list_seen;
     r.skip = -INFINITY;                                              // sweep 1: neither the maximum nor the smallest finite value
-    {
-        const int nseen = list_seen ? s_nseen : 0;
-#pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++) {
-            const int i = tid + k * NUC_BLOCK;
-            seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
+    // What must precede the first visit of sweep 1 but not its first loads: run by the row visitor with the first stage
+    // in flight (barriers that wait for LDS only).
+    auto prologue = [&]() {
+        if (r.penal)
+            for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
+        for (int i = tid; i < NUC_BINS; i += NUC_BLOCK) mass[i] = 0ull;
+        if (tid == 0) {
+            s_n = 0;
+            s_over = 0;
+            s_win = 0ull;
+            s_nseen = 0;
         }
-        float raw[NUC_SEEN];
+        lds_barrier();
+        // The ids the history holds, each once (whoever sets an id's bit first lists it): at most NUC_SEEN per thread, kept
+        // in registers with their penalised logits for the whole kernel. The sweeps then see a constant in place of a seen
+        // logit (chosen per sweep so that it contributes nothing) and visit the seen ids apart, every lane busy; applying the
+        // penalty inside the sweep costs a whole wave the penalty arithmetic whenever one of its lanes holds a seen id, which
+        // with a long history is nearly always. A history too long for the registers keeps the penalty inside the sweeps.
+        if (list_seen) {
+            int hv[NUC_SEEN];                                            // (all of the thread's history loads in flight together)
 #pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++) raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
+            for (int k = 0; k < NUC_SEEN; k++) {
+                const int i = tid + k * NUC_BLOCK;
+                hv[k] = i < hlen ? h[i] : -2;
+            }
 #pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++)
-            seen_y[k] = seen_id[k] >= 0 ? penalise_seen(raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
-    }
+            for (int k = 0; k < NUC_SEEN; k++) {
+                const int t = hv[k];
+                bool first = false;
+                if (t >= 0 && t < V) {
+                    const u32 bit = 1u << (t & 31);
+                    const u32 old = atomicOr(&bm[t >> 5], bit);
+                    first = !(old & bit);
+                } else if (t != -2) {
+                    atomicOr(a.status, 1);
+                }
+                // one addition to the list's length per wave
+                const u64 mk = __ballot(first);
+                if (mk) {
+                    const u32 rank = __builtin_amdgcn_mbcnt_hi((u32)(mk >> 32), __builtin_amdgcn_mbcnt_lo((u32)mk, 0u));
+                    int base = 0;
+                    if (first && rank == 0u) base = atomicAdd(&s_nseen, __popcll(mk));
+                    base = __builtin_amdgcn_readlane(base, __builtin_ctzll(mk));
+                    if (first) seen_list[base + (int)rank] = (u32)t;
+                }
+            }
+        } else {
+            for (int i = tid; i < hlen; i += NUC_BLOCK) {
+                const int t = h[i];
+                if (t < 0 || t >= V) atomicOr(a.status, 1);
+                else if (r.penal) atomicOr(&bm[t >> 5], 1u << (t & 31));
+            }
+        }
+        lds_barrier();
+        {
+            const int nseen = list_seen ? s_nseen : 0;
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++) {
+                const int i = tid + k * NUC_BLOCK;
+                seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
+            }
+            float raw[NUC_SEEN];
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++) raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++)
+                seen_y[k] = seen_id[k] >= 0 ? penalise_seen(raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
+        }
+    };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
-    auto sweep = [&](auto nt, auto f) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f);
+    auto sweep = [&](auto nt, auto f, auto pre) {
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f, pre);
         if (r.masked) {
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++)
@@ -357,7 +361,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         sweep(Cached(), [&](int, float y) {
             mx = fmaxf(mx, y);
             mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
-        });
+        }, prologue);
         mx = block_max_f32<NUC_BLOCK>(mx, &scr);
         mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
         r.m = uniform_f32(nuc_z(r, mx));
@@ -382,19 +386,19 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             if (!nuc_ordinary(y)) z = canon(y);
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        });
+        }, NucNoPre());
     } else if (r.rcp != 0.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        });
+        }, NucNoPre());
     } else {
         sweep(Cached(), [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        });
+        }, NucNoPre());
     }
     __syncthreads();
     BORN_STAMP(a, row, 3);
@@ -472,11 +476,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         };
         // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
         if (nint == 1) {
-            sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+            sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); }, NucNoPre());
         } else {
             sweep(Streamed(), [&](int j, float y) {
                 append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
-            });
+            }, NucNoPre());
         }
         const u32 count = __hip_atomic_load(wcount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
         if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
