@@ -86,12 +86,14 @@ template <bool NT>
 __device__ __forceinline__ nuc_f32x4 nuc_load4(const nuc_f32x4 *p) {
     return NT ? __builtin_nontemporal_load(p) : *p;
 }
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, class F4, class F1, class PRE = NucNoPre>
+// PLAIN: the caller knows that the row has no penalties (a loop of its own without the penalty code: the visitor's
+// test of r.penal at every visit cost the single-sweep kernel 5 %).
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F4, class F1, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
         float y[4] = {q[0], q[1], q[2], q[3]};
-        if (r.penal) {
+        if (!PLAIN && r.penal) {
             // One seen element per turn, the lowest first: with a long history nearly every wave has some lane with a seen
             // id among its four, but a lane rarely holds two, so the wave computes one penalty per visit, not four.
             u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
@@ -119,7 +121,7 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     };
     auto visit1 = [&](int j) {
         float y = r.x[j];
-        if (r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = r.masked ? r.skip : penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
+        if (!PLAIN && r.penal && ((bm[j >> 5] >> (j & 31)) & 1u)) y = r.masked ? r.skip : penalise_seen(y, r.rep, r.counts, j, r.freq, r.pres);
         f1(j, y);
     };
     if (r.vec) {
@@ -785,21 +787,21 @@ __global__ __launch_bounds__(NUC_BLOCK_MAX) void token_logprob_kernel(SampleArgs
         st *= (double)__expf(mt - mnew);                             // exp(-inf) = 0: nothing finite was seen so far
         mt = mnew;
     };
-    nuc_foreach4<NUC_BLOCK, true, false>(r, bm,
-        [&](int, const float (&y)[4]) {
-            float z[4];
+    auto four = [&](int, const float (&y)[4]) {
+        float z[4];
 #pragma unroll
-            for (int t = 0; t < 4; t++) z[t] = zof(y[t]);
-            const float m4 = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
-            if (m4 > mt) raise(m4);
-            st += (double)((term(z[0], mt) + term(z[1], mt)) + (term(z[2], mt) + term(z[3], mt)));
-        },
-        [&](int, float y) {
-            const float z = zof(y);
-            if (z > mt) raise(z);
-            st += (double)term(z, mt);
-        },
-        build_bitmap);
+        for (int t = 0; t < 4; t++) z[t] = zof(y[t]);
+        const float m4 = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
+        if (m4 > mt) raise(m4);
+        st += (double)((term(z[0], mt) + term(z[1], mt)) + (term(z[2], mt) + term(z[3], mt)));
+    };
+    auto one = [&](int, float y) {
+        const float z = zof(y);
+        if (z > mt) raise(z);
+        st += (double)term(z, mt);
+    };
+    if (r.penal) nuc_foreach4<NUC_BLOCK, true, false, false>(r, bm, four, one, build_bitmap);
+    else nuc_foreach4<NUC_BLOCK, true, false, true>(r, bm, four, one, build_bitmap);
 
     const float m = block_max_f32<NUC_BLOCK>(mt, &scr);
     double part = mt == m ? st : st * exp((double)mt - (double)m);   // a thread without elements: st = 0
