@@ -9,9 +9,10 @@
 namespace born {
 
 // ---------------------------------------------------------------------------
-// argmax: B * S workgroups of 256 threads scan 8192 logits each with 128-bit loads and write one
+// argmax, small batches: B * S workgroups of 256 threads scan 8192 logits each with 128-bit loads and write one
 // (value, index) partial; a second, tiny launch merges the S partials of each row (a kernel
 // boundary is the cheapest correct way to pass data between workgroups on this multi-XCD part).
+// From 64 rows on: argmax_row_kernel, a row per workgroup in one launch.
 // A NaN never wins (the reference's comparisons are false for it) unless it sits at index 0,
 // where the reference's loop returns 0.
 // ---------------------------------------------------------------------------
@@ -94,8 +95,63 @@ __global__ __launch_bounds__(64) void argmax_merge_kernel(const float *__restric
     if (threadIdx.x == 0) tokens[row] = argmax_token(b, logits[(long long)row * stride]);
 }
 
+// Batches that fill a fair part of the device on their own: one workgroup of 1024 threads per row, one launch
+// (64 rows x 32000: 7.1 us as two launches, of which the second only merges four partials per row).
+typedef float argmax_f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(1024) void argmax_row_kernel(const float *__restrict__ logits, int V, long long stride,
+                                                          int *__restrict__ tokens) {
+    __shared__ ArgPair sh[16];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float *x = logits + (long long)row * stride;
+    const bool vec = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
+    ArgPair best = {-INFINITY, 0x7FFFFFFF};
+    // a thread meets its indices in ascending order, so "strictly greater" keeps the first of equals; NaN compares false
+    auto take = [&](float v, int j) {
+        if (v > best.v) {
+            best.v = v;
+            best.i = j;
+        }
+    };
+    if (vec) {
+        const int n4 = V >> 2;
+        const argmax_f32x4 *x4 = reinterpret_cast<const argmax_f32x4 *>(x);
+        int i = tid;
+        for (; i + 3 * 1024 < n4; i += 4 * 1024) {                    // four loads in flight per thread
+            argmax_f32x4 f[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) f[u] = __builtin_nontemporal_load(x4 + i + u * 1024);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) take(f[u][c], ((i + u * 1024) << 2) + c);
+        }
+        for (; i < n4; i += 1024) {
+            const argmax_f32x4 f = __builtin_nontemporal_load(x4 + i);
+#pragma unroll
+            for (int c = 0; c < 4; c++) take(f[c], (i << 2) + c);
+        }
+        for (int j = (n4 << 2) + tid; j < V; j += 1024) take(x[j], j);
+    } else {
+        for (int j = tid; j < V; j += 1024) take(x[j], j);
+    }
+    best = wave_best(best);
+    if (lane_id() == 0) sh[wave_id()] = best;
+    __syncthreads();
+    if (tid == 0) {
+        ArgPair b = sh[0];
+        for (int w = 1; w < 16; w++) b = better(b, sh[w]);
+        tokens[row] = argmax_token(b, x[0]);
+    }
+}
+
+constexpr int ARGMAX_ROW_KERNEL_BATCH = 64;     // from this many rows on, a row per workgroup
+
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st) {
+    if (B >= ARGMAX_ROW_KERNEL_BATCH) {
+        hipLaunchKernelGGL(argmax_row_kernel, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, tokens);
+        return hipGetLastError();
+    }
     int S = (V + ARGMAX_SEG - 1) / ARGMAX_SEG;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3((unsigned)(B * S)), dim3(256), 0, st, logits, V, stride, S, tokens,
                        part_val, part_idx);

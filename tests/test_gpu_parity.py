@@ -105,9 +105,15 @@ def test_argmax_reference_kats_and_tie_rule(oracle, rocm):
     assert _argmax(rocm, x).tolist() == [2, 0, 1, 2]
     x = np.array([[5, 5, 5], [1, 7, 7], [np.nan, 9, 1], [1, np.nan, 0], [-np.inf, -np.inf, -np.inf]], dtype=np.float32)
     assert _argmax(rocm, x).tolist() == oracle.argmax_ref(x).tolist() == [0, 1, 0, 0, 0]
+    assert _argmax(rocm, np.tile(x, (16, 1))).tolist() == [0, 1, 0, 0, 0] * 16         # 80 rows: the row-per-workgroup kernel
+    wide = np.full((64, 9000), -np.inf, np.float32)
+    wide[1, 8999] = 3.0; wide[2, 0] = np.nan; wide[2, 5] = 9.0; wide[3, 4096:4100] = 7.0; wide[4, :] = np.nan
+    assert _argmax(rocm, wide).tolist() == oracle.argmax_ref(wide).tolist()
 
 
-@pytest.mark.parametrize("B,V,stride", [(64, 32000, None), (7, 8193, None), (5, 1001, 1003), (3, 128256, None), (2, 5, 8)])
+@pytest.mark.parametrize("B,V,stride", [(64, 32000, None), (7, 8193, None), (5, 1001, 1003), (3, 128256, None), (2, 5, 8),
+                                        (63, 32000, None), (64, 8193, None), (70, 1001, 1003), (65, 5, 8), (64, 16384, 16388),
+                                        (96, 128256, None), (64, 1, None), (64, 20001, 20004)])
 def test_argmax_random_and_ties(oracle, rocm, B, V, stride):
     rng = np.random.default_rng(V)
     x = rng.standard_normal((B, V), dtype=np.float32)
