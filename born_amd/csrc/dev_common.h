@@ -105,8 +105,16 @@ __device__ __forceinline__ float emass(float z, float m, float dcut = 80.0f) {
     float d = (z == m) ? 0.0f : m - z;
     return expneg(d, dcut);
 }
-// trunc(e * 2^S): e has 24 significant bits, so e * 2^S (S <= 61) is exact in fp32
-__device__ __forceinline__ u64 qfix(float e, float scale) { return (u64)(e * scale); }
+// trunc(e * 2^S): e has 24 significant bits, so x = e * 2^S (S <= 61) is exact in fp32.  The two 32-bit halves are
+// taken apart in five instructions (the compiler's float -> u64 conversion is seven): hi = trunc(x / 2^32) is exact
+// and has at most 24 significant bits, so it converts back exactly, and x - hi * 2^32 is the exact low part (one
+// fused multiply-add whose result is representable), truncated by its conversion.
+__device__ __forceinline__ u64 qfix(float e, float scale) {
+    const float x = e * scale;
+    const u32 hi = (u32)(x * 2.3283064365386963e-10f);
+    const u32 lo = (u32)__fmaf_rn(-(float)hi, 4294967296.0f, x);
+    return ((u64)hi << 32) | (u64)lo;
+}
 __device__ __forceinline__ float mass_scale(int S) { return __uint_as_float((u32)(S + 127) << 23); }
 
 // ---- built-in uniform stream ------------------------------------------------

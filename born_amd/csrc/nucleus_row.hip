@@ -99,10 +99,12 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
             if (r.masked) {
                 if (bits) {
-                    y[0] = (bits & 1u) ? r.skip : y[0];
-                    y[1] = (bits & 2u) ? r.skip : y[1];
-                    y[2] = (bits & 4u) ? r.skip : y[2];
-                    y[3] = (bits & 8u) ? r.skip : y[3];
+                    const u32 sk = __float_as_uint(r.skip);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {                    // a bit field extract and a bitwise select per element
+                        const u32 m = (u32)((int)(bits << (31 - t)) >> 31);
+                        y[t] = __uint_as_float((sk & m) | (__float_as_uint(y[t]) & ~m));
+                    }
                 }
                 bits = 0u;
             }
@@ -357,12 +359,13 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     typedef std::integral_constant<bool, true> Streamed;             // the row's last sweep: non-temporal loads
 
     BORN_STAMP(a, row, 1);
-    // ---- sweep 1: maximum and smallest finite penalised logit
+    // ---- sweep 1: maximum of the penalised logits, and about how far below it they reach
     {
         float mx = -INFINITY, mn = INFINITY;
-        sweep(Cached(), [&](int, float y) {
+        // (the smallest value only sizes the bins: every fourth id is looked at, spread over the whole row)
+        sweep(Cached(), [&](int j, float y) {
             mx = fmaxf(mx, y);
-            mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
+            if ((j & 3) == 0) mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
         }, prologue);
         mx = block_max_f32<NUC_BLOCK>(mx, &scr);
         mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
@@ -385,7 +388,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     if (r.T == 1.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
             float z = y;                                             // a logit of ordinary magnitude is its own canonical form
-            if (!nuc_ordinary(y)) z = canon(y);
+            if (!nuc_ordinary(y)) {
+                asm volatile("" ::: "memory");                       // (keeps this a branch: as selects it is paid by every logit)
+                z = canon(y);
+            }
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
