@@ -44,7 +44,14 @@ __device__ __forceinline__ void spec_foreach(const float *x, int V, bool vec, F 
 // RESIDENT: V <= SPEC_RESIDENT_V, V % 4 == 0 and the rows 16-byte aligned.
 // z = canon(x / T); UNIT: T == 1, where the division is the identity and is not computed at all.
 template <bool UNIT>
-__device__ __forceinline__ float spec_z(float x, float T) { return UNIT ? canon(x) : z_of(x, T); }
+__device__ __forceinline__ float spec_z(float x, float T) {
+    if (!UNIT) return z_of(x, T);
+    // a logit of ordinary magnitude (2^-100 <= |x| < 2^100) is its own canonical form: one integer range test, and a
+    // branch that waves of ordinary logits never take, instead of three compares and selects on every logit
+    if (((__float_as_uint(x) & 0x7FFFFFFFu) - (27u << 23)) < (200u << 23)) return x;
+    asm volatile("" ::: "memory");                                   // (keeps the rest behind a branch)
+    return canon(x);
+}
 
 template <bool RESIDENT, bool UNIT>
 __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
@@ -87,11 +94,21 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
             }
         }
         m = block_max_f32<SPEC_BLOCK>(m, &scr);
+        if (m > -INFINITY) {                                         // (uniform) m - z is a number: +inf for a masked logit, no mass
 #pragma unroll
-        for (int i = 0; i < SPEC_NF4; i++) {
-            if (i * SPEC_BLOCK + tid < n4) {
+            for (int i = 0; i < SPEC_NF4; i++) {
+                if (i * SPEC_BLOCK + tid < n4) {
 #pragma unroll
-                for (int c = 0; c < 4; c++) sum += qfix(emass(t[i][c], m), scale);
+                    for (int c = 0; c < 4; c++) sum += qfix(expneg(m - t[i][c]), scale);
+                }
+            }
+        } else {                                                     // nothing finite: (-inf) - (-inf) := 0 for every logit
+#pragma unroll
+            for (int i = 0; i < SPEC_NF4; i++) {
+                if (i * SPEC_BLOCK + tid < n4) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) sum += qfix(emass(t[i][c], m), scale);
+                }
             }
         }
     } else {
