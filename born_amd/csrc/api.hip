@@ -660,6 +660,13 @@ static int spec_verify_impl(born_sampler *s, const float *target, int64_t target
     a.u_acc = u_accept;
     a.u_res = u_residual;
     a.T = s->cfg.temperature;
+    if (a.T != 1.0f) {                                               // (host arithmetic only; the answer is kept per temperature)
+        if (s->div_T != a.T) {
+            s->div_rcp = division_shortcut_reciprocal(a.T);
+            s->div_T = a.T;
+        }
+        a.rcp_T = s->div_rcp;
+    }
     a.n_accepted = n_accepted_out;
     a.next_token = next_token_out;
     a.mp = s->sp_mp; a.mq = s->sp_mq;

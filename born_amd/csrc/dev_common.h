@@ -73,6 +73,24 @@ __device__ __forceinline__ float penalise_counted(float x, float r, bool counted
 // z from a (possibly penalised) logit: temperature then canonicalisation
 __device__ __forceinline__ float z_of(float y, float T) { return canon(T == 1.0f ? y : y / T); }
 
+// The division shortcut (division.cpp decides on the host for which T it is exact; rcp = RN(1 / T) then, else 0):
+// for a logit of ordinary magnitude, 2^-100 <= |y| < 2^100, a multiply and two fused multiply-adds give the correctly
+// rounded y / T, a finite non-zero number that is its own canonical form; anything else takes z_of behind a branch
+// that waves of ordinary logits never take.
+__device__ __forceinline__ bool ordinary_magnitude(float y) {
+    return ((__float_as_uint(y) & 0x7FFFFFFFu) - (27u << 23)) < (200u << 23);
+}
+__device__ __forceinline__ float z_of_shortcut(float y, float T, float rcp) {
+    const float q = __fmul_rn(y, rcp);
+    const float e = __fmaf_rn(-q, T, y);
+    float z = __fmaf_rn(e, rcp, q);
+    if (!ordinary_magnitude(y)) {
+        asm volatile("" ::: "memory");                               // (keeps the division behind a branch)
+        z = z_of(y, T);
+    }
+    return z;
+}
+
 // next representable float below x (x finite or +inf, not NaN); nextbelow(-FLT_MAX) = -inf
 __device__ __forceinline__ float next_below(float x) {
     if (x == 0.0f) return -1.401298464e-45f;

@@ -86,6 +86,7 @@ struct SpecArgs {
     const int *draft_tokens;
     const float *u_acc, *u_res;
     float T;
+    float rcp_T;                  // RN(1 / T) where the division shortcut is exact for T (division.cpp), else 0
     int *n_accepted, *next_token;
     // workspace: per (b, i) row statistics
     float *mp, *mq;

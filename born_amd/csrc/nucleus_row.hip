@@ -59,11 +59,8 @@ __device__ __forceinline__ float nuc_d(const NucRow &r, float z) { return r.dege
 __device__ __forceinline__ int nuc_bin(const NucRow &r, float d) {
     return (int)fminf(d * r.sbin, (float)(NUC_BINS - 1));          // monotone in d; NaN, inf and all beyond the span -> last bin
 }
-// z for a logit of ordinary magnitude by the division shortcut (r.rcp != 0): equal to nuc_z for 2^-100 <= |y| < 2^100,
-// which `ordinary` tests; the result is finite and not zero, so it is its own canonical form.
-__device__ __forceinline__ bool nuc_ordinary(float y) {
-    return ((__float_as_uint(y) & 0x7FFFFFFFu) - (27u << 23)) < (200u << 23);
-}
+// (the magnitude test of the division shortcut and of the unit-temperature path: dev_common.h)
+__device__ __forceinline__ bool nuc_ordinary(float y) { return ordinary_magnitude(y); }
 __device__ __forceinline__ float nuc_z_shortcut(const NucRow &r, float y) {
     const float q = __fmul_rn(y, r.rcp);
     const float e = __fmaf_rn(-q, r.T, y);

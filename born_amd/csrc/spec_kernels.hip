@@ -44,11 +44,11 @@ __device__ __forceinline__ void spec_foreach(const float *x, int V, bool vec, F 
 // RESIDENT: V <= SPEC_RESIDENT_V, V % 4 == 0 and the rows 16-byte aligned.
 // z = canon(x / T); UNIT: T == 1, where the division is the identity and is not computed at all.
 template <bool UNIT>
-__device__ __forceinline__ float spec_z(float x, float T) {
-    if (!UNIT) return z_of(x, T);
+__device__ __forceinline__ float spec_z(float x, float T, float rcp) {
+    if (!UNIT) return rcp != 0.0f ? z_of_shortcut(x, T, rcp) : z_of(x, T);
     // a logit of ordinary magnitude (2^-100 <= |x| < 2^100) is its own canonical form: one integer range test, and a
     // branch that waves of ordinary logits never take, instead of three compares and selects on every logit
-    if (((__float_as_uint(x) & 0x7FFFFFFFu) - (27u << 23)) < (200u << 23)) return x;
+    if (ordinary_magnitude(x)) return x;
     asm volatile("" ::: "memory");                                   // (keeps the rest behind a branch)
     return canon(x);
 }
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     const float *x = is_bonus ? a.bonus + (long long)row * a.b_seq
                               : (is_draft ? a.draft + (long long)(row / a.G) * a.d_seq : a.target + (long long)(row / a.G) * a.t_seq) +
                                     (long long)(row % a.G) * V;
-    const float T = a.T;
+    const float T = a.T, rcp = a.rcp_T;
     const float scale = mass_scale(a.mass_shift);
     // The draft token and its logit are two dependent loads: requested now, used after the reductions (at the end of
     // the kernel they would be two memory round trips nothing overlaps).
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
         for (int i = 0; i < SPEC_NF4; i++) {
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                t[i][c] = spec_z<UNIT>(t[i][c], T);                  // the -inf fill stays -inf
+                t[i][c] = spec_z<UNIT>(t[i][c], T, rcp);                  // the -inf fill stays -inf
                 m = fmaxf(m, t[i][c]);
             }
         }
@@ -113,9 +113,9 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
         }
     } else {
         const bool vec = a.aligned != 0;
-        spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, spec_z<UNIT>(v, T)); });
+        spec_foreach(x, V, vec, [&](float v) { m = fmaxf(m, spec_z<UNIT>(v, T, rcp)); });
         m = block_max_f32<SPEC_BLOCK>(m, &scr);
-        spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(spec_z<UNIT>(v, T), m), scale); });
+        spec_foreach(x, V, vec, [&](float v) { sum += qfix(emass(spec_z<UNIT>(v, T, rcp), m), scale); });
     }
     u64 Z;
     block_inclusive_scan_u64<SPEC_BLOCK>(sum, &scr, &Z);
@@ -132,10 +132,13 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
 }
 
 // ip = 1 / Zp and iq = 1 / Zq are formed once per row; each product below is one fp64 rounding.
-__device__ __forceinline__ u64 residual_mass(float t, float d, float T, float mp, float mq, float scale, double ip,
+__device__ __forceinline__ float spec_z_any(float x, float T, float rcp) {
+    return rcp != 0.0f ? z_of_shortcut(x, T, rcp) : z_of(x, T);      // (uniform; z_of itself skips the division at T = 1)
+}
+__device__ __forceinline__ u64 residual_mass(float t, float d, float T, float rcp, float mp, float mq, float scale, double ip,
                                              double iq, double scale_d) {
-    double pj = (double)qfix(emass(z_of(t, T), mp), scale) * ip;
-    double qj = (double)qfix(emass(z_of(d, T), mq), scale) * iq;
+    double pj = (double)qfix(emass(spec_z_any(t, T, rcp), mp), scale) * ip;
+    double qj = (double)qfix(emass(spec_z_any(d, T, rcp), mq), scale) * iq;
     double r = pj > qj ? pj - qj : 0.0;
     return (u64)(r * scale_d);
 }
@@ -170,7 +173,7 @@ __device__ __forceinline__ void spec_run(int V, int c, int tid, int &j0, int &j1
 
 struct SpecRow {
     const float *xt, *xd;
-    float T, mp, mq, scale;
+    float T, rcp, mp, mq, scale;
     double Zp, Zq, scale_d;       // Zp, Zq: reciprocals of the integer normalisers
     bool plain;                   // bonus row: the mass of id j is the row's own integer mass, there is no draft
 };
@@ -178,6 +181,7 @@ struct SpecRow {
 __device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
     SpecRow r;
     r.T = a.T;
+    r.rcp = a.rcp_T;
     r.scale = mass_scale(a.mass_shift);
     r.scale_d = ldexp(1.0, a.mass_shift);
     r.plain = i == a.G;
@@ -197,8 +201,8 @@ __device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
     return r;
 }
 __device__ __forceinline__ u64 spec_mass(const SpecRow &r, float t, float d) {
-    if (r.plain) return qfix(emass(z_of(t, r.T), r.mp), r.scale);    // uniform per row
-    return residual_mass(t, d, r.T, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+    if (r.plain) return qfix(emass(spec_z_any(t, r.T, r.rcp), r.mp), r.scale);    // uniform per row
+    return residual_mass(t, d, r.T, r.rcp, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
 }
 constexpr int SPEC_RUN = 8;                   // run lengths up to this are loaded before any arithmetic
 __device__ __forceinline__ u64 spec_run_mass(const SpecRow &r, int j0, int j1) {
