@@ -436,17 +436,18 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
     } else if (launched == 1u) {
         keep_first(launch_topk_row(a, st));
-    } else if (launched == 2u) {
-        if (a.T != 1.0f) {                                           // (host arithmetic only: nothing is launched or waited for)
+    } else {
+        // the kernels that divide every logit by the temperature take the shortcut where it is exact for this temperature
+        // (host arithmetic only: nothing is launched or waited for; per-row temperatures, above, always divide)
+        if (a.T != 1.0f) {
             if (s->div_T != a.T) {
                 s->div_rcp = division_shortcut_reciprocal(a.T);
                 s->div_T = a.T;
             }
             a.rcp_T = s->div_rcp;
         }
-        keep_first(launch_nucleus_row(a, st, nullptr, s->path == 2));
-    } else {
-        keep_first(launch_sample_wide(a, st));
+        if (launched == 2u) keep_first(launch_nucleus_row(a, st, nullptr, s->path == 2));
+        else keep_first(launch_sample_wide(a, st));
     }
     if (table) keep_first(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st));
     if (launch_err != hipSuccess) return hip_fail(launch_err, "sample: kernel launch");

@@ -88,6 +88,7 @@ __device__ __forceinline__ bool row_config(SampleArgs &a, const RowConfigs &rc, 
     RowValues v;
     const bool mine = row_config_values(a, rc, row, my_route, v, invalid);
     a.T = v.T;
+    a.rcp_T = 0.0f;                                                  // (the shortcut is decided per temperature on the host: a row of its own divides)
     a.top_k = v.top_k;
     a.top_p = v.top_p;
     a.rep = v.rep;

@@ -16,7 +16,7 @@ struct WideCtx {
     const BORN_GLOBAL float *x;
     int V;
     bool vec, has_hist, count_mode;
-    float T, rep, m, scale, dcut;
+    float T, rcp, rep, m, scale, dcut;   // rcp: RN(1 / T) where the division shortcut is exact for T, else 0
     const unsigned *counts;  // occurrences of each id in the row's history (frequency / presence penalties), or null
     float freq, pres;
     const lds_u32 *bm;
@@ -35,6 +35,7 @@ __device__ __forceinline__ int wide_bin(float d) {
 // z of a penalised logit (uniform branch: no division at temperature 1)
 __device__ __forceinline__ float wide_z(const WideCtx &c, float y) {
     if (c.T == 1.0f) return canon(y);
+    if (c.rcp != 0.0f) return z_of_shortcut(y, c.T, c.rcp);
     return canon(y / c.T);
 }
 
@@ -336,6 +337,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     c.V = V;
     c.vec = ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
     c.T = uniform_f32(a.T);
+    c.rcp = uniform_f32(a.rcp_T);
     c.rep = uniform_f32(a.rep);
     c.scale = uniform_f32(mass_scale(a.mass_shift));
     c.dcut = a.dcut;
