@@ -43,7 +43,9 @@ def _check_against_oracle(oracle, rocm, x, u, T=1.0, k=0, p=1.0, rep=1.0, hist=N
     diff = got["tokens"] != tr["tokens"]
     assert not (diff & ~tr["near"]).any(), "token differs from the fp64 truth on a row not flagged near a CDF step"
     assert tr["near"].mean() <= max_near_frac
-    same = ~diff
+    # (a row whose top-p / min-p cut lies within the tolerance of an element boundary may keep one element more or fewer
+    # in the truth layer than in the fixed-point layer: same token, another normaliser; the truth layer flags such rows)
+    same = ~diff & ~tr["near_cut"]
     assert np.allclose(got["probs"][same], tr["probs"][same], rtol=1e-5, atol=0), "probability off by more than 1e-5 relative"
     if nuc:
         assert np.array_equal(got["n_nucleus"], fx["n_nucleus"])
