@@ -196,3 +196,40 @@ def test_large_vocabularies_against_oracle(oracle, rocm, V):
                 fx = oracle.sample(x, u, 0.8, k, p, rep, hist, mode=oracle.MODE_FIXED, min_p=min_p, freq=freq, pres=pres)
             assert np.array_equal(out["tokens"], fx["tokens"]), (V, k, p, rep, path)
             assert np.array_equal(out["probs"].view(np.uint32), fx["probs"].view(np.uint32)), (V, k, p, rep, path)
+
+
+def test_wide_seeded_sweep_on_request(oracle, rocm):
+    """The sweep above with as many further seeded chunks as BORN_SWEEP_CHUNKS asks for (skipped when unset), weighted
+    towards the kernel without a top-k cut: temperatures the division shortcut takes and refuses, histories up to 5000
+    tokens, draws from the very end of the rank order, logits of unusual magnitude; all three kernel selections.
+    BORN_SWEEP_SEED moves the seeds.  (About 140 cases a second; a run of 150 000 cases found nothing in the kernels
+    and one tolerance of these tests.)"""
+    import os
+    chunks = int(os.environ.get("BORN_SWEEP_CHUNKS", "0"))
+    if chunks <= 0:
+        pytest.skip("set BORN_SWEEP_CHUNKS to run it")
+    seed0 = int(os.environ.get("BORN_SWEEP_SEED", "2000000"))
+    odd = np.array([0.0, -0.0, 1e-45, 3e-31, 2 ** -100, 2 ** -101, 1.2e30, 2 ** 100, -3e38], dtype=np.float32)
+    for chunk in range(chunks):
+        rng = np.random.default_rng(seed0 + chunk)
+        for i in range(10):
+            c = _draw_case(rng)
+            if rng.random() < 0.7:
+                c["k"] = 0
+            c["T"] = float(rng.choice([0.25, 0.35, 0.5, 0.7, 0.8, 1.0, 1.2, 1.3, 1.9999999, 2.0, 5.0]))
+            if rng.random() < 0.3:
+                c["V"] = int(rng.integers(1, 40000))
+            if rng.random() < 0.3:
+                c["H"] = int(rng.integers(1, 5000))
+            x, u, hist, hist_len = _inputs(rng, c)
+            if rng.random() < 0.3:
+                u[-1] = np.float32(1.0) - np.float32(2.0 ** -24)
+            if rng.random() < 0.2 and x.size > 8:
+                at = rng.integers(0, x.size, size=8)
+                x.reshape(-1)[at] = rng.choice(odd, size=8)
+            for path in (0, 2, 1):
+                try:
+                    _check_against_oracle(oracle, rocm, x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, path=path,
+                                          min_p=c["min_p"], freq=c["freq"], pres=c["pres"])
+                except Exception as e:
+                    raise AssertionError(f"seed {seed0 + chunk} case {i} path {path}: {c}: {type(e).__name__}: {e}") from None
