@@ -11,11 +11,11 @@ the one the metric is quoted on).  Prints ONE JSON line.
                step finds its logits in the Infinity Cache)
   roofline     that kernel: algorithmic bytes of one step divided by its average launch duration,
                measured here with HIP events on the launch stream over the timed region
-  timing       W warm-up steps, then exactly K timed steps between two events, a synchronisation on
-               either side; the last warm-up step is launched behind the opening synchronisation and
-               the opening event behind it, so that the region holds K launch-to-launch steps and not
-               the latency of a first launch on an idle device (that figure is printed beside it as
-               ms_per_step_idle_start)
+  timing       W untimed warm-up steps, then exactly K timed steps between two events on the launch
+               stream, a synchronisation on either side.  The spread measurement (30 groups of 10
+               steps, its own figures) runs before the warm-up: a step is 27 us, W = 5 steps are
+               0.14 ms, and a device that idled during the host's set-up is not at its working clocks
+               after that little work
   cpu_baseline the CPU oracle's reference-arithmetic mode timed on this box's host, one thread,
                on a bounded sample of the same workload
 
@@ -49,13 +49,13 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 # file under profiles/ that holds the counters; a run whose dominant kernel is not listed prints null.
 PMC_TRAFFIC = {
     ("C3", "topk_row_kernel"): {
-        "bytes": int(64581.8 * (128256 / 64146.2) * 1024 + 24.0 * 1024),
+        "bytes": int(64581.8 * (128256 / 64145.8) * 1024 + 24.0 * 1024),
         "measured_on": "born::topk_row_kernel<true, false>, workload C3",
         "source": "profiles/topk_row_kernel_c3_hbm_traffic.txt",
     },
     # (the probe of that run copied a C5 logits buffer: 608 256 KiB read and written)
     ("C5", "nucleus_row_kernel"): {
-        "bytes": int(1013597.0 * (608256 / 304147.1) * 1024 + 4198.8 * 1024),
+        "bytes": int(1013617.6 * (608256 / 304146.9) * 1024 + 4198.9 * 1024),
         "measured_on": "born::nucleus_row_kernel<512, false>, workload C5 (what the L2s fetch, the Infinity Cache's share included)",
         "source": "profiles/nucleus_row_kernel_c5_counters.txt",
     },
@@ -258,15 +258,9 @@ def main():
         if rc:
             _capi.check(rc)
 
-    def timed(k, lead):
-        """ms per step over exactly k steps, between two events on the launch stream, a synchronisation on either side.
-        lead: one untimed step is launched behind the opening synchronisation and the opening event is recorded behind
-        it while it still runs, so the region starts when that step ends and holds k launch-to-launch steps. Without
-        it the region starts on an idle device and also holds the latency of the first launch (host and command
-        processor, 3 - 10 us depending on the box: up to 0.5 us per step of a 20-step region, none of it kernel time)."""
+    def timed(k):
+        """ms per step over exactly k steps, between two events on the launch stream, a synchronisation on either side."""
         torch.cuda.synchronize()
-        if lead:
-            step()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(k):
@@ -293,12 +287,11 @@ def main():
     # Measured first: a step is 27 us, so W = 5 warm-up steps are 0.14 ms, and a device that idled while the host prepared
     # the run needs a few ms of work to be back at its working clocks (measured: the first 25 steps after a pause run
     # 1 % slower than the next 20 at C3, 8 % at C5).
-    groups = sorted(timed(10, lead=True) for _ in range(30))
-    # W warm-up steps, the last of them the lead step of the timed region; then exactly K timed steps
-    for _ in range(max(0, args.warmup - 1)):
+    groups = sorted(timed(10) for _ in range(30))
+    # W untimed warm-up steps, then exactly K timed steps
+    for _ in range(args.warmup):
         step()
-    ms = timed(args.steps, lead=args.warmup >= 1)
-    ms_idle_start = timed(args.steps, lead=False)      # the same K steps started on an idle device, reported beside it
+    ms = timed(args.steps)
     spread = {"median": groups[len(groups) // 2], "p10": groups[len(groups) // 10], "p90": groups[(9 * len(groups)) // 10],
               "sample": "30 groups of 10 steps, ms per step, measured before the warm-up and the timed region"}
     smp.Status(stream)
@@ -313,9 +306,9 @@ def main():
     # read back above confirm it: rows settled by the single-pass kernel, by its exact selection, by the other two
     kernel_name = ("topk_row_kernel" if 1 <= w.top_k <= 128 else "nucleus_row_kernel" if w.top_k == 0 else "sample_wide_kernel") \
         if args.path == 0 else "sample_wide_kernel"
-    # (the checked call, the warm-up, the two timed regions, the 30 groups with their lead steps; the chained and the
-    # fused steps of the LM-head leg count too)
-    launches = 1 + max(args.warmup, 0) + 2 * args.steps + 330 + (0 if producer is None else 2 * (producer["iters"] + 1))
+    # (the checked call, the 30 groups, the warm-up, the timed region; the chained and the fused steps of the LM-head leg
+    # count too)
+    launches = 1 + 300 + args.warmup + args.steps + (0 if producer is None else 2 * (producer["iters"] + 1))
     if kernel_name == "topk_row_kernel":
         confirmed = counters["topk_rows"] + counters["fallback_rows"] == B * launches and counters["general_rows"] == 0
     else:
@@ -332,10 +325,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms,
-        "ms_per_step_timing": "HIP events on the launch stream around exactly K steps, a synchronisation on either side; the opening event is "
-                              "recorded behind the last warm-up step while it runs, so the region holds K launch-to-launch steps",
-        "ms_per_step_idle_start": ms_idle_start,
-        "ms_per_step_idle_start_note": "the same K steps with the opening event recorded on an idle device: adds the first launch's latency",
+        "ms_per_step_timing": "HIP events on the launch stream around exactly K steps, a synchronisation on either side, behind W warm-up steps; "
+                              "the 30 groups of ms_per_step_spread run before the warm-up, so the device is at its working clocks",
         "ms_per_step_spread": spread,
         "higher_is_better": True,
         "scaling": "weak",
@@ -476,12 +467,9 @@ def main_other(args, torch, S, synth, w, dev):
         step = lambda: smp.Verify(t, d, B, G, V, dt, ua, ur, na, nt, stream=stream)
         units, alg_bytes, kernel_name = B * G, 2 * B * G * V * 4 + 4 * B * G * 2 + 4 * B * 3, "spec_stats_kernel (+ residual, pick)"
         workload = f"C4: speculative verify, {B} sequences x {G} positions x vocab {V}, T={w.temperature}; \"tokens\" are verified draft positions"
-    # as for the headline configuration: the last warm-up step is the lead step of the timed region
-    for _ in range(max(0, args.warmup - 1)):
+    for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    if args.warmup >= 1:
-        step()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(args.steps):
