@@ -411,7 +411,7 @@ def main_extras(args, torch, S, synth, dev):
 
     if args.config == "C3x":
         base, minp, fp = mk(), mk(MinP=0.05), mk(FrequencyPenalty=0.3, PresencePenalty=0.5)
-        k100, k128, k129 = mk(top_k=100), mk(top_k=128), mk(top_k=129)
+        k100, k128, k129, k0 = mk(top_k=100), mk(top_k=128), mk(top_k=129), mk(top_k=0)
         Ts = torch.full((B,), w.temperature, device=dev)
         ks = torch.full((B,), w.top_k, dtype=torch.int32, device=dev)
         ps = torch.full((B,), w.top_p, device=dev)
@@ -421,6 +421,7 @@ def main_extras(args, torch, S, synth, dev):
             "C3 shape, top_k 100": lambda: k100.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 shape, top_k 128": lambda: k128.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 shape, top_k 129 (the general kernel)": lambda: k129.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 0 (top-p alone: the three-sweep kernel)": lambda: k0.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + min_p 0.05": lambda: minp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 with per-row arrays (same values in every row)":

@@ -426,16 +426,41 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     const bool cut = cfg_p < 1.0f;
     u64 tp = Zk;
     int w0, w1, w2;
+    bool unpredicted = false;                                        // the draw's bin could not be narrowed down to two
     if (cut) {
         tp = top_p_target(cfg_p, Zk);
         w0 = nuc_first_reaching(cum, tp);
         const u64 hi = cum[w0] < Zk ? cum[w0] : Zk;
         w1 = nuc_first_reaching(cum, draw_target(u, tp));
         w2 = nuc_first_reaching(cum, draw_target(u, hi));
-        if (w2 - w1 > 1) w1 = w2 = w0;
+        unpredicted = w2 - w1 > 1;
+        if (unpredicted) w1 = w2 = w0;
     } else {
         w0 = w1 = w2 = nuc_first_reaching(cum, draw_target(u, Zk));
     }
+    // Where that prediction gives up (a peaked row: the cut's bin holds so much of the mass that the draw may fall
+    // anywhere, and a draw outside the gathered bins costs further sweeps of the row), a small nucleus is gathered
+    // whole, every bin down to the cut's: the draw then needs no predicted bin.  A bin's mass over the smallest mass a
+    // logit in it can have bounds the number of its logits.
+    bool whole = false;
+    if (unpredicted && !r.degenerate && w0 < NUC_BINS - 1) {
+        const float per_bin = 1.44269504f / r.sbin;                  // bin b holds d < (b + 1) / sbin: masses above scale * 2^-((b + 1) * per_bin)
+        if (__builtin_amdgcn_exp2f(-(float)(w0 + 1) * per_bin) * r.scale >= 1024.0f) {   // (integer truncation is then below 0.1 %)
+            float bound = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NUC_PER; t++) {
+                const int b = tid * NUC_PER + t;
+                if (b <= w0) {
+                    const u64 mb = cum[b] - (b ? cum[b - 1] : 0ull);
+                    bound += (float)mb / (__builtin_amdgcn_exp2f(-(float)(b + 1) * per_bin) * r.scale * 0.98f);
+                }
+            }
+            // (summed in sixteenths, each thread's share rounded up)
+            const u32 total = block_sum_u32<NUC_BLOCK>((u32)fminf(ceilf(bound * 16.0f), 1048576.0f), &scr);
+            whole = total <= (u32)(16 * NUC_CAP / 2);                 // (half the capacity: the lists are per wave, the logits fall as they may)
+        }
+    }
+    if (whole) w1 = w2 = w0;
 
     BORN_STAMP(a, row, 4);
     // ---- sweep 3: stage the logits inside the wanted bins' ranges, then classify them exactly
@@ -444,6 +469,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         nuc_range(r, w0, lo0, hi0);
         nuc_range(r, w1, lo1, hi1);
         nuc_range(r, w2, lo2, hi2);
+        if (whole) hi0 = hi1 = hi2 = INFINITY;                       // every bin down to the cut's
         // The three value ranges as disjoint intervals in ascending order, overlapping ones merged (the draw's two bins
         // are neighbours, and often the cut's bin is one of them): most rows test one or two intervals per logit.
         // An unused interval is (+inf, -inf), which only a NaN passes (as it passes a real one: classified below).
@@ -499,7 +525,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 const float z = nuc_z(r, __uint_as_float(c.x));
                 const float d = nuc_d(r, z);
                 const int b = nuc_bin(r, d);
-                const int slot = b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+                const int slot = whole ? (b <= w0 ? 0 : -1) : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
                 if (slot >= 0) {
                     take = true;
                     key = make_key64(z, (int)c.y);
@@ -563,7 +589,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         const u64 target = phase == 0 ? tp : draw_target(u, Zp);
         const int b = phase == 0 ? w0 : nuc_first_reaching(cum, target);
         u64 base = b ? cum[b - 1] : 0ull;
-        const int slot = !listed ? -1 : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+        const int slot = !listed ? -1 : whole ? (b <= w0 ? 0 : -1) : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+        if (whole && slot == 0) base = 0ull;                         // the list starts at the row's maximum
         if (slot < 0) {
             u64 prefix = 0ull;
             int plen = 0;

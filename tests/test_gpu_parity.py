@@ -734,6 +734,33 @@ def test_three_sweep_kernel_seen_ids_visited_apart(oracle, rocm, V, H, scale, pa
         assert got["counters"]["general_rows"] == B
 
 
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
+@pytest.mark.parametrize("V,peaks,lift", [(4096, 3, 14.0), (32000, 20, 9.0), (50000, 200, 6.0), (128256, 20, 9.0), (20000, 700, 7.0)])
+def test_three_sweep_kernel_peaked_rows_gather_the_nucleus_whole(oracle, rocm, V, peaks, lift, path):
+    """Top-p alone on peaked rows (what a trained model emits): a few lifted logits carry nearly all of the mass, the
+    cut's bin holds so much of it that the draw's bin cannot be predicted, and the kernel gathers the whole nucleus
+    (every bin down to the cut's) when the bins' masses bound its size by half the list. From a handful of peaks to
+    more than the bound allows (the row then takes the older route), with and without penalties on the peaks
+    themselves: bit-exact against the oracle."""
+    rng = np.random.default_rng(V + peaks)
+    B = 12
+    x = (rng.standard_normal((B, V)) * 1.5).astype(np.float32)
+    hist = rng.integers(0, V, size=(B, 64)).astype(np.int32)
+    for b in range(B):
+        at = rng.choice(V, size=peaks, replace=False)
+        x[b, at] += rng.uniform(lift * 0.6, lift * 1.3, size=peaks).astype(np.float32)
+        hist[b, :8] = at[:8] if peaks >= 8 else np.resize(at, 8)     # some of the peaks are penalised
+    x[1, :] = x[1, 0]                                                  # a flat row among them
+    x[2, rng.choice(V, size=2, replace=False)] = 40.0                  # two equal maxima far above the rest
+    hl = np.full(B, hist.shape[1], dtype=np.int32)
+    u = rng.random(B, dtype=np.float32)
+    u[0] = np.float32(1.0) - np.float32(2.0 ** -24)
+    u[3] = 0.0
+    for (T, p, rep) in [(0.7, 0.9, 1.15), (1.0, 0.5, 1.0), (1.0, 0.99, 1.3), (1.4, 0.999, 1.0), (0.5, 0.2, 2.0)]:
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, 0, p, rep, hist, hl, path=path)
+        assert got["counters"]["general_rows"] == B
+
+
 def test_three_sweep_kernel_random_case_that_lost_staged_entries(oracle, rocm):
     # the case a wide seeded sweep of test_random_row_layouts_against_oracle found (its chunk 1096, third case)
     import test_gpu_parity_random as R
