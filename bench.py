@@ -55,7 +55,7 @@ PMC_TRAFFIC = {
     },
     # (the probe of that run copied a C5 logits buffer: 608 256 KiB read and written)
     ("C5", "nucleus_row_kernel"): {
-        "bytes": int(1013617.6 * (608256 / 304146.9) * 1024 + 4198.9 * 1024),
+        "bytes": int(1015062.7 * (608256 / 304146.8) * 1024 + 6246.5 * 1024),
         "measured_on": "born::nucleus_row_kernel<512, false>, workload C5 (what the L2s fetch, the Infinity Cache's share included)",
         "source": "profiles/nucleus_row_kernel_c5_counters.txt",
     },
