@@ -201,7 +201,7 @@ def test_large_vocabularies_against_oracle(oracle, rocm, V):
 def test_wide_seeded_sweep_on_request(oracle, rocm):
     """The sweep above with as many further seeded chunks as BORN_SWEEP_CHUNKS asks for (skipped when unset), weighted
     towards the kernel without a top-k cut: temperatures the division shortcut takes and refuses, histories up to 5000
-    tokens, draws from the very end of the rank order, logits of unusual magnitude; all three kernel selections.
+    tokens, draws from the very end of the rank order, logits of unusual magnitude, peaked rows; all three kernel selections.
     BORN_SWEEP_SEED moves the seeds.  (About 140 cases a second; a run of 150 000 cases found nothing in the kernels
     and one tolerance of these tests.)"""
     import os
@@ -227,6 +227,11 @@ def test_wide_seeded_sweep_on_request(oracle, rocm):
             if rng.random() < 0.2 and x.size > 8:
                 at = rng.integers(0, x.size, size=8)
                 x.reshape(-1)[at] = rng.choice(odd, size=8)
+            if rng.random() < 0.3 and x.shape[1] > 64:
+                # peaked rows: a few lifted logits carry the mass (the kernel without a top-k cut gathers such a nucleus whole)
+                for b in range(x.shape[0]):
+                    peaks = int(rng.integers(1, 40))
+                    x[b, rng.choice(x.shape[1], size=peaks, replace=False)] += rng.uniform(4.0, 14.0, size=peaks).astype(np.float32)
             for path in (0, 2, 1):
                 try:
                     _check_against_oracle(oracle, rocm, x, u, c["T"], c["k"], c["p"], c["rep"], hist, hist_len, path=path,
