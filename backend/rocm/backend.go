@@ -26,7 +26,7 @@ type Tensor struct {
 
 // Device is the value a device-aware tensor.Device enum would carry for this backend; the reference's enum
 // (internal/tensor/raw.go:14-20: CPU, CUDA, Vulkan, Metal, WebGPU) has no ROCm member, so the package defines its own
-// until one is added there (INTEGRATION.md shows the one-line change).
+// until one is added there (one more constant after WebGPU in that enum, and a case in its String method).
 type Device int
 
 // ROCm is the only device of this backend.
