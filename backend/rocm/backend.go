@@ -121,6 +121,10 @@ func (b *Backend) binary(op string, fn binaryFn, x, y *Tensor) *Tensor {
 	if err != nil {
 		panic(fmt.Sprintf("%s: failed to create result tensor: %v", op, err))
 	}
+	// The operands stay reachable until the launch is enqueued: their last Go use is the read of Buf.ptr above, and a
+	// tensor whose finalizer ran in between would have its device memory freed under the kernel.
+	defer runtime.KeepAlive(x)
+	defer runtime.KeepAlive(y)
 	if err := call(func() C.int {
 		return fn((*C.float)(x.Buf.ptr), xs, xn, (*C.float)(y.Buf.ptr), ys, yn, (*C.float)(res.Buf.ptr), nil)
 	}); err != nil {
@@ -170,6 +174,8 @@ func (b *Backend) MatMul(x, y *Tensor) *Tensor {
 	if err != nil {
 		panic(fmt.Sprintf("matmul: failed to create result tensor: %v", err))
 	}
+	defer runtime.KeepAlive(x) // (see binary: operands must outlive the enqueue)
+	defer runtime.KeepAlive(y)
 	if err := MatMul(x.Buf, x.Shape, y.Buf, y.Shape, res.Buf, nil); err != nil {
 		panic(fmt.Sprintf("matmul: %v", err))
 	}
@@ -198,6 +204,8 @@ func (b *Backend) Conv2D(input, kernel *Tensor, stride, padding int) *Tensor {
 	}
 	is, _ := cShape(input.Shape)
 	ks, _ := cShape(kernel.Shape)
+	defer runtime.KeepAlive(input)
+	defer runtime.KeepAlive(kernel)
 	// call() panics with the library's "conv2d: input channels ... != kernel channels ..."
 	if err := call(func() C.int { return C.born_rocm_conv2d((*C.float)(input.Buf.ptr), is, (*C.float)(kernel.Buf.ptr), ks, C.int32_t(stride),
 		C.int32_t(padding), (*C.float)(res.Buf.ptr), nil, nil) }); err != nil {
@@ -226,6 +234,7 @@ func (b *Backend) MaxPool2D(input *Tensor, kernelSize, stride int) *Tensor {
 		panic(fmt.Sprintf("maxpool2d: failed to create output: %v", err))
 	}
 	is, _ := cShape(input.Shape)
+	defer runtime.KeepAlive(input)
 	if err := call(func() C.int { return C.born_rocm_maxpool2d((*C.float)(input.Buf.ptr), is, C.int32_t(kernelSize), C.int32_t(stride),
 		(*C.float)(res.Buf.ptr), nil, nil) }); err != nil {
 		panic(fmt.Sprintf("maxpool2d: %v", err))
@@ -235,12 +244,23 @@ func (b *Backend) MaxPool2D(input *Tensor, kernelSize, stride int) *Tensor {
 
 // Reshape returns a tensor with the same data but a different shape (a copy, as in the reference).
 func (b *Backend) Reshape(t *Tensor, newShape []int) *Tensor {
+	// validated before anything is allocated, in the reference's order and words (internal/backend/cpu/backend.go:137-146,
+	// Shape.Validate internal/tensor/shape.go:21-28): every extent positive, then the element counts equal
+	for i, d := range newShape {
+		if d <= 0 {
+			panic(fmt.Sprintf("reshape: invalid shape: invalid dimension at index %d: %d (must be > 0)", i, d))
+		}
+	}
+	if numElements(newShape) != numElements(t.Shape) {
+		panic(fmt.Sprintf("reshape: incompatible shapes: %v -> %v (different number of elements)", t.Shape, newShape))
+	}
 	res, err := NewTensor(newShape)
 	if err != nil {
 		panic(fmt.Sprintf("reshape: %v", err))
 	}
 	ts, tn := cShape(t.Shape)
 	ns, nn := cShape(newShape)
+	defer runtime.KeepAlive(t)
 	if err := call(func() C.int { return C.born_rocm_reshape((*C.float)(t.Buf.ptr), ts, tn, ns, nn, (*C.float)(res.Buf.ptr), nil) }); err != nil {
 		panic(fmt.Sprintf("reshape: %v", err))
 	}
@@ -274,6 +294,7 @@ func (b *Backend) Transpose(t *Tensor, axes ...int) *Tensor {
 		panic(fmt.Sprintf("transpose: %v", err))
 	}
 	ts, tn := cShape(t.Shape)
+	defer runtime.KeepAlive(t)
 	// call() panics with the library's "transpose: invalid axis ..." / "transpose: duplicate axis ..."
 	if err := call(func() C.int { return C.born_rocm_transpose((*C.float)(t.Buf.ptr), ts, tn, &cax[0], (*C.float)(res.Buf.ptr), nil) }); err != nil {
 		panic(fmt.Sprintf("transpose: %v", err))

@@ -1,3 +1,3 @@
 module github.com/born-ml/born/backend/rocm
 
-go 1.23
+go 1.25

@@ -11,6 +11,7 @@ import (
 	"fmt"
 	"math"
 	"math/rand"
+	"runtime"
 	"unsafe"
 )
 
@@ -102,6 +103,7 @@ func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]i
 		panic(fmt.Sprintf("Linear.Forward: expected input with %d features, got %d", l.inFeatures, shape[1]))
 	}
 	batch := shape[0]
+	defer runtime.KeepAlive(s)
 	out, err := Alloc(int64(4 * batch))
 	if err != nil {
 		return nil, err
@@ -123,7 +125,9 @@ func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]i
 // s.Sample draws from Forward(input)[b], and the [batch, out_features] logits are never written.  The sampler's
 // configuration must be one the single-pass kernel serves (1 <= TopK <= 128, RepetitionPenalty >= 1, no frequency or
 // presence penalty).  A row the fused step cannot settle comes back as -1; the whole call is then repeated over
-// materialised logits (Forward + Sample), so the caller always gets the tokens of the unfused pair.
+// materialised logits (Forward + Sample) with the draw counter of the built-in uniform stream set back to its value
+// before the fused call, so the caller always gets the tokens of the unfused pair and a seeded run consumes one
+// step per call either way.
 func (l *Linear) ForwardSample(s *Sampler, input DeviceBuffer, shape []int, history DeviceBuffer, histStride int,
 	histLen, uniforms DeviceBuffer) ([]int32, error) {
 	if len(shape) != 2 {
@@ -133,7 +137,9 @@ func (l *Linear) ForwardSample(s *Sampler, input DeviceBuffer, shape []int, hist
 		panic(fmt.Sprintf("Linear.Forward: expected input with %d features, got %d", l.inFeatures, shape[1]))
 	}
 	batch := shape[0]
+	defer runtime.KeepAlive(s)
 	out := s.results(batch)
+	step := s.Step() // the draws this call consumes when uniforms is the built-in stream
 	if err := call(func() C.int {
 		return C.born_rocm_linear_sample(s.h, (*C.float)(input.ptr), C.int64_t(batch), C.int64_t(l.inFeatures),
 			C.int64_t(l.inFeatures), (*C.float)(l.weight.ptr), C.int64_t(l.outFeatures), C.int64_t(l.inFeatures),
@@ -166,6 +172,9 @@ func (l *Linear) ForwardSample(s *Sampler, input DeviceBuffer, shape []int, hist
 	if err := l.Forward(input, shape, logits, nil); err != nil {
 		return nil, err
 	}
+	// the fused call advanced the draw counter although a row did not settle: set it back, so that Sample draws the same
+	// uniforms and the generation consumes one step whether or not this fallback ran
+	s.SetStep(step)
 	return s.Sample(logits, batch, l.outFeatures, history, histStride, histLen, uniforms)
 }
 

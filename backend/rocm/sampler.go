@@ -146,6 +146,23 @@ func (s *Sampler) Close() {
 	}
 }
 
+// Step returns the draw counter of the built-in uniform stream: a call that is given no uniforms draws row b's uniform
+// from (Seed, step, b) and advances the counter by one.  SetStep sets it, so that a call can be repeated with the
+// same draws (Linear.ForwardSample's fallback does).
+func (s *Sampler) Step() int64 {
+	var v C.int64_t
+	if err := call(func() C.int { return C.born_rocm_sampler_get_step(s.h, &v) }); err != nil {
+		panic("sampler: " + err.Error())
+	}
+	return int64(v)
+}
+
+func (s *Sampler) SetStep(step int64) {
+	if err := call(func() C.int { return C.born_rocm_sampler_set_step(s.h, C.int64_t(step)) }); err != nil {
+		panic("sampler: " + err.Error())
+	}
+}
+
 // results returns the handle's own device buffer for the int32 results of a step (no allocation per call: an
 // allocation synchronises the device, which a decode loop cannot afford).
 func (s *Sampler) results(batch int) DeviceBuffer {
@@ -195,6 +212,7 @@ func (s *Sampler) Sample(logits DeviceBuffer, batch, vocab int, history DeviceBu
 	if batch <= 0 || vocab <= 0 {
 		panic("sampler: Sample: batch and vocab must be > 0")
 	}
+	defer runtime.KeepAlive(s) // the finalizer frees the handle and `out`: s stays reachable until the results are read
 	out := s.results(batch)
 	if err = call(func() C.int { return C.born_rocm_sample(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
 		(*C.int32_t)(history.ptr), (*C.int32_t)(histLen.ptr), C.int64_t(histStride), (*C.float)(uniforms.ptr),
@@ -210,6 +228,7 @@ func (s *Sampler) Sample(logits DeviceBuffer, batch, vocab int, history DeviceBu
 
 // Argmax is the greedy decode: reference argmax per row (internal/nn/cross_entropy.go:241-251).
 func (s *Sampler) Argmax(logits DeviceBuffer, batch, vocab int) ([]int32, error) {
+	defer runtime.KeepAlive(s)
 	out := s.results(batch)
 	if err := call(func() C.int { return C.born_rocm_argmax(s.h, (*C.float)(logits.ptr), C.int64_t(batch), C.int64_t(vocab), C.int64_t(vocab),
 		(*C.int32_t)(out.ptr), nil) }); err != nil {
@@ -224,6 +243,7 @@ func (s *Sampler) Argmax(logits DeviceBuffer, batch, vocab int) ([]int32, error)
 // token of sequence b was accepted.
 func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
 	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
+	defer runtime.KeepAlive(s)
 	out := s.results(batch)
 	na := (*C.int32_t)(out.ptr)
 	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
@@ -244,6 +264,7 @@ func (s *Sampler) Verify(target, draft DeviceBuffer, batch, gamma, vocab int, dr
 // token from it (nextToken is never -1).
 func (s *Sampler) VerifyBonus(target, draft DeviceBuffer, batch, gamma, vocab int, draftTokens, uAccept,
 	uResidual DeviceBuffer) (nAccepted, nextToken []int32, err error) {
+	defer runtime.KeepAlive(s)
 	out := s.results(batch)
 	na := (*C.int32_t)(out.ptr)
 	nt := (*C.int32_t)(unsafe.Add(out.ptr, 4*batch))
@@ -282,6 +303,7 @@ const (
 // from the status check that follows the copy of the tokens.
 func (s *Sampler) SampleRows(logits DeviceBuffer, batch, vocab int, history DeviceBuffer, histStride int,
 	histLen, uniforms DeviceBuffer, rows RowConfigs) ([]int32, error) {
+	defer runtime.KeepAlive(s)
 	out := s.results(batch)
 	var err error
 	// the struct holds device addresses only (C memory as far as cgo's pointer rules are concerned)

@@ -44,6 +44,8 @@ SYMBOLS = {
     "born_rocm_sampler_get_config": (C.c_int, [_vp, C.POINTER(SamplerConfigC)]),
     "born_rocm_sampler_set_config": (C.c_int, [_vp, C.POINTER(SamplerConfigC)]),
     "born_rocm_sampler_set_path": (C.c_int, [_vp, C.c_int32]),
+    "born_rocm_sampler_get_step": (C.c_int, [_vp, C.POINTER(_i64)]),
+    "born_rocm_sampler_set_step": (C.c_int, [_vp, _i64]),
     "born_rocm_sampler_status": (C.c_int, [_vp, _vp]),
     "born_rocm_sampler_counters": (C.c_int, [_vp, _vp, C.POINTER(_i64), C.POINTER(_i64), C.POINTER(_i64)]),
     "born_rocm_argmax": (C.c_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),

@@ -234,6 +234,18 @@ int born_rocm_sampler_set_path(born_sampler *s, int32_t path) {
     return BORN_ROCM_OK;
 }
 
+int born_rocm_sampler_get_step(const born_sampler *s, int64_t *step_out) {
+    if (!s || !step_out) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: get_step: null argument");
+    *step_out = (int64_t)s->step;
+    return BORN_ROCM_OK;
+}
+int born_rocm_sampler_set_step(born_sampler *s, int64_t step) {
+    if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_step: null handle");
+    if (step < 0) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: set_step: step must be >= 0, got %lld", (long long)step);
+    s->step = (unsigned long long)step;
+    return BORN_ROCM_OK;
+}
+
 int born_rocm_sampler_status(born_sampler *s, void *stream) {
     if (!s) return fail(BORN_ROCM_ERR_ARGUMENT, "sampler: status: null handle");
     int st = 0;
@@ -807,11 +819,26 @@ int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int6
         HIP_TRY(hipStreamIsCapturing(st, &capturing));
         if (capturing != hipStreamCaptureStatusNone)
             return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: the first call on a handle allocates its workspace; make it outside a stream capture");
+        // all four buffers or none: a failure part of the way frees what it got, so that the next call starts over
+        // without leaking (the handle's pointers are set only once every allocation has succeeded)
         const size_t rows = (size_t)s->max_batch;
-        HIP_TRY(hipMalloc((void **)&s->lm_samp, rows * LM_SAMPLE_MAX * sizeof(float)));
-        HIP_TRY(hipMalloc((void **)&s->lm_thr, rows * sizeof(float)));
-        HIP_TRY(hipMalloc((void **)&s->lm_cnt, rows * LM_CAND_PITCH * sizeof(unsigned)));
-        HIP_TRY(hipMalloc((void **)&s->lm_cand, rows * LM_CAND_CAP * sizeof(uint2)));
+        const size_t bytes[4] = {rows * LM_SAMPLE_MAX * sizeof(float), rows * sizeof(float), rows * LM_CAND_PITCH * sizeof(unsigned),
+                                 rows * LM_CAND_CAP * sizeof(uint2)};
+        void *got[4] = {nullptr, nullptr, nullptr, nullptr};
+        hipError_t e = hipSuccess;
+        for (int i = 0; i < 4 && e == hipSuccess; i++) {
+            e = hipMalloc(&got[i], bytes[i]);
+            if (e == hipSuccess) e = hipMemset(got[i], 0, bytes[i]);
+        }
+        if (e != hipSuccess) {
+            for (void *p : got)
+                if (p) (void)hipFree(p);
+            return hip_fail(e, "linear_sample: workspace allocation");
+        }
+        s->lm_samp = (float *)got[0];
+        s->lm_thr = (float *)got[1];
+        s->lm_cnt = (unsigned *)got[2];
+        s->lm_cand = (uint2 *)got[3];
     }
     // 1. the product over every sstep-th weight row (no bias: the threshold kernel adds it)
     const int64_t sstep = (out_features + LM_SAMPLE_MAX - 1) / LM_SAMPLE_MAX;

@@ -101,10 +101,12 @@ def ForwardSample(sampler, layer, input, input_shape, history, histLen, uniforms
 
 def ForwardSampleHost(sampler, layer, input, input_shape, history, histLen, uniforms, hist_stride=0):
     """ForwardSample with the tokens and probabilities copied back, and the fallback a caller owes the rows the fused
-    step could not settle: the whole call is repeated as Forward + Sample over materialised logits.  Returns
-    (tokens, probs, fell_back)."""
+    step could not settle: the whole call is repeated as Forward + Sample over materialised logits, with the draw
+    counter of the built-in uniform stream set back first, so that the tokens are those of the unfused pair whether
+    or not the fallback ran.  Returns (tokens, probs, fell_back)."""
     batch = int(input_shape[0])
     tok, pr = DeviceBuffer(4 * batch), DeviceBuffer(4 * batch)
+    step = sampler.Step()                                            # the draws this call consumes (built-in stream)
     ForwardSample(sampler, layer, input, input_shape, history, histLen, uniforms, tok, pr, hist_stride)
     tokens = tok.to_numpy(np.int32, (batch,))
     fell_back = bool((tokens < 0).any())
@@ -116,6 +118,7 @@ def ForwardSampleHost(sampler, layer, input, input_shape, history, histLen, unif
                 raise
         logits = DeviceBuffer(4 * batch * layer.outFeatures)
         layer.Forward(input, input_shape, logits)
+        sampler.SetStep(step)                                        # the same uniforms again: one step consumed either way
         sampler.Sample(logits, batch, layer.outFeatures, history, histLen, uniforms, tok, pr, hist_stride=hist_stride)
         tokens = tok.to_numpy(np.int32, (batch,))
     return tokens, pr.to_numpy(np.float32, (batch,)), fell_back

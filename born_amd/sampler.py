@@ -163,6 +163,15 @@ class Sampler:
         the kernel for TopK 0 whatever the batch (by default: for batches of more rows than the device has CUs)."""
         _check(_capi.lib().born_rocm_sampler_set_path(self._h, int(path)))
 
+    def Step(self):
+        """The draw counter of the built-in uniform stream (calls without `uniforms` advance it by one)."""
+        v = C.c_int64()
+        _check(_capi.lib().born_rocm_sampler_get_step(self._h, C.byref(v)))
+        return v.value
+
+    def SetStep(self, step):
+        _check(_capi.lib().born_rocm_sampler_set_step(self._h, int(step)))
+
     def Status(self, stream=None):
         """Raises BornRocmError(ERR_DATA) if a kernel met an out-of-range history id / draft token."""
         _check(_capi.lib().born_rocm_sampler_status(self._h, stream))

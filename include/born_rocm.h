@@ -96,6 +96,17 @@ int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows
  * All implement the same fixed-point pipeline and must return identical results; tests compare them. */
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
 
+/* The draw counter of the built-in uniform stream: a call that is given no `uniforms` draws row b's uniform from
+ * (cfg.seed, step, b) and then advances `step` by one (born_rocm_sample, born_rocm_sample_rows,
+ * born_rocm_linear_sample; calls that are given uniforms leave it alone).  Reading and setting it lets a caller
+ * repeat a call with the same draws: the fallback after born_rocm_linear_sample reports an unsettled row sets the
+ * counter back to what it was before that call, so that born_rocm_linear + born_rocm_sample draw the very uniforms
+ * the fused call used and the generation consumes one step either way.  Host state only: nothing is enqueued.  No
+ * counterpart in the reference snapshot (its only generator is the process-global unseeded one,
+ * internal/tensor/creation.go:92-93). */
+int born_rocm_sampler_get_step(const born_sampler *s, int64_t *step_out);
+int born_rocm_sampler_set_step(born_sampler *s, int64_t step);
+
 /* Greedy decode: index of the maximum of each row, lowest index on ties — `argmax`,
  * internal/nn/cross_entropy.go:241-251 (the per-row step of nn.Accuracy, :261-284). */
 int born_rocm_argmax(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
@@ -117,6 +128,9 @@ int born_rocm_log_softmax(born_sampler *s, const float *logits, int64_t batch, i
  *   uniforms  fp32 [batch] in [0,1) or NULL (=> built-in stream from cfg.seed and the handle's draw counter)
  *   tokens_out int32 [batch]; probs_out fp32 [batch] or NULL (probability of the sampled token in the
  *   renormalised nucleus)
+ *   The logits buffer must span batch * row_stride elements (the last row included): rows that start 16-byte aligned
+ *   with a row_stride that is a multiple of 4 are read in whole 128-bit blocks, so up to 3 floats past `vocab`
+ *   (inside the row's pitch) are loaded and ignored when vocab is not a multiple of 4.
  *   nucleus outputs (all three NULL, or all three set with nucleus_cap > 0): the first
  *   min(n, nucleus_cap) survivors of each row in rank order; produced when 1 <= top_k <= 4096
  *   (nucleus_len_out[b] = -1 otherwise). */
@@ -266,8 +280,11 @@ int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int6
  * it (value and column); the sampling step runs over the list and proves that nothing outside it can belong to the
  * row's top_k.  A row it cannot settle (a list of more than 4096, fewer than top_k candidates above the bound, a
  * history of more than 1024 tokens with a penalty) gets token -1 and born_rocm_sampler_status returns
- * BORN_ROCM_ERR_DATA: the caller then runs born_rocm_linear + born_rocm_sample for that call.  The first call on a
- * handle allocates about 36 KiB of workspace per row of max_batch (outside a stream capture). */
+ * BORN_ROCM_ERR_DATA: the caller then runs born_rocm_linear + born_rocm_sample for that call.  With uniforms == NULL
+ * the fused call has advanced the handle's draw counter whether or not every row settled: a caller that falls back
+ * first sets the counter to its value before the fused call (born_rocm_sampler_get_step / _set_step), so that the
+ * unfused pair draws the same uniforms and the tokens stay those of a run that never used the fused call.  The first
+ * call on a handle allocates about 36 KiB of workspace per row of max_batch (outside a stream capture). */
 int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
                             const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
                             const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,

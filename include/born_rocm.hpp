@@ -73,6 +73,15 @@ public:
         return tokens;
     }
 
+    // The draw counter of the built-in uniform stream (a call without uniforms advances it by one).  Setting it back to
+    // its value before a call repeats that call's draws: what the fallback after an unsettled Linear::ForwardSample does.
+    int64_t Step() const {
+        int64_t v = 0;
+        check(born_rocm_sampler_get_step(h_, &v));
+        return v;
+    }
+    void SetStep(int64_t step) { check(born_rocm_sampler_set_step(h_, step)); }
+
     // The same step for callers that cannot allocate (born_rocm_sample_static): no handle, every buffer the caller's,
     // at most 4096 rows; `status_dev` (optional) is an int32 device word the status bits are OR-ed into.
     static void SampleStatic(const SamplerConfig &cfg, const float *logits_dev, int64_t batch, int64_t vocab,
@@ -187,7 +196,8 @@ public:
     }
     // The layer and the sampling step in one call (born_rocm_linear_sample): tokens_dev[b] is what the sampler draws
     // from Forward(input)[b], the logits never written; a row the fused step cannot settle gets token -1 (the caller
-    // then runs Forward + Sampler::Sample for the call).
+    // then runs Forward + Sampler::Sample for the call, after sampler.SetStep(the value of sampler.Step() before this
+    // call) when the built-in uniform stream is in use, so that both draw the same uniforms).
     void ForwardSample(const Sampler &sampler, const float *input_dev, int64_t batch, int64_t features, const int32_t *history_dev,
                        int64_t hist_stride, const int32_t *hist_len_dev, const float *uniforms_dev, int32_t *tokens_dev,
                        float *probs_dev = nullptr, void *stream = nullptr) const {

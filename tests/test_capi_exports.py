@@ -37,6 +37,8 @@ def test_argument_checks_need_no_gpu():
     assert L.born_rocm_sampler_create(None, 0, 10, None) == _capi.ERR_ARGUMENT
     assert b"null output" in L.born_rocm_last_error()
     assert L.born_rocm_sampler_set_path(None, 0) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_sampler_set_step(None, 0) == _capi.ERR_ARGUMENT
+    assert L.born_rocm_sampler_get_step(None, None) == _capi.ERR_ARGUMENT
     assert L.born_rocm_expneg(None, None, 0, None) == _capi.ERR_ARGUMENT
     assert L.born_rocm_sampler_destroy(None) == _capi.OK
 

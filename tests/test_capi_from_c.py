@@ -51,6 +51,8 @@ int main(void) {
     EXPECT(born_rocm_sample(0, x, 1, 4, 4, 0, 0, 0, u, tok, 0, 0, 0, 0, 0, 0) == BORN_ROCM_ERR_ARGUMENT);
     EXPECT(born_rocm_argmax(0, x, 1, 4, 4, tok, 0) == BORN_ROCM_ERR_ARGUMENT);
     EXPECT(born_rocm_sampler_set_path(0, 0) == BORN_ROCM_ERR_ARGUMENT);
+    EXPECT(born_rocm_sampler_set_step(0, 0) == BORN_ROCM_ERR_ARGUMENT);
+    EXPECT(born_rocm_sampler_get_step(0, 0) == BORN_ROCM_ERR_ARGUMENT);
     EXPECT(born_rocm_sampler_destroy(0) == BORN_ROCM_OK);
     EXPECT(born_rocm_exp(0, 0, 4, 0) == BORN_ROCM_ERR_ARGUMENT);
     EXPECT(born_rocm_exp(x, x, -1, 0) == BORN_ROCM_ERR_ARGUMENT);

@@ -419,6 +419,41 @@ def test_lm_head_sampling_fused_penalised_favourites_and_unsettled_rows(rocm, li
     assert not settled.any()
 
 
+def test_lm_head_sampling_fused_built_in_stream_survives_a_fallback(rocm, lin):
+    """With the built-in uniform stream (uniforms = None) a seeded generation must not depend on whether a fused call
+    fell back: the wrapper sets the draw counter back before it repeats the call unfused, so that call and every later
+    one draw what a twin handle that never used the fused call draws."""
+    M, K, N = 6, 128, 6000
+    rng = np.random.default_rng(4242)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * (2.0 / np.sqrt(K))).astype(np.float32)
+    cfg = rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.3, Seed=777)
+    dw = rocm.DeviceBuffer.from_numpy(w)
+    layer = lin.Linear(K, N, dw, None)
+    fused = rocm.NewSampler(cfg, max_batch=M, max_vocab=N)
+    twin = rocm.NewSampler(cfg, max_batch=M, max_vocab=N)
+    long_hist = rocm.DeviceBuffer.from_numpy(rng.integers(0, N, size=(M, 1500)).astype(np.int32))   # no row can settle
+    short_hist = rocm.DeviceBuffer.from_numpy(rng.integers(0, N, size=(M, 40)).astype(np.int32))
+    dx = rocm.DeviceBuffer.from_numpy(x)
+    logits = rocm.DeviceBuffer(4 * M * N)
+    layer.Forward(dx, (M, K), logits)
+    tok = rocm.DeviceBuffer(4 * M)
+    fell = []
+    for step, (hist, H) in enumerate([(short_hist, 40), (long_hist, 1500), (short_hist, 40), (long_hist, 1500), (short_hist, 40)]):
+        assert fused.Step() == step == twin.Step()
+        got, _, fell_back = lin.ForwardSampleHost(fused, layer, dx, (M, K), hist, None, None, hist_stride=H)
+        fell.append(fell_back)
+        twin.Sample(logits, M, N, hist, None, None, tok, None, hist_stride=H)
+        want = tok.to_numpy(np.int32, (M,))
+        assert np.array_equal(got, want), (step, got, want)
+    assert fell == [False, True, False, True, False]
+    assert fused.Step() == 5 == twin.Step()
+    with pytest.raises(rocm.SamplerPanic):
+        fused.SetStep(-1)
+    fused.Close()
+    twin.Close()
+
+
 def test_lm_head_sampling_fused_argument_errors(rocm, lin):
     from born_amd import _capi
     M, K, N = 4, 64, 500

@@ -99,3 +99,62 @@ def test_static_entry_point_limits(rocm):
     with pytest.raises(_capi.BornRocmError) as e:                            # counting a 5000-token history needs the table
         S.SampleStatic(S.SamplerConfig(TopK=5, FrequencyPenalty=0.5), dx, 2, 1000, h, None, du, tok, hist_stride=5000)
     assert e.value.code == _capi.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("cfg_kw", [
+    dict(Temperature=0.7, TopK=50, TopP=0.9, RepetitionPenalty=1.15),                       # the single-pass kernel
+    dict(Temperature=1.2, TopP=0.95, RepetitionPenalty=1.05),                               # the three-sweep kernel
+    dict(Temperature=0.9, TopK=300, TopP=0.9),                                              # the general kernel
+])
+def test_static_entry_point_allocates_nothing_and_can_be_captured(rocm, cfg_kw):
+    """The property the entry point exists for.  (a) The device's free memory (hipMemGetInfo, read through torch) is the
+    same before and after two calls.  (b) A call is recorded into a HIP graph after one warm call: an allocation, a free
+    or a synchronisation inside the capture would invalidate it.  The graph is then replayed three times, with eager
+    work (new uniforms uploaded, the handle-based call, synchronisations) between the replays, and every replay must
+    equal the eager handle-based result for the uniforms it saw."""
+    import torch
+    S = rocm
+    cfg = S.SamplerConfig(**cfg_kw)
+    B, V, H = 40, 12000, 64
+    x, u, h = _rows(11, B, V, H)
+    dev = torch.device("cuda:0")
+    tx, th = torch.from_numpy(x).to(dev), torch.from_numpy(h).to(dev)
+    tu = torch.from_numpy(u).to(dev)
+    tok_s = torch.full((B,), -7, dtype=torch.int32, device=dev)
+    pr_s = torch.zeros(B, device=dev)
+    tok_h = torch.empty(B, dtype=torch.int32, device=dev)
+    pr_h = torch.empty(B, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    smp = S.NewSampler(cfg, max_batch=B, max_vocab=V)
+    cur = lambda: torch.cuda.current_stream().cuda_stream
+
+    def static_call():
+        S.SampleStatic(cfg, tx, B, V, th, None, tu, tok_s, pr_s, status_out=status, hist_stride=H, stream=cur())
+
+    static_call()                                                            # the warm call: looks up the array's address
+    torch.cuda.synchronize()
+    # (a) nothing allocated, nothing freed
+    free_before = torch.cuda.mem_get_info()[0]
+    static_call()
+    static_call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    # (b) under stream capture
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=side):
+        static_call()
+    rng = np.random.default_rng(5)
+    for replay in range(3):
+        u_new = rng.random(B, dtype=np.float32)
+        tu.copy_(torch.from_numpy(u_new))                                    # eager work between the replays
+        tok_s.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        smp.Sample(tx, B, V, th, None, tu, tok_h, pr_h, hist_stride=H, stream=cur())
+        torch.cuda.synchronize()
+        assert torch.equal(tok_s, tok_h), (replay, (tok_s != tok_h).nonzero().flatten()[:8].tolist())
+        assert torch.equal(pr_s.view(torch.int32), pr_h.view(torch.int32)), replay
+    assert int(status.item()) == 0
+    smp.Close()
