@@ -101,60 +101,91 @@ def test_static_entry_point_limits(rocm):
     assert e.value.code == _capi.ERR_UNSUPPORTED
 
 
+def _hip():
+    """The HIP runtime the library itself is linked against (already mapped into this process), through ctypes."""
+    import ctypes as C
+    _capi.lib()
+    with open("/proc/self/maps") as f:
+        paths = sorted({line.split()[-1] for line in f if "libamdhip64" in line})
+    assert paths, "the HIP runtime is not mapped"
+    hip = C.CDLL(paths[0])
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    return hip
+
+
 @pytest.mark.parametrize("cfg_kw", [
     dict(Temperature=0.7, TopK=50, TopP=0.9, RepetitionPenalty=1.15),                       # the single-pass kernel
     dict(Temperature=1.2, TopP=0.95, RepetitionPenalty=1.05),                               # the three-sweep kernel
-    dict(Temperature=0.9, TopK=300, TopP=0.9),                                              # the general kernel
+    dict(Temperature=0.9, TopK=600, TopP=0.9),                                              # the general kernel
 ])
 def test_static_entry_point_allocates_nothing_and_can_be_captured(rocm, cfg_kw):
-    """The property the entry point exists for.  (a) The device's free memory (hipMemGetInfo, read through torch) is the
-    same before and after two calls.  (b) A call is recorded into a HIP graph after one warm call: an allocation, a free
-    or a synchronisation inside the capture would invalidate it.  The graph is then replayed three times, with eager
-    work (new uniforms uploaded, the handle-based call, synchronisations) between the replays, and every replay must
-    equal the eager handle-based result for the uniforms it saw."""
-    import torch
+    """The property the entry point exists for.  (a) The device's free memory (hipMemGetInfo) is the same before and
+    after two calls.  (b) After one warm call, a call is recorded into a HIP graph: an allocation, a free or a
+    synchronisation inside the capture would invalidate it.  The graph is then replayed three times, with eager work
+    (new uniforms uploaded, the handle-based call, synchronisations) between the replays, and every replay must equal
+    the eager handle-based result for the uniforms it saw."""
+    import ctypes as C
     S = rocm
+    hip = _hip()
     cfg = S.SamplerConfig(**cfg_kw)
     B, V, H = 40, 12000, 64
     x, u, h = _rows(11, B, V, H)
-    dev = torch.device("cuda:0")
-    tx, th = torch.from_numpy(x).to(dev), torch.from_numpy(h).to(dev)
-    tu = torch.from_numpy(u).to(dev)
-    tok_s = torch.full((B,), -7, dtype=torch.int32, device=dev)
-    pr_s = torch.zeros(B, device=dev)
-    tok_h = torch.empty(B, dtype=torch.int32, device=dev)
-    pr_h = torch.empty(B, device=dev)
-    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    dx, dh, du = S.DeviceBuffer.from_numpy(x), S.DeviceBuffer.from_numpy(h), S.DeviceBuffer.from_numpy(u)
+    tok_s, pr_s, tok_h, pr_h = (S.DeviceBuffer(4 * B) for _ in range(4))
+    status = S.DeviceBuffer.from_numpy(np.zeros(1, np.int32))
     smp = S.NewSampler(cfg, max_batch=B, max_vocab=V)
-    cur = lambda: torch.cuda.current_stream().cuda_stream
+    stream = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(stream)) == 0                         # (default priority)
 
-    def static_call():
-        S.SampleStatic(cfg, tx, B, V, th, None, tu, tok_s, pr_s, status_out=status, hist_stride=H, stream=cur())
+    def static_call(st):
+        S.SampleStatic(cfg, dx, B, V, dh, None, du, tok_s, pr_s, status_out=status, hist_stride=H, stream=st)
 
-    static_call()                                                            # the warm call: looks up the array's address
-    torch.cuda.synchronize()
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    static_call(stream)                                                      # the warm call: looks up the array's address
+    assert hip.hipStreamSynchronize(stream) == 0
     # (a) nothing allocated, nothing freed
-    free_before = torch.cuda.mem_get_info()[0]
-    static_call()
-    static_call()
-    torch.cuda.synchronize()
-    assert torch.cuda.mem_get_info()[0] == free_before
-    # (b) under stream capture
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    with torch.cuda.graph(graph, stream=side):
-        static_call()
+    before = free_bytes()
+    static_call(stream)
+    static_call(stream)
+    assert hip.hipStreamSynchronize(stream) == 0
+    assert free_bytes() == before
+    # (b) under stream capture (mode 0 = global: an allocation by any thread invalidates the capture)
+    graph, graph_exec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0
+    try:
+        static_call(stream)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0 and graph.value, "the capture was invalidated"
+    assert hip.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, 0) == 0
     rng = np.random.default_rng(5)
+    poison = np.full(B, -7, np.int32)
     for replay in range(3):
         u_new = rng.random(B, dtype=np.float32)
-        tu.copy_(torch.from_numpy(u_new))                                    # eager work between the replays
-        tok_s.fill_(-7)
-        torch.cuda.synchronize()
-        graph.replay()
-        torch.cuda.synchronize()
-        smp.Sample(tx, B, V, th, None, tu, tok_h, pr_h, hist_stride=H, stream=cur())
-        torch.cuda.synchronize()
-        assert torch.equal(tok_s, tok_h), (replay, (tok_s != tok_h).nonzero().flatten()[:8].tolist())
-        assert torch.equal(pr_s.view(torch.int32), pr_h.view(torch.int32)), replay
-    assert int(status.item()) == 0
+        _capi.check(_capi.lib().born_rocm_h2d(du.ptr, u_new.ctypes.data, u_new.nbytes, None))      # eager work between the replays
+        _capi.check(_capi.lib().born_rocm_h2d(tok_s.ptr, poison.ctypes.data, poison.nbytes, None))
+        assert hip.hipGraphLaunch(graph_exec, stream) == 0
+        assert hip.hipStreamSynchronize(stream) == 0
+        smp.Sample(dx, B, V, dh, None, du, tok_h, pr_h, hist_stride=H)
+        smp.Status()
+        got, want = tok_s.to_numpy(np.int32, (B,)), tok_h.to_numpy(np.int32, (B,))
+        assert np.array_equal(got, want), (replay, np.nonzero(got != want)[0][:8])
+        assert np.array_equal(pr_s.to_numpy(np.uint32, (B,)), pr_h.to_numpy(np.uint32, (B,))), replay
+    assert int(status.to_numpy(np.int32, (1,))[0]) == 0
+    hip.hipGraphExecDestroy(graph_exec)
+    hip.hipGraphDestroy(graph)
+    hip.hipStreamDestroy(stream)
     smp.Close()
