@@ -123,7 +123,7 @@ func (l *Linear) ForwardArgmax(s *Sampler, input DeviceBuffer, shape []int) ([]i
 
 // ForwardSample is the layer and the sampling step in one call (born_rocm_linear_sample): tokens[b] is what
 // s.Sample draws from Forward(input)[b], and the [batch, out_features] logits are never written.  The sampler's
-// configuration must be one the single-pass kernel serves (1 <= TopK <= 128, RepetitionPenalty >= 1, no frequency or
+// configuration must be one the fused step serves (1 <= TopK <= 128, RepetitionPenalty >= 1, no frequency or
 // presence penalty).  A row the fused step cannot settle comes back as -1; the whole call is then repeated over
 // materialised logits (Forward + Sample) with the draw counter of the built-in uniform stream set back to its value
 // before the fused call, so the caller always gets the tokens of the unfused pair and a seeded run consumes one

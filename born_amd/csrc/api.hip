@@ -167,6 +167,7 @@ int born_rocm_sampler_create(const born_sampler_config *cfg, int64_t max_batch, 
     std::call_once(g_cfg_once, [] {
         g_cfg_err = configure_kernels();
         if (g_cfg_err == hipSuccess) g_cfg_err = configure_nucleus();
+        if (g_cfg_err == hipSuccess) g_cfg_err = configure_topk_row();
     });
     if (g_cfg_err != hipSuccess) return hip_fail(g_cfg_err, "configure_kernels");
 
@@ -593,6 +594,7 @@ int born_rocm_sample_static(const born_sampler_config *cfg, const float *logits,
     std::call_once(g_cfg_once, [] {
         g_cfg_err = configure_kernels();
         if (g_cfg_err == hipSuccess) g_cfg_err = configure_nucleus();
+        if (g_cfg_err == hipSuccess) g_cfg_err = configure_topk_row();
     });
     if (g_cfg_err != hipSuccess) return hip_fail(g_cfg_err, "configure_kernels");
     unsigned long long *ws = nullptr;
@@ -808,10 +810,10 @@ int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int6
         w_stride * (int64_t)((out_features + LM_SAMPLE_MAX - 1) / LM_SAMPLE_MAX) > ((int64_t)1 << 40))
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: shape too large");
     const int top_k = (s->cfg.top_k <= 0 || s->cfg.top_k >= out_features) ? 0 : s->cfg.top_k;
-    if (top_k < 1 || top_k > TOPK_MAX_K || out_features > ROW_MAX_VOCAB || (history && s->cfg.repetition_penalty < 1.0f) ||
+    if (top_k < 1 || top_k > LM_MAX_K || out_features > ROW_MAX_VOCAB || (history && s->cfg.repetition_penalty < 1.0f) ||
         counts_history(s->cfg))
         return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: the fused step serves 1 <= top_k <= %d over at most %d columns with a repetition "
-                    "penalty >= 1 and no frequency / presence penalty; use born_rocm_linear + born_rocm_sample", TOPK_MAX_K, ROW_MAX_VOCAB);
+                    "penalty >= 1 and no frequency / presence penalty; use born_rocm_linear + born_rocm_sample", LM_MAX_K, ROW_MAX_VOCAB);
     hipStream_t st = (hipStream_t)stream;
     if (!s->lm_cand) {
         if (s->fixed_workspace) return fail(BORN_ROCM_ERR_UNSUPPORTED, "linear_sample: this handle cannot allocate its workspace");

@@ -7,7 +7,8 @@ namespace born {
 
 // The single-pass top-k kernel (one workgroup per row).
 constexpr int TOPK_LOCAL_COUNT_HISTORY = 4096;   // longest history whose occurrences it counts in LDS
-constexpr int TOPK_MAX_K = 128;            // largest top_k it serves (its last wave holds two survivors per lane)
+constexpr int TOPK_MAX_K = 512;            // largest top_k it serves (its last wave holds up to eight survivors per lane)
+constexpr int LM_MAX_K = 128;              // largest top_k of the sampling step fused into the LM head
 constexpr int ROW_MAX_VOCAB = 393216;      // largest vocabulary it takes (its history bitmap is 48 KiB of LDS)
 
 // Geometry of the general (any k, any p) kernel: one workgroup per row.
@@ -158,6 +159,7 @@ hipError_t launch_hist_counts(const int *history, const int *hist_len, long long
                               bool clear, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
+hipError_t configure_topk_row();   // one-time function attributes (dynamic LDS above 64 KiB)
 // Sampling fused into the LM head, in three steps around the GEMM that lists the candidates:
 //   thr[row] = the kth largest of samp[row][0..nsamp) + bias[j * sstep] (-inf if there are fewer); cand_cnt[row] = 0
 hipError_t launch_lm_threshold(const float *samp, long long ld, int B, int nsamp, const float *bias, int sstep, int kth, float *thr,

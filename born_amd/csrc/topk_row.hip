@@ -1,18 +1,23 @@
-// One-launch sampler for 1 <= top_k <= 128 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
+// One-launch sampler for 1 <= top_k <= 512 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
 // of 1024 threads per row.
 //
 // The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 logits, the
-// loads of one stage in flight while the stage before it is examined.
+// loads of three stages in flight.  A stage is not a contiguous piece of the row: the row is cut into chunks
+// of 64 float4 (1 KiB, what one wave instruction loads) and stage s takes the chunks (u * 16 + w) * nstage + s
+// for the four loads u of the sixteen waves w, so that every stage is an even sample of the whole row by
+// position.  Rows whose large logits sit late in vocabulary order (sorted ascending, a step up near the end, a
+// slow rise) then look to the pass like any other row.
 //
 //   T   A threshold that the row's top_k-th largest logit is known to reach.  First from the first stage alone:
 //       every wave takes the a-th largest of its lane maxima, and the w-th largest of the wave results has
 //       >= w * a >= top_k logits of that stage at or above it.
 //   L   Every logit >= T met from then on is appended, exact value and id, to the list of the wave that met it
 //       (ballot + lane rank, no atomics): one compare per logit in the common case.
-//   T'  Every three stages, with the next stages' loads in flight, the lists' entries are binned by key distance
-//       above T (one LDS atomic each); the highest bin boundary with >= top_k + 16 entries at or above it becomes
-//       the new T and every wave drops its entries below it.  The lists so end the pass with little more than
-//       top_k + 16 entries between them, and nothing has to be thinned out after the last load.
+//   T'  After the first stage and then every three stages, with the next stages' loads in flight, the lists'
+//       entries are binned by key distance above T (one LDS atomic each); the highest bin boundary with >= top_k
+//       + margin entries at or above it becomes the new T and every wave drops its entries below it.  The lists
+//       so end the pass with little more than top_k + margin entries between them, and nothing has to be
+//       thinned out after the last load.
 //   Any logit outside the lists is below T, and so is its z after a penalty (repetition_penalty >= 1
 //   only lowers a logit) and the monotone division by the temperature.  Every wave turns its own entries into rank
 //   keys (probing its hash of the history) and appends them to one array; the row is proven if top_k candidates
@@ -36,18 +41,10 @@
 
 namespace born {
 
-#ifndef BORN_ROW_BLOCK
-#define BORN_ROW_BLOCK 1024
-#endif
-constexpr int ROW_BLOCK = BORN_ROW_BLOCK;
+constexpr int ROW_BLOCK = 1024;
 constexpr int ROW_WAVES = ROW_BLOCK / WAVE;
 constexpr int ROW_U = 4096 / ROW_BLOCK;       // 128-bit loads per thread and stage: a stage is 16384 logits
-constexpr int ROW_WCAP = 256;                 // list entries per wave
-constexpr int ROW_CAP = 512;                  // candidates the tail can hold
-constexpr int ROW_SLOTS = 1024;               // hash slots (load factor <= 0.5)
-constexpr int ROW_MARGIN = 16;                // entries a raised threshold keeps beyond top_k
 constexpr int ROW_HSLOTS = 2048;              // slots of the history hash (at most ROW_BLOCK tokens: load factor <= 0.5)
-__device__ __forceinline__ u32 row_hash(u32 id) { return (id * 2654435761u) >> (32 - 10); }
 __device__ __forceinline__ u32 row_hhash(u32 id) { return (id * 2654435761u) >> (32 - 11); }
 // A slot of a history hash: id + 1 in the low bits, the number of occurrences above them (kept only when the
 // frequency / presence penalties are counted by the kernel itself).
@@ -62,41 +59,53 @@ static_assert(FB_HSLOTS == (1 << 13), "fb_hhash produces 13 bits");
 template <bool LOCAL>
 __device__ __forceinline__ u32 hslot_id(u32 e) { return LOCAL ? (e & HSLOT_ID_MASK) : e; }
 static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS >= 2 * ROW_BLOCK, "row_hhash produces 11 bits; load factor <= 0.5");
-static_assert(ROW_SLOTS == (1 << 10), "row_hash produces 10 bits");
-static_assert(ROW_CAP <= ROW_BLOCK, "one thread per candidate");
-static_assert(ROW_WCAP % WAVE == 0, "lists are scanned in whole wave strides");
 
-// LDS pool (u64 words), laid out once for the proof and once for the exact selection
-constexpr int ROW_POOL = 8064 + (ROW_BLOCK < 1024 ? 2048 : 0);   // (a smaller workgroup pads its pool so that a compute unit holds one)
-constexpr int OFF_L = 0;                      // [ROW_WAVES][ROW_WCAP] uint2
-constexpr int OFF_C = OFF_L + ROW_WAVES * ROW_WCAP;   // [ROW_CAP] uint2
-constexpr int OFF_K = OFF_C + ROW_CAP;        // [ROW_CAP] u64
-constexpr int OFF_TAB = OFF_K + ROW_CAP;      // [ROW_SLOTS] u32
-constexpr int OFF_SORTED = OFF_TAB + ROW_SLOTS / 2;   // [TOPK_MAX_K] u64
-constexpr int OFF_HTAB = OFF_SORTED + TOPK_MAX_K;   // [ROW_HSLOTS] u32
-static_assert(OFF_HTAB + ROW_HSLOTS / 2 <= ROW_POOL, "proof layout fits the pool");
 constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
-constexpr int FB_DIGIT = ROW_BLOCK >= 1024 ? 11 : 10;   // key bits per sweep: two digits per thread
-constexpr int OFF_FB_HIST = FB_BITMAP;        // [1 << FB_DIGIT] u32
-constexpr int OFF_FB_LIST = OFF_FB_HIST + (1 << FB_DIGIT) / 2;
-constexpr int FB_LIST_CAP = ROW_BLOCK >= 1024 ? 768 : 512;
-constexpr int OFF_FB_SORTED = OFF_FB_LIST + FB_LIST_CAP;
-static_assert(OFF_FB_SORTED + TOPK_MAX_K <= ROW_POOL, "selection layout fits the pool");
-static_assert(TOPK_MAX_K <= 2 * WAVE, "the last wave holds at most two survivors per lane");
-static_assert(FB_LIST_CAP <= ROW_BLOCK, "one thread per gathered key");
+constexpr int FB_DIGIT = 11;                  // key bits per sweep: two digits per thread
 static_assert((long long)FB_BITMAP * 64 >= ROW_MAX_VOCAB, "one bitmap bit per id");
 static_assert(FB_HSLOTS / 2 <= FB_BITMAP, "the history hash takes the bitmap's place");
 
+constexpr int TOPK_SMALL_K = 128;             // up to here the candidates are ranked by counting and the last wave holds two per lane
+
+// Sizes of an instance and the layout of its LDS pool (u64 words), once for the proof and once for the exact selection.
+//   KC 0: top_k <= 128.  KC 1: top_k <= 512 (and the per-row instances, whose rows may ask for either).
+//   KC 2: the finish over a list of candidates (cand_row_kernel).
+template <int KC>
+struct RowGeom {
+    static constexpr int WCAP = KC == 2 ? 256 : 512;                 // list entries per wave
+    static constexpr int CAP = KC == 1 ? 1024 : 512;                 // candidates the finish can hold
+    static constexpr int MAXK = KC == 1 ? TOPK_MAX_K : TOPK_SMALL_K; // largest top_k
+    static constexpr int SLOTS = 2 * CAP;                            // hash slots of the candidates' ids (load factor <= 0.5)
+    static constexpr int SLOT_BITS = KC == 1 ? 11 : 10;
+    static constexpr int FB_LIST = KC == 1 ? 1024 : 768;             // keys the exact selection ranks
+    static constexpr int OFF_L = 0;                                  // [ROW_WAVES][WCAP] uint2
+    static constexpr int OFF_C = OFF_L + ROW_WAVES * WCAP;           // [CAP] uint2
+    static constexpr int OFF_K = OFF_C + CAP;                        // [CAP] u64
+    static constexpr int OFF_TAB = OFF_K + CAP;                      // [SLOTS] u32
+    static constexpr int OFF_SORTED = OFF_TAB + SLOTS / 2;           // [MAXK] u64
+    static constexpr int OFF_HTAB = OFF_SORTED + MAXK;               // [ROW_HSLOTS] u32
+    static constexpr int PROOF_END = OFF_HTAB + ROW_HSLOTS / 2;
+    static constexpr int OFF_FB_HIST = FB_BITMAP;                    // [1 << FB_DIGIT] u32
+    static constexpr int OFF_FB_LIST = OFF_FB_HIST + (1 << FB_DIGIT) / 2;
+    static constexpr int OFF_FB_SORTED = OFF_FB_LIST + FB_LIST;
+    static constexpr int FB_END = OFF_FB_SORTED + MAXK;
+    static constexpr int POOL = PROOF_END > FB_END ? PROOF_END : FB_END;
+    static_assert(SLOTS == (1 << SLOT_BITS), "the hash of a candidate id produces SLOT_BITS bits");
+    static_assert(CAP <= ROW_BLOCK && FB_LIST <= ROW_BLOCK, "one thread per candidate");
+    static_assert(WCAP % (4 * WAVE) == 0, "lists are compacted four wave strides at a time");
+    static_assert(MAXK <= 8 * WAVE, "the last wave holds at most eight survivors per lane");
+    static_assert(CAP % 32 == 0 && ROW_WAVES * WCAP >= CAP, "the ranked keys are read 32 at a time; the lists' space is reused for them");
+    __device__ static __forceinline__ u32 hash(u32 id) { return (id * 2654435761u) >> (32 - SLOT_BITS); }
+};
+static_assert(TOPK_MAX_K == 512, "RowGeom<1> and its last wave are sized for 512");
+// Entries a raised threshold keeps beyond top_k (what the penalties may push below the bound without losing the proof).
+__device__ __forceinline__ int row_margin(int k) { return k <= TOPK_SMALL_K ? 16 : k >> 3; }
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-// One stage = ROW_U consecutive blocks of ROW_BLOCK float4.  row_load_fast: the stage lies wholly inside the
-// row (no branches, so the loads of the next stage can stay in flight while this one is examined).
-__device__ __forceinline__ void row_load_fast(f32x4 (&v)[ROW_U], const float *x, int stage, int tid) {
-#pragma unroll
-    for (int u = 0; u < ROW_U; u++)
-        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + ((stage * ROW_U + u) * ROW_BLOCK + tid));
-}
-// row_load_any: the row's ragged end, unaligned rows, and anything past the end (-inf fill).
+// row_load_any: one stage of ROW_U consecutive blocks of ROW_BLOCK float4 in row order, for the row's ragged end,
+// unaligned rows, and anything past the end (-inf fill).  Used by the sweeps of the exact selection and by rows that
+// 128-bit loads cannot take.
 template <bool VEC>
 __device__ __forceinline__ void row_load_any(f32x4 (&v)[ROW_U], const float *x, int V, int stage, int tid) {
 #pragma unroll
@@ -110,27 +119,91 @@ __device__ __forceinline__ void row_load_any(f32x4 (&v)[ROW_U], const float *x, 
         }
     }
 }
+// The same for a stage that lies wholly inside the row (no branches, so the loads of the next stage can stay in flight
+// while this one is examined).
+__device__ __forceinline__ void row_load_fast(f32x4 (&v)[ROW_U], const float *x, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + ((stage * ROW_U + u) * ROW_BLOCK + tid));
+}
 
-// Appends the logits >= tw of one stage to the wave's list.  tw >= -FLT_MAX, so -inf (the fill past the end of
-// the row included) and NaN never pass.  `count` is wave-uniform.
-__device__ __forceinline__ void row_filter(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid) {
+// Appends the elements >= tw of one float4 to the wave's list.  tw >= -FLT_MAX, so -inf and NaN never pass.  `count`
+// is wave-uniform; idof(c) is the id of element c (evaluated only for elements that pass); MASKED: elements whose id
+// is not below V count as -inf (the row's ragged end).
+template <int WCAP, bool MASKED, class IdOf>
+__device__ __forceinline__ void row_filter4(const f32x4 v, float tw, uint2 *list, u32 &count, int V, IdOf idof) {
 #pragma unroll
-    for (int u = 0; u < ROW_U; u++) {
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const float xv = v[u][c];
-            const bool pass = xv >= tw;
-            const u64 m = __ballot(pass);
-            if (m) {                                                 // wave-uniform
-                if (pass) {
-                    const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
-                    if (pos < (u32)ROW_WCAP)
-                        list[pos] = make_uint2(__float_as_uint(xv), (u32)(((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c));
-                }
-                count += (u32)__popcll(m);
+    for (int c = 0; c < 4; c++) {
+        const float xv = v[c];
+        const bool pass = MASKED ? (xv >= tw && idof(c) < V) : (xv >= tw);
+        const u64 m = __ballot(pass);
+        if (m) {                                                     // wave-uniform
+            if (pass) {
+                const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+                if (pos < (u32)WCAP) list[pos] = make_uint2(__float_as_uint(xv), (u32)idof(c));
             }
+            count += (u32)__popcll(m);
         }
     }
+}
+
+// Where the 128-bit loads of the pass lie.  The row is cut into chunks of WAVE float4 (what one wave instruction
+// loads, 1 KiB); stage s of the pass takes, for load u of wave w, chunk (u * ROW_WAVES + w) * nstage + s: the 64 chunks
+// of a stage are spread evenly over the row, so every stage is a sample of the whole row by position.  nstage * 64
+// chunk places cover the row; those at or beyond `cend` hold nothing, the one between `cfull` and `cend` (if any)
+// holds the row's ragged end.
+struct RowMap {
+    int nstage;                   // stages of the pass
+    int n4;                       // float4 blocks that hold an element of the row
+    int cfull, cend;              // chunks wholly inside the row; chunks that hold any element
+    int w, l;                     // this thread's wave (wave-uniform) and lane
+};
+#ifndef BORN_ROW_SEQUENTIAL
+__device__ __forceinline__ int row_chunk(const RowMap &m, int s, int u) { return (u * ROW_WAVES + m.w) * m.nstage + s; }
+#else
+// (measurement builds: the stages in row order)
+__device__ __forceinline__ int row_chunk(const RowMap &m, int s, int u) { return (s * ROW_U + u) * ROW_WAVES + m.w; }
+#endif
+// The loads of stage s.  A chunk place beyond the row (or a stage beyond the last) re-reads the row's last block
+// instead of branching around its load, so that the loads of later stages can stay in flight: a load under a
+// condition makes the compiler wait for every load in flight.  The row starts 16-byte aligned and its pitch is a
+// multiple of four floats, so the last block lies inside the pitch.
+__device__ __forceinline__ void row_load_perm(f32x4 (&v)[ROW_U], const float *x, const RowMap &m, int s) {
+    const int last = m.n4 - 1;
+    const int off = s < m.nstage ? m.l : m.n4;                       // (a stage past the last one: every lane reads the last block)
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++) {
+        const int i4 = min(row_chunk(m, s, u) * WAVE + off, last);
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i4);
+    }
+}
+// Appends the logits >= tw of stage s to the wave's list.
+template <int WCAP>
+__device__ __forceinline__ void row_filter_perm(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, const RowMap &m, int s, int V) {
+    bool whole = true;                                               // wave-uniform: every chunk of the wave's stage lies wholly inside the row
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++) whole = whole && row_chunk(m, s, u) < m.cfull;
+    if (whole) {
+#pragma unroll
+        for (int u = 0; u < ROW_U; u++) {
+            const int ch = row_chunk(m, s, u);
+            row_filter4<WCAP, false>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < ROW_U; u++) {
+            const int ch = row_chunk(m, s, u);
+            if (ch < m.cfull) row_filter4<WCAP, false>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
+            else if (ch < m.cend) row_filter4<WCAP, true>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
+        }
+    }
+}
+// The same for a stage in row order (rows that 128-bit loads cannot take; elements past the end were filled with -inf).
+template <int WCAP>
+__device__ __forceinline__ void row_filter_seq(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+        row_filter4<WCAP, false>(v[u], tw, list, count, 0, [&](int c) { return ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c; });
 }
 
 // The need-th largest of the 16 wave results in `wthr` (LDS), computed redundantly by every wave in its first
@@ -145,8 +218,8 @@ __device__ __forceinline__ u32 row_pick(const u32 *wthr, int need) {
     return wave_max_u32((l < ROW_WAVES && ge >= need) ? mine : 0u);
 }
 
-// Visits every element of the row as f(id, logit), the loads of one stage in flight while the stage before it
-// is visited.
+// Visits every element of the row as f(id, logit), in row order, the loads of one stage in flight while the stage
+// before it is visited.
 template <bool VEC, class F>
 __device__ __forceinline__ void row_foreach(const float *x, int V, int tid, F f) {
     const int n4 = (V + 3) >> 2;
@@ -183,14 +256,14 @@ __device__ __forceinline__ void row_foreach(const float *x, int V, int tid, F f)
 
 // Exact selection of the row's top_k rank keys for any input (every thread of the workgroup calls it).
 // pool: the workgroup's LDS pool; s_n, s_x: two shared ints.
-template <bool VEC, bool LOCAL>
+template <bool VEC, bool LOCAL, class G>
 __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, const float *x, int hlen, const int *h, float u_row,
                                                  u64 *pool, int *s_n, int *s_x) {
     const int tid = threadIdx.x, V = a.V, k = a.top_k;
     u32 *bm = reinterpret_cast<u32 *>(pool);
-    u32 *hist = reinterpret_cast<u32 *>(pool + OFF_FB_HIST);
-    u64 *list = pool + OFF_FB_LIST;
-    u64 *sorted = pool + OFF_FB_SORTED;
+    u32 *hist = reinterpret_cast<u32 *>(pool + G::OFF_FB_HIST);
+    u64 *list = pool + G::OFF_FB_LIST;
+    u64 *sorted = pool + G::OFF_FB_SORTED;
     const unsigned *counts = a.hist_counts ? a.hist_counts + (long long)row * V : nullptr;
     constexpr bool local = LOCAL;                                    // occurrences are counted here, in a hash of the history
     const bool counted = counts || local;
@@ -279,7 +352,7 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
         prefix = (prefix << db) | (u64)D;
         plen += db;
         __syncthreads();
-        if (above + (int)cntD <= FB_LIST_CAP || plen == 64) break;
+        if (above + (int)cntD <= G::FB_LIST || plen == 64) break;
     }
     // gather the keys at or above the bucket: `above` + the bucket's, at least top_k of them
     const u64 lo_key = plen == 64 ? prefix : prefix << (64 - plen);
@@ -289,11 +362,11 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
         const u64 key = rank_key(j, xv);
         if (key >= lo_key) {
             const int pos = atomicAdd(&s_n[0], 1);
-            if (pos < FB_LIST_CAP) list[pos] = key;
+            if (pos < G::FB_LIST) list[pos] = key;
         }
     });
     __syncthreads();
-    const int n = min(s_n[0], FB_LIST_CAP);
+    const int n = min(s_n[0], G::FB_LIST);
     if (tid < n) {
         const u64 key = list[tid];
         int r = 0;
@@ -308,26 +381,6 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
 }
 
-// Block indices clamped into the row: a stage that reaches past the row's end (or lies wholly beyond it) re-reads the
-// row's last block instead of branching around its loads, so that the loads of later stages can stay in flight.  The
-// row starts 16-byte aligned and its pitch is a multiple of four floats (VEC), so the last block lies inside the pitch.
-__device__ __forceinline__ void row_load_clamped(f32x4 (&v)[ROW_U], const float *x, int n4, int stage, int tid) {
-#pragma unroll
-    for (int u = 0; u < ROW_U; u++) {
-        const int i4 = min((stage * ROW_U + u) * ROW_BLOCK + tid, n4 - 1);
-        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i4);
-    }
-}
-// row_filter for a stage that may reach past the row's end: elements at or beyond V count as -inf.
-__device__ __forceinline__ void row_filter_masked(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid, int V) {
-    f32x4 m[ROW_U];
-#pragma unroll
-    for (int u = 0; u < ROW_U; u++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) m[u][c] = (((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c < V) ? v[u][c] : -INFINITY;
-    row_filter(m, tw, list, count, stage, tid);
-}
-
 constexpr int ROW_TBINS = 256;                // bins of the threshold histogram (four per lane)
 static_assert(ROW_TBINS == 4 * WAVE && ROW_TBINS <= ROW_BLOCK, "one 128-bit read per lane covers the bins");
 
@@ -340,11 +393,12 @@ static_assert(ROW_TBINS == 4 * WAVE && ROW_TBINS <= ROW_BLOCK, "one 128-bit read
 //   H: this round's bins (all zero on entry); Hclear: the next round's bins, zeroed here (with three sets in rotation
 //   they were last read two rounds ago, before the previous round's barrier);
 //   Mnext: where this round's largest key is published for the next round.
+template <int WCAP>
 __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, int want, u32 smax, u32 *H, u32 *Hclear, u32 *Mnext,
                                             int *s_over, int tid) {
     const int l = lane_id();
-    if (count > (u32)ROW_WCAP && l == 0) *s_over = 1;
-    const int cw = (int)min(count, (u32)ROW_WCAP);
+    if (count > (u32)WCAP && l == 0) *s_over = 1;
+    const int cw = (int)min(count, (u32)WCAP);
     const u32 range = smax > twkey ? smax - twkey : 0u;
     const int sh = max(0, 24 - (int)__clz(range));                   // (range >> sh) < ROW_TBINS
     u32 mx = 0u;
@@ -372,45 +426,61 @@ __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey,
     if (c < need) { bin--; c += hz; if (c < need) { bin--; c += hy; if (c < need) bin--; } }
     const u32 nk = twkey + ((u32)bin << sh);                         // at most the key of an entry of that bin: no overflow
     if (nk <= twkey) return;
-    // in-place compaction of the wave's own list: every read is issued before the first write
-    uint2 ent[ROW_WCAP / WAVE];
-    bool keep[ROW_WCAP / WAVE];
-#pragma unroll
-    for (int r = 0; r < ROW_WCAP / WAVE; r++) {
-        const int e = l + r * WAVE;
-        keep[r] = false;
-        if (e < cw) {
-            ent[r] = list[e];
-            keep[r] = ordkey(__uint_as_float(ent[r].x)) >= nk;
-        }
-    }
+    // in-place compaction of the wave's own list, four wave strides at a time: within a group every read is issued
+    // before the first write, and a group writes only below the entries it has read (kept <= the group's first entry)
     u32 kept = 0u;
+    for (int g = 0; g * WAVE < cw; g += 4) {                         // wave-uniform
+        uint2 ent[4];
+        bool keep[4];
 #pragma unroll
-    for (int r = 0; r < ROW_WCAP / WAVE; r++) {
-        if (r * WAVE < cw) {                                         // wave-uniform
-            const u64 m = __ballot(keep[r]);
-            if (keep[r]) list[kept + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u))] = ent[r];
-            kept += (u32)__popcll(m);
+        for (int r = 0; r < 4; r++) {
+            const int e = l + (g + r) * WAVE;
+            keep[r] = false;
+            if (e < cw) {
+                ent[r] = list[e];
+                keep[r] = ordkey(__uint_as_float(ent[r].x)) >= nk;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            if ((g + r) * WAVE < cw) {                               // wave-uniform
+                const u64 m = __ballot(keep[r]);
+                if (keep[r]) list[kept + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u))] = ent[r];
+                kept += (u32)__popcll(m);
+            }
         }
     }
     count = kept;
     twkey = nk;
 }
 
+// Waves whose first load of the first stage holds an element of the row.
+__device__ __forceinline__ int row_active_waves(const RowMap &m) {
+#ifndef BORN_ROW_SEQUENTIAL
+    return min(ROW_WAVES, (m.cend + m.nstage - 1) / m.nstage);
+#else
+    return min(ROW_WAVES, m.cend);
+#endif
+}
+
 // LOCAL: the frequency / presence penalties are on and the kernel counts the occurrences itself (SampleArgs::local_counts).
-template <bool VEC, bool LOCAL>
+// KC: the instance's sizes (RowGeom).
+template <bool VEC, bool LOCAL, int KC>
 __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
-    __shared__ u64 pool[ROW_POOL];
-    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);       // per-wave lists of (logit bits, id) >= the threshold
-    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);       // long histories: the candidates; .y bit 31 = id occurs in the history
-    u64 *const K = pool + OFF_K;                                     // the candidates' rank keys
-    u32 *const tab = reinterpret_cast<u32 *>(pool + OFF_TAB);
+    using G = RowGeom<KC>;
+    extern __shared__ __align__(16) u64 row_pool[];                 // G::POOL words
+    u64 *const pool = row_pool;
+    uint2 *const L = reinterpret_cast<uint2 *>(pool + G::OFF_L);    // per-wave lists of (logit bits, id) >= the threshold
+    uint2 *const C = reinterpret_cast<uint2 *>(pool + G::OFF_C);    // long histories: the candidates; .y bit 31 = id occurs in the history
+    u64 *const K = pool + G::OFF_K;                                  // the candidates' rank keys
+    u32 *const tab = reinterpret_cast<u32 *>(pool + G::OFF_TAB);
     u32 *const Khi = tab;                                            // the candidates' z alone, once the hash of their ids has served
-    u64 *const sorted = pool + OFF_SORTED;
-    u32 *const htab = reinterpret_cast<u32 *>(pool + OFF_HTAB);
+    u64 *const sorted = pool + G::OFF_SORTED;
+    u32 *const htab = reinterpret_cast<u32 *>(pool + G::OFF_HTAB);
     __shared__ u32 s_wthr[ROW_WAVES], s_wmax[ROW_WAVES];
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
     __shared__ u32 s_max[2];
+    __shared__ u32 s_kmax, s_kmin;
     __shared__ int s_n, s_valid, s_over, s_next;
     __shared__ int s_x[1 + ROW_WAVES];
 #ifdef BORN_PHASE_TIMING
@@ -434,7 +504,13 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int n4 = (V + 3) >> 2;
     const int iters = (n4 + ROW_BLOCK - 1) / ROW_BLOCK;             // float4 blocks per thread
     const int nstage = (iters + ROW_U - 1) / ROW_U;
-    const int nfull = (V >> 2) / (ROW_U * ROW_BLOCK);                // stages made of whole float4 blocks inside the row
+    RowMap m;
+    m.nstage = nstage;
+    m.n4 = n4;
+    m.cfull = V / (4 * WAVE);
+    m.cend = (V + 4 * WAVE - 1) / (4 * WAVE);
+    m.w = __builtin_amdgcn_readfirstlane(wave_id());
+    m.l = lane_id();
 
     // Order of the requests: this thread's first history entry (used last, but loads return in order and it must
     // not wait behind the row), then the row's first three stages; the LDS tables are cleared behind them.
@@ -443,9 +519,9 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int h0 = (tid < hlen) ? h[tid] : -1;
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
     if (VEC) {
-        row_load_clamped(va, x, n4, 0, tid);
-        row_load_clamped(vb, x, n4, 1, tid);                         // in flight during the search for the first threshold
-        row_load_clamped(vc, x, n4, 2, tid);
+        row_load_perm(va, x, m, 0);
+        row_load_perm(vb, x, m, 1);                                  // in flight during the search for the first threshold
+        row_load_perm(vc, x, m, 2);
     } else {
         row_load_any<false>(va, x, V, 0, tid);
     }
@@ -457,8 +533,10 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         s_next = 0;
         s_max[0] = 0u;
         s_max[1] = 0u;
+        s_kmax = 0u;
+        s_kmin = 0xFFFFFFFFu;
     }
-    for (int i = tid; i < ROW_SLOTS; i += ROW_BLOCK) tab[i] = 0u;
+    for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
     if (tid < ROW_TBINS) s_bins[0][tid] = 0u;                        // every round clears the bins of the next
     // A history of at most ROW_BLOCK tokens is hashed while the first loads are in flight, and the candidates
     // probe it at the end; a longer one probes a hash of the candidates instead.
@@ -469,7 +547,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const bool hfast = penal && hlen <= ROW_BLOCK;
     u32 *const ccnt = htab;                                          // a long history: occurrences by candidate (the hash is unused then)
     for (int i = tid; i < ROW_HSLOTS; i += ROW_BLOCK) htab[i] = 0u;
-    if (tid < TOPK_MAX_K) sorted[tid] = 0ull;
+    if (tid < G::MAXK) sorted[tid] = 0ull;
 
     ROW_STAMP(0);
     // The row's uniform is one scalar load whose result the compiler waits for on the spot: after the row's first
@@ -481,22 +559,29 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 
     // ---- the first threshold, from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per
     // wave and the need = ceil(top_k / a)-th largest of the wave results
-    const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
+    const int act = VEC ? row_active_waves(m) : min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
     const int aw = min(WAVE, (k + act - 1) / act);                   // lanes of one wave
-    const int need = (k + aw - 1) / aw;                              // <= act, but for top_k > 64 on a row of one wave: no threshold then
+    const int need = (k + aw - 1) / aw;                              // <= act, but for a top_k beyond the lanes that hold data: no threshold then
     {
         float lm = -INFINITY;
-        if (nfull > 0) {
+        if (VEC) {
+#pragma unroll
+            for (int u = 0; u < ROW_U; u++) {
+                const int ch = row_chunk(m, 0, u);
+                if (ch < m.cfull) {                                  // wave-uniform
+#pragma unroll
+                    for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
+                } else if (ch < m.cend) {                            // the row's ragged end
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        if ((ch * WAVE + m.l) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
+                }
+            }
+        } else {                                                     // (elements past the end were filled with -inf)
 #pragma unroll
             for (int u = 0; u < ROW_U; u++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
-        } else {                                                     // the row ends inside the first stage
-#pragma unroll
-            for (int u = 0; u < ROW_U; u++)
-#pragma unroll
-                for (int c = 0; c < 4; c++)
-                    if ((u * ROW_BLOCK + tid) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
+                for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);
         }
         const u32 lk = ordkey(lm);
         const u32 wk = wave_kth_largest_bound(lk, aw, 14);
@@ -526,17 +611,17 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // for the counting argument); nothing is listed and the row goes to the exact selection
     const bool have_tw = twkey > ordkey(-INFINITY);
     float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
-    const int want = k + ROW_MARGIN;                                 // entries a raised threshold keeps at least
+    const int want = k + row_margin(k);                              // entries a raised threshold keeps at least
 
-    // ---- the pass over the row.  Every three stages the threshold is raised from what the lists hold by then, so
-    // that they end the pass with little more than `want` entries between them.
-    uint2 *list = L + wave_id() * ROW_WCAP;
+    // ---- the pass over the row.  After the first stage and then every three stages the threshold is raised from what
+    // the lists hold by then, so that they end the pass with little more than `want` entries between them.
+    uint2 *list = L + wave_id() * G::WCAP;
     u32 count = 0;
     int round = 0;
     auto tighten = [&]() {
         if (have_tw) {                                               // workgroup-uniform
             const u32 smax = max(max0, s_max[round & 1]);
-            row_tighten(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+            row_tighten<G::WCAP>(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
             tw = ordkey_inv(twkey);
             round++;
         }
@@ -549,40 +634,42 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // The row is proven if top_k candidates have z strictly above that bound.
     u32 zb = 0u;
     if (VEC) {
-        // at the loop head va, vb, vc = stages s, s + 1, s + 2 are requested: two stages stay in flight while one
-        // is examined.  The stages of the loop lie wholly inside the row; the last three (the last of which may reach
-        // past its end) are examined without new requests.
-        int s = 0;
+        // va, vb, vc = stages 0, 1, 2 are requested: two stages stay in flight while one is examined.  The first stage is
+        // an even sample of the row like every other, and the threshold the counting argument drew from it can be far
+        // below what the stage's own logits allow (a few waves may hold all the large ones): it is raised at once.
+        row_filter_perm<G::WCAP>(va, tw, list, count, m, 0, V);
+        row_load_perm(va, x, m, 3);
+#ifndef BORN_ROW_NO_ROUND0
+        tighten();
+#endif
+        // at the loop head vb, vc, va = stages s, s + 1, s + 2
+        int s = 1;
         while (s + 3 < nstage) {
-            row_filter(va, tw, list, count, s, tid);
-            row_load_clamped(va, x, n4, s + 3, tid);
-            row_filter(vb, tw, list, count, s + 1, tid);
-            row_load_clamped(vb, x, n4, s + 4, tid);
-            row_filter(vc, tw, list, count, s + 2, tid);
-            row_load_clamped(vc, x, n4, s + 5, tid);
+            row_filter_perm<G::WCAP>(vb, tw, list, count, m, s, V);
+            row_load_perm(vb, x, m, s + 3);
+            row_filter_perm<G::WCAP>(vc, tw, list, count, m, s + 1, V);
+            row_load_perm(vc, x, m, s + 4);
+            row_filter_perm<G::WCAP>(va, tw, list, count, m, s + 2, V);
+            row_load_perm(va, x, m, s + 5);
             s += 3;
             tighten();
         }
         if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T)); // the threshold is final
-        auto last_stages = [&](const f32x4 (&v)[ROW_U], int st) {
-            if (st >= nstage) return;                                // wave-uniform
-            if (st < nfull) row_filter(v, tw, list, count, st, tid); else row_filter_masked(v, tw, list, count, st, tid, V);
-        };
-        last_stages(va, s);
-        last_stages(vb, s + 1);
-        last_stages(vc, s + 2);
+        if (s < nstage) row_filter_perm<G::WCAP>(vb, tw, list, count, m, s, V);          // wave-uniform conditions
+        if (s + 1 < nstage) row_filter_perm<G::WCAP>(vc, tw, list, count, m, s + 1, V);
+        if (s + 2 < nstage) row_filter_perm<G::WCAP>(va, tw, list, count, m, s + 2, V);
     } else {
         // rows that 128-bit loads cannot take: one stage at a time, then one raise of the threshold
-        row_filter(va, tw, list, count, 0, tid);
+        row_filter_seq<G::WCAP>(va, tw, list, count, 0, tid);
         for (int s = 1; s < nstage; s++) {
             row_load_any<false>(va, x, V, s, tid);
-            row_filter(va, tw, list, count, s, tid);
+            row_filter_seq<G::WCAP>(va, tw, list, count, s, tid);
         }
         tighten();
         if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));
     }
-    if (count > (u32)ROW_WCAP && lane_id() == 0) s_over = 1;
-    const int cw = (int)min(count, (u32)ROW_WCAP);
+    if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
+    const int cw = (int)min(count, (u32)G::WCAP);
     ROW_STAMP(1);
 #ifdef BORN_PHASE_TIMING
     __shared__ u64 s_wend[ROW_WAVES];
@@ -598,12 +685,12 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
         for (int e = lane_id(); e < cw; e += WAVE) {
             const u32 pos = base + (u32)e;
-            if (pos < (u32)ROW_CAP) {
+            if (pos < (u32)G::CAP) {
                 const uint2 c = list[e];
                 C[pos] = c;
                 if (!fast) {                                         // a long history probes a hash of the candidate ids
-                    u32 slot = row_hash(c.y);
-                    while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (ROW_SLOTS - 1);
+                    u32 slot = G::hash(c.y);
+                    while (atomicCAS(&tab[slot], 0u, pos + 1u) != 0u) slot = (slot + 1) & (G::SLOTS - 1);
                 }
             }
         }
@@ -611,7 +698,11 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __syncthreads();
     ROW_STAMP(2);
     const int n = s_n;
-    bool ok = have_tw && !s_over && n >= k && n <= ROW_CAP;
+    bool ok = have_tw && !s_over && n >= k && n <= G::CAP;
+    // top_k beyond TOPK_SMALL_K: the candidates are ranked through buckets of z (below), whose counters take the
+    // threshold rounds' first set of bins (no round runs any more)
+    const bool bucketed = KC == 1 && k > TOPK_SMALL_K;
+    if (bucketed && tid < ROW_TBINS) s_bins[0][tid] = 0u;
     if (!fast) {
         // report ids out of range, flag the candidates that were already emitted
         for (int i = tid; i < hlen; i += ROW_BLOCK) {
@@ -621,7 +712,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
                 continue;
             }
             if (!ok) continue;
-            u32 slot = row_hash((u32)tk);
+            u32 slot = G::hash((u32)tk);
             for (;;) {
                 const u32 e = tab[slot];
                 if (e == 0u) break;
@@ -630,13 +721,15 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
                     if (local) atomicAdd(&ccnt[e - 1], 1u);
                     break;
                 }
-                slot = (slot + 1) & (ROW_SLOTS - 1);
+                slot = (slot + 1) & (G::SLOTS - 1);
             }
         }
         __syncthreads();
     }
     // ---- exact z and rank key of every candidate, one thread each
-    if (ok && tid < n) {
+    u32 zkey = 0u;
+    const bool cand = ok && tid < n;
+    if (cand) {
         const uint2 c = C[tid];
         float y = __uint_as_float(c.x);
         bool seen = (c.y & 0x80000000u) != 0u;
@@ -660,17 +753,69 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             y = penalise_counted(y, a.rep, counted, occ, a.freq, a.pres);
         }
         const float z = z_of(y, a.T);
+        zkey = ordkey(z);
         K[tid] = make_key64(z, (int)(c.y & 0x7FFFFFFFu));
-        Khi[tid] = ordkey(z);
-        const int nk = __popcll(__ballot(ordkey(z) > zb));           // the active lanes of this wave
+        Khi[tid] = zkey;
+        const int nk = __popcll(__ballot(zkey > zb));                // the active lanes of this wave
         if (nk && lane_id() == 0) atomicAdd(&s_valid, nk);           // (lane 0 is active whenever a lane of its wave is)
     }
     if (ok && tid >= n && tid < ((n + 31) & ~31)) Khi[tid] = 0u;     // the rank sort reads z in groups of 32: below any real one
+    if (bucketed && ok && tid < ((n + WAVE - 1) & ~(WAVE - 1))) {    // whole waves: the span of z among the candidates
+        const u32 mx = wave_max_u32(cand ? zkey : 0u), mn = wave_min_u32(cand ? zkey : 0xFFFFFFFFu);
+        if (lane_id() == 0) {
+            atomicMax(&s_kmax, mx);
+            atomicMin(&s_kmin, mn);
+        }
+    }
     __syncthreads();
     ROW_STAMP(3);
     ok = ok && s_valid >= k;
     if (!ok) {                                                       // wave-uniform, workgroup-uniform
-        row_select_exact<VEC, LOCAL>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
+        row_select_exact<VEC, LOCAL, G>(a, row, x, hlen, h, u_row, pool, &s_n, s_x);
+        return;
+    }
+
+    if (bucketed) {
+        // ---- rank through buckets: a candidate's rank is the number of candidates in the buckets of larger z plus its
+        // rank inside its own bucket, found by comparing whole keys (z descending, id ascending; unique) with the few
+        // dozen candidates that share the bucket.  Counting against all n candidates, as below, is n * n compares:
+        // several microseconds at top_k 512.
+        u32 *const cnt = s_bins[0], *const start = s_bins[1];
+        u64 *const grouped = pool + G::OFF_L;                        // (the lists have been moved out)
+        const u32 kmax = s_kmax, range = kmax - s_kmin;
+        const int sh = max(0, 24 - (int)__clz(range));               // (range >> sh) < ROW_TBINS
+        u32 bkt = 0u, pos = 0u;
+        u64 key = 0ull;
+        if (tid < n) {
+            key = K[tid];
+            bkt = (kmax - zkey) >> sh;                               // bucket 0 holds the largest z
+            pos = atomicAdd(&cnt[bkt], 1u);
+        }
+        __syncthreads();
+        if (tid < WAVE) {                                            // where each bucket starts in rank order
+            const uint4 c4 = reinterpret_cast<const uint4 *>(cnt)[tid];
+            const u32 s4 = c4.x + c4.y + c4.z + c4.w;
+            const u32 ex = wave_inclusive_scan_u32(s4) - s4;
+            reinterpret_cast<uint4 *>(start)[tid] = make_uint4(ex, ex + c4.x, ex + c4.x + c4.y, ex + c4.x + c4.y + c4.z);
+        }
+        __syncthreads();
+        u32 st = 0u;
+        if (tid < n) {
+            st = start[bkt];
+            grouped[st + pos] = key;
+        }
+        __syncthreads();
+        if (tid < n) {
+            const u32 c = cnt[bkt];
+            u32 r = st;
+            for (u32 j = 0; j < c; j++) r += grouped[st + j] > key ? 1u : 0u;
+            if (r < (u32)k) sorted[r] = key;
+        }
+        __syncthreads();
+        ROW_STAMP(6);
+        if (tid >= WAVE) return;
+        finish_sorted_by_wave(sorted, k, a, row, u_row);
+        ROW_STAMP(7);
         return;
     }
 
@@ -734,13 +879,14 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 // the unfused pair for those calls.
 // ---------------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const float *thr, const unsigned *cand_cnt, const uint2 *cand, int cap) {
-    __shared__ u64 pool[ROW_POOL];
-    uint2 *const L = reinterpret_cast<uint2 *>(pool + OFF_L);
-    uint2 *const C = reinterpret_cast<uint2 *>(pool + OFF_C);
-    u64 *const K = pool + OFF_K;
-    u32 *const Khi = reinterpret_cast<u32 *>(pool + OFF_TAB);
-    u64 *const sorted = pool + OFF_SORTED;
-    u32 *const htab = reinterpret_cast<u32 *>(pool + OFF_HTAB);
+    using G = RowGeom<2>;
+    __shared__ u64 pool[G::PROOF_END];
+    uint2 *const L = reinterpret_cast<uint2 *>(pool + G::OFF_L);
+    uint2 *const C = reinterpret_cast<uint2 *>(pool + G::OFF_C);
+    u64 *const K = pool + G::OFF_K;
+    u32 *const Khi = reinterpret_cast<u32 *>(pool + G::OFF_TAB);
+    u64 *const sorted = pool + G::OFF_SORTED;
+    u32 *const htab = reinterpret_cast<u32 *>(pool + G::OFF_HTAB);
     __shared__ u32 s_wmax[ROW_WAVES];
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
     __shared__ u32 s_max[2];
@@ -763,10 +909,10 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         s_max[0] = 0u;
         s_max[1] = 0u;
     }
-    for (int i = tid; i < ROW_SLOTS; i += ROW_BLOCK) Khi[i] = 0u;
+    for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) Khi[i] = 0u;
     for (int i = tid; i < ROW_HSLOTS; i += ROW_BLOCK) htab[i] = 0u;
     if (tid < ROW_TBINS) s_bins[0][tid] = 0u;
-    if (tid < TOPK_MAX_K) sorted[tid] = 0ull;
+    if (tid < G::MAXK) sorted[tid] = 0ull;
     // ids of the history outside the vocabulary are reported whatever becomes of the row
     for (int i = tid; i < hlen; i += ROW_BLOCK) {
         const int t = i == tid ? h0 : h[i];
@@ -801,8 +947,8 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
     }
     const u32 max0 = wave_max_u32(lane_id() < ROW_WAVES ? s_wmax[lane_id()] : 0u);
     u32 twkey = ordkey(t0);                                          // every logit outside the list has a smaller key
-    const int want = k + ROW_MARGIN;
-    uint2 *list = L + wave_id() * ROW_WCAP;
+    const int want = k + row_margin(k);
+    uint2 *list = L + wave_id() * G::WCAP;
     u32 count = 0;
     int round = 0;
     for (unsigned base = 0; base < cnt; base += ROW_BLOCK) {         // workgroup-uniform
@@ -816,26 +962,26 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         const u64 m = __ballot(pass);
         if (pass) {
             const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
-            if (pos < (u32)ROW_WCAP) list[pos] = c;
+            if (pos < (u32)G::WCAP) list[pos] = c;
         }
         count += (u32)__popcll(m);
         const u32 smax = max(max0, s_max[round & 1]);
-        row_tighten(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+        row_tighten<G::WCAP>(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
         round++;
     }
-    if (count > (u32)ROW_WCAP && lane_id() == 0) s_over = 1;
-    const int cw = (int)min(count, (u32)ROW_WCAP);
+    if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
+    const int cw = (int)min(count, (u32)G::WCAP);
     const u32 zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));       // bound of z for everything outside the lists
     {
         u32 base = 0u;
         if (lane_id() == 0 && cw) base = (u32)atomicAdd(&s_n, cw);
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
         for (int e = lane_id(); e < cw; e += WAVE)
-            if (base + (u32)e < (u32)ROW_CAP) C[base + e] = list[e];
+            if (base + (u32)e < (u32)G::CAP) C[base + e] = list[e];
     }
     __syncthreads();
     const int n = s_n;
-    bool ok = !s_over && n >= k && n <= ROW_CAP;
+    bool ok = !s_over && n >= k && n <= G::CAP;
     if (ok && tid < n) {                                             // exact z and rank key of every candidate
         const uint2 c = C[tid];
         float y = __uint_as_float(c.x);
@@ -899,17 +1045,19 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
     if (tid == 0) count_row(a.counters, row, 0);
 }
 
+
 hipError_t launch_cand_rows(const SampleArgs &a, const float *thr, const unsigned *cand_cnt, const uint2 *cand, int cand_cap,
                             hipStream_t st) {
     hipLaunchKernelGGL(cand_row_kernel, dim3((unsigned)a.B), dim3(ROW_BLOCK), 0, st, a, thr, cand_cnt, cand, cand_cap);
     return hipGetLastError();
 }
 
-template <bool VEC, bool LOCAL>
+template <bool VEC, bool LOCAL, int KC>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_kernel(SampleArgs a) {
-    topk_row_body<VEC, LOCAL>(a);
+    topk_row_body<VEC, LOCAL, KC>(a);
 }
-// The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
+// The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.  A row
+// may ask for any top_k the kernel serves, so these instances have the larger sizes.
 template <bool VEC, bool LOCAL>
 __global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, RowConfigs rc) {
     bool invalid;
@@ -918,16 +1066,21 @@ __global__ __launch_bounds__(ROW_BLOCK) void topk_row_rows_kernel(SampleArgs a, 
         row_config_reject(a, (int)blockIdx.x);
         return;
     }
-    topk_row_body<VEC, LOCAL>(a);
+    topk_row_body<VEC, LOCAL, 1>(a);
 }
+
+template <int KC>
+constexpr size_t row_pool_bytes() { return (size_t)RowGeom<KC>::POOL * sizeof(u64); }
 
 template <bool VEC, bool LOCAL>
 static void launch_topk_row_as(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
     const dim3 gr((unsigned)a.B), bl(ROW_BLOCK);
     if (rows)
-        hipLaunchKernelGGL((topk_row_rows_kernel<VEC, LOCAL>), gr, bl, 0, st, a, *rows);
+        hipLaunchKernelGGL((topk_row_rows_kernel<VEC, LOCAL>), gr, bl, row_pool_bytes<1>(), st, a, *rows);
+    else if (a.top_k > TOPK_SMALL_K)
+        hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL, 1>), gr, bl, row_pool_bytes<1>(), st, a);
     else
-        hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL>), gr, bl, 0, st, a);
+        hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL, 0>), gr, bl, row_pool_bytes<0>(), st, a);
 }
 
 hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
@@ -938,6 +1091,27 @@ hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs
         if (a.local_counts) launch_topk_row_as<false, true>(a, st, rows); else launch_topk_row_as<false, false>(a, st, rows);
     }
     return hipGetLastError();
+}
+
+// The LDS pools are dynamic allocations beyond 64 KiB: every instance is told so once.
+template <bool VEC, bool LOCAL>
+static hipError_t configure_topk_row_as() {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(topk_row_kernel<VEC, LOCAL, 0>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)row_pool_bytes<0>());
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(topk_row_kernel<VEC, LOCAL, 1>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)row_pool_bytes<1>());
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(topk_row_rows_kernel<VEC, LOCAL>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)row_pool_bytes<1>());
+    return e;
+}
+hipError_t configure_topk_row() {
+    hipError_t e = configure_topk_row_as<true, false>();
+    if (e == hipSuccess) e = configure_topk_row_as<true, true>();
+    if (e == hipSuccess) e = configure_topk_row_as<false, false>();
+    if (e == hipSuccess) e = configure_topk_row_as<false, true>();
+    return e;
 }
 
 }  // namespace born

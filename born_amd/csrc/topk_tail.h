@@ -123,10 +123,90 @@ __device__ __forceinline__ void finish_sorted_wave2(const u64 *list, int ns, con
     }
 }
 
-// One survivor per lane up to a wave of them, two beyond.
+// The same for ns <= N * 64 survivors: lane l holds entries N * l .. N * l + N - 1 and their running sum, the scan runs
+// over the lane totals.
+template <int N>
+__device__ __forceinline__ void finish_sorted_waveN(const u64 *list, int ns, const SampleArgs &a, int row, float u) {
+    const int l = lane_id();
+    const float m = key64_z(list[0]);
+    const float scale = mass_scale(a.mass_shift);
+    float e[N];
+    u64 cum[N], key[N];
+    bool live[N];
+    u64 lane_total = 0ull;
+#pragma unroll
+    for (int t = 0; t < N; t++) {
+        const int i = N * l + t;
+        live[t] = false;
+        e[t] = 0.0f;
+        key[t] = 0ull;
+        if (i < ns) {
+            key[t] = list[i];
+            const float z = key64_z(key[t]);
+            const float d = (z == m) ? 0.0f : m - z;
+            live[t] = d <= a.dcut;
+            e[t] = expneg(d, a.dcut);
+            lane_total += qfix(e[t], scale);
+        }
+        cum[t] = lane_total;
+    }
+    const u64 incl = wave_inclusive_scan_u62(lane_total);           // (a row's masses sum below 2^62)
+    const u64 excl = incl - lane_total;
+#pragma unroll
+    for (int t = 0; t < N; t++) cum[t] += excl;
+    const u64 Zk = readlane_u64(incl, WAVE - 1);
+    int np = ns;
+    if (a.dcut < 80.0f) {                                            // min-p: its survivors are a prefix of the rank order
+        np = 0;
+#pragma unroll
+        for (int t = 0; t < N; t++) np += __popcll(__ballot(live[t]));
+    }
+    u64 Zp = Zk;
+    if (a.top_p < 1.0f) {
+        const u64 tp = top_p_target(a.top_p, Zk);
+        int c = 0;
+#pragma unroll
+        for (int t = 0; t < N; t++) c += __popcll(__ballot(N * l + t < np && cum[t] < tp));
+        np = c + 1;
+    }
+    if (np < ns || a.top_p < 1.0f) {                                 // the normaliser of the first np survivors
+        const int last = __builtin_amdgcn_readfirstlane(np - 1);
+        u64 mine = 0ull;
+#pragma unroll
+        for (int t = 0; t < N; t++) mine = (N * l + t == last) ? cum[t] : mine;
+        Zp = readlane_u64(mine, last / N);
+    }
+    const u64 td = draw_target(u, Zp);
+    int pick = 0;
+#pragma unroll
+    for (int t = 0; t < N; t++) pick += __popcll(__ballot(N * l + t < np && cum[t] < td));
+#pragma unroll
+    for (int t = 0; t < N; t++) {
+        const int i = N * l + t;
+        if (i == pick) {
+            a.tokens[row] = key64_id(key[t]);
+            if (a.probs) a.probs[row] = prob_of(e[t], Zp, a.mass_shift);
+        }
+        if (a.nuc_len && i < np && i < a.nuc_cap) {
+            a.nuc_ids[(long long)row * a.nuc_cap + i] = key64_id(key[t]);
+            a.nuc_probs[(long long)row * a.nuc_cap + i] = prob_of(e[t], Zp, a.mass_shift);
+        }
+    }
+    if (a.nuc_len) {
+        if (l == 0) a.nuc_len[row] = np;
+        for (int i = np + l; i < a.nuc_cap; i += WAVE) {
+            a.nuc_ids[(long long)row * a.nuc_cap + i] = -1;
+            a.nuc_probs[(long long)row * a.nuc_cap + i] = 0.0f;
+        }
+    }
+}
+
+// One survivor per lane up to a wave of them, two up to 128, four and eight beyond (ns <= 512).
 __device__ __forceinline__ void finish_sorted_by_wave(const u64 *list, int ns, const SampleArgs &a, int row, float u) {
     if (ns <= WAVE) finish_sorted_wave(list, ns, a, row, u);
-    else finish_sorted_wave2(list, ns, a, row, u);
+    else if (ns <= 2 * WAVE) finish_sorted_wave2(list, ns, a, row, u);
+    else if (ns <= 4 * WAVE) finish_sorted_waveN<4>(list, ns, a, row, u);
+    else finish_sorted_waveN<8>(list, ns, a, row, u);
 }
 
 }  // namespace born

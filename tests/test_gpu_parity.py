@@ -158,7 +158,7 @@ def test_softmax_operators(oracle, rocm):
 
 
 # ---------------------------------------------------------------- sampling: single-pass top-k kernel
-# path 0 = the default kernel selection (1 <= top_k <= 128: one workgroup per row, one launch)
+# path 0 = the default kernel selection (1 <= top_k <= 512: one workgroup per row, one launch)
 
 TOPK_PATHS = [0]
 
@@ -180,13 +180,22 @@ TOPK_PATHS = [0]
     (9, 777, 0.9, 127, 0.99, 1.5, 2000),
     (4, 200, 1.0, 128, 0.9, 1.1, 10),            # a row of one wave: no first-stage threshold for top_k > 64
     (4, 129, 0.8, 128, 0.7, 1.0, 0),
+    (32, 128256, 0.7, 129, 0.9, 1.15, 512),      # beyond 128: ranked through buckets, four survivors per lane
+    (32, 128256, 0.7, 256, 0.9, 1.15, 512),
+    (32, 128256, 0.7, 512, 0.9, 1.15, 512),      # eight survivors per lane
+    (16, 32000, 1.0, 257, 1.0, 1.0, 0),
+    (16, 50257, 1.1, 400, 0.95, 1.2, 1500),      # history longer than the workgroup
+    (9, 2000, 0.9, 512, 0.99, 1.5, 3000),        # a quarter of the vocabulary survives the cut
+    (9, 777, 0.9, 300, 0.99, 1.5, 2000),
+    (4, 600, 0.8, 512, 0.7, 1.0, 0),             # a row of three waves: no first-stage threshold
+    (6, 16385, 0.7, 333, 0.9, 1.3, 64),          # one element in the second stage
 ])
 def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
     rng = np.random.default_rng(B * 1000003 + V)
     x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
-    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(128, max(k, 1)), path=path)
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(512, max(k, 1)), path=path)
     c = got["counters"]
     if rep < 1.0 and H:          # a boosting penalty is served by the general kernel
         assert c["general_rows"] == B
@@ -274,7 +283,7 @@ def test_topk_kernel_rows_that_stress_the_streamed_threshold(oracle, rocm, kind,
     u = rng.random(B, dtype=np.float32)
     top = np.argsort(-x, axis=1, kind="stable")[:, :H // 2].astype(np.int32)      # half the history penalises the winners
     hist = np.concatenate([top, rng.integers(0, V, size=(B, H - H // 2)).astype(np.int32)], axis=1)
-    for k, p, rep in [(50, 0.9, 1.3), (128, 1.0, 1.0), (1, 1.0, 2.0)]:
+    for k, p, rep in [(50, 0.9, 1.3), (128, 1.0, 1.0), (1, 1.0, 2.0), (300, 0.95, 1.2)]:
         want = oracle.sample(x, u, 0.7, k, p, rep, hist if rep != 1.0 else None, mode=oracle.MODE_FIXED, nuc_cap=min(k, 64))
         s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.7, TopK=k, TopP=p, RepetitionPenalty=rep), max_batch=B, max_vocab=V)
         xp = np.full((B, V + pad), 1e38, np.float32)                                  # padding must never be read as data
@@ -321,17 +330,17 @@ def test_kernel_selection_by_shape(oracle, rocm):
 
 
 # ---------------------------------------------------------------- sampling: kernel without a top-k cut (path 0, top_k 0)
-# and the general kernel (path 0 for top_k > 128, path 1 for everything)
+# and the general kernel (path 0 for top_k > 512, path 1 for everything)
 
 @pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("B,V,T,k,p,rep,H", [
     (64, 32000, 1.0, 0, 1.0, 1.0, 0),            # C2 multinomial shape
     (16, 152064, 1.2, 0, 0.99, 1.05, 2048),      # C5 shape, 16 rows
-    (16, 32000, 0.9, 500, 0.9, 1.1, 64),         # top_k above the single-pass limit
+    (16, 32000, 0.9, 700, 0.9, 1.1, 64),         # top_k above the single-pass limit
     (8, 50000, 1.0, 20000, 0.8, 1.0, 0),         # top_k too large to list: count descent
     (8, 50000, 1.0, 20000, 1.0, 1.0, 0),
     (16, 4097, 0.6, 0, 0.3, 1.0, 0),
-    (16, 1000, 2.0, 200, 1.0, 1.2, 50),
+    (16, 1000, 2.0, 600, 1.0, 1.2, 50),
     (5, 2, 1.0, 0, 0.9, 1.0, 0),
     (5, 1, 1.0, 0, 0.9, 1.0, 0),
 ])
@@ -390,7 +399,7 @@ def test_min_p_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, min_p, path):
     x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.0)).astype(np.float32)
     u = rng.random(B, dtype=np.float32)
     hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
-    nuc = k if 1 <= k <= 128 else 0
+    nuc = k if 1 <= k <= 512 else 0
     _, fx, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=nuc, path=path, min_p=min_p)
     if nuc and min_p >= 0.05:
         assert (fx["n_nucleus"] < k).any(), "the case is meant to have min-p bind"
@@ -437,7 +446,8 @@ def test_min_p_is_validated(rocm):
     (16, 32000, 1.0, 20, 0.9, 1.1, 128, -0.4, 0.2, "general"),   # a negative penalty raises logits: general kernel
     (16, 32000, 1.0, 0, 1.0, 1.0, 256, 0.4, 0.4, "nucleus"),     # no top-k: three-sweep kernel
     (16, 152064, 1.2, 0, 0.99, 1.05, 2048, 0.1, 0.6, "nucleus"), # C5 shape
-    (16, 32000, 0.9, 500, 0.9, 1.1, 64, 0.25, 0.25, "general"),
+    (16, 32000, 0.9, 500, 0.9, 1.1, 64, 0.25, 0.25, "topk"),       # beyond 128: the single-pass kernel's larger sizes
+    (16, 32000, 0.9, 700, 0.9, 1.1, 64, 0.25, 0.25, "general"),
     (8, 50000, 1.0, 20000, 0.8, 1.0, 300, 0.5, 0.5, "general"),
     (8, 1001, 1.0, 0, 0.9, 1.0, 5000, 0.05, 1.0, "nucleus"),     # unaligned rows, history much longer than the vocabulary
     (8, 1001, 1.0, 10, 0.9, 1.0, 5000, 0.05, 1.0, "topk"),
@@ -453,14 +463,14 @@ def test_frequency_and_presence_penalties_against_oracle(oracle, rocm, B, V, T, 
     hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)        # heavy repeats of the small ids
     x[:, :8] += np.float32(4.0)                                             # ... which are also the likely tokens
     hist_len = rng.integers(H // 2, H + 1, size=B).astype(np.int32)
-    nuc = k if 1 <= k <= 128 else 0
+    nuc = k if 1 <= k <= 512 else 0
     got, fx, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, hist_len, nuc=nuc, path=path, freq=freq, pres=pres)
     plain = oracle.sample(x, u, T, k, p, rep, hist, hist_len, mode=oracle.MODE_FIXED)
     assert (plain["tokens"] != fx["tokens"]).any() or not np.array_equal(plain["probs"], fx["probs"]), "the penalties are meant to matter"
     c = got["counters"]
     if path != 1 and route == "topk":
         assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
-    if path != 1 and route == "general" and 1 <= k <= 128:
+    if path != 1 and route == "general":
         assert c["general_rows"] == B
 
 
@@ -915,7 +925,7 @@ def _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path=0, min_ps=None, freqs=
 
 @pytest.mark.parametrize("path", [0, 1, 2])
 def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
-    # one batch, every row its own settings, covering the three kernels' territories (top-k <= 128, no top-k cut,
+    # one batch, every row its own settings, covering the three kernels' territories (top-k <= 512, no top-k cut,
     # top-k > 64, a boosting penalty < 1); each row must equal the oracle under that row's settings
     rng = np.random.default_rng(77)
     B, V, H = 24, 9000, 48
@@ -923,7 +933,7 @@ def test_per_row_configurations_match_per_row_handles(oracle, rocm, path):
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, (B, H)).astype(np.int32)
     Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
-    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 300, V, V + 5, -3], B).astype(np.int32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 300, 512, 513, 900, V, V + 5, -3], B).astype(np.int32)
     ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
     reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
     s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path)
@@ -957,7 +967,7 @@ def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq
     u = rng.random(B, dtype=np.float32)
     hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
     Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
-    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 129, 300, V], B).astype(np.int32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 129, 300, 512, 700, V], B).astype(np.int32)
     ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
     reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
     s, tok, pr = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, MinP=min_p, FrequencyPenalty=freq, PresencePenalty=pres)
@@ -983,7 +993,7 @@ def test_per_row_min_p_and_additive_penalties(oracle, rocm, path):
     u = rng.random(B, dtype=np.float32)
     hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
     Ts = rng.choice([0.5, 0.7, 1.0, 1.3], B).astype(np.float32)
-    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 129, 300, V], B).astype(np.int32)
+    ks = rng.choice([0, 1, 5, 40, 64, 65, 128, 129, 300, 512, 700, V], B).astype(np.int32)
     ps = rng.choice([1.0, 0.9, 0.5, 0.99], B).astype(np.float32)
     reps = rng.choice([1.0, 1.15, 2.0, 0.8], B).astype(np.float32)
     mps = rng.choice([0.0, 0.0, 0.01, 0.1, 0.5], B).astype(np.float32)
@@ -1038,16 +1048,16 @@ def test_per_row_promised_kinds_of_row(oracle, rocm, path):
                              mode=oracle.MODE_FIXED)["tokens"][0]
 
     # every row a small top-k, and the caller says so: only the single-pass kernel runs (under path 1 the general one)
-    ks = rng.choice([1, 5, 40, 64, 90, 128], B).astype(np.int32)
+    ks = rng.choice([1, 5, 40, 64, 90, 128, 200, 512], B).astype(np.int32)
     s, tok, _ = _sample_rows(rocm, x, u, hist, Ts, ks, ps, reps, path, row_kinds=_capi.ROWS_SMALL_TOP_K)
     s.Status()
     assert [int(t) for t in tok] == [int(want(b, ks[b])) for b in range(B)]
     c = s.Counters()
     assert (c["general_rows"] == 0) if path != 1 else (c["topk_rows"] + c["fallback_rows"] == 0)
     s.Close()
-    # two kinds promised, a third occurs in rows 3 and 11 (top_k 300), and row 7 is invalid: those rows are reported
+    # two kinds promised, a third occurs in rows 3 and 11 (top_k 600), and row 7 is invalid: those rows are reported
     ks2 = rng.choice([0, 5, 50], B).astype(np.int32)
-    ks2[3] = ks2[11] = 300
+    ks2[3] = ks2[11] = 600
     Tbad = Ts.copy()
     Tbad[7] = -1.0
     s, tok, _ = _sample_rows(rocm, x, u, hist, Tbad, ks2, ps, reps, path, row_kinds=_capi.ROWS_SMALL_TOP_K | _capi.ROWS_NO_TOP_K)

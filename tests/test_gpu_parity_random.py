@@ -21,7 +21,7 @@ def _draw_case(rng):
     V = int(rng.choice([1, 2, 3, 7, 64, 65, 130, 257, 1000, 1001, 4095, 4096, 4100, 8193, 16388, 20000, 32000, 50257, 100003]))
     B = int(rng.integers(1, 9))
     T = float(rng.choice([0.25, 0.5, 0.7, 1.0, 1.0, 1.3, 2.0, 5.0]))
-    k = int(rng.choice([0, 0, 1, 2, 5, 40, 50, 64, 65, 100, 127, 128, 129, 1000, V, V + 3]))
+    k = int(rng.choice([0, 0, 1, 2, 5, 40, 50, 64, 65, 100, 127, 128, 129, 200, 256, 257, 400, 512, 513, 1000, V, V + 3]))
     p = float(rng.choice([1.0, 1.0, 0.99, 0.95, 0.9, 0.5, 0.1, 0.01]))
     rep = float(rng.choice([1.0, 1.0, 1.1, 1.5, 3.0, 0.8]))
     min_p = float(rng.choice([0.0, 0.0, 0.0, 0.01, 0.05, 0.3, 0.9]))

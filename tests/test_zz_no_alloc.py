@@ -56,7 +56,8 @@ def _both(rocm, cfg, x, u, h):
 @pytest.mark.parametrize("cfg_kw", [
     dict(Temperature=0.7, TopK=50, TopP=0.9, RepetitionPenalty=1.15),                       # the single-pass kernel
     dict(Temperature=1.2, TopP=0.95, RepetitionPenalty=1.05),                               # no top-k cut: the three-sweep kernel
-    dict(Temperature=0.9, TopK=300, TopP=0.9),                                              # the general kernel
+    dict(Temperature=0.9, TopK=300, TopP=0.9),                                              # the single-pass kernel's larger sizes
+    dict(Temperature=0.9, TopK=700, TopP=0.9),                                              # the general kernel
     dict(Temperature=0.8, TopK=40, TopP=0.95, FrequencyPenalty=0.3, PresencePenalty=0.2),   # occurrences counted in the kernel
 ])
 def test_static_entry_point_equals_the_handle_one_on_two_calls_in_a_row(rocm, oracle, cfg_kw):
