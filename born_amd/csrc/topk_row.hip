@@ -34,6 +34,9 @@
 // histories of at most TOPK_LOCAL_COUNT_HISTORY tokens the LOCAL instances count them where the
 // history is hashed anyway (the count rides in the high bits of the slot); otherwise the counts
 // come from a table by id that the caller's launches raise and clear around this one.
+#ifndef BORN_ROW_SCHED
+#define BORN_ROW_SCHED 1
+#endif
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
@@ -72,7 +75,7 @@ constexpr int TOPK_SMALL_K = 128;             // up to here the candidates are r
 //   KC 2: the finish over a list of candidates (cand_row_kernel).
 template <int KC>
 struct RowGeom {
-    static constexpr int WCAP = KC == 2 ? 256 : 512;                 // list entries per wave
+    static constexpr int WCAP = KC == 1 ? 768 : 256;                 // list entries per wave
     static constexpr int CAP = KC == 1 ? 1024 : 512;                 // candidates the finish can hold
     static constexpr int MAXK = KC == 1 ? TOPK_MAX_K : TOPK_SMALL_K; // largest top_k
     static constexpr int SLOTS = 2 * CAP;                            // hash slots of the candidates' ids (load factor <= 0.5)
@@ -127,83 +130,173 @@ __device__ __forceinline__ void row_load_fast(f32x4 (&v)[ROW_U], const float *x,
         v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + ((stage * ROW_U + u) * ROW_BLOCK + tid));
 }
 
-// Appends the elements >= tw of one float4 to the wave's list.  tw >= -FLT_MAX, so -inf and NaN never pass.  `count`
-// is wave-uniform; idof(c) is the id of element c (evaluated only for elements that pass); MASKED: elements whose id
-// is not below V count as -inf (the row's ragged end).
-template <int WCAP, bool MASKED, class IdOf>
-__device__ __forceinline__ void row_filter4(const f32x4 v, float tw, uint2 *list, u32 &count, int V, IdOf idof) {
+// Block indices clamped into the row: a stage that reaches past the row's end (or lies wholly beyond it) re-reads the
+// row's last block instead of branching around its loads, so that the loads of later stages can stay in flight (a load
+// under a condition makes the compiler wait for every load in flight).  The row starts 16-byte aligned and its pitch
+// is a multiple of four floats (VEC), so the last block lies inside the pitch.
+__device__ __forceinline__ void row_load_clamped(f32x4 (&v)[ROW_U], const float *x, int n4, int stage, int tid) {
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-        const float xv = v[c];
-        const bool pass = MASKED ? (xv >= tw && idof(c) < V) : (xv >= tw);
-        const u64 m = __ballot(pass);
-        if (m) {                                                     // wave-uniform
-            if (pass) {
-                const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
-                if (pos < (u32)WCAP) list[pos] = make_uint2(__float_as_uint(xv), (u32)idof(c));
+    for (int u = 0; u < ROW_U; u++) {
+        const int i4 = min((stage * ROW_U + u) * ROW_BLOCK + tid, n4 - 1);
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i4);
+    }
+}
+
+constexpr int ROW_TBINS = 256;                // bins of a threshold histogram (four per lane)
+static_assert(ROW_TBINS == 4 * WAVE && ROW_TBINS <= ROW_BLOCK, "one 128-bit read per lane covers the bins");
+
+// Second half of a raise of the threshold: H holds the number of the wave's own (or of all the lists') entries per bin
+// of (key - base) >> sh.  The highest bin boundary with at least `want` entries at or above it is a lower bound of the
+// row's want-th largest logit; returns its key, or 0 if the bins hold fewer than `want` entries.  Wave-uniform.
+__device__ __forceinline__ u32 row_bins_crossing(const u32 *H, int want, u32 base, int sh) {
+    const int l = lane_id();
+    const uint4 h = reinterpret_cast<const uint4 *>(H)[WAVE - 1 - l];   // lane 0 holds the four highest bins
+    const u32 s4 = h.x + h.y + h.z + h.w;
+    const u32 incl = wave_inclusive_scan_u32(s4);                    // entries in this lane's bins and all higher ones
+    const u32 total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
+    if (total < (u32)want) return 0u;
+    const int L = __ffsll((long long)__ballot(incl >= (u32)want)) - 1;   // the lane whose bins hold the crossing
+    const u32 excl = (u32)__builtin_amdgcn_readlane((int)(incl - s4), L);
+    const u32 hw = (u32)__builtin_amdgcn_readlane((int)h.w, L), hz = (u32)__builtin_amdgcn_readlane((int)h.z, L);
+    const u32 hy = (u32)__builtin_amdgcn_readlane((int)h.y, L);
+    const u32 need = (u32)want - excl;                               // >= 1
+    int bin = 4 * (WAVE - 1 - L) + 3;
+    u32 c = hw;
+    if (c < need) { bin--; c += hz; if (c < need) { bin--; c += hy; if (c < need) bin--; } }
+    return base + ((u32)bin << sh);                                  // at most the key of an entry of that bin: no overflow
+}
+// Drops the entries below key nk from the wave's own list, in place, four wave strides at a time: within a group every
+// read is issued before the first write, and a group writes only below the entries it has read.
+template <int WCAP>
+__device__ __forceinline__ void row_list_compact(uint2 *list, u32 &count, u32 nk) {
+    const int l = lane_id();
+    const int cw = (int)min(count, (u32)WCAP);
+    u32 kept = 0u;
+    for (int g = 0; g * WAVE < cw; g += 4) {                         // wave-uniform
+        uint2 ent[4];
+        bool keep[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int e = l + (g + r) * WAVE;
+            keep[r] = false;
+            if (e < cw) {
+                ent[r] = list[e];
+                keep[r] = ordkey(__uint_as_float(ent[r].x)) >= nk;
             }
-            count += (u32)__popcll(m);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            if ((g + r) * WAVE < cw) {                               // wave-uniform
+                const u64 m = __ballot(keep[r]);
+                if (keep[r]) list[kept + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u))] = ent[r];
+                kept += (u32)__popcll(m);
+            }
+        }
+    }
+    count = kept;
+}
+
+// Appends the logits >= tw of one stage to the wave's list.  tw >= -FLT_MAX, so -inf (the fill past the end of the row
+// included) and NaN never pass.  `count` is wave-uniform; entries beyond the list's capacity are counted, not stored.
+template <int WCAP>
+__device__ __forceinline__ void row_filter(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid) {
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float xv = v[u][c];
+            const bool pass = xv >= tw;
+            const u64 m = __ballot(pass);
+            if (m) {                                                 // wave-uniform
+                if (pass) {
+                    const u32 pos = count + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+                    if (pos < (u32)WCAP)
+                        list[pos] = make_uint2(__float_as_uint(xv), (u32)(((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c));
+                }
+                count += (u32)__popcll(m);
+            }
         }
     }
 }
 
-// Where the 128-bit loads of the pass lie.  The row is cut into chunks of WAVE float4 (what one wave instruction
-// loads, 1 KiB); stage s of the pass takes, for load u of wave w, chunk (u * ROW_WAVES + w) * nstage + s: the 64 chunks
-// of a stage are spread evenly over the row, so every stage is a sample of the whole row by position.  nstage * 64
-// chunk places cover the row; those at or beyond `cend` hold nothing, the one between `cfull` and `cend` (if any)
-// holds the row's ragged end.
-struct RowMap {
-    int nstage;                   // stages of the pass
-    int n4;                       // float4 blocks that hold an element of the row
-    int cfull, cend;              // chunks wholly inside the row; chunks that hold any element
-    int w, l;                     // this thread's wave (wave-uniform) and lane
-};
-#ifndef BORN_ROW_SEQUENTIAL
-__device__ __forceinline__ int row_chunk(const RowMap &m, int s, int u) { return (u * ROW_WAVES + m.w) * m.nstage + s; }
-#else
-// (measurement builds: the stages in row order)
-__device__ __forceinline__ int row_chunk(const RowMap &m, int s, int u) { return (s * ROW_U + u) * ROW_WAVES + m.w; }
-#endif
-// The loads of stage s.  A chunk place beyond the row (or a stage beyond the last) re-reads the row's last block
-// instead of branching around its load, so that the loads of later stages can stay in flight: a load under a
-// condition makes the compiler wait for every load in flight.  The row starts 16-byte aligned and its pitch is a
-// multiple of four floats, so the last block lies inside the pitch.
-__device__ __forceinline__ void row_load_perm(f32x4 (&v)[ROW_U], const float *x, const RowMap &m, int s) {
-    const int last = m.n4 - 1;
-    const int off = s < m.nstage ? m.l : m.n4;                       // (a stage past the last one: every lane reads the last block)
-#pragma unroll
-    for (int u = 0; u < ROW_U; u++) {
-        const int i4 = min(row_chunk(m, s, u) * WAVE + off, last);
-        v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x) + i4);
-    }
-}
-// Appends the logits >= tw of stage s to the wave's list.
+// A stage did not fit the wave's list (the row's large logits come late in row order: sorted ascending, a step up near
+// the end, a slow rise): the wave raises a threshold of its own, by itself, and examines the stage again.  The list's
+// first c0 entries (what it held before the stage) and the stage's logits >= the threshold, still in registers, are
+// all logits of the row and more than `want` of them, so the want-th largest of them is a lower bound of the row's
+// want-th largest logit: it becomes the wave's threshold, and the old entries below it are dropped.  Thresholds so
+// differ between waves; the bound of the proof is the largest of them.  W: 256 bins of the wave's own.  No barrier:
+// a wave's LDS traffic is in order.  Returns false if the keys at hand cannot be told apart (equal logits by the
+// hundred): the list stays overflowed and the row goes to the exact selection.
 template <int WCAP>
-__device__ __forceinline__ void row_filter_perm(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, const RowMap &m, int s, int V) {
-    bool whole = true;                                               // wave-uniform: every chunk of the wave's stage lies wholly inside the row
-#pragma unroll
-    for (int u = 0; u < ROW_U; u++) whole = whole && row_chunk(m, s, u) < m.cfull;
-    if (whole) {
-#pragma unroll
-        for (int u = 0; u < ROW_U; u++) {
-            const int ch = row_chunk(m, s, u);
-            row_filter4<WCAP, false>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
-        }
-    } else {
-#pragma unroll
-        for (int u = 0; u < ROW_U; u++) {
-            const int ch = row_chunk(m, s, u);
-            if (ch < m.cfull) row_filter4<WCAP, false>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
-            else if (ch < m.cend) row_filter4<WCAP, true>(v[u], tw, list, count, V, [&](int c) { return (ch * WAVE + m.l) * 4 + c; });
-        }
+__device__ __forceinline__ bool row_raise_from_stage(const f32x4 (&v)[ROW_U], uint2 *list, u32 &c0, u32 &twkey, int want, u32 *W) {
+    const int l = lane_id();
+    const float tw = ordkey_inv(twkey);
+    u32 mx = 0u, mn = 0xFFFFFFFFu;
+    for (int e = l; e < (int)c0; e += WAVE) {
+        const u32 key = ordkey(__uint_as_float(list[e].x));
+        mx = max(mx, key);
+        mn = min(mn, key);
     }
-}
-// The same for a stage in row order (rows that 128-bit loads cannot take; elements past the end were filled with -inf).
-template <int WCAP>
-__device__ __forceinline__ void row_filter_seq(const f32x4 (&v)[ROW_U], float tw, uint2 *list, u32 &count, int stage, int tid) {
 #pragma unroll
     for (int u = 0; u < ROW_U; u++)
-        row_filter4<WCAP, false>(v[u], tw, list, count, 0, [&](int c) { return ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c; });
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const u32 key = ordkey(v[u][c]);
+            if (v[u][c] >= tw) {
+                mx = max(mx, key);
+                mn = min(mn, key);
+            }
+        }
+    mx = wave_max_u32(mx);
+    mn = wave_min_u32(mn);
+    const int sh = max(0, 24 - (int)__clz(mx - mn));                 // ((mx - mn) >> sh) < ROW_TBINS
+    reinterpret_cast<uint4 *>(W)[l] = make_uint4(0u, 0u, 0u, 0u);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int e = l; e < (int)c0; e += WAVE) atomicAdd(&W[(ordkey(__uint_as_float(list[e].x)) - mn) >> sh], 1u);
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float xv = v[u][c];
+            asm volatile("" : "+v"(xv));                             // (keeps the keys of the first pass from being held in registers until here)
+            if (xv >= tw) atomicAdd(&W[(ordkey(xv) - mn) >> sh], 1u);
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const u32 nk = row_bins_crossing(W, want, mn, sh);
+    if (nk <= twkey) return false;
+    row_list_compact<WCAP>(list, c0, nk);
+    twkey = nk;
+    return true;
+}
+
+// One stage of the pass: its logits >= the wave's threshold join the wave's list; if they do not fit, the wave raises
+// its threshold and examines the stage again (the common case pays one scalar compare for this).  MASKED: the stage may
+// reach past the row's end; elements at or beyond V count as -inf.
+template <int WCAP, bool MASKED>
+__device__ __forceinline__ void row_stage(const f32x4 (&v)[ROW_U], float &tw, u32 &twkey, uint2 *list, u32 &count, int stage, int tid, int V,
+                                          int want, u32 *W) {
+    f32x4 m[ROW_U];
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) m[u][c] = (!MASKED || ((stage * ROW_U + u) * ROW_BLOCK + tid) * 4 + c < V) ? v[u][c] : -INFINITY;
+    u32 c0 = count;                                                  // (wave-uniform, <= WCAP unless an earlier stage gave up)
+    row_filter<WCAP>(m, tw, list, count, stage, tid);
+    if (__builtin_expect(count > (u32)WCAP, 0)) {
+        // (examined a second time by a second copy of the filter, not by a loop around one: inside a loop the compiler
+        // keeps the sixteen ids of the stage in registers)
+        if (c0 <= (u32)WCAP && row_raise_from_stage<WCAP>(m, list, c0, twkey, want, W)) {
+            tw = ordkey_inv(twkey);
+            count = c0;
+            int st = stage, t2 = tid;
+            asm volatile("" : "+v"(st), "+v"(t2));                   // (or the sixteen ids of the stage are kept in registers for this second use)
+            row_filter<WCAP>(m, tw, list, count, st, t2);            // (a second overflow stands: equal logits by the hundred,
+                                                                     // or logits around zero, where the bins of the key crowd)
+        }
+    }
 }
 
 // The need-th largest of the 16 wave results in `wthr` (LDS), computed redundantly by every wave in its first
@@ -381,86 +474,41 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
     }
 }
 
-constexpr int ROW_TBINS = 256;                // bins of the threshold histogram (four per lane)
-static_assert(ROW_TBINS == 4 * WAVE && ROW_TBINS <= ROW_BLOCK, "one 128-bit read per lane covers the bins");
-
-// Raises the threshold in the middle of the pass (every thread of the workgroup calls it, between two stages; global
-// loads stay in flight).  The lists hold every logit >= the threshold among the stages seen so far.  All of their
-// entries are binned by key distance above the threshold; the highest bin boundary with at least `want` entries at
-// or above it is a lower bound of the row's want-th largest logit, so it becomes the new threshold and every wave
-// drops the entries below it from its own list.  The bin width follows the largest key listed one round earlier
-// (`smax`: waves must agree on it, so it cannot be this round's); later, larger keys share the top bin.
+// Raises the common threshold in the middle of the pass (every thread of the workgroup calls it, between two stages;
+// global loads stay in flight).  The lists hold every logit >= the threshold among the stages seen so far (a wave that
+// raised its own threshold holds fewer: still logits of the row).  All of their entries are binned by key distance
+// above the common threshold `gkey`; the highest bin boundary with at least `want` entries at or above it is a lower
+// bound of the row's want-th largest logit, so it becomes the new common threshold, and every wave whose own
+// threshold `twkey` is lower adopts it and drops the entries below it from its own list.  The bin width follows the
+// largest key listed one round earlier (`smax`: waves must agree on it, so it cannot be this round's); later, larger
+// keys share the top bin.
 //   H: this round's bins (all zero on entry); Hclear: the next round's bins, zeroed here (with three sets in rotation
 //   they were last read two rounds ago, before the previous round's barrier);
 //   Mnext: where this round's largest key is published for the next round.
 template <int WCAP>
-__device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, int want, u32 smax, u32 *H, u32 *Hclear, u32 *Mnext,
-                                            int *s_over, int tid) {
+__device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, u32 &gkey, int want, u32 smax, u32 *H, u32 *Hclear,
+                                            u32 *Mnext, int *s_over, int tid) {
     const int l = lane_id();
     if (count > (u32)WCAP && l == 0) *s_over = 1;
     const int cw = (int)min(count, (u32)WCAP);
-    const u32 range = smax > twkey ? smax - twkey : 0u;
+    const u32 range = smax > gkey ? smax - gkey : 0u;
     const int sh = max(0, 24 - (int)__clz(range));                   // (range >> sh) < ROW_TBINS
     u32 mx = 0u;
     for (int e = l; e < cw; e += WAVE) {
         const u32 key = ordkey(__uint_as_float(list[e].x));
         mx = max(mx, key);
-        if (key >= twkey) atomicAdd(&H[min((key - twkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
+        if (key >= gkey) atomicAdd(&H[min((key - gkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
     }
     mx = wave_max_u32(mx);
     if (l == 0 && mx) atomicMax(Mnext, mx);
     if (tid < ROW_TBINS) Hclear[tid] = 0u;
     lds_barrier();
-    const uint4 h = reinterpret_cast<const uint4 *>(H)[WAVE - 1 - l];   // lane 0 holds the four highest bins
-    const u32 s4 = h.x + h.y + h.z + h.w;
-    const u32 incl = wave_inclusive_scan_u32(s4);                    // entries in this lane's bins and all higher ones
-    const u32 total = (u32)__builtin_amdgcn_readlane((int)incl, WAVE - 1);
-    if (total < (u32)want) return;                                   // wave-uniform, the same in every wave
-    const int L = __ffsll((long long)__ballot(incl >= (u32)want)) - 1;   // the lane whose bins hold the crossing
-    const u32 excl = (u32)__builtin_amdgcn_readlane((int)(incl - s4), L);
-    const u32 hw = (u32)__builtin_amdgcn_readlane((int)h.w, L), hz = (u32)__builtin_amdgcn_readlane((int)h.z, L);
-    const u32 hy = (u32)__builtin_amdgcn_readlane((int)h.y, L);
-    const u32 need = (u32)want - excl;                               // >= 1
-    int bin = 4 * (WAVE - 1 - L) + 3;
-    u32 c = hw;
-    if (c < need) { bin--; c += hz; if (c < need) { bin--; c += hy; if (c < need) bin--; } }
-    const u32 nk = twkey + ((u32)bin << sh);                         // at most the key of an entry of that bin: no overflow
-    if (nk <= twkey) return;
-    // in-place compaction of the wave's own list, four wave strides at a time: within a group every read is issued
-    // before the first write, and a group writes only below the entries it has read (kept <= the group's first entry)
-    u32 kept = 0u;
-    for (int g = 0; g * WAVE < cw; g += 4) {                         // wave-uniform
-        uint2 ent[4];
-        bool keep[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int e = l + (g + r) * WAVE;
-            keep[r] = false;
-            if (e < cw) {
-                ent[r] = list[e];
-                keep[r] = ordkey(__uint_as_float(ent[r].x)) >= nk;
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            if ((g + r) * WAVE < cw) {                               // wave-uniform
-                const u64 m = __ballot(keep[r]);
-                if (keep[r]) list[kept + __builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u))] = ent[r];
-                kept += (u32)__popcll(m);
-            }
-        }
-    }
-    count = kept;
+    const u32 nk = row_bins_crossing(H, want, gkey, sh);             // the same in every wave
+    if (nk <= gkey) return;
+    gkey = nk;
+    if (nk <= twkey) return;                                         // (this wave's own threshold is higher already)
+    row_list_compact<WCAP>(list, count, nk);
     twkey = nk;
-}
-
-// Waves whose first load of the first stage holds an element of the row.
-__device__ __forceinline__ int row_active_waves(const RowMap &m) {
-#ifndef BORN_ROW_SEQUENTIAL
-    return min(ROW_WAVES, (m.cend + m.nstage - 1) / m.nstage);
-#else
-    return min(ROW_WAVES, m.cend);
-#endif
 }
 
 // LOCAL: the frequency / presence penalties are on and the kernel counts the occurrences itself (SampleArgs::local_counts).
@@ -479,8 +527,9 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     u32 *const htab = reinterpret_cast<u32 *>(pool + G::OFF_HTAB);
     __shared__ u32 s_wthr[ROW_WAVES], s_wmax[ROW_WAVES];
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
+    __shared__ __align__(16) u32 s_wbins[ROW_WAVES][ROW_TBINS];      // a wave's own bins, for a raise of its own threshold
     __shared__ u32 s_max[2];
-    __shared__ u32 s_kmax, s_kmin;
+    __shared__ u32 s_kmax, s_kmin, s_twmax;
     __shared__ int s_n, s_valid, s_over, s_next;
     __shared__ int s_x[1 + ROW_WAVES];
 #ifdef BORN_PHASE_TIMING
@@ -504,24 +553,32 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int n4 = (V + 3) >> 2;
     const int iters = (n4 + ROW_BLOCK - 1) / ROW_BLOCK;             // float4 blocks per thread
     const int nstage = (iters + ROW_U - 1) / ROW_U;
-    RowMap m;
-    m.nstage = nstage;
-    m.n4 = n4;
-    m.cfull = V / (4 * WAVE);
-    m.cend = (V + 4 * WAVE - 1) / (4 * WAVE);
-    m.w = __builtin_amdgcn_readfirstlane(wave_id());
-    m.l = lane_id();
+    const int nfull = (V >> 2) / (ROW_U * ROW_BLOCK);                // stages made of whole float4 blocks inside the row
 
     // Order of the requests: this thread's first history entry (used last, but loads return in order and it must
     // not wait behind the row), then the row's first three stages; the LDS tables are cleared behind them.
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
+    // The row's last stage is examined first, the others follow in row order: what raises the threshold fastest in a
+    // row whose large logits come late (sorted ascending, a step up near the end, a slow rise) is seen at once, and a
+    // row whose large logits come early meets them in the stage after.  Not when the last stage is too short to give
+    // every wave a full load: the first threshold comes from the first stage examined.
+    const int last = nstage - 1;
+#ifdef BORN_ROW_NO_LAST_FIRST
+    const bool last_first = false;                                   // (measurement builds)
+#else
+    const bool last_first = VEC && nstage > 1 && n4 - last * (ROW_U * ROW_BLOCK) >= ROW_BLOCK;
+#endif
+    const int first = last_first ? last : 0;
+    // the stage examined in place t >= 1 (a place past the last one: a stage past the row's end, whose loads all re-read
+    // the row's last block)
+    auto stage_at = [&](int t) { return last_first ? (t < nstage ? t - 1 : nstage) : t; };
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
     if (VEC) {
-        row_load_perm(va, x, m, 0);
-        row_load_perm(vb, x, m, 1);                                  // in flight during the search for the first threshold
-        row_load_perm(vc, x, m, 2);
+        row_load_clamped(va, x, n4, first, tid);
+        row_load_clamped(vb, x, n4, stage_at(1), tid);               // in flight during the search for the first threshold
+        row_load_clamped(vc, x, n4, stage_at(2), tid);
     } else {
         row_load_any<false>(va, x, V, 0, tid);
     }
@@ -535,6 +592,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         s_max[1] = 0u;
         s_kmax = 0u;
         s_kmin = 0xFFFFFFFFu;
+        s_twmax = 0u;
     }
     for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
     if (tid < ROW_TBINS) s_bins[0][tid] = 0u;                        // every round clears the bins of the next
@@ -559,29 +617,22 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 
     // ---- the first threshold, from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per
     // wave and the need = ceil(top_k / a)-th largest of the wave results
-    const int act = VEC ? row_active_waves(m) : min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
+    const int act = min(ROW_WAVES, (min(n4 - first * (ROW_U * ROW_BLOCK), ROW_BLOCK) + WAVE - 1) / WAVE);   // (its first load)
     const int aw = min(WAVE, (k + act - 1) / act);                   // lanes of one wave
     const int need = (k + aw - 1) / aw;                              // <= act, but for a top_k beyond the lanes that hold data: no threshold then
     {
         float lm = -INFINITY;
-        if (VEC) {
-#pragma unroll
-            for (int u = 0; u < ROW_U; u++) {
-                const int ch = row_chunk(m, 0, u);
-                if (ch < m.cfull) {                                  // wave-uniform
-#pragma unroll
-                    for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
-                } else if (ch < m.cend) {                            // the row's ragged end
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        if ((ch * WAVE + m.l) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
-                }
-            }
-        } else {                                                     // (elements past the end were filled with -inf)
+        if (!VEC || first < nfull) {                                 // (without 128-bit loads, elements past the end were filled with -inf)
 #pragma unroll
             for (int u = 0; u < ROW_U; u++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);
+                for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
+        } else {                                                     // the row ends inside this stage
+#pragma unroll
+            for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (((first * ROW_U + u) * ROW_BLOCK + tid) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
         }
         const u32 lk = ordkey(lm);
         const u32 wk = wave_kth_largest_bound(lk, aw, 14);
@@ -613,15 +664,18 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     float tw = have_tw ? ordkey_inv(twkey) : INFINITY;
     const int want = k + row_margin(k);                              // entries a raised threshold keeps at least
 
-    // ---- the pass over the row.  After the first stage and then every three stages the threshold is raised from what
-    // the lists hold by then, so that they end the pass with little more than `want` entries between them.
+    // ---- the pass over the row.  Every three stages the common threshold is raised from what the lists hold by then, so
+    // that they end the pass with little more than `want` entries between them.  A wave whose list cannot take a stage
+    // (the row's large logits come late in row order) raises a threshold of its own, `twkey` >= the common `gkey`.
     uint2 *list = L + wave_id() * G::WCAP;
+    u32 *const W = s_wbins[wave_id()];
     u32 count = 0;
+    u32 gkey = twkey;
     int round = 0;
     auto tighten = [&]() {
         if (have_tw) {                                               // workgroup-uniform
             const u32 smax = max(max0, s_max[round & 1]);
-            row_tighten<G::WCAP>(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
             tw = ordkey_inv(twkey);
             round++;
         }
@@ -629,47 +683,49 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // A history that fits the workgroup was hashed above and the candidates probe it; otherwise the candidates' ids are
     // hashed and the history probes them.
     const bool fast = !penal || hfast;
-    // A logit outside the lists has a key of at most twkey - 1 (twkey > the key of -inf, so that is the key of a float
-    // or of -inf), and so has its z: a penalty only lowers a logit and the division by the temperature is monotone.
-    // The row is proven if top_k candidates have z strictly above that bound.
-    u32 zb = 0u;
     if (VEC) {
-        // va, vb, vc = stages 0, 1, 2 are requested: two stages stay in flight while one is examined.  The first stage is
-        // an even sample of the row like every other, and the threshold the counting argument drew from it can be far
-        // below what the stage's own logits allow (a few waves may hold all the large ones): it is raised at once.
-        row_filter_perm<G::WCAP>(va, tw, list, count, m, 0, V);
-        row_load_perm(va, x, m, 3);
-#ifndef BORN_ROW_NO_ROUND0
-        tighten();
-#endif
-        // at the loop head vb, vc, va = stages s, s + 1, s + 2
-        int s = 1;
-        while (s + 3 < nstage) {
-            row_filter_perm<G::WCAP>(vb, tw, list, count, m, s, V);
-            row_load_perm(vb, x, m, s + 3);
-            row_filter_perm<G::WCAP>(vc, tw, list, count, m, s + 1, V);
-            row_load_perm(vc, x, m, s + 4);
-            row_filter_perm<G::WCAP>(va, tw, list, count, m, s + 2, V);
-            row_load_perm(va, x, m, s + 5);
+        // va, vb, vc hold places s, s + 1, s + 2 of the order of examination: two stages stay in flight while one is
+        // examined.  Only the row's last stage may reach past its end: it is examined under a mask, in place 0 or in one
+        // of the last places, which are kept out of the loop (so that the loop's stages are all of one kind).
+        auto examine = [&](const f32x4 (&v)[ROW_U], int t) {
+            const int st = t == 0 ? first : stage_at(t);
+            if (st == last) row_stage<G::WCAP, true>(v, tw, twkey, list, count, st, tid, V, want, W);   // wave-uniform
+            else row_stage<G::WCAP, false>(v, tw, twkey, list, count, st, tid, V, want, W);
+        };
+        int s = 0;
+        if (nstage > 3) {                                            // (places 1 and 2 are not the row's last stage then)
+            examine(va, 0);
+            row_load_clamped(va, x, n4, stage_at(3), tid);
+            row_stage<G::WCAP, false>(vb, tw, twkey, list, count, stage_at(1), tid, V, want, W);
+            row_load_clamped(vb, x, n4, stage_at(4), tid);
+            row_stage<G::WCAP, false>(vc, tw, twkey, list, count, stage_at(2), tid, V, want, W);
+            row_load_clamped(vc, x, n4, stage_at(5), tid);
+            s = 3;
+            tighten();
+        }
+        while (s + 3 < nstage) {                                     // (places s .. s + 2 < nstage - 1: never the row's last stage)
+            row_stage<G::WCAP, false>(va, tw, twkey, list, count, stage_at(s), tid, V, want, W);
+            row_load_clamped(va, x, n4, stage_at(s + 3), tid);
+            row_stage<G::WCAP, false>(vb, tw, twkey, list, count, stage_at(s + 1), tid, V, want, W);
+            row_load_clamped(vb, x, n4, stage_at(s + 4), tid);
+            row_stage<G::WCAP, false>(vc, tw, twkey, list, count, stage_at(s + 2), tid, V, want, W);
+            row_load_clamped(vc, x, n4, stage_at(s + 5), tid);
             s += 3;
             tighten();
         }
-        if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T)); // the threshold is final
-        if (s < nstage) row_filter_perm<G::WCAP>(vb, tw, list, count, m, s, V);          // wave-uniform conditions
-        if (s + 1 < nstage) row_filter_perm<G::WCAP>(vc, tw, list, count, m, s + 1, V);
-        if (s + 2 < nstage) row_filter_perm<G::WCAP>(va, tw, list, count, m, s + 2, V);
+        if (s < nstage) examine(va, s);                              // wave-uniform; the last places are examined without new requests
+        if (s + 1 < nstage) examine(vb, s + 1);
+        if (s + 2 < nstage) examine(vc, s + 2);
     } else {
         // rows that 128-bit loads cannot take: one stage at a time, then one raise of the threshold
-        row_filter_seq<G::WCAP>(va, tw, list, count, 0, tid);
+        row_stage<G::WCAP, false>(va, tw, twkey, list, count, 0, tid, V, want, W);
         for (int s = 1; s < nstage; s++) {
             row_load_any<false>(va, x, V, s, tid);
-            row_filter_seq<G::WCAP>(va, tw, list, count, s, tid);
+            row_stage<G::WCAP, false>(va, tw, twkey, list, count, s, tid, V, want, W);
         }
         tighten();
-        if (have_tw) zb = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));
     }
     if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
-    const int cw = (int)min(count, (u32)G::WCAP);
     ROW_STAMP(1);
 #ifdef BORN_PHASE_TIMING
     __shared__ u64 s_wend[ROW_WAVES];
@@ -679,9 +735,13 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // ---- C: every wave moves its entries into one array (one LDS atomic per wave reserves the range).  What follows
     // is the work of as many threads as there are candidates, so most waves only pass the barriers: an instruction
     // that all sixteen waves execute costs the compute unit sixteen issue slots.
-    {
+    int cw = (int)min(count, (u32)G::WCAP);
+    auto join = [&]() {
         u32 base = 0u;
-        if (lane_id() == 0 && cw) base = (u32)atomicAdd(&s_n, cw);
+        if (lane_id() == 0) {
+            if (cw) base = (u32)atomicAdd(&s_n, cw);
+            if (twkey != gkey) atomicMax(&s_twmax, twkey);           // (a threshold of the wave's own)
+        }
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
         for (int e = lane_id(); e < cw; e += WAVE) {
             const u32 pos = base + (u32)e;
@@ -694,10 +754,30 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
                 }
             }
         }
-    }
+    };
+    join();
     __syncthreads();
     ROW_STAMP(2);
-    const int n = s_n;
+    int n = s_n;
+    // More candidates than the finish holds: waves that raised thresholds of their own end the pass with up to a full
+    // list each.  The common threshold is raised (each round refines the bins 256-fold) until they fit, or no round
+    // changes anything any more (equal logits by the thousand: the exact selection's case).
+    for (int it = 0; it < 5 && have_tw && !s_over && n > G::CAP; it++) {   // workgroup-uniform
+        __syncthreads();                                             // (every thread has read s_n and s_over)
+        if (tid == 0) s_n = 0;
+        if (!fast)
+            for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
+        tighten();                                                   // (its barrier orders the clears before the joins)
+        cw = (int)min(count, (u32)G::WCAP);
+        join();
+        __syncthreads();
+        n = s_n;
+    }
+    // A logit outside the lists has a key below the threshold of the wave that met it (thresholds only rise), so at most
+    // the largest threshold's key - 1 (the thresholds lie above the key of -inf, so that is the key of a float or of
+    // -inf), and so has its z: a penalty only lowers a logit and the division by the temperature is monotone.
+    // The row is proven if top_k candidates have z strictly above that bound.
+    const u32 zb = have_tw ? ordkey(z_of(ordkey_inv(max(gkey, s_twmax) - 1u), a.T)) : 0u;
     bool ok = have_tw && !s_over && n >= k && n <= G::CAP;
     // top_k beyond TOPK_SMALL_K: the candidates are ranked through buckets of z (below), whose counters take the
     // threshold rounds' first set of bins (no round runs any more)
@@ -946,7 +1026,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         }
     }
     const u32 max0 = wave_max_u32(lane_id() < ROW_WAVES ? s_wmax[lane_id()] : 0u);
-    u32 twkey = ordkey(t0);                                          // every logit outside the list has a smaller key
+    u32 twkey = ordkey(t0), gkey = twkey;                            // every logit outside the list has a smaller key (the waves share one threshold here)
     const int want = k + row_margin(k);
     uint2 *list = L + wave_id() * G::WCAP;
     u32 count = 0;
@@ -966,7 +1046,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         }
         count += (u32)__popcll(m);
         const u32 smax = max(max0, s_max[round & 1]);
-        row_tighten<G::WCAP>(list, count, twkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+        row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
         round++;
     }
     if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
