@@ -34,9 +34,6 @@
 // histories of at most TOPK_LOCAL_COUNT_HISTORY tokens the LOCAL instances count them where the
 // history is hashed anyway (the count rides in the high bits of the slot); otherwise the counts
 // come from a table by id that the caller's launches raise and clear around this one.
-#ifndef BORN_ROW_SCHED
-#define BORN_ROW_SCHED 1
-#endif
 #include "dev_common.h"
 #include "kernels.h"
 #include "topk_tail.h"
@@ -529,7 +526,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
     __shared__ __align__(16) u32 s_wbins[ROW_WAVES][ROW_TBINS];      // a wave's own bins, for a raise of its own threshold
     __shared__ u32 s_max[2];
-    __shared__ u32 s_kmax, s_kmin, s_twmax;
+    __shared__ u32 s_kmax, s_kmin, s_zb;
     __shared__ int s_n, s_valid, s_over, s_next;
     __shared__ int s_x[1 + ROW_WAVES];
 #ifdef BORN_PHASE_TIMING
@@ -560,16 +557,12 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
-    // The row's last stage is examined first, the others follow in row order: what raises the threshold fastest in a
-    // row whose large logits come late (sorted ascending, a step up near the end, a slow rise) is seen at once, and a
-    // row whose large logits come early meets them in the stage after.  Not when the last stage is too short to give
-    // every wave a full load: the first threshold comes from the first stage examined.
+    // The row's last stage is examined first, the others follow in row order: the first threshold then comes from the
+    // end of the row, which is what a row whose large logits come late (sorted ascending, a step up near the end, a slow
+    // rise) needs, and a row whose large logits come early meets them in the stage after.  Not when the last stage is
+    // too short to give every wave a full load: the first threshold comes from the first stage examined.
     const int last = nstage - 1;
-#ifdef BORN_ROW_NO_LAST_FIRST
-    const bool last_first = false;                                   // (measurement builds)
-#else
     const bool last_first = VEC && nstage > 1 && n4 - last * (ROW_U * ROW_BLOCK) >= ROW_BLOCK;
-#endif
     const int first = last_first ? last : 0;
     // the stage examined in place t >= 1 (a place past the last one: a stage past the row's end, whose loads all re-read
     // the row's last block)
@@ -592,7 +585,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         s_max[1] = 0u;
         s_kmax = 0u;
         s_kmin = 0xFFFFFFFFu;
-        s_twmax = 0u;
+        s_zb = 0u;
     }
     for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
     if (tid < ROW_TBINS) s_bins[0][tid] = 0u;                        // every round clears the bins of the next
@@ -683,6 +676,18 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     // A history that fits the workgroup was hashed above and the candidates probe it; otherwise the candidates' ids are
     // hashed and the history probes them.
     const bool fast = !penal || hfast;
+    // A logit outside the lists has a key below the threshold of the wave that met it (thresholds only rise), so at most
+    // that threshold's key - 1 (the thresholds lie above the key of -inf, so that is the key of a float or of -inf), and
+    // so has its z: a penalty only lowers a logit and the division by the temperature is monotone.  `zbw` is that bound
+    // for this wave's threshold; the bound for the row is the largest of the waves' (z is monotone in the threshold).
+    // The row is proven if top_k candidates have z strictly above it.
+    u32 zbw = 0u, zbw_of = 0u;
+    auto bound = [&]() {
+        if (have_tw && zbw_of != twkey) {                            // wave-uniform
+            zbw = ordkey(z_of(ordkey_inv(twkey - 1u), a.T));
+            zbw_of = twkey;
+        }
+    };
     if (VEC) {
         // va, vb, vc hold places s, s + 1, s + 2 of the order of examination: two stages stay in flight while one is
         // examined.  Only the row's last stage may reach past its end: it is examined under a mask, in place 0 or in one
@@ -713,6 +718,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             s += 3;
             tighten();
         }
+        bound();                                                     // (while the last loads are in flight; repeated below if the threshold still moves)
         if (s < nstage) examine(va, s);                              // wave-uniform; the last places are examined without new requests
         if (s + 1 < nstage) examine(vb, s + 1);
         if (s + 2 < nstage) examine(vc, s + 2);
@@ -725,6 +731,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         }
         tighten();
     }
+    bound();
     if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
     ROW_STAMP(1);
 #ifdef BORN_PHASE_TIMING
@@ -740,7 +747,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         u32 base = 0u;
         if (lane_id() == 0) {
             if (cw) base = (u32)atomicAdd(&s_n, cw);
-            if (twkey != gkey) atomicMax(&s_twmax, twkey);           // (a threshold of the wave's own)
+            atomicMax(&s_zb, zbw);
         }
         base = (u32)__builtin_amdgcn_readfirstlane((int)base);
         for (int e = lane_id(); e < cw; e += WAVE) {
@@ -768,16 +775,13 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         if (!fast)
             for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
         tighten();                                                   // (its barrier orders the clears before the joins)
+        bound();
         cw = (int)min(count, (u32)G::WCAP);
         join();
         __syncthreads();
         n = s_n;
     }
-    // A logit outside the lists has a key below the threshold of the wave that met it (thresholds only rise), so at most
-    // the largest threshold's key - 1 (the thresholds lie above the key of -inf, so that is the key of a float or of
-    // -inf), and so has its z: a penalty only lowers a logit and the division by the temperature is monotone.
-    // The row is proven if top_k candidates have z strictly above that bound.
-    const u32 zb = have_tw ? ordkey(z_of(ordkey_inv(max(gkey, s_twmax) - 1u), a.T)) : 0u;
+    const u32 zb = s_zb;                                             // the largest of the waves' bounds
     bool ok = have_tw && !s_over && n >= k && n <= G::CAP;
     // top_k beyond TOPK_SMALL_K: the candidates are ranked through buckets of z (below), whose counters take the
     // threshold rounds' first set of bins (no round runs any more)
