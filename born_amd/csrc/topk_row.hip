@@ -216,54 +216,72 @@ __device__ __forceinline__ void row_filter(const f32x4 (&v)[ROW_U], float tw, ui
     }
 }
 
-// A stage did not fit the wave's list (the row's large logits come late in row order: sorted ascending, a step up near
-// the end, a slow rise): the wave raises a threshold of its own, by itself, and examines the stage again.  The list's
-// first c0 entries (what it held before the stage) and the stage's logits >= the threshold, still in registers, are
-// all logits of the row and more than `want` of them, so the want-th largest of them is a lower bound of the row's
-// want-th largest logit: it becomes the wave's threshold, and the old entries below it are dropped.  Thresholds so
-// differ between waves; the bound of the proof is the largest of them.  W: 256 bins of the wave's own.  No barrier:
-// a wave's LDS traffic is in order.  Returns false if the keys at hand cannot be told apart (equal logits by the
-// hundred): the list stays overflowed and the row goes to the exact selection.
+// A stage did not fit the wave's list (the row's large logits sit where the first threshold did not look): the wave
+// raises a threshold of its own, by itself, and examines the stage again.  The list's first c0 entries (what it held
+// before the stage) and the stage's logits >= the threshold, still in registers, are all logits of the row and more
+// than `want` of them (`fresh` counts the stage's), so the want-th largest of them is a lower bound of the row's
+// want-th largest logit.  They are binned by value (256 bins, linear in the logit, where bins of the order key would
+// crowd around zero); the smallest key in the highest bins that hold `want` between them becomes the
+// wave's threshold, and the old entries below it are dropped.  Thresholds so differ between waves; the bound of the
+// proof is the largest of them.  W: 256 bins of the wave's own.  No barrier: a wave's LDS traffic is in order.
+// Selects, not branches: the lanes' conditions stay out of the scalar registers.  Returns false if the values at hand
+// cannot be told apart (equal logits by the hundred, an infinite span): the list stays overflowed and the row goes to
+// the exact selection.
 template <int WCAP>
-__device__ __forceinline__ bool row_raise_from_stage(const f32x4 (&v)[ROW_U], uint2 *list, u32 &c0, u32 &twkey, int want, u32 *W) {
+__device__ __forceinline__ bool row_raise_from_stage(const f32x4 (&v)[ROW_U], uint2 *list, u32 &c0, u32 fresh, u32 &twkey, int want, u32 *W) {
     const int l = lane_id();
     const float tw = ordkey_inv(twkey);
-    u32 mx = 0u, mn = 0xFFFFFFFFu;
-    for (int e = l; e < (int)c0; e += WAVE) {
-        const u32 key = ordkey(__uint_as_float(list[e].x));
-        mx = max(mx, key);
-        mn = min(mn, key);
+    float hi = -INFINITY, lo = INFINITY;
+    // The bins span the stage's own logits when those alone number `want` (the threshold sought then lies among them,
+    // and old entries below them share the lowest bin), else the old entries as well.
+    if (fresh < (u32)want) {                                         // wave-uniform
+        for (int e = l; e < (int)c0; e += WAVE) lo = fminf(lo, __uint_as_float(list[e].x));
     }
+    for (int e = l; e < (int)c0; e += WAVE) hi = fmaxf(hi, __uint_as_float(list[e].x));
 #pragma unroll
     for (int u = 0; u < ROW_U; u++)
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            const u32 key = ordkey(v[u][c]);
-            if (v[u][c] >= tw) {
-                mx = max(mx, key);
-                mn = min(mn, key);
-            }
+            const float xv = v[u][c];
+            hi = fmaxf(hi, xv);                                      // (the largest of all is the largest of those that pass; fmaxf drops NaN)
+            lo = fminf(lo, xv >= tw ? xv : INFINITY);
         }
-    mx = wave_max_u32(mx);
-    mn = wave_min_u32(mn);
-    const int sh = max(0, 24 - (int)__clz(mx - mn));                 // ((mx - mn) >> sh) < ROW_TBINS
+    hi = ordkey_inv(wave_max_u32(ordkey(hi)));
+    lo = ordkey_inv(wave_min_u32(ordkey(lo)));
+    const float scale = (float)(ROW_TBINS - 1) / (hi - lo);          // (a span of zero or infinity: every logit lands in one bin, and the raise fails below)
+    auto bin_of = [&](float xv) { return max(0, min((int)((xv - lo) * scale), ROW_TBINS - 1)); };   // monotone in xv; NaN -> 0
     reinterpret_cast<uint4 *>(W)[l] = make_uint4(0u, 0u, 0u, 0u);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    for (int e = l; e < (int)c0; e += WAVE) atomicAdd(&W[(ordkey(__uint_as_float(list[e].x)) - mn) >> sh], 1u);
+    for (int e = l; e < (int)c0; e += WAVE) atomicAdd(&W[bin_of(__uint_as_float(list[e].x))], 1u);
 #pragma unroll
     for (int u = 0; u < ROW_U; u++)
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             float xv = v[u][c];
-            asm volatile("" : "+v"(xv));                             // (keeps the keys of the first pass from being held in registers until here)
-            if (xv >= tw) atomicAdd(&W[(ordkey(xv) - mn) >> sh], 1u);
+            asm volatile("" : "+v"(xv));                             // (keeps the first pass's values from being held in registers until here)
+            atomicAdd(&W[bin_of(xv)], xv >= tw ? 1u : 0u);           // (a logit below the threshold adds nothing, wherever it lands)
         }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const u32 nk = row_bins_crossing(W, want, mn, sh);
-    if (nk <= twkey) return false;
+    const int bin = (int)row_bins_crossing(W, want, 0u, 0);          // the lowest of the highest bins that hold `want` entries between them
+    // the smallest key in those bins: exactly the entries of those bins reach it (the bins are monotone in the logit)
+    u32 nk = 0xFFFFFFFFu;
+    for (int e = l; e < (int)c0; e += WAVE) {
+        const float xv = __uint_as_float(list[e].x);
+        nk = min(nk, bin_of(xv) >= bin ? ordkey(xv) : 0xFFFFFFFFu);
+    }
+#pragma unroll
+    for (int u = 0; u < ROW_U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float xv = v[u][c];
+            asm volatile("" : "+v"(xv));
+            nk = min(nk, (xv >= tw && bin_of(xv) >= bin) ? ordkey(xv) : 0xFFFFFFFFu);
+        }
+    nk = wave_min_u32(nk);
+    if (nk <= twkey || nk == 0xFFFFFFFFu) return false;
     row_list_compact<WCAP>(list, c0, nk);
     twkey = nk;
     return true;
@@ -285,13 +303,12 @@ __device__ __forceinline__ void row_stage(const f32x4 (&v)[ROW_U], float &tw, u3
     if (__builtin_expect(count > (u32)WCAP, 0)) {
         // (examined a second time by a second copy of the filter, not by a loop around one: inside a loop the compiler
         // keeps the sixteen ids of the stage in registers)
-        if (c0 <= (u32)WCAP && row_raise_from_stage<WCAP>(m, list, c0, twkey, want, W)) {
+        if (c0 <= (u32)WCAP && row_raise_from_stage<WCAP>(m, list, c0, count - c0, twkey, want, W)) {
             tw = ordkey_inv(twkey);
             count = c0;
             int st = stage, t2 = tid;
             asm volatile("" : "+v"(st), "+v"(t2));                   // (or the sixteen ids of the stage are kept in registers for this second use)
-            row_filter<WCAP>(m, tw, list, count, st, t2);            // (a second overflow stands: equal logits by the hundred,
-                                                                     // or logits around zero, where the bins of the key crowd)
+            row_filter<WCAP>(m, tw, list, count, st, t2);            // (a second overflow stands: equal logits by the hundred)
         }
     }
 }
@@ -557,19 +574,17 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     const int hlen = a.history ? min((int)(a.hist_len ? a.hist_len[row] : (int)a.hist_stride), (int)a.hist_stride) : 0;
     const int *h = a.history + (long long)row * a.hist_stride;
     const int h0 = (tid < hlen) ? h[tid] : -1;
-    // The row's last stage is examined first, the others follow in row order: the first threshold then comes from the
-    // end of the row, which is what a row whose large logits come late (sorted ascending, a step up near the end, a slow
-    // rise) needs, and a row whose large logits come early meets them in the stage after.  Not when the last stage is
-    // too short to give every wave a full load: the first threshold comes from the first stage examined.
+    // The row's last stage is examined second, right after its first; the others follow in row order.  Both ends of the
+    // row are then known to the first raise of the threshold: a row whose large logits come late (sorted ascending, a
+    // step up near the end, a slow rise) pays one stage that overflows the lists (below), not one per stage.  The first
+    // threshold still comes from the row's first stage, where a vocabulary keeps its frequent tokens.
     const int last = nstage - 1;
-    const bool last_first = VEC && nstage > 1 && n4 - last * (ROW_U * ROW_BLOCK) >= ROW_BLOCK;
-    const int first = last_first ? last : 0;
-    // the stage examined in place t >= 1 (a place past the last one: a stage past the row's end, whose loads all re-read
+    // the stage examined in place t (a place past the last one: a stage past the row's end, whose loads all re-read
     // the row's last block)
-    auto stage_at = [&](int t) { return last_first ? (t < nstage ? t - 1 : nstage) : t; };
+    auto stage_at = [&](int t) { return !VEC || nstage < 3 || t == 0 ? t : t == 1 ? last : t < nstage ? t - 1 : nstage; };
     f32x4 va[ROW_U], vb[ROW_U], vc[ROW_U];
     if (VEC) {
-        row_load_clamped(va, x, n4, first, tid);
+        row_load_clamped(va, x, n4, 0, tid);
         row_load_clamped(vb, x, n4, stage_at(1), tid);               // in flight during the search for the first threshold
         row_load_clamped(vc, x, n4, stage_at(2), tid);
     } else {
@@ -610,22 +625,22 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
 
     // ---- the first threshold, from the first stage: with `act` waves holding data, a = ceil(top_k / act) lanes per
     // wave and the need = ceil(top_k / a)-th largest of the wave results
-    const int act = min(ROW_WAVES, (min(n4 - first * (ROW_U * ROW_BLOCK), ROW_BLOCK) + WAVE - 1) / WAVE);   // (its first load)
+    const int act = min(ROW_WAVES, (min(n4, ROW_BLOCK) + WAVE - 1) / WAVE);
     const int aw = min(WAVE, (k + act - 1) / act);                   // lanes of one wave
     const int need = (k + aw - 1) / aw;                              // <= act, but for a top_k beyond the lanes that hold data: no threshold then
     {
         float lm = -INFINITY;
-        if (!VEC || first < nfull) {                                 // (without 128-bit loads, elements past the end were filled with -inf)
+        if (!VEC || nfull > 0) {                                     // (without 128-bit loads, elements past the end were filled with -inf)
 #pragma unroll
             for (int u = 0; u < ROW_U; u++)
 #pragma unroll
                 for (int c = 0; c < 4; c++) lm = fmaxf(lm, va[u][c]);    // fmaxf drops NaN
-        } else {                                                     // the row ends inside this stage
+        } else {                                                     // the row ends inside the first stage
 #pragma unroll
             for (int u = 0; u < ROW_U; u++)
 #pragma unroll
                 for (int c = 0; c < 4; c++)
-                    if (((first * ROW_U + u) * ROW_BLOCK + tid) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
+                    if ((u * ROW_BLOCK + tid) * 4 + c < V) lm = fmaxf(lm, va[u][c]);
         }
         const u32 lk = ordkey(lm);
         const u32 wk = wave_kth_largest_bound(lk, aw, 14);
@@ -690,18 +705,18 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     };
     if (VEC) {
         // va, vb, vc hold places s, s + 1, s + 2 of the order of examination: two stages stay in flight while one is
-        // examined.  Only the row's last stage may reach past its end: it is examined under a mask, in place 0 or in one
-        // of the last places, which are kept out of the loop (so that the loop's stages are all of one kind).
+        // examined.  Only the row's last stage may reach past its end: it is examined under a mask, in place 1 or (short
+        // rows) in the last place, which are kept out of the loop (so that the loop's stages are all of one kind).
         auto examine = [&](const f32x4 (&v)[ROW_U], int t) {
-            const int st = t == 0 ? first : stage_at(t);
+            const int st = stage_at(t);
             if (st == last) row_stage<G::WCAP, true>(v, tw, twkey, list, count, st, tid, V, want, W);   // wave-uniform
             else row_stage<G::WCAP, false>(v, tw, twkey, list, count, st, tid, V, want, W);
         };
         int s = 0;
-        if (nstage > 3) {                                            // (places 1 and 2 are not the row's last stage then)
-            examine(va, 0);
+        if (nstage > 3) {                                            // (place 1 is the row's last stage, places 0 and 2 are whole)
+            row_stage<G::WCAP, false>(va, tw, twkey, list, count, 0, tid, V, want, W);
             row_load_clamped(va, x, n4, stage_at(3), tid);
-            row_stage<G::WCAP, false>(vb, tw, twkey, list, count, stage_at(1), tid, V, want, W);
+            row_stage<G::WCAP, true>(vb, tw, twkey, list, count, last, tid, V, want, W);
             row_load_clamped(vb, x, n4, stage_at(4), tid);
             row_stage<G::WCAP, false>(vc, tw, twkey, list, count, stage_at(2), tid, V, want, W);
             row_load_clamped(vc, x, n4, stage_at(5), tid);
