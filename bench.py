@@ -71,6 +71,67 @@ METRIC = {
 }
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or platform.machine()
+
+
+def go_twin():
+    """The Go twin of the CPU baseline (backend/rocm/cpu_ref_test.go), if this box has a Go toolchain: run in a child
+    process of its own, reported with GOMAXPROCS.  No toolchain: says so."""
+    import shutil
+    import subprocess
+    go = shutil.which("go")
+    if not go:
+        return {"go": "absent"}
+    procs = os.environ.get("GOMAXPROCS") or str(len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
+    try:
+        r = subprocess.run([go, "test", "-run", "^$", "-bench", "CPURef", "-benchtime", "3x", "./backend/rocm"], cwd=ROOT, capture_output=True,
+                           text=True, timeout=180, env=dict(os.environ, GOMAXPROCS=procs, GOFLAGS="-mod=mod"))
+    except (OSError, subprocess.TimeoutExpired) as e:
+        return {"go": go, "error": str(e)[:200]}
+    out = {"go": go, "GOMAXPROCS": int(procs), "returncode": r.returncode}
+    lines = [ln for ln in r.stdout.splitlines() if ln.startswith("Benchmark")]
+    if lines:
+        out["benchmarks"] = lines[:8]
+    else:
+        out["output_tail"] = (r.stdout + r.stderr)[-400:]
+    return out
+
+
+def parity_block(w, tokens_host, probs_host, rows=16):
+    """The oracle as the checker on a slice of the batch, outside the timed region: how many of the sampled rows equal
+    the fixed-point layer (must be all), how many the fp64 layer flags as lying within 1e-6 of a CDF step, how many
+    differ from the fp64 layer (all of those must be flagged)."""
+    from oracle import pyoracle
+    B = w.logits.shape[0]
+    idx = sorted(set(np.linspace(0, B - 1, num=min(rows, B)).astype(int).tolist()))
+    x = np.ascontiguousarray(w.logits[idx])
+    u = np.ascontiguousarray(w.uniforms[idx])
+    h = None if w.history is None else np.ascontiguousarray(w.history[idx])
+    fx = pyoracle.sample(x, u, w.temperature, w.top_k, w.top_p, w.rep, h, mode=pyoracle.MODE_FIXED)
+    tr = pyoracle.sample(x, u, w.temperature, w.top_k, w.top_p, w.rep, h, mode=pyoracle.MODE_TRUTH)
+    got, gp = tokens_host[idx], probs_host[idx]
+    differ = got != tr["tokens"]
+    same = ~differ & ~tr["near_cut"]
+    rel = np.abs(gp[same].astype(np.float64) - tr["probs"][same]) / np.maximum(tr["probs"][same], 1e-300)
+    return {"rows_checked": len(idx), "rows": idx,
+            "tokens_equal_fixed_point_layer": int((got == fx["tokens"]).sum()),
+            "probabilities_bit_equal_fixed_point_layer": int((gp.view(np.uint32) == fx["probs"].view(np.uint32)).sum()),
+            "rows_flagged_within_1e-6_of_a_cdf_step": int(tr["near"].sum()),
+            "tokens_differing_from_fp64_layer": int(differ.sum()),
+            "of_those_not_flagged": int((differ & ~tr["near"]).sum()),
+            "max_relative_probability_error_vs_fp64": float(rel.max()) if rel.size else 0.0,
+            "checker": "oracle/born_oracle.c (fixed-point layer and fp64 layer), not part of the timed region"}
+
+
 def cpu_baseline(w, seconds=12.0):
     """Times the oracle's reference-arithmetic mode (the checker, used here only as the CPU baseline)."""
     from oracle import pyoracle
@@ -85,7 +146,7 @@ def cpu_baseline(w, seconds=12.0):
         pyoracle.sample(x, u, w.temperature, w.top_k, w.top_p, w.rep, h, mode=pyoracle.MODE_REF32)
         n += rows
     dt = time.perf_counter() - t0
-    out = {"value": n / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+    out = {"value": n / dt, "unit": "tokens/s", "cores": 1, "kind": "port", "cpu_model": cpu_model(),
            "sample": f"{n} rows of the same workload ({rows}-row slices repeated for {dt:.1f} s), "
                      "C restatement of a Born-style scalar sampler (fp64 exp cast to fp32, sequential fp32 sums, heap top-k), 1 thread"}
     # The same port row-parallel over the host cores this process may use (rows are independent; the C call
@@ -107,6 +168,7 @@ def cpu_baseline(w, seconds=12.0):
     dt = time.perf_counter() - t0
     out["all_cores"] = {"value": done / dt, "unit": "tokens/s", "cores": cores,
                         "sample": f"{done} rows, {cores} threads each repeating the {rows}-row slice for {dt:.1f} s"}
+    out["go_twin"] = go_twin()
     return out
 
 
@@ -269,7 +331,13 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / k
 
-    # The LM-head leg runs first (its own figures, never part of the headline): the W warm-up steps and the K timed
+    # The literal reading of the flags first: W warm-up steps straight after the host's set-up (the device has idled),
+    # then K timed steps.  Reported beside the headline as ms_per_step_idle_start.
+    for _ in range(args.warmup):
+        step()
+    ms_idle_start = timed(args.steps)
+
+    # The LM-head leg runs next (its own figures, never part of the headline): the W warm-up steps and the K timed
     # steps below then run on a device that is already at its working clocks, as in a serving loop.
     producer = None
     if not args.no_producer and args.config == "C3":
@@ -308,7 +376,8 @@ def main():
         if args.path == 0 else "sample_wide_kernel"
     # (the checked call, the 30 groups, the warm-up, the timed region; the chained and the fused steps of the LM-head leg
     # count too)
-    launches = 1 + 300 + args.warmup + args.steps + (0 if producer is None else 2 * (producer["iters"] + 1))
+    launches = 1 + 300 + 2 * (args.warmup + args.steps) + (0 if producer is None else 2 * (producer["iters"] + 1))
+    warmup_effective = launches - args.steps - (0 if producer is None else producer["iters"] + 1)   # (the fused steps do not run this kernel)
     if kernel_name == "topk_row_kernel":
         confirmed = counters["topk_rows"] + counters["fallback_rows"] == B * launches and counters["general_rows"] == 0
     else:
@@ -324,7 +393,10 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_effective": warmup_effective,
         "ms_per_step": ms,
+        "ms_per_step_idle_start": ms_idle_start,
+        "ms_per_step_idle_start_note": "the same K steps behind the same W warm-up steps, taken straight after set-up, before anything else ran on the device",
         "ms_per_step_timing": "HIP events on the launch stream around exactly K steps, a synchronisation on either side, behind W warm-up steps; "
                               "the 30 groups of ms_per_step_spread run before the warm-up, so the device is at its working clocks",
         "ms_per_step_spread": spread,
@@ -346,6 +418,7 @@ def main():
     if producer is not None:
         out["producer"] = producer
     if not args.no_cpu:
+        out["parity"] = parity_block(w, tok_host, probs.cpu().numpy())
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
 
@@ -411,7 +484,22 @@ def main_extras(args, torch, S, synth, dev):
 
     if args.config == "C3x":
         base, minp, fp = mk(), mk(MinP=0.05), mk(FrequencyPenalty=0.3, PresencePenalty=0.5)
-        k100, k128, k129, k0 = mk(top_k=100), mk(top_k=128), mk(top_k=129), mk(top_k=0)
+        k100, k128, k129, k256, k512, k513, k0 = mk(top_k=100), mk(top_k=128), mk(top_k=129), mk(top_k=256), mk(top_k=512), mk(top_k=513), mk(top_k=0)
+        # rows whose large logits sit where a threshold drawn from the row's first logits does not look (same shape, same
+        # history and uniforms): sorted ascending; a step up in the last tenth; a bump around the middle
+        rng = np.random.default_rng(synth.BASE_SEED)
+        i = np.arange(V, dtype=np.float64)
+        shaped = {"ascending": np.tile(i / V * 20 - 10, (B, 1)) + rng.standard_normal((B, V)) * 1e-3,
+                  "late_step": rng.standard_normal((B, V)), "mid_bump": rng.standard_normal((B, V))}
+        shaped["late_step"][:, V - V // 10:] += 30
+        shaped["mid_bump"][:, V // 2:V // 2 + V // 10] += 30
+        shaped = {name: [torch.from_numpy(x.astype(np.float32)).to(dev) for _ in range(2)] for name, x in shaped.items()}
+
+        def shaped_case(name, smp):
+            def f():
+                c[0] += 1
+                smp.Sample(shaped[name][c[0] % 2], B, V, h, None, u, tok, pr, hist_stride=H, stream=stream)
+            return f
         Ts = torch.full((B,), w.temperature, device=dev)
         ks = torch.full((B,), w.top_k, dtype=torch.int32, device=dev)
         ps = torch.full((B,), w.top_p, device=dev)
@@ -420,7 +508,15 @@ def main_extras(args, torch, S, synth, dev):
             "C3": lambda: base.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 shape, top_k 100": lambda: k100.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 shape, top_k 128": lambda: k128.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
-            "C3 shape, top_k 129 (the general kernel)": lambda: k129.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 129": lambda: k129.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 256": lambda: k256.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 512": lambda: k512.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 shape, top_k 513 (the general kernel)": lambda: k513.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 settings, rows sorted ascending": shaped_case("ascending", base),
+            "C3 settings, rows with a step up in their last tenth": shaped_case("late_step", base),
+            "C3 settings, rows with a bump around their middle": shaped_case("mid_bump", base),
+            "C3 settings, rows sorted ascending, top_k 512": shaped_case("ascending", k512),
+            "C3 settings, rows with a step up in their last tenth, top_k 256": shaped_case("late_step", k256),
             "C3 shape, top_k 0 (top-p alone: the three-sweep kernel)": lambda: k0.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + min_p 0.05": lambda: minp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
@@ -441,6 +537,10 @@ def main_extras(args, torch, S, synth, dev):
         tok.zero_()
     for name, fn in cases.items():
         out["us"][name] = timed(fn, args.steps, args.warmup)
+    if args.config == "C3x":
+        # rows the single-pass kernel handed to its exact selection, over every step of every case above (0: none did)
+        out["exact_selection_rows_total"] = {name: smp.Counters(stream)["fallback_rows"] for name, smp in
+                                             (("handle of the C3 settings (all its cases)", base), ("top_k 256", k256), ("top_k 512", k512))}
     out["algorithmic_bytes_per_step"] = w.algorithmic_bytes()
     print(json.dumps(out))
 

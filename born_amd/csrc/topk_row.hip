@@ -246,8 +246,13 @@ __device__ __forceinline__ bool row_raise_from_stage(const f32x4 (&v)[ROW_U], ui
             hi = fmaxf(hi, xv);                                      // (the largest of all is the largest of those that pass; fmaxf drops NaN)
             lo = fminf(lo, xv >= tw ? xv : INFINITY);
         }
-    hi = ordkey_inv(wave_max_u32(ordkey(hi)));
+    // The bins end at the eighth largest of the lanes' maxima, not at the largest logit of all: a few logits far above
+    // the rest (one token close to certain) would stretch the bins until everything else shared one.  What lies above
+    // shares the top bin.
+    const float top = ordkey_inv(wave_max_u32(ordkey(hi)));
+    hi = ordkey_inv(wave_kth_largest_bound(ordkey(hi), 8, 10));
     lo = ordkey_inv(wave_min_u32(ordkey(lo)));
+    if (!(hi > lo)) hi = top;                                        // wave-uniform
     const float scale = (float)(ROW_TBINS - 1) / (hi - lo);          // (a span of zero or infinity: every logit lands in one bin, and the raise fails below)
     auto bin_of = [&](float xv) { return max(0, min((int)((xv - lo) * scale), ROW_TBINS - 1)); };   // monotone in xv; NaN -> 0
     reinterpret_cast<uint4 *>(W)[l] = make_uint4(0u, 0u, 0u, 0u);
@@ -499,9 +504,12 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
 //   H: this round's bins (all zero on entry); Hclear: the next round's bins, zeroed here (with three sets in rotation
 //   they were last read two rounds ago, before the previous round's barrier);
 //   Mnext: where this round's largest key is published for the next round.
+//   span_out (optional): receives the width of a bin when the threshold was raised to a bin boundary below the top bin:
+//   the want-th largest key then lies within that distance above the new threshold, which a following round may take as
+//   its range (0 otherwise).
 template <int WCAP>
 __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, u32 &gkey, int want, u32 smax, u32 *H, u32 *Hclear,
-                                            u32 *Mnext, int *s_over, int tid) {
+                                            u32 *Mnext, int *s_over, int tid, u32 *span_out = nullptr) {
     const int l = lane_id();
     if (count > (u32)WCAP && l == 0) *s_over = 1;
     const int cw = (int)min(count, (u32)WCAP);
@@ -519,10 +527,55 @@ __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey,
     lds_barrier();
     const u32 nk = row_bins_crossing(H, want, gkey, sh);             // the same in every wave
     if (nk <= gkey) return;
+    // (the top bin also holds every key beyond the range: a crossing there says nothing about how far above it lies)
+    if (span_out) *span_out = ((nk - gkey) >> sh) < (u32)(ROW_TBINS - 1) ? 1u << sh : 0u;
     gkey = nk;
     if (nk <= twkey) return;                                         // (this wave's own threshold is higher already)
     row_list_compact<WCAP>(list, count, nk);
     twkey = nk;
+}
+
+// Candidates with equal z (first wave only, after the rank sort by z).  They counted the same rank r0: one of them sits
+// in sorted[r0] and the places behind it stayed empty (`sorted` starts as zeros, no key is zero); equal z across the
+// cut shows as nobody having counted exactly top_k (`cut_unseen`).  Those candidates, a handful at most, are listed
+// and ranked again among themselves by their whole keys (z descending, id ascending; unique); the others are in place.
+//   K, Khi: the candidates' keys and their z alone; R: the ranks they counted; T: room for the list (n words).
+__device__ __forceinline__ void row_resolve_ties(const u64 *K, const u32 *Khi, const u32 *R, u32 *T, u64 *sorted, int n, int k,
+                                                 bool cut_unseen) {
+    const int l = lane_id();
+    bool hole = false;
+    for (int i = l; i < k; i += WAVE) hole |= sorted[i] == 0ull;
+    if (__ballot(hole) == 0ull && !cut_unseen) return;               // wave-uniform
+    int m = 0;
+    for (int c0 = 0; c0 < n; c0 += WAVE) {                           // wave-uniform
+        const int c = c0 + l;
+        bool tied = false;
+        if (c < n) {
+            const u32 r = R[c];
+            if (r < (u32)k) tied = sorted[r] != K[c] || (r + 1u < (u32)k ? sorted[r + 1u] == 0ull : cut_unseen);
+        }
+        const u64 b = __ballot(tied);
+        if (tied) T[m + (int)__builtin_amdgcn_mbcnt_hi((u32)(b >> 32), __builtin_amdgcn_mbcnt_lo((u32)b, 0u))] = (u32)c;
+        m += __popcll(b);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int i0 = 0; i0 < m; i0 += WAVE) {                           // wave-uniform
+        const int i = i0 + l;
+        const u32 c = T[min(i, m - 1)];
+        const u64 key = K[c];
+        const u32 zk = Khi[c];
+        u32 pos = R[c];
+        for (int j = 0; j < m; j++) {                                // (wave-uniform addresses)
+            const u32 cj = T[j];
+            pos += (Khi[cj] == zk && K[cj] > key) ? 1u : 0u;
+        }
+        if (i < m && pos < (u32)k) sorted[pos] = key;                // (nothing read above is written here)
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // LOCAL: the frequency / presence penalties are on and the kernel counts the occurrences itself (SampleArgs::local_counts).
@@ -782,14 +835,22 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     ROW_STAMP(2);
     int n = s_n;
     // More candidates than the finish holds: waves that raised thresholds of their own end the pass with up to a full
-    // list each.  The common threshold is raised (each round refines the bins 256-fold) until they fit, or no round
-    // changes anything any more (equal logits by the thousand: the exact selection's case).
+    // list each.  The common threshold is raised until they fit, each round over the range of the bin the last one
+    // found the want-th largest key in (256 times finer each time, whatever lies far above), or no round changes
+    // anything any more (equal logits by the thousand: the exact selection's case).
+    u32 span = 0u;
     for (int it = 0; it < 5 && have_tw && !s_over && n > G::CAP; it++) {   // workgroup-uniform
         __syncthreads();                                             // (every thread has read s_n and s_over)
         if (tid == 0) s_n = 0;
         if (!fast)
             for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
-        tighten();                                                   // (its barrier orders the clears before the joins)
+        {                                                            // (the round's barrier orders the clears before the joins)
+            const u32 smax = span ? (u32)min((u64)gkey + (u64)(span - 1u), (u64)0xFFFFFFFFull) : max(max0, s_max[round & 1]);
+            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over,
+                                 tid, &span);
+            tw = ordkey_inv(twkey);
+            round++;
+        }
         bound();
         cw = (int)min(count, (u32)G::WCAP);
         join();
@@ -919,10 +980,9 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     }
 
     // ---- rank sort: every candidate counts the candidates with a larger z (32-bit compares; 64-bit ones run at a
-    // quarter of the rate) and the top_k take their place in rank order.  Candidates with equal z would count the same
-    // and leave the next place empty (`sorted` starts as zeros, no key is zero): the first wave then repeats the count
-    // with the whole keys (z descending, id ascending; unique).  Equal z across the cut shows as nobody counting
-    // exactly top_k.
+    // quarter of the rate) and the top_k take their place in rank order.  Candidates with equal z count the same; the
+    // first wave puts them right (row_resolve_ties).
+    u32 *const R = reinterpret_cast<u32 *>(C);                       // the ranks counted (the candidates' list has served)
     if (tid < n) {
         const u32 khi = Khi[tid];
         const uint4 *K4 = reinterpret_cast<const uint4 *>(Khi);      // wave-uniform addresses: four z per read,
@@ -937,29 +997,17 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         }
         if (r < k) sorted[r] = K[tid];
         else if (r == k) s_next = 1;
+        R[tid] = (u32)r;
     }
     __syncthreads();
     ROW_STAMP(6);
     if (tid >= WAVE) return;                                         // the first wave alone goes on
-    {
-        bool hole = false;
-        for (int i = tid; i < k; i += WAVE) hole |= sorted[i] == 0ull;
-        if (__ballot(hole) != 0ull || (n > k && s_next == 0)) {      // wave-uniform
-            for (int c = tid; c < n; c += WAVE) {
-                const u64 key = K[c];
-                int r = 0;
-                for (int j = 0; j < n; j++) r += K[j] > key ? 1 : 0;
-                if (r < k) sorted[r] = key;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
-    }
+    row_resolve_ties(K, Khi, R, R + G::CAP, sorted, n, k, n > k && s_next == 0);
     finish_sorted_by_wave(sorted, k, a, row, u_row);
     ROW_STAMP(7);
 #ifdef BORN_PHASE_TIMING
     for (int w = 0; w < ROW_WAVES; w++) stamp_[5] = max(stamp_[5], s_wend[w]);   // the last wave to end its pass
+    stamp_[4] = (u64)n | ((u64)round << 32);                         // (slot 4 carries no stamp: the candidates and the rounds)
     if (tid == 0)
         for (int i = 0; i < 8; i++) a.counters[COUNTER_ROW_BASE + COUNTER_ROW_STRIDE * row + i] = stamp_[i];
     if (tid == 0 && row == 0) { a.counters[8 + 16] = (u64)n; a.counters[8 + 17] = (u64)round; a.counters[8 + 19] = __builtin_readcyclecounter() - cyc0_; a.counters[8 + 20] = stamp_[7] - stamp_[0]; }
@@ -1122,24 +1170,11 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         }
         if (r < k) sorted[r] = K[tid];
         else if (r == k) s_next = 1;
+        reinterpret_cast<u32 *>(C)[tid] = (u32)r;                    // (the candidates' list has served)
     }
     __syncthreads();
     if (tid >= WAVE) return;
-    {
-        bool hole = false;
-        for (int i = tid; i < k; i += WAVE) hole |= sorted[i] == 0ull;
-        if (__ballot(hole) != 0ull || (n > k && s_next == 0)) {      // equal z among the candidates: whole keys decide
-            for (int c = tid; c < n; c += WAVE) {
-                const u64 key = K[c];
-                int r = 0;
-                for (int j = 0; j < n; j++) r += K[j] > key ? 1 : 0;
-                if (r < k) sorted[r] = key;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
-    }
+    row_resolve_ties(K, Khi, reinterpret_cast<const u32 *>(C), reinterpret_cast<u32 *>(C) + G::CAP, sorted, n, k, n > k && s_next == 0);   // equal z among the candidates
     finish_sorted_by_wave(sorted, k, a, row, u_row);
     if (tid == 0) count_row(a.counters, row, 0);
 }
