@@ -381,6 +381,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     }
 
     BORN_STAMP(a, row, 2);
+#if defined(BORN_NUC_STOP_AFTER) && BORN_NUC_STOP_AFTER == 1
+    // (measurement builds only: the row ends after the named sweep, for per-sweep instruction counts; results are wrong)
+    if (tid == 0) a.tokens[row] = __float_as_int(r.sbin) & 1;
+    return;
+#endif
     // ---- sweep 2: integer masses by bin
     if (r.T == 1.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
@@ -407,6 +412,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     }
     __syncthreads();
     BORN_STAMP(a, row, 3);
+#if defined(BORN_NUC_STOP_AFTER) && BORN_NUC_STOP_AFTER == 2
+    if (tid == 0) a.tokens[row] = (int)(mass[0] & 1ull);
+    return;
+#endif
     u64 Zk;
     {
         u64 v[NUC_PER], local = 0;

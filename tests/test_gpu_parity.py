@@ -1144,12 +1144,12 @@ def test_argument_errors_panic_like_the_go_layer(rocm):
 # ---------------------------------------------------------------- the benchmark configurations
 
 def test_config_c1_steps(oracle, rocm):
-    """C1: batch 1, vocab 32000, fresh logits per step; 40 of the 1000 steps against both oracle layers."""
+    """C1: batch 1, vocab 32000, fresh logits per step; 200 of the 1000 steps (every fifth) against both oracle layers."""
     from born_amd import synth
     s = rocm.NewSampler(rocm.SamplerConfig(Temperature=0.8, TopK=40, TopP=0.95, RepetitionPenalty=1.1), max_batch=1,
                         max_vocab=32000)
     near = 0
-    for step in range(40):
+    for step in range(0, 1000, 5):
         w = synth.c1(step)
         got = rocm.sample_host(s, w.logits, w.uniforms, w.history)
         fx = oracle.sample(w.logits, w.uniforms, 0.8, 40, 0.95, 1.1, w.history, mode=oracle.MODE_FIXED)
@@ -1157,7 +1157,7 @@ def test_config_c1_steps(oracle, rocm):
         assert got["tokens"][0] == fx["tokens"][0] and got["probs"][0] == fx["probs"][0], step
         assert got["tokens"][0] == tr["tokens"][0] or tr["near"][0]
         near += int(tr["near"][0])
-    assert near <= 2
+    assert near <= 6
 
 
 def test_config_c2_greedy_and_multinomial(oracle, rocm):
@@ -1204,8 +1204,8 @@ def test_config_c4_full(oracle, rocm):
 
 
 def test_config_c5_slice_and_full_size_properties(oracle, rocm):
-    """C5 (wide nucleus, vocabulary 152064): 24 rows against the oracle; the full 1024-row batch through
-    size-independent properties (determinism, row independence, range)."""
+    """C5 (wide nucleus, vocabulary 152064): 64 rows from across the batch against the oracle; the full 1024-row batch
+    through size-independent properties (determinism, row independence, range)."""
     from born_amd import synth
     w = synth.c5(rows=1024)
     B, V = w.logits.shape
@@ -1218,15 +1218,21 @@ def test_config_c5_slice_and_full_size_properties(oracle, rocm):
     sl = slice(500, 524)
     part = rocm.sample_host(s, w.logits[sl], w.uniforms[sl], w.history[sl])
     assert np.array_equal(part["tokens"], full["tokens"][sl])                       # rows are independent
-    fx = oracle.sample(w.logits[sl], w.uniforms[sl], w.temperature, 0, w.top_p, w.rep, w.history[sl], mode=oracle.MODE_FIXED)
-    tr = oracle.sample(w.logits[sl], w.uniforms[sl], w.temperature, 0, w.top_p, w.rep, w.history[sl], mode=oracle.MODE_TRUTH)
-    assert np.array_equal(part["tokens"], fx["tokens"])
-    assert np.array_equal(part["probs"].view(np.uint32), fx["probs"].view(np.uint32))
-    diff = part["tokens"] != tr["tokens"]
+    assert np.array_equal(part["probs"].view(np.uint32), full["probs"][sl].view(np.uint32))
+    # 64 rows drawn across the batch (its first and last eight and 48 others) against both oracle layers
+    rng = np.random.default_rng(synth.BASE_SEED + 5)
+    idx = np.unique(np.concatenate([np.arange(8), np.arange(B - 8, B), rng.choice(np.arange(8, B - 8), 48, replace=False)]))
+    x, u, h = np.ascontiguousarray(w.logits[idx]), w.uniforms[idx], np.ascontiguousarray(w.history[idx])
+    fx = oracle.sample(x, u, w.temperature, 0, w.top_p, w.rep, h, mode=oracle.MODE_FIXED)
+    tr = oracle.sample(x, u, w.temperature, 0, w.top_p, w.rep, h, mode=oracle.MODE_TRUTH)
+    got_t, got_p = full["tokens"][idx], full["probs"][idx]
+    assert np.array_equal(got_t, fx["tokens"])
+    assert np.array_equal(got_p.view(np.uint32), fx["probs"].view(np.uint32))
+    diff = got_t != tr["tokens"]
     assert not (diff & ~tr["near"]).any()
     # CDF steps are about 1e-5 wide on these flat rows, so the 1e-6 criterion flags many rows by itself; what is held
     # to a bound is the number of tokens that actually differ from the fp64 layer (a draw within ~3e-7 of a step)
-    assert int(diff.sum()) <= 2, f"{int(diff.sum())} of 24 tokens differ from the fp64 layer"
-    assert np.allclose(part["probs"][~diff], tr["probs"][~diff], rtol=1e-5)
-    print(f"C5 slice: {int(tr['near'].sum())} of 24 rows flagged near a CDF step, {int(diff.sum())} tokens differ from the truth layer")
+    assert int(diff.sum()) <= 4, f"{int(diff.sum())} of {idx.size} tokens differ from the fp64 layer"
+    assert np.allclose(got_p[~diff], tr["probs"][~diff], rtol=1e-5)
+    print(f"C5: {int(tr['near'].sum())} of {idx.size} rows flagged near a CDF step, {int(diff.sum())} tokens differ from the truth layer")
     s.Status()
