@@ -102,9 +102,9 @@ __device__ __forceinline__ float next_below(float x) {
 
 // exp(-d), d >= 0; see the spec, section 6.  dcut <= 80: the distance beyond which the mass is zero (80, or the
 // min-p bound -ln(min_p) when that is smaller).
-__device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
-    const bool in = d <= dcut;                                    // false for NaN too
-    float x = in ? -d : 0.0f;                                     // (a select at each end instead of a branch around the polynomial)
+// (the polynomial itself, of x = -d; no range test: the result is exp(x) as specified for -87 <= x <= 0 and some
+// deterministic value anywhere else)
+__device__ __forceinline__ float expneg_core(float x) {
     float k = rintf(x * 1.44269504f);
     float r = fmaf(k, -0.693145752f, x);
     r = fmaf(k, -1.42860677e-06f, r);
@@ -116,7 +116,11 @@ __device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
     float r2 = r * r;
     y = fmaf(y, r2, r);
     y = y + 1.0f;
-    const float e = __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
+    return __uint_as_float(__float_as_uint(y) + ((u32)(int)k << 23));   // exact scaling by 2^k (result normal)
+}
+__device__ __forceinline__ float expneg(float d, float dcut = 80.0f) {
+    const bool in = d <= dcut;                                    // false for NaN too
+    const float e = expneg_core(in ? -d : 0.0f);                  // (a select at each end instead of a branch around the polynomial)
     return in ? e : 0.0f;
 }
 __device__ __forceinline__ float emass(float z, float m, float dcut = 80.0f) {
@@ -131,6 +135,15 @@ __device__ __forceinline__ u64 qfix(float e, float scale) {
     const float x = e * scale;
     const u32 hi = (u32)(x * 2.3283064365386963e-10f);
     const u32 lo = (u32)__fmaf_rn(-(float)hi, 4294967296.0f, x);
+    return ((u64)hi << 32) | (u64)lo;
+}
+// The same from scale32 = 2^(S - 32): t = e * 2^(S - 32) is exact, its integer part is the high word and its fractional
+// part (exact: t >= 0) times 2^32 the low word.  One instruction fewer; the kernels whose sweeps are bound by the
+// vector ALU use it.
+__device__ __forceinline__ u64 qfix32(float e, float scale32) {
+    const float t = e * scale32;
+    const u32 hi = (u32)t;
+    const u32 lo = (u32)(__builtin_amdgcn_fractf(t) * 4294967296.0f);
     return ((u64)hi << 32) | (u64)lo;
 }
 __device__ __forceinline__ float mass_scale(int S) { return __uint_as_float((u32)(S + 127) << 23); }

@@ -74,6 +74,10 @@ __device__ __forceinline__ float nuc_z_shortcut(const NucRow &r, float y) {
 // blocks left over are a third of the row; measured slower on long ones and in the single-sweep kernel).
 // `pre` runs once before the first element is visited, with the first stage's loads already in flight (work that
 // must precede the visits but not the loads: building the history bitmap).
+template <bool NT, bool REVERSE>
+struct NucMode {                                                   // how a sweep reads the row
+    static constexpr bool value = NT, rev = REVERSE;
+};
 struct NucNoPre {
     __device__ __forceinline__ void operator()() const {}
 };
@@ -85,7 +89,7 @@ __device__ __forceinline__ nuc_f32x4 nuc_load4(const nuc_f32x4 *p) {
 }
 // PLAIN: the caller knows that the row has no penalties (a loop of its own without the penalty code: the visitor's
 // test of r.penal at every visit cost the single-sweep kernel 5 %).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F4, class F1, class PRE = NucNoPre>
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, bool REV = false, class F4, class F1, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
@@ -130,20 +134,23 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             const int nfull = n4 / (NUC_U * NUC_BLOCK);
             const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
             if (nfull > 0) {
+                // REV: the whole stages from the row's end to its start (a sweep that follows a forward one finds
+                // the end of the row, read last, still in the caches)
+                auto at = [&](int s) { return REV ? nfull - 1 - s : s; };
                 nuc_f32x4 va[NUC_U], vb[NUC_U];
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + u * NUC_BLOCK + tid);
+                for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(0) * NUC_U + u) * NUC_BLOCK + tid);
                 pre();
                 for (int s = 0; s + 1 < nfull; s++) {
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + ((s + 1) * NUC_U + u) * NUC_BLOCK + tid);
+                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + (at(s + 1) * NUC_U + u) * NUC_BLOCK + tid);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(s) * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
                 }
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) visit4(va[u], (((nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
             } else {
                 pre();
             }
@@ -186,9 +193,9 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     }
 }
 // Visits every element of the row as f(id, penalised logit).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, class F, class PRE = NucNoPre>
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool REV = false, bool PLAIN = false, class F, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f, PRE pre = PRE()) {
-    nuc_foreach4<NUC_BLOCK, NT, AHEAD>(r, bm, [&](int j, const float (&y)[4]) {
+    nuc_foreach4<NUC_BLOCK, NT, AHEAD, PLAIN, REV>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
     }, f, pre);
@@ -271,7 +278,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     static_assert(NUC_SEEN * NUC_BLOCK * sizeof(u32) <= 2 * NUC_CAP * sizeof(u64), "the list of seen ids fits the gathered entries' storage");
     const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
     int seen_id[NUC_SEEN];
-    float seen_y[NUC_SEEN];
+    float seen_y[NUC_SEEN], seen_raw[NUC_SEEN];
+    bool lin = false;
     r.masked = list_seen;
     r.skip = -INFINITY;                                              // sweep 1: neither the maximum nor the smallest finite value
     // What must precede the first visit of sweep 1 but not its first loads: run by the row visitor with the first stage
@@ -335,25 +343,33 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 const int i = tid + k * NUC_BLOCK;
                 seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
             }
-            float raw[NUC_SEEN];
 #pragma unroll
-            for (int k = 0; k < NUC_SEEN; k++) raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
+            for (int k = 0; k < NUC_SEEN; k++) seen_raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++)
-                seen_y[k] = seen_id[k] >= 0 ? penalise_seen(raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
+                seen_y[k] = seen_id[k] >= 0 ? penalise_seen(seen_raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
         }
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
     auto sweep = [&](auto nt, auto f, auto pre) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f, pre);
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, decltype(nt)::rev>(r, bm, f, pre);
         if (r.masked) {
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++)
                 if (seen_id[k] >= 0) f(seen_id[k], seen_y[k]);
         }
     };
-    typedef std::integral_constant<bool, false> Cached;             // the row is read again: ordinary loads
-    typedef std::integral_constant<bool, true> Streamed;             // the row's last sweep: non-temporal loads
+    // every element of the row as f(id, logit as stored): no penalty, no look at the history bitmap
+    auto sweep_plain = [&](auto nt, auto f) {
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, decltype(nt)::rev, true>(r, bm, f, NucNoPre());
+    };
+    typedef NucMode<false, false> Cached;                            // the row is read again: ordinary loads
+#ifdef BORN_NUC_ZIGZAG
+    typedef NucMode<false, true> CachedBack;                         // .. from its end to its start
+#else
+    typedef Cached CachedBack;
+#endif
+    typedef NucMode<true, false> Streamed;                           // the row's last sweep: non-temporal loads
 
     BORN_STAMP(a, row, 1);
     // ---- sweep 1: maximum of the penalised logits, and about how far below it they reach
@@ -378,6 +394,42 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         // mass and ranked last, next to the id's real entry). A maximum that leaves no such value: penalties inside the sweeps.
         if (r.masked && fabsf(r.m) < 1e6f) r.skip = uniform_f32((r.m - 200.0f) * r.T);
         else r.masked = false;
+        // The usual row (a maximum of ordinary size, a temperature whose division has the shortcut, no min-p bound, a history
+        // short enough to be listed): sweeps 2 and 3 read the logits as stored, without the history bitmap, and what the
+        // seen ids contribute is set right apart, see below.
+        const float amx = fabsf(uniform_f32(mx)), am = fabsf(r.m);
+        lin = !r.degenerate && am >= 0x1p-40f && am < 0x1p90f && amx < 0x1p90f && (r.T == 1.0f || r.rcp != 0.0f) &&
+              r.dcut == 80.0f && (!r.penal || r.masked);
+    }
+    // In such a row the mass of a logit y needs no test of y at all. With x = z' - m, z' the three-instruction quotient
+    // (y itself at temperature 1), the mass is that of exp(clamp(x, -87, 0)), and every kind of y comes out as specified:
+    //   2^-100 <= |y| < 2^100  z' is the correctly rounded quotient, x = -d exactly;
+    //   zeros and |y| < 2^-100  z' stays below 2^-78, half an ulp of m or less: x = -m, as with the exact z;
+    //   -inf, NaN               x is -inf or a NaN (the quotient of -inf is inf - inf); the clamp (a median of three, which
+    //                           returns the smallest operand when one is a NaN) gives -87: no mass;
+    //   y <= -2^100             z' is -inf or within 2^-20 of the quotient, below -2^80: no mass;
+    //   +inf, y >= 2^100        not in such a row (the maximum is below 2^90).
+    // Beyond d = 80 the specified mass is 0, and so is trunc(exp(x) * 2^S) down to the clamp (S <= 61).  A seen id's
+    // stored logit may exceed the penalised maximum: clamped to x = 0, some mass that the correction takes out again.
+    const float scale32 = r.scale * 2.3283064365386963e-10f, nsbin = -r.sbin;
+    auto lin_z = [&](float y) { return r.T == 1.0f ? y : nuc_z_shortcut(r, y); };
+    auto lin_put = [&](float z, auto minus) {
+        const float x = z - r.m;
+        const u64 q = qfix32(expneg_core(__builtin_amdgcn_fmed3f(x, -87.0f, 0.0f)), scale32);
+        const int b = (int)__builtin_amdgcn_fmed3f(x * nsbin, 0.0f, (float)(NUC_BINS - 1));
+        atomicAdd(&mass[b], decltype(minus)::value ? 0ull - q : q);
+    };
+    typedef std::integral_constant<bool, false> Plus;
+    typedef std::integral_constant<bool, true> Minus;
+    if (lin && r.penal) {
+        // The histogram is a sum of integers modulo 2^64: sweep 2 adds every id's stored logit, so each seen id's stored
+        // logit is taken out (by the same arithmetic, to the bit) and its penalised logit put in, here, in any order.
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++)
+            if (seen_id[k] >= 0) {
+                lin_put(lin_z(seen_raw[k]), Minus());
+                lin_put(lin_z(seen_y[k]), Plus());
+            }
     }
 
     BORN_STAMP(a, row, 2);
@@ -387,8 +439,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     return;
 #endif
     // ---- sweep 2: integer masses by bin
-    if (r.T == 1.0f && !r.degenerate) {
-        sweep(Cached(), [&](int, float y) {
+    if (lin) {
+        if (r.T == 1.0f) sweep_plain(CachedBack(), [&](int, float y) { lin_put(y, Plus()); });
+        else sweep_plain(CachedBack(), [&](int, float y) { lin_put(nuc_z_shortcut(r, y), Plus()); });
+    } else if (r.T == 1.0f && !r.degenerate) {
+        sweep(CachedBack(), [&](int, float y) {
             float z = y;                                             // a logit of ordinary magnitude is its own canonical form
             if (!nuc_ordinary(y)) {
                 asm volatile("" ::: "memory");                       // (keeps this a branch: as selects it is paid by every logit)
@@ -398,14 +453,14 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
     } else if (r.rcp != 0.0f && !r.degenerate) {
-        sweep(Cached(), [&](int, float y) {
+        sweep(CachedBack(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
     } else {
-        sweep(Cached(), [&](int, float y) {
+        sweep(CachedBack(), [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
@@ -515,7 +570,26 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             }
         };
         // (bitwise and / or of the compares: the short-circuit forms compiled to a nest of branches per logit)
-        if (nint == 1) {
+        if (lin) {
+            // (the stored logits; a seen id's stored logit that passes is dropped below, its penalised logit is offered
+            // here under the id with the top bit set)
+            if (nint == 1) {
+                sweep_plain(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+            } else {
+                sweep_plain(Streamed(), [&](int j, float y) {
+                    append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
+                });
+            }
+            if (r.penal) {
+#pragma unroll
+                for (int k = 0; k < NUC_SEEN; k++)
+                    if (seen_id[k] >= 0) {
+                        const float y = seen_y[k];
+                        append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y,
+                               (int)((u32)seen_id[k] | 0x80000000u));
+                    }
+            }
+        } else if (nint == 1) {
             sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); }, NucNoPre());
         } else {
             sweep(Streamed(), [&](int j, float y) {
@@ -530,11 +604,16 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             bool take = false;
             u64 key = 0ull, qs = 0ull;
             if (e < cw) {
-                const uint2 c = list[e];
+                uint2 c = list[e];
+                bool stale = false;                                  // a seen id's stored logit
+                if (lin && r.penal) {
+                    if (c.y & 0x80000000u) c.y &= 0x7FFFFFFFu;
+                    else stale = (bm[c.y >> 5] >> (c.y & 31)) & 1u;
+                }
                 const float z = nuc_z(r, __uint_as_float(c.x));
                 const float d = nuc_d(r, z);
                 const int b = nuc_bin(r, d);
-                const int slot = whole ? (b <= w0 ? 0 : -1) : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
+                const int slot = stale ? -1 : whole ? (b <= w0 ? 0 : -1) : b == w0 ? 0 : b == w1 ? 1 : b == w2 ? 2 : -1;
                 if (slot >= 0) {
                     take = true;
                     key = make_key64(z, (int)c.y);
@@ -910,7 +989,11 @@ static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConf
 
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows, bool two_per_cu) {
     // More rows than CUs, and two rows' LDS fit one CU: 512 threads per row, two rows to a CU at a time.
+#ifdef BORN_NUC_FORCE_1024
+    if (false) launch_nucleus_of<512>(a, st, rows);                  // (measurement builds only)
+#else
     if ((two_per_cu || a.B > cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU) launch_nucleus_of<512>(a, st, rows);
+#endif
     else launch_nucleus_of<1024>(a, st, rows);
     return hipGetLastError();
 }

@@ -721,9 +721,13 @@ def test_three_sweep_kernel_division_shortcut_and_unusual_magnitudes(oracle, roc
     x = (rng.standard_normal((B, V)) * 2.5).astype(np.float32)
     odd = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 3e-31, -3e-31, 7.9e-31, 2 ** -100, -(2 ** -100), 2 ** -101, 1.2e30, -1.2e30,
                     2 ** 100, 2 ** 99, -(2 ** 100), 3e38, -3e38, np.inf, -np.inf, np.nan], dtype=np.float32)
+    # values that leave the row's maximum ordinary (such rows take the sweeps that test no logit's magnitude)
+    low = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 3e-31, -3e-31, 7.9e-31, 2 ** -100, -(2 ** -100), 2 ** -101, -1.2e30,
+                    -(2 ** 100), -(2 ** 99), -3e38, -np.inf, np.nan], dtype=np.float32)
     for b in range(1, B):
         at = rng.choice(V, size=40 * b, replace=False)
-        x[b, at] = rng.choice(odd if b % 3 else odd[:17], size=at.size)        # (rows b % 3 == 0: no infinities, no huge values)
+        # (rows b % 3 == 0: no infinities, no huge values; b % 3 == 1: nothing above the ordinary maximum)
+        x[b, at] = rng.choice(odd[:17] if b % 3 == 0 else low if b % 3 == 1 else odd, size=at.size)
     x[5, :] = rng.choice(np.array([0.0, -0.0, 1e-45, 2 ** -101, 3e-31], dtype=np.float32), size=V)   # nothing of ordinary magnitude
     u = rng.random(B, dtype=np.float32)
     hist = rng.integers(0, V, size=(B, 64)).astype(np.int32)
@@ -754,6 +758,27 @@ def test_three_sweep_kernel_seen_ids_visited_apart(oracle, rocm, V, H, scale, pa
     for (T, p, rep, freq, pres) in [(3.0, 1.0, 1.3, 0.0, 0.0), (1.2, 0.999, 1.05, 0.0, 0.0), (2.0, 1.0, 1.0, 0.3, 0.2),
                                     (0.8, 0.9, 2.0, 0.1, 0.0)]:
         got, _, _ = _check_against_oracle(oracle, rocm, x, u, T * scale, 0, p, rep, hist, hl, path=path, freq=freq, pres=pres)
+        assert got["counters"]["general_rows"] == B
+
+
+@pytest.mark.parametrize("path", NUCLEUS_PATHS)
+@pytest.mark.parametrize("T", [1.0, 0.8, 1.9999999])
+def test_three_sweep_kernel_seen_logits_above_the_penalised_maximum(oracle, rocm, T, path):
+    """Rows whose largest stored logits belong to ids of the history, far above everything else, so that after the
+    penalty the maximum is another logit or a much smaller value: the sweeps that read the logits as stored meet
+    values above the maximum they work from, up to overflow of the exponential, and what they add for them must
+    come out again exactly. Also with unusual values among the seen ids. Bit-exact against the oracle."""
+    rng = np.random.default_rng(int(T * 1000) + 5)
+    B, V, H = 10, 9001, 200
+    x = rng.standard_normal((B, V)).astype(np.float32)
+    hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
+    tops = [60.0, 25.0, 300.0, 3000.0, 1e9, 12.0, 88.5, 1e30, 40.0, 14.0]
+    for b in range(B):
+        x[b, hist[b, :3 + b % 4]] = np.float32(tops[b]) * (1 + 0.01 * np.arange(3 + b % 4, dtype=np.float32))
+        x[b, hist[b, 10:20]] = np.array([0.0, -0.0, 1e-45, -np.inf, np.nan, -3e38, 2 ** -101, -1e-39, 5.0, -5.0], dtype=np.float32)
+    u = rng.random(B, dtype=np.float32)
+    for p, rep, freq, pres in [(0.95, 10.0, 0.0, 0.0), (1.0, 1.3, 0.0, 0.0), (0.9, 100.0, 0.0, 0.0), (0.99, 1.0, 2.0, 30.0)]:
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, 0, p, rep, hist, path=path, freq=freq, pres=pres)
         assert got["counters"]["general_rows"] == B
 
 
