@@ -99,13 +99,13 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             // id among its four, but a lane rarely holds two, so the wave computes one penalty per visit, not four.
             u32 bits = (bm[j >> 5] >> (j & 31)) & 0xFu;
             if (r.masked) {
-                if (bits) {
-                    const u32 sk = __float_as_uint(r.skip);
+                // a sign-extended bit field extract and a bitwise select per element, unconditionally: a branch around
+                // them is taken by nearly every wave once the history has a few hundred ids
+                const u32 sk = __float_as_uint(r.skip);
 #pragma unroll
-                    for (int t = 0; t < 4; t++) {                    // a bit field extract and a bitwise select per element
-                        const u32 m = (u32)((int)(bits << (31 - t)) >> 31);
-                        y[t] = __uint_as_float((sk & m) | (__float_as_uint(y[t]) & ~m));
-                    }
+                for (int t = 0; t < 4; t++) {
+                    const u32 m = (u32)((int)(bits << (31 - t)) >> 31);
+                    y[t] = __uint_as_float((sk & m) | (__float_as_uint(y[t]) & ~m));
                 }
                 bits = 0u;
             }
@@ -137,20 +137,30 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
                 // REV: the whole stages from the row's end to its start (a sweep that follows a forward one finds
                 // the end of the row, read last, still in the caches)
                 auto at = [&](int s) { return REV ? nfull - 1 - s : s; };
+                // Two stages a turn, each loaded while the other is visited, so that no register is copied; the last
+                // one or two stages in a loop of their own.
                 nuc_f32x4 va[NUC_U], vb[NUC_U];
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(0) * NUC_U + u) * NUC_BLOCK + tid);
                 pre();
-                for (int s = 0; s + 1 < nfull; s++) {
+                int s = 0;
+                for (; s + 2 < nfull; s += 2) {
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + (at(s + 1) * NUC_U + u) * NUC_BLOCK + tid);
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(s) * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
-                }
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(s + 2) * NUC_U + u) * NUC_BLOCK + tid);
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(nfull - 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(vb[u], ((at(s + 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                }
+                for (;;) {
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(s) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    if (++s >= nfull) break;
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(s) * NUC_U + u) * NUC_BLOCK + tid);
+                }
             } else {
                 pre();
             }
@@ -242,7 +252,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     extern __shared__ __align__(16) u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ int s_n, s_over, s_nseen;
-    __shared__ u64 s_win, s_mass;
+    __shared__ u64 s_win, s_mass, s_slot0[4];
     __shared__ u32 s_wcount[NUC_WAVES];
 
     u64 *const mass = nuc_dyn;                                                   // [NUC_BINS] masses, then cumulative
@@ -363,7 +373,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     auto sweep_plain = [&](auto nt, auto f) {
         nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, decltype(nt)::rev, true>(r, bm, f, NucNoPre());
     };
+#ifdef BORN_NUC_ALL_NT
+    typedef NucMode<true, false> Cached;
+#else
     typedef NucMode<false, false> Cached;                            // the row is read again: ordinary loads
+#endif
 #ifdef BORN_NUC_ZIGZAG
     typedef NucMode<false, true> CachedBack;                         // .. from its end to its start
 #else
@@ -646,22 +660,54 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     }
     __syncthreads();
 
-    // ---- cumulative mass of every listed entry within its bin, in rank order
+    // ---- cumulative mass of every listed entry within its bin, in rank order.  The bins' value ranges are disjoint, so
+    // the rank order of the whole list goes bin by bin: an entry counts the keys above its own (all distinct: the id is
+    // part of the key) and moves to that place; one scan of the masses in that order gives every entry the mass at and
+    // above it, and where a bin begins the scan holds what the bins listed before it add up to.
     u64 mykey = 0ull, mine = 0ull;                                   // inclusive mass at and above this entry in its bin
     int myslot = -1;
-    if (tid < n) {
-        mykey = fkey[tid];
-        myslot = (int)(fq[tid] >> 62);
-        // four entries a turn, their eight words read with four 128-bit LDS loads before any is used (one dependent
-        // read per entry made this loop wait for LDS: a few hundred entries took longer than a sweep of the row)
-        const ulonglong2 *k2 = reinterpret_cast<const ulonglong2 *>(fkey), *q2 = reinterpret_cast<const ulonglong2 *>(fq);
-        for (int j = 0; j < n4; j += 4) {
-            const ulonglong2 ka = k2[j >> 1], kb = k2[(j >> 1) + 1], qa = q2[j >> 1], qb = q2[(j >> 1) + 1];
-            const u64 ks[4] = {ka.x, ka.y, kb.x, kb.y}, qs[4] = {qa.x, qa.y, qb.x, qb.y};
+    if (n <= 2 * WAVE) {
+        // (a short list: every entry sums the masses of its bin's entries at and above it; no barrier, no scan)
+        if (tid < n) {
+            mykey = fkey[tid];
+            myslot = (int)(fq[tid] >> 62);
+            const ulonglong2 *k2 = reinterpret_cast<const ulonglong2 *>(fkey), *q2 = reinterpret_cast<const ulonglong2 *>(fq);
+            for (int j = 0; j < n4; j += 4) {
+                const ulonglong2 ka = k2[j >> 1], kb = k2[(j >> 1) + 1], qa = q2[j >> 1], qb = q2[(j >> 1) + 1];
+                const u64 ks[4] = {ka.x, ka.y, kb.x, kb.y}, qs[4] = {qa.x, qa.y, qb.x, qb.y};
 #pragma unroll
-            for (int t = 0; t < 4; t++)
-                if ((int)(qs[t] >> 62) == myslot && ks[t] >= mykey) mine += qs[t] & 0x3FFFFFFFFFFFFFFFull;
+                for (int t = 0; t < 4; t++)
+                    if ((int)(qs[t] >> 62) == myslot && ks[t] >= mykey) mine += qs[t] & 0x3FFFFFFFFFFFFFFFull;
+            }
         }
+    } else {
+        u64 *const skey = reinterpret_cast<u64 *>(stage), *const sq = skey + NUC_CAP;       // the staging lists are spent
+        static_assert(2 * NUC_CAP <= NUC_WAVES * NUC_WCAP, "the ordered entries fit the staging lists' storage");
+        if (tid < n) {
+            const u64 key = fkey[tid];
+            int rank = 0;
+            // four keys a turn, read with two 128-bit LDS loads before any is used
+            const ulonglong2 *k2 = reinterpret_cast<const ulonglong2 *>(fkey);
+            for (int j = 0; j < n4; j += 4) {
+                const ulonglong2 ka = k2[j >> 1], kb = k2[(j >> 1) + 1];
+                rank += (int)(ka.x > key) + (int)(ka.y > key) + (int)(kb.x > key) + (int)(kb.y > key);
+            }
+            skey[rank] = key;
+            sq[rank] = fq[tid];
+        }
+        __syncthreads();
+        u64 q = 0ull;
+        if (tid < n) {
+            mykey = skey[tid];
+            const u64 w = sq[tid];
+            myslot = (int)(w >> 62);
+            q = w & 0x3FFFFFFFFFFFFFFFull;
+        }
+        u64 listed_mass;
+        const u64 incl = block_inclusive_scan_u64<NUC_BLOCK>(q, &scr, &listed_mass);
+        if (tid < n && (tid == 0 || (int)(sq[tid - 1] >> 62) != myslot)) s_slot0[myslot] = incl - q;
+        __syncthreads();
+        if (tid < n) mine = incl - s_slot0[myslot];
     }
     __syncthreads();                                                 // the lists may be overwritten from here on
 
