@@ -179,18 +179,34 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + tid, lastb));
                 pre();
-                for (int s = 0; s + 1 < nst; s++) {
+                int s = 0;
+                for (; s + 2 < nst; s += 2) {                        // (two whole stages a turn: no register is copied)
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + min(((s + 1) * NUC_U + u) * NUC_BLOCK + tid, lastb));
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
-                }
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(((s + 2) * NUC_U + u) * NUC_BLOCK + tid, lastb));
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) {
-                    const int i = ((nst - 1) * NUC_U + u) * NUC_BLOCK + tid;
-                    if (i < n4) visit4(va[u], i << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(vb[u], (((s + 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                }
+                // the last one or two stages, the very last whole or partial
+                if (s + 1 < nst) {
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + min(((s + 1) * NUC_U + u) * NUC_BLOCK + tid, lastb));
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) {
+                        const int i = ((s + 1) * NUC_U + u) * NUC_BLOCK + tid;
+                        if (i < n4) visit4(vb[u], i << 2);
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) {
+                        const int i = (s * NUC_U + u) * NUC_BLOCK + tid;
+                        if (i < n4) visit4(va[u], i << 2);
+                    }
                 }
             } else {
                 pre();
