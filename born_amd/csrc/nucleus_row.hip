@@ -305,11 +305,22 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
     int seen_id[NUC_SEEN];
     float seen_y[NUC_SEEN], seen_raw[NUC_SEEN];
+    unsigned seen_cnt[NUC_SEEN];
     bool lin = false;
     r.masked = list_seen;
     r.skip = -INFINITY;                                              // sweep 1: neither the maximum nor the smallest finite value
     // What must precede the first visit of sweep 1 but not its first loads: run by the row visitor with the first stage
     // in flight (barriers that wait for LDS only).
+    // (all of the thread's history loads are requested here, before the sweep's first loads: in flight together, their
+    // latency behind the clearing of the tables)
+    int hv[NUC_SEEN];
+    if (list_seen) {
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++) {
+            const int i = tid + k * NUC_BLOCK;
+            hv[k] = i < hlen ? h[i] : -2;
+        }
+    }
     auto prologue = [&]() {
         if (r.penal)
             for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
@@ -327,12 +338,6 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         // penalty inside the sweep costs a whole wave the penalty arithmetic whenever one of its lanes holds a seen id, which
         // with a long history is nearly always. A history too long for the registers keeps the penalty inside the sweeps.
         if (list_seen) {
-            int hv[NUC_SEEN];                                            // (all of the thread's history loads in flight together)
-#pragma unroll
-            for (int k = 0; k < NUC_SEEN; k++) {
-                const int i = tid + k * NUC_BLOCK;
-                hv[k] = i < hlen ? h[i] : -2;
-            }
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++) {
                 const int t = hv[k];
@@ -369,11 +374,16 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 const int i = tid + k * NUC_BLOCK;
                 seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
             }
+            // (requested here, used after the sweep: their latency, and the occurrence counts', behind the sweep)
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++) seen_raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
+            if (COUNTED) {
 #pragma unroll
-            for (int k = 0; k < NUC_SEEN; k++)
-                seen_y[k] = seen_id[k] >= 0 ? penalise_seen(seen_raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
+                for (int k = 0; k < NUC_SEEN; k++) seen_cnt[k] = seen_id[k] >= 0 ? r.counts[seen_id[k]] : 0u;
+            }
+#ifdef BORN_NUC_STAMP_PROLOGUE
+            BORN_STAMP(a, row, 2);
+#endif
         }
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
@@ -406,16 +416,26 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     {
         float mx = -INFINITY, mn = INFINITY;
         // (the smallest value only sizes the bins: every fourth id is looked at, spread over the whole row)
-        sweep(Cached(), [&](int j, float y) {
+        auto top = [&](int j, float y) {
             mx = fmaxf(mx, y);
             if ((j & 3) == 0) mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
-        }, prologue);
+        };
+        nuc_foreach<NUC_BLOCK, Cached::value, NUC_BLOCK == 1024, false>(r, bm, top, prologue);
+        // the seen ids' logits, requested by the prologue, are first needed here
+#pragma unroll
+        for (int k = 0; k < NUC_SEEN; k++)
+            seen_y[k] = seen_id[k] >= 0 ? penalise_counted(seen_raw[k], r.rep, COUNTED, seen_cnt[k], r.freq, r.pres) : 0.0f;
+        if (r.masked) {
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++)
+                if (seen_id[k] >= 0) top(seen_id[k], seen_y[k]);
+        }
         mx = block_max_f32<NUC_BLOCK>(mx, &scr);
         mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
         r.m = uniform_f32(nuc_z(r, mx));
         r.degenerate = r.m == -INFINITY;                             // nothing finite: every d is 0 by definition
         const float zmin = mn < INFINITY ? nuc_z(r, mn) : r.m;
-        const float span = r.degenerate ? 0.0f : r.m - zmin;         // >= 0
+        const float span = r.degenerate ? 0.0f : fmaxf(r.m - zmin, 0.0f);
         // the bins cover the logits that can carry mass: the row's span, at most 32, at most the min-p bound
         r.range = uniform_f32(fminf(fminf(32.0f, span * 1.0001f + 1e-3f), r.dcut * 1.0001f + 1e-3f));
         r.sbin = uniform_f32((float)NUC_BINS / r.range);
@@ -462,7 +482,9 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             }
     }
 
+#ifndef BORN_NUC_STAMP_PROLOGUE
     BORN_STAMP(a, row, 2);
+#endif
 #if defined(BORN_NUC_STOP_AFTER) && BORN_NUC_STOP_AFTER == 1
     // (measurement builds only: the row ends after the named sweep, for per-sweep instruction counts; results are wrong)
     if (tid == 0) a.tokens[row] = __float_as_int(r.sbin) & 1;

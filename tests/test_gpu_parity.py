@@ -762,14 +762,16 @@ def test_three_sweep_kernel_seen_ids_visited_apart(oracle, rocm, V, H, scale, pa
 
 
 @pytest.mark.parametrize("path", NUCLEUS_PATHS)
-@pytest.mark.parametrize("T", [1.0, 0.8, 1.9999999])
-def test_three_sweep_kernel_seen_logits_above_the_penalised_maximum(oracle, rocm, T, path):
+@pytest.mark.parametrize("T,V", [(1.0, 9001), (0.8, 9001), (1.9999999, 9001), (0.8, 40003), (1.0, 70000)])
+def test_three_sweep_kernel_seen_logits_above_the_penalised_maximum(oracle, rocm, T, V, path):
     """Rows whose largest stored logits belong to ids of the history, far above everything else, so that after the
     penalty the maximum is another logit or a much smaller value: the sweeps that read the logits as stored meet
     values above the maximum they work from, up to overflow of the exponential, and what they add for them must
-    come out again exactly. Also with unusual values among the seen ids. Bit-exact against the oracle."""
-    rng = np.random.default_rng(int(T * 1000) + 5)
-    B, V, H = 10, 9001, 200
+    come out again exactly; and the first sweep, which keeps a maximum per stage of the row and reads again the
+    stages whose maximum a seen id holds, reads several of them again. Also with unusual values among the seen ids.
+    Bit-exact against the oracle."""
+    rng = np.random.default_rng(int(T * 1000) + 5 + V)
+    B, H = 10, 200
     x = rng.standard_normal((B, V)).astype(np.float32)
     hist = rng.integers(0, V, size=(B, H)).astype(np.int32)
     tops = [60.0, 25.0, 300.0, 3000.0, 1e9, 12.0, 88.5, 1e30, 40.0, 14.0]
