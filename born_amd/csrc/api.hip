@@ -445,8 +445,12 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
         rows.path = s->path;
         rows.launched = launched;
         if (launched & 1u) keep_first(launch_topk_row(a, st, &rows));
-        if (launched & 2u) keep_first(launch_nucleus_row(a, st, &rows, s->path == 2));
-        if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
+        if ((launched & 6u) == 6u) {
+            keep_first(launch_nucleus_and_general_rows(a, st, rows, s->path == 2));
+        } else {
+            if (launched & 2u) keep_first(launch_nucleus_row(a, st, &rows, s->path == 2));
+            if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
+        }
     } else if (launched == 1u) {
         keep_first(launch_topk_row(a, st));
     } else {

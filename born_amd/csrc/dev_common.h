@@ -206,16 +206,6 @@ __device__ __forceinline__ float uniform_f32(float v) { return __int_as_float(__
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }
 __device__ __forceinline__ int wave_id() { return (int)(threadIdx.x >> 6); }
 
-__device__ __forceinline__ float wave_max_f32(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-    return v;
-}
-__device__ __forceinline__ u32 wave_sum_u32(u32 v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
-}
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
 // load still in flight (its workgroup-scope fence covers global memory), which would serialise
 // a software pipeline that keeps the next tile's loads outstanding across the barrier.
@@ -231,6 +221,29 @@ __device__ __forceinline__ void lds_barrier() {
 template <int CTRL, int ROW_MASK = 0xF>
 __device__ __forceinline__ u32 dpp_u32(u32 old, u32 src) {
     return (u32)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, ROW_MASK, 0xF, false);
+}
+
+// Wave-wide maximum (NaNs ignored, as fmaxf does) and sum, the same value in every lane: four DPP steps inside each
+// row of 16 lanes, then one lane per row read back (no lane-index registers, which a shuffle keeps alive for the
+// whole kernel).
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, __uint_as_float(dpp_u32<0xB1>(__float_as_uint(v), __float_as_uint(v))));
+    v = fmaxf(v, __uint_as_float(dpp_u32<0x4E>(__float_as_uint(v), __float_as_uint(v))));
+    v = fmaxf(v, __uint_as_float(dpp_u32<0x141>(__float_as_uint(v), __float_as_uint(v))));
+    v = fmaxf(v, __uint_as_float(dpp_u32<0x140>(__float_as_uint(v), __float_as_uint(v))));
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ u32 wave_sum_u32(u32 v) {
+    v += dpp_u32<0xB1>(v, v);                                        // pairs, quads, eights (half-row mirror), sixteens (row mirror)
+    v += dpp_u32<0x4E>(v, v);
+    v += dpp_u32<0x141>(v, v);
+    v += dpp_u32<0x140>(v, v);
+    return (u32)__builtin_amdgcn_readlane((int)v, 0) + (u32)__builtin_amdgcn_readlane((int)v, 16) +
+           (u32)__builtin_amdgcn_readlane((int)v, 32) + (u32)__builtin_amdgcn_readlane((int)v, 48);
 }
 
 // Wave-wide maximum / minimum as a wave-uniform value: four DPP steps inside each row of 16
@@ -295,13 +308,19 @@ __device__ __forceinline__ u64 shfl_u64(u64 v, int src) {
     u32 lo = __shfl((u32)v, src, WAVE), hi = __shfl((u32)(v >> 32), src, WAVE);
     return ((u64)hi << 32) | lo;
 }
+// (the 32-bit scan's steps on both halves, the carry in the 64-bit addition)
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ u64 dpp_u64(u64 v) {
+    const u32 lo = dpp_u32<CTRL, ROW_MASK>(0u, (u32)v), hi = dpp_u32<CTRL, ROW_MASK>(0u, (u32)(v >> 32));
+    return ((u64)hi << 32) | lo;
+}
 __device__ __forceinline__ u64 wave_inclusive_scan_u64(u64 v) {
-    int l = lane_id();
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {
-        u64 t = shfl_up_u64(v, o);
-        if (l >= o) v += t;
-    }
+    v += dpp_u64<0x111>(v);
+    v += dpp_u64<0x112>(v);
+    v += dpp_u64<0x114>(v);
+    v += dpp_u64<0x118>(v);
+    v += dpp_u64<0x142, 0xA>(v);
+    v += dpp_u64<0x143, 0xC>(v);
     return v;
 }
 

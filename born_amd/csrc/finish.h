@@ -10,7 +10,7 @@ namespace born {
 // `ns` are the top-k survivors.  Computes the integer CDF, the top-p cut and the draw.
 // ---------------------------------------------------------------------------
 template <int BLOCK, int ITEMS>
-__device__ void finish_sorted(const u64 *list, int ns, const SampleArgs &a, int row, BlockScratch *scr) {
+__device__ __forceinline__ void finish_sorted(const u64 *list, int ns, const SampleArgs &a, int row, BlockScratch *scr) {
     const int tid = threadIdx.x;
     const float scale = mass_scale(a.mass_shift);
     const float m = key64_z(list[0]);

@@ -171,6 +171,7 @@ hipError_t launch_cand_rows(const SampleArgs &a, const float *thr, const unsigne
 hipError_t launch_sample_wide(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
 // two_per_cu: 512 threads per row whatever the batch (else: only for batches of more rows than the device has CUs)
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr, bool two_per_cu = false);
+hipError_t launch_nucleus_and_general_rows(const SampleArgs &a, hipStream_t st, const RowConfigs &rows, bool two_per_cu);
 hipError_t configure_nucleus();
 size_t nucleus_lds_bytes(int V);
 hipError_t launch_spec_verify(const SpecArgs &a, hipStream_t st);

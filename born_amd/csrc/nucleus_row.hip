@@ -14,10 +14,21 @@
 //            first entry in rank order whose cumulative mass reaches a target is found with an LDS max.
 // A wanted bin too full for the lists (heavy ties, masked rows) is refined in place by a radix descent over
 // the rank keys of that bin, 11 bits per sweep.
+#include <algorithm>
 #include <type_traits>
 #include "dev_common.h"
+#include "finish.h"
 #include "kernels.h"
 #include "row_config.h"
+
+// (the general kernel's row body, for the kernel below that takes a row of either kind)
+#define BORN_WIDE_BLOCK 1024
+#define BORN_WIDE_NS wide_in_nucleus
+#define BORN_WIDE_BODY_ONLY
+#include "sample_wide_impl.h"
+#undef BORN_WIDE_BODY_ONLY
+#undef BORN_WIDE_BLOCK
+#undef BORN_WIDE_NS
 
 namespace born {
 
@@ -898,6 +909,29 @@ __global__ __launch_bounds__(BLOCK, 4) void nucleus_row_rows_kernel(SampleArgs a
     }
     nucleus_row_body<BLOCK, COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres, 0.0f);   // (a row's own temperature: no shortcut)
 }
+// Per-row configurations of any kind: the rows without a top-k cut and the rows of the general kernel in one launch (a
+// launch whose workgroups all find their rows to be another kernel's still costs its 7 us at 256 rows).
+template <bool COUNTED>
+__global__ __launch_bounds__(1024) void nucleus_or_general_rows_kernel(SampleArgs a, RowConfigs rc) {
+    extern __shared__ __align__(16) u64 either_dyn[];                // (the same storage as the three-sweep body's)
+    __shared__ BlockScratch wide_scr;
+    __shared__ int wide_int[8];
+    __shared__ u64 wide_u64[4];
+    const int row = (int)blockIdx.x;
+    RowValues v;
+    bool invalid;
+    if (row_config_values(a, rc, row, ROUTE_NUCLEUS, v, invalid)) {   // workgroup-uniform, before any barrier
+        if (invalid) row_config_reject(a, row);
+        else nucleus_row_body<1024, COUNTED>(a, v.T, v.top_p, v.rep, v.dcut, v.freq, v.pres, 0.0f);
+        return;
+    }
+    if (!row_config(a, rc, row, ROUTE_GENERAL, invalid)) return;
+    if (invalid) {
+        row_config_reject(a, row);
+        return;
+    }
+    wide_in_nucleus::wide_row<COUNTED>(a, row, (lds_u64 *)either_dyn, (BORN_LDS BlockScratch *)&wide_scr, (lds_int *)wide_int, (lds_u64 *)wide_u64);
+}
 
 // ---------------------------------------------------------------------------------------------------------
 // Log-probability of one given token per row under the softmax of the row's penalised, temperature-scaled
@@ -1071,6 +1105,24 @@ static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConf
     }
 }
 
+// Whether launch_nucleus_row would give this batch 512 threads per row.
+static bool nucleus_two_per_cu(const SampleArgs &a, bool two_per_cu) {
+    return (two_per_cu || a.B > cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU;
+}
+// The rows without a top-k cut and the general kernel's rows of a batch with per-row configurations: one launch where
+// the former would get a workgroup of 1024 threads anyway, else the two kernels one after the other.
+hipError_t launch_nucleus_and_general_rows(const SampleArgs &a, hipStream_t st, const RowConfigs &rows, bool two_per_cu) {
+    if (nucleus_two_per_cu(a, two_per_cu)) {
+        const hipError_t e = launch_nucleus_row(a, st, &rows, two_per_cu);
+        if (e != hipSuccess) return e;
+        return launch_sample_wide(a, st, &rows);
+    }
+    const size_t lds = std::max(nucleus_lds_bytes_of<1024>(a.V), wide_lds_bytes(a.V));
+    if (a.hist_counts) hipLaunchKernelGGL(nucleus_or_general_rows_kernel<true>, dim3((unsigned)a.B), dim3(1024), lds, st, a, rows);
+    else hipLaunchKernelGGL(nucleus_or_general_rows_kernel<false>, dim3((unsigned)a.B), dim3(1024), lds, st, a, rows);
+    return hipGetLastError();
+}
+
 hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows, bool two_per_cu) {
     // More rows than CUs, and two rows' LDS fit one CU: 512 threads per row, two rows to a CU at a time.
 #ifdef BORN_NUC_FORCE_1024
@@ -1097,6 +1149,13 @@ hipError_t configure_nucleus() {
                           reinterpret_cast<const void *>(nucleus_row_rows_kernel<512, true>)};
     for (const void *k : half) {
         const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds512);
+        if (e != hipSuccess) return e;
+    }
+    const int lds_both = (int)std::max(nucleus_lds_bytes((int)WIDE_MAX_VOCAB), wide_lds_bytes((int)WIDE_MAX_VOCAB));
+    const void *both[] = {reinterpret_cast<const void *>(nucleus_or_general_rows_kernel<false>),
+                          reinterpret_cast<const void *>(nucleus_or_general_rows_kernel<true>)};
+    for (const void *k : both) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_both);
         if (e != hipSuccess) return e;
     }
     return hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -1,5 +1,7 @@
 // Body of the general sampling kernel, instantiated once per workgroup size by sample_wide.hip:
 // BORN_WIDE_BLOCK threads per workgroup, everything inside namespace born::BORN_WIDE_NS.
+// (BORN_WIDE_BODY_ONLY: the row's body without the kernels and their launchers, for a kernel of another file that
+// calls it.)
 namespace born {
 namespace BORN_WIDE_NS {
 
@@ -237,7 +239,7 @@ __device__ __forceinline__ void wide_sort(const WideCtx &c, int n) {
 
 // Radix descent inside one over-full bin: refine by 11 key bits per sweep until the
 // remaining set fits the list.  The sub-histograms live in the list's storage.
-__device__ __noinline__ Found wide_descend(const WideCtx &c, int b, bool by_count, u64 target, u64 base_mass, u64 base_cnt) {
+__device__ __forceinline__ Found wide_descend(const WideCtx &c, int b, bool by_count, u64 target, u64 base_mass, u64 base_cnt) {
     lds_u64 *smass = c.list;                                       // [WIDE_SUB_BINS]
     lds_u32 *scnt = (lds_u32 *)(c.list + WIDE_SUB_BINS);           // [WIDE_SUB_BINS]
     u64 prefix = 0;
@@ -317,10 +319,9 @@ __device__ __forceinline__ Found wide_find(const WideCtx &c, WideHeld &held, boo
             held.n = n;
         }
     }
-    if (descend) {                       // over-full bin (ties, masked rows): refined out of line, on a copy of the
-        const WideCtx cc = c;            // context so that the original never has its address taken
-        return wide_descend(cc, b, by_count, target, base_mass, base_cnt);
-    }
+    // (an over-full bin (ties, masked rows) is refined in line: a call would give the kernel a stack, and a kernel with
+    // a stack pays some 10 us per launch for it, whether a row ever descends or not)
+    if (descend) return wide_descend(c, b, by_count, target, base_mass, base_cnt);
     return wide_resolve(c, held.n, b, by_count, target, base_mass, base_cnt);
 }
 
@@ -477,6 +478,7 @@ __device__ __forceinline__ void wide_row(const SampleArgs &a, const int row, lds
     if (tid == 0) count_row(a.counters, row, 2);
 }
 
+#ifndef BORN_WIDE_BODY_ONLY
 // One workgroup per row of the batch.
 template <bool COUNTED>
 __global__ __launch_bounds__(WIDE_BLOCK) void sample_wide_kernel(SampleArgs a) {
@@ -527,6 +529,8 @@ hipError_t configure() {
     }
     return hipSuccess;
 }
+
+#endif  // BORN_WIDE_BODY_ONLY
 
 }  // namespace BORN_WIDE_NS
 }  // namespace born
