@@ -53,6 +53,30 @@ __device__ __forceinline__ float spec_z(float x, float T, float rcp) {
     return canon(x);
 }
 
+// The usual row: a maximum m = z(largest logit) of ordinary size (2^-40 <= |m| < 2^60) and, away from temperature 1, a
+// temperature whose division has the three-instruction shortcut.  The integer mass of a logit x of such a row needs no
+// test of x: with z' the shortcut's quotient (x itself at temperature 1), it is that of exp(clamp(z' - m, -87, 0)):
+//   2^-100 <= |x| < 2^100  z' is the correctly rounded quotient, a canonical z;
+//   zeros, |x| < 2^-100    z' stays below 2^-78, less than half an ulp of m: z' - m = -m, as with the exact z;
+//   -inf, NaN              z' - m is -inf or a NaN; the clamp (a median of three, which returns the smallest operand
+//                          when one is a NaN) gives -87: no mass, as specified for z = -inf;
+//   x <= -2^100            z' is -inf or far below m - 80: no mass;
+//   +inf, x >= 2^100       not in such a row.
+// Beyond d = 80 the specified mass is 0, and so is trunc(exp(-d) * 2^S) down to the clamp (S <= 61).
+__device__ __forceinline__ bool spec_usual_row(float m, float T, float rcp) {
+    const float am = fabsf(m);
+    return am >= 0x1p-40f && am < 0x1p60f && (T == 1.0f || rcp != 0.0f);
+}
+template <bool UNIT>
+__device__ __forceinline__ u64 spec_usual_mass(float x, float m, float T, float rcp, float scale32) {
+    float z = x;
+    if (!UNIT) {
+        const float q = __fmul_rn(x, rcp), e = __fmaf_rn(-q, T, x);
+        z = __fmaf_rn(e, rcp, q);
+    }
+    return qfix32(expneg_core(__builtin_amdgcn_fmed3f(z - m, -87.0f, 0.0f)), scale32);
+}
+
 template <bool RESIDENT, bool UNIT>
 __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
     __shared__ BlockScratch scr;
@@ -85,21 +109,29 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
             const spec_f32x4 fill = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
             t[i] = j < n4 ? __builtin_nontemporal_load(reinterpret_cast<const spec_f32x4 *>(x) + j) : fill;
         }
+        // (z is a non-decreasing function of the logit: the maximum of the logits as stored, NaNs ignored, gives m)
 #pragma unroll
         for (int i = 0; i < SPEC_NF4; i++) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                t[i][c] = spec_z<UNIT>(t[i][c], T, rcp);                  // the -inf fill stays -inf
-                m = fmaxf(m, t[i][c]);
-            }
+            for (int c = 0; c < 4; c++) m = fmaxf(m, t[i][c]);
         }
         m = block_max_f32<SPEC_BLOCK>(m, &scr);
-        if (m > -INFINITY) {                                         // (uniform) m - z is a number: +inf for a masked logit, no mass
+        m = UNIT ? canon(m) : spec_z<false>(m, T, rcp);
+        if (spec_usual_row(m, T, rcp)) {                             // (uniform)
+            const float scale32 = scale * 2.3283064365386963e-10f;
 #pragma unroll
             for (int i = 0; i < SPEC_NF4; i++) {
                 if (i * SPEC_BLOCK + tid < n4) {
 #pragma unroll
-                    for (int c = 0; c < 4; c++) sum += qfix(expneg(m - t[i][c]), scale);
+                    for (int c = 0; c < 4; c++) sum += spec_usual_mass<UNIT>(t[i][c], m, T, rcp, scale32);
+                }
+            }
+        } else if (m > -INFINITY) {                                  // (uniform) m - z is a number: +inf for a masked logit, no mass
+#pragma unroll
+            for (int i = 0; i < SPEC_NF4; i++) {
+                if (i * SPEC_BLOCK + tid < n4) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) sum += qfix(expneg(m - spec_z<UNIT>(t[i][c], T, rcp)), scale);
                 }
             }
         } else {                                                     // nothing finite: (-inf) - (-inf) := 0 for every logit
@@ -107,7 +139,7 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
             for (int i = 0; i < SPEC_NF4; i++) {
                 if (i * SPEC_BLOCK + tid < n4) {
 #pragma unroll
-                    for (int c = 0; c < 4; c++) sum += qfix(emass(t[i][c], m), scale);
+                    for (int c = 0; c < 4; c++) sum += qfix(emass(spec_z<UNIT>(t[i][c], T, rcp), m), scale);
                 }
             }
         }
@@ -135,10 +167,26 @@ __global__ __launch_bounds__(SPEC_BLOCK) void spec_stats_kernel(SpecArgs a) {
 __device__ __forceinline__ float spec_z_any(float x, float T, float rcp) {
     return rcp != 0.0f ? z_of_shortcut(x, T, rcp) : z_of(x, T);      // (uniform; z_of itself skips the division at T = 1)
 }
+// USUAL: both rows are usual ones (spec_usual_row): the masses without a test of the logits.
+template <bool USUAL>
 __device__ __forceinline__ u64 residual_mass(float t, float d, float T, float rcp, float mp, float mq, float scale, double ip,
                                              double iq, double scale_d) {
-    double pj = (double)qfix(emass(spec_z_any(t, T, rcp), mp), scale) * ip;
-    double qj = (double)qfix(emass(spec_z_any(d, T, rcp), mq), scale) * iq;
+    u64 mt, md;
+    if (USUAL) {
+        const float scale32 = scale * 2.3283064365386963e-10f;
+        if (T == 1.0f) {                                             // (uniform)
+            mt = spec_usual_mass<true>(t, mp, T, rcp, scale32);
+            md = spec_usual_mass<true>(d, mq, T, rcp, scale32);
+        } else {
+            mt = spec_usual_mass<false>(t, mp, T, rcp, scale32);
+            md = spec_usual_mass<false>(d, mq, T, rcp, scale32);
+        }
+    } else {
+        mt = qfix(emass(spec_z_any(t, T, rcp), mp), scale);
+        md = qfix(emass(spec_z_any(d, T, rcp), mq), scale);
+    }
+    double pj = (double)mt * ip;
+    double qj = (double)md * iq;
     double r = pj > qj ? pj - qj : 0.0;
     return (u64)(r * scale_d);
 }
@@ -176,6 +224,7 @@ struct SpecRow {
     float T, rcp, mp, mq, scale;
     double Zp, Zq, scale_d;       // Zp, Zq: reciprocals of the integer normalisers
     bool plain;                   // bonus row: the mass of id j is the row's own integer mass, there is no draft
+    bool usual;                   // both maxima are of ordinary size and the division has its shortcut: masses without tests
 };
 // Position i of sequence b; i == G is the bonus row.
 __device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
@@ -198,11 +247,13 @@ __device__ __forceinline__ SpecRow spec_row(const SpecArgs &a, int b, int i) {
         r.Zp = 1.0 / (double)a.Zp[row];
         r.Zq = 1.0 / (double)a.Zq[row];
     }
+    r.usual = spec_usual_row(r.mp, r.T, r.rcp) && spec_usual_row(r.mq, r.T, r.rcp);
     return r;
 }
 __device__ __forceinline__ u64 spec_mass(const SpecRow &r, float t, float d) {
     if (r.plain) return qfix(emass(spec_z_any(t, r.T, r.rcp), r.mp), r.scale);    // uniform per row
-    return residual_mass(t, d, r.T, r.rcp, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+    if (r.usual) return residual_mass<true>(t, d, r.T, r.rcp, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
+    return residual_mass<false>(t, d, r.T, r.rcp, r.mp, r.mq, r.scale, r.Zp, r.Zq, r.scale_d);
 }
 constexpr int SPEC_RUN = 8;                   // run lengths up to this are loaded before any arithmetic
 __device__ __forceinline__ u64 spec_run_mass(const SpecRow &r, int j0, int j1) {

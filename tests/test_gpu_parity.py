@@ -910,6 +910,43 @@ def test_spec_verify_special_cases(oracle, rocm):
     s.Status()                                                             # the status word clears once read
 
 
+@pytest.mark.parametrize("T", [1.0, 0.8, 1.9999999])
+@pytest.mark.parametrize("V", [32000, 3001, 40000])
+def test_spec_verify_unusual_logits(oracle, rocm, T, V):
+    """Zeros of both signs, denormals, tiny and hugely negative values, -inf (masked tokens) and NaNs mixed into both
+    models' rows under maxima of ordinary size (the kernels then compute every mass without a test of the logit), rows
+    with +inf or huge maxima (which take the tested arithmetic), and a draft that masks what the target prefers:
+    accept counts and tokens bit-exact against the oracle, resident, scalar and two-sweep rows, with and without the
+    division shortcut (1.9999999 has none)."""
+    rng = np.random.default_rng(V + int(T * 100))
+    B, G = 8, 3
+    t = (rng.standard_normal((B, G + 1, V)) * 2).astype(np.float32)
+    dr = (t[:, :G] + 0.7 * rng.standard_normal((B, G, V))).astype(np.float32)
+    low = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 3e-31, -3e-31, 2 ** -100, -(2 ** -100), 2 ** -101, -1.2e30, -(2 ** 100),
+                    -3e38, -np.inf, np.nan], dtype=np.float32)
+    for b in range(B):
+        for g in range(G + 1):
+            at = rng.choice(V, size=50 + 10 * b, replace=False)
+            t[b, g, at] = rng.choice(low, size=at.size)
+            if g < G:
+                at = rng.choice(V, size=50 + 10 * b, replace=False)
+                dr[b, g, at] = rng.choice(low, size=at.size)
+    t[6, 1, 17] = np.inf                                                  # rows outside the usual kind
+    dr[6, 2, 5] = 3e38
+    t[7, 0, 99] = 2.0 ** 101
+    dr[5, 0, np.argsort(t[5, 0])[-40:]] = -np.inf                          # the draft masks the target's favourites
+    d = rng.integers(0, V, size=(B, G)).astype(np.int32)
+    ua, ur = rng.random((B, G), dtype=np.float32), rng.random(B, dtype=np.float32)
+    s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T), max_batch=B, max_vocab=V)
+    got = rocm.verify_host(s, t, dr, d, ua, ur, bonus=True)
+    tt, bonus = np.ascontiguousarray(t[:, :G]), np.ascontiguousarray(t[:, G])
+    fx = oracle.spec_verify(tt, dr, d, ua, ur, temperature=T, mode=oracle.MODE_FIXED, bonus=bonus)
+    assert np.array_equal(got["n_accepted"], fx["n_accepted"]), (T, V)
+    assert np.array_equal(got["next_token"], fx["next_token"]), (T, V)
+    s.Status()
+    s.Close()
+
+
 def test_spec_verify_bonus_draw(oracle, rocm):
     # target given as [B, G + 1, V] (the bonus row is the last position, addressed through sequence strides)
     rng = np.random.default_rng(31)
