@@ -1,4 +1,4 @@
-// Sampler for top_k disabled (full-vocabulary multinomial and top-p): one workgroup of 1024 threads per
+// Sampler for top_k disabled (full-vocabulary multinomial and top-p): one workgroup of 1024 or 512 threads per
 // row, three sweeps over the row (docs/SAMPLING_SPEC.md, fixed-point layer).
 //
 //   sweep 1  maximum and smallest finite value of the penalised logits (z is a non-decreasing function of
@@ -10,10 +10,16 @@
 //   sweep 3  gather: a compare of the penalised logit against the wanted bins' value ranges (widened, so
 //            that it can only over-select) stages about 1 % of the row in per-wave LDS lists (ballot + lane
 //            rank); the staged entries are then classified exactly.
-//   resolve  every gathered entry sums the masses of the entries of its bin that rank at or above it; the
-//            first entry in rank order whose cumulative mass reaches a target is found with an LDS max.
+//   resolve  the gathered entries are put in rank order by counting, one scan of their masses gives every entry
+//            the mass at and above it within its bin (a short list: summed directly); the first entry in rank
+//            order whose cumulative mass reaches a target is found with an LDS max.
 // A wanted bin too full for the lists (heavy ties, masked rows) is refined in place by a radix descent over
 // the rank keys of that bin, 11 bits per sweep.
+// In the usual row (a maximum of ordinary size, a temperature whose division has the three-instruction shortcut, no
+// min-p bound, a history short enough to be listed) sweeps 2 and 3 read the logits as stored: no history bitmap, no
+// test of a logit's magnitude, clamps in place of selects; what the seen ids contribute is corrected apart (the
+// histogram is a sum of integers, so a stored logit's mass comes out again exactly).  The sweeps are then bound by
+// the three reads of the row from HBM, not by the vector ALU.
 #include <algorithm>
 #include <type_traits>
 #include "dev_common.h"
@@ -190,34 +196,18 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
 #pragma unroll
                 for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + tid, lastb));
                 pre();
-                int s = 0;
-                for (; s + 2 < nst; s += 2) {                        // (two whole stages a turn: no register is copied)
+                for (int s = 0; s + 1 < nst; s++) {
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + min(((s + 1) * NUC_U + u) * NUC_BLOCK + tid, lastb));
 #pragma unroll
                     for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(((s + 2) * NUC_U + u) * NUC_BLOCK + tid, lastb));
-#pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(vb[u], (((s + 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) va[u] = vb[u];
                 }
-                // the last one or two stages, the very last whole or partial
-                if (s + 1 < nst) {
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + min(((s + 1) * NUC_U + u) * NUC_BLOCK + tid, lastb));
-#pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
-#pragma unroll
-                    for (int u = 0; u < NUC_U; u++) {
-                        const int i = ((s + 1) * NUC_U + u) * NUC_BLOCK + tid;
-                        if (i < n4) visit4(vb[u], i << 2);
-                    }
-                } else {
-#pragma unroll
-                    for (int u = 0; u < NUC_U; u++) {
-                        const int i = (s * NUC_U + u) * NUC_BLOCK + tid;
-                        if (i < n4) visit4(va[u], i << 2);
-                    }
+                for (int u = 0; u < NUC_U; u++) {
+                    const int i = ((nst - 1) * NUC_U + u) * NUC_BLOCK + tid;
+                    if (i < n4) visit4(va[u], i << 2);
                 }
             } else {
                 pre();
@@ -316,22 +306,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     const bool list_seen = r.penal && hlen <= NUC_SEEN * NUC_BLOCK;
     int seen_id[NUC_SEEN];
     float seen_y[NUC_SEEN], seen_raw[NUC_SEEN];
-    unsigned seen_cnt[NUC_SEEN];
     bool lin = false;
     r.masked = list_seen;
     r.skip = -INFINITY;                                              // sweep 1: neither the maximum nor the smallest finite value
     // What must precede the first visit of sweep 1 but not its first loads: run by the row visitor with the first stage
     // in flight (barriers that wait for LDS only).
-    // (all of the thread's history loads are requested here, before the sweep's first loads: in flight together, their
-    // latency behind the clearing of the tables)
-    int hv[NUC_SEEN];
-    if (list_seen) {
-#pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++) {
-            const int i = tid + k * NUC_BLOCK;
-            hv[k] = i < hlen ? h[i] : -2;
-        }
-    }
     auto prologue = [&]() {
         if (r.penal)
             for (int i = tid; i < ((V + 31) >> 5); i += NUC_BLOCK) bm[i] = 0u;
@@ -349,6 +328,12 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         // penalty inside the sweep costs a whole wave the penalty arithmetic whenever one of its lanes holds a seen id, which
         // with a long history is nearly always. A history too long for the registers keeps the penalty inside the sweeps.
         if (list_seen) {
+            int hv[NUC_SEEN];                                            // (all of the thread's history loads in flight together)
+#pragma unroll
+            for (int k = 0; k < NUC_SEEN; k++) {
+                const int i = tid + k * NUC_BLOCK;
+                hv[k] = i < hlen ? h[i] : -2;
+            }
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++) {
                 const int t = hv[k];
@@ -385,16 +370,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 const int i = tid + k * NUC_BLOCK;
                 seen_id[k] = i < nseen ? (int)seen_list[i] : -1;
             }
-            // (requested here, used after the sweep: their latency, and the occurrence counts', behind the sweep)
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++) seen_raw[k] = seen_id[k] >= 0 ? r.x[seen_id[k]] : 0.0f;
-            if (COUNTED) {
 #pragma unroll
-                for (int k = 0; k < NUC_SEEN; k++) seen_cnt[k] = seen_id[k] >= 0 ? r.counts[seen_id[k]] : 0u;
-            }
-#ifdef BORN_NUC_STAMP_PROLOGUE
-            BORN_STAMP(a, row, 2);
-#endif
+            for (int k = 0; k < NUC_SEEN; k++)
+                seen_y[k] = seen_id[k] >= 0 ? penalise_seen(seen_raw[k], r.rep, r.counts, seen_id[k], r.freq, r.pres) : 0.0f;
         }
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
@@ -427,26 +407,16 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     {
         float mx = -INFINITY, mn = INFINITY;
         // (the smallest value only sizes the bins: every fourth id is looked at, spread over the whole row)
-        auto top = [&](int j, float y) {
+        sweep(Cached(), [&](int j, float y) {
             mx = fmaxf(mx, y);
             if ((j & 3) == 0) mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
-        };
-        nuc_foreach<NUC_BLOCK, Cached::value, NUC_BLOCK == 1024, false>(r, bm, top, prologue);
-        // the seen ids' logits, requested by the prologue, are first needed here
-#pragma unroll
-        for (int k = 0; k < NUC_SEEN; k++)
-            seen_y[k] = seen_id[k] >= 0 ? penalise_counted(seen_raw[k], r.rep, COUNTED, seen_cnt[k], r.freq, r.pres) : 0.0f;
-        if (r.masked) {
-#pragma unroll
-            for (int k = 0; k < NUC_SEEN; k++)
-                if (seen_id[k] >= 0) top(seen_id[k], seen_y[k]);
-        }
+        }, prologue);
         mx = block_max_f32<NUC_BLOCK>(mx, &scr);
         mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
         r.m = uniform_f32(nuc_z(r, mx));
         r.degenerate = r.m == -INFINITY;                             // nothing finite: every d is 0 by definition
         const float zmin = mn < INFINITY ? nuc_z(r, mn) : r.m;
-        const float span = r.degenerate ? 0.0f : fmaxf(r.m - zmin, 0.0f);
+        const float span = r.degenerate ? 0.0f : r.m - zmin;         // >= 0
         // the bins cover the logits that can carry mass: the row's span, at most 32, at most the min-p bound
         r.range = uniform_f32(fminf(fminf(32.0f, span * 1.0001f + 1e-3f), r.dcut * 1.0001f + 1e-3f));
         r.sbin = uniform_f32((float)NUC_BINS / r.range);
@@ -493,9 +463,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             }
     }
 
-#ifndef BORN_NUC_STAMP_PROLOGUE
     BORN_STAMP(a, row, 2);
-#endif
 #if defined(BORN_NUC_STOP_AFTER) && BORN_NUC_STOP_AFTER == 1
     // (measurement builds only: the row ends after the named sweep, for per-sweep instruction counts; results are wrong)
     if (tid == 0) a.tokens[row] = __float_as_int(r.sbin) & 1;

@@ -1,29 +1,33 @@
 // One-launch sampler for 1 <= top_k <= 512 (docs/SAMPLING_SPEC.md, fixed-point layer): one workgroup
 // of 1024 threads per row.
 //
-// The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 logits, the
-// loads of three stages in flight.  A stage is not a contiguous piece of the row: the row is cut into chunks
-// of 64 float4 (1 KiB, what one wave instruction loads) and stage s takes the chunks (u * 16 + w) * nstage + s
-// for the four loads u of the sixteen waves w, so that every stage is an even sample of the whole row by
-// position.  Rows whose large logits sit late in vocabulary order (sorted ascending, a step up near the end, a
-// slow rise) then look to the pass like any other row.
+// The row is streamed from HBM once with 128-bit non-temporal loads in stages of 16384 consecutive logits, the
+// loads of three stages in flight.  The stages are examined in the order first, last, second, third, ...: a row
+// whose large logits sit at the end of the vocabulary (sorted ascending, a step up near the end) shows them to
+// the threshold before the bulk of the row is filtered against it.
 //
 //   T   A threshold that the row's top_k-th largest logit is known to reach.  First from the first stage alone:
 //       every wave takes the a-th largest of its lane maxima, and the w-th largest of the wave results has
 //       >= w * a >= top_k logits of that stage at or above it.
 //   L   Every logit >= T met from then on is appended, exact value and id, to the list of the wave that met it
 //       (ballot + lane rank, no atomics): one compare per logit in the common case.
-//   T'  After the first stage and then every three stages, with the next stages' loads in flight, the lists'
-//       entries are binned by key distance above T (one LDS atomic each); the highest bin boundary with >= top_k
-//       + margin entries at or above it becomes the new T and every wave drops its entries below it.  The lists
-//       so end the pass with little more than top_k + margin entries between them, and nothing has to be
-//       thinned out after the last load.
+//   T'  Every three stages, with the next stages' loads in flight, the lists' entries are binned by key distance
+//       above T (one LDS atomic each); the highest bin boundary with >= top_k + margin entries at or above it
+//       becomes the new T and every wave drops its entries below it.
+//   T"  A wave whose list would overflow inside a stage (late-large logits: the common threshold is stale) raises
+//       a threshold of its own first: it bins the stage's own logits by value between the threshold and a robust
+//       maximum (the 8th largest lane maximum), takes the highest boundary with enough of them above it, drops its
+//       list entries below that, and filters the stage again.  The wave's threshold never falls below the common one,
+//       so the bound of the proof is the largest threshold any wave ended with.
+//   After the last load the lists hold a few times top_k entries; final rounds of T' (each refining inside the bin
+//   the boundary fell into) bring them down to what the rank sort takes.
 //   Any logit outside the lists is below T, and so is its z after a penalty (repetition_penalty >= 1
 //   only lowers a logit) and the monotone division by the temperature.  Every wave turns its own entries into rank
 //   keys (probing its hash of the history) and appends them to one array; the row is proven if top_k candidates
-//   end up with z strictly above that bound.  A rank sort orders them and one wave computes the integer CDF, the
-//   top-p cut and the draw.  (A history longer than the workgroup is not hashed: the candidates' ids are, and the
-//   history probes them.)
+//   end up with z strictly above that bound.  A rank sort orders them (by counting for top_k <= 128, by buckets of
+//   the key above that; candidates of equal z are ranked among themselves from a short list) and one wave computes
+//   the integer CDF, the top-p cut and the draw, up to eight candidates per lane.  (A history longer than the
+//   workgroup is not hashed: the candidates' ids are, and the history probes them.)
 // Rows that cannot be proven (fewer than top_k finite logits, heavy ties, list overflow, penalised
 // tokens dropping below the bound) are finished by the same workgroup with an exact selection that
 // works for any input: a radix descent over the 64-bit rank keys (z descending, id ascending; the
