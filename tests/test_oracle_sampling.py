@@ -193,7 +193,8 @@ def _torch_sample(x, u, T, k, p, rep, hist, min_p=0.0, freq=0.0, pres=0.0):
 
 
 @pytest.mark.parametrize("T,k,p,rep", [(1.0, 0, 1.0, 1.0), (0.8, 40, 0.95, 1.1), (0.7, 50, 0.9, 1.15),
-                                         (1.2, 0, 0.99, 1.05), (1.0, 5, 1.0, 1.0), (1.5, 0, 0.5, 0.8)])
+                                         (1.2, 0, 0.99, 1.05), (1.0, 5, 1.0, 1.0), (1.5, 0, 0.5, 0.8),
+                                         (0.9, 129, 0.97, 1.1), (1.0, 256, 1.0, 1.0), (0.7, 512, 0.95, 1.2)])
 def test_against_torch_restatement(oracle, T, k, p, rep):
     rng = np.random.default_rng(7)
     B, V, H = 48, 1000, 32
