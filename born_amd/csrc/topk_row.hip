@@ -520,10 +520,32 @@ __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey,
     const u32 range = smax > gkey ? smax - gkey : 0u;
     const int sh = max(0, 24 - (int)__clz(range));                   // (range >> sh) < ROW_TBINS
     u32 mx = 0u;
-    for (int e = l; e < cw; e += WAVE) {
-        const u32 key = ordkey(__uint_as_float(list[e].x));
-        mx = max(mx, key);
-        if (key >= gkey) atomicAdd(&H[min((key - gkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
+    if (cw <= 2 * WAVE) {                                            // wave-uniform: the usual, short list
+        for (int e = l; e < cw; e += WAVE) {
+            const u32 key = ordkey(__uint_as_float(list[e].x));
+            mx = max(mx, key);
+            if (key >= gkey) atomicAdd(&H[min((key - gkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
+        }
+    } else {
+        // A long list is what a wave's own raise leaves behind: its entries lie close together next to the range, and
+        // thousands of atomics would go to one word.  Lanes that share a bin add once between them, twice over.
+        for (int e = l; e < cw; e += WAVE) {
+            const u32 key = ordkey(__uint_as_float(list[e].x));
+            mx = max(mx, key);
+            bool todo = key >= gkey;
+            const u32 bin = todo ? min((key - gkey) >> sh, (u32)(ROW_TBINS - 1)) : 0u;
+#pragma unroll
+            for (int turn = 0; turn < 2; turn++) {
+                const u64 open = __ballot(todo);
+                if (!open) break;                                    // (wave-uniform)
+                const u32 first = (u32)__builtin_amdgcn_readlane((int)bin, __builtin_ctzll(open));
+                const bool same = todo && bin == first;
+                const u64 mk = __ballot(same);
+                if (same && __builtin_ctzll(mk) == l) atomicAdd(&H[first], (u32)__popcll(mk));
+                todo = todo && !same;
+            }
+            if (todo) atomicAdd(&H[bin], 1u);
+        }
     }
     mx = wave_max_u32(mx);
     if (l == 0 && mx) atomicMax(Mnext, mx);
