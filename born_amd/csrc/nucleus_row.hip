@@ -91,10 +91,6 @@ __device__ __forceinline__ float nuc_z_shortcut(const NucRow &r, float y) {
 // blocks left over are a third of the row; measured slower on long ones and in the single-sweep kernel).
 // `pre` runs once before the first element is visited, with the first stage's loads already in flight (work that
 // must precede the visits but not the loads: building the history bitmap).
-template <bool NT, bool REVERSE>
-struct NucMode {                                                   // how a sweep reads the row
-    static constexpr bool value = NT, rev = REVERSE;
-};
 struct NucNoPre {
     __device__ __forceinline__ void operator()() const {}
 };
@@ -106,7 +102,7 @@ __device__ __forceinline__ nuc_f32x4 nuc_load4(const nuc_f32x4 *p) {
 }
 // PLAIN: the caller knows that the row has no penalties (a loop of its own without the penalty code: the visitor's
 // test of r.penal at every visit cost the single-sweep kernel 5 %).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, bool REV = false, class F4, class F1, class PRE = NucNoPre>
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F4, class F1, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
@@ -151,32 +147,29 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
             const int nfull = n4 / (NUC_U * NUC_BLOCK);
             const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
             if (nfull > 0) {
-                // REV: the whole stages from the row's end to its start (a sweep that follows a forward one finds
-                // the end of the row, read last, still in the caches)
-                auto at = [&](int s) { return REV ? nfull - 1 - s : s; };
                 // Two stages a turn, each loaded while the other is visited, so that no register is copied; the last
                 // one or two stages in a loop of their own.
                 nuc_f32x4 va[NUC_U], vb[NUC_U];
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(0) * NUC_U + u) * NUC_BLOCK + tid);
+                for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + u * NUC_BLOCK + tid);
                 pre();
                 int s = 0;
                 for (; s + 2 < nfull; s += 2) {
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + (at(s + 1) * NUC_U + u) * NUC_BLOCK + tid);
+                    for (int u = 0; u < NUC_U; u++) vb[u] = nuc_load4<NT>(x4 + ((s + 1) * NUC_U + u) * NUC_BLOCK + tid);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(s) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(s + 2) * NUC_U + u) * NUC_BLOCK + tid);
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + ((s + 2) * NUC_U + u) * NUC_BLOCK + tid);
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(vb[u], ((at(s + 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(vb[u], (((s + 1) * NUC_U + u) * NUC_BLOCK + tid) << 2);
                 }
                 for (;;) {
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((at(s) * NUC_U + u) * NUC_BLOCK + tid) << 2);
+                    for (int u = 0; u < NUC_U; u++) visit4(va[u], ((s * NUC_U + u) * NUC_BLOCK + tid) << 2);
                     if (++s >= nfull) break;
 #pragma unroll
-                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (at(s) * NUC_U + u) * NUC_BLOCK + tid);
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + (s * NUC_U + u) * NUC_BLOCK + tid);
                 }
             } else {
                 pre();
@@ -220,9 +213,9 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
     }
 }
 // Visits every element of the row as f(id, penalised logit).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool REV = false, bool PLAIN = false, class F, class PRE = NucNoPre>
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F, class PRE = NucNoPre>
 __device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f, PRE pre = PRE()) {
-    nuc_foreach4<NUC_BLOCK, NT, AHEAD, PLAIN, REV>(r, bm, [&](int j, const float (&y)[4]) {
+    nuc_foreach4<NUC_BLOCK, NT, AHEAD, PLAIN>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
     }, f, pre);
@@ -379,7 +372,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
     auto sweep = [&](auto nt, auto f, auto pre) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, decltype(nt)::rev>(r, bm, f, pre);
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f, pre);
         if (r.masked) {
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++)
@@ -388,19 +381,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     };
     // every element of the row as f(id, logit as stored): no penalty, no look at the history bitmap
     auto sweep_plain = [&](auto nt, auto f) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, decltype(nt)::rev, true>(r, bm, f, NucNoPre());
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, true>(r, bm, f, NucNoPre());
     };
-#ifdef BORN_NUC_ALL_NT
-    typedef NucMode<true, false> Cached;
-#else
-    typedef NucMode<false, false> Cached;                            // the row is read again: ordinary loads
-#endif
-#ifdef BORN_NUC_ZIGZAG
-    typedef NucMode<false, true> CachedBack;                         // .. from its end to its start
-#else
-    typedef Cached CachedBack;
-#endif
-    typedef NucMode<true, false> Streamed;                           // the row's last sweep: non-temporal loads
+    typedef std::integral_constant<bool, false> Cached;             // the row is read again: ordinary loads
+    typedef std::integral_constant<bool, true> Streamed;             // the row's last sweep: non-temporal loads
 
     BORN_STAMP(a, row, 1);
     // ---- sweep 1: maximum of the penalised logits, and about how far below it they reach
@@ -471,10 +455,10 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 #endif
     // ---- sweep 2: integer masses by bin
     if (lin) {
-        if (r.T == 1.0f) sweep_plain(CachedBack(), [&](int, float y) { lin_put(y, Plus()); });
-        else sweep_plain(CachedBack(), [&](int, float y) { lin_put(nuc_z_shortcut(r, y), Plus()); });
+        if (r.T == 1.0f) sweep_plain(Cached(), [&](int, float y) { lin_put(y, Plus()); });
+        else sweep_plain(Cached(), [&](int, float y) { lin_put(nuc_z_shortcut(r, y), Plus()); });
     } else if (r.T == 1.0f && !r.degenerate) {
-        sweep(CachedBack(), [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             float z = y;                                             // a logit of ordinary magnitude is its own canonical form
             if (!nuc_ordinary(y)) {
                 asm volatile("" ::: "memory");                       // (keeps this a branch: as selects it is paid by every logit)
@@ -484,14 +468,14 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
     } else if (r.rcp != 0.0f && !r.degenerate) {
-        sweep(CachedBack(), [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
     } else {
-        sweep(CachedBack(), [&](int, float y) {
+        sweep(Cached(), [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
         }, NucNoPre());
