@@ -513,18 +513,27 @@ __device__ __forceinline__ void row_select_exact(const SampleArgs &a, int row, c
 //   its range (0 otherwise).
 template <int WCAP>
 __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey, u32 &gkey, int want, u32 smax, u32 *H, u32 *Hclear,
-                                            u32 *Mnext, int *s_over, int tid, u32 *span_out = nullptr) {
+                                            u32 *Mnext, u32 *TW, u32 &twlow, int round, int *s_over, int tid, u32 *span_out = nullptr) {
     const int l = lane_id();
     if (count > (u32)WCAP && l == 0) *s_over = 1;
     const int cw = (int)min(count, (u32)WCAP);
-    const u32 range = smax > gkey ? smax - gkey : 0u;
+    // The bins start at the common threshold, or above it at the smallest threshold any wave held when it entered the
+    // last round (published before that round's barrier, so every wave reads the same value now; thresholds only rise):
+    // where every wave has raised a threshold of its own, the lists' entries lie far above the common one, and bins
+    // that start there would all but share one bin.  TW: three words in rotation, one collecting for the next round
+    // (read behind this round's barrier into `twlow`, which the wave keeps), one being reset, one idle.
+    u32 base = gkey;
+    if (twlow != 0xFFFFFFFFu && twlow > base && twlow <= smax) base = twlow;
+    if (l == 0) atomicMin(&TW[(round + 1) % 3], twkey);
+    if (tid == 0) TW[(round + 2) % 3] = 0xFFFFFFFFu;
+    const u32 range = smax > base ? smax - base : 0u;
     const int sh = max(0, 24 - (int)__clz(range));                   // (range >> sh) < ROW_TBINS
     u32 mx = 0u;
     if (cw <= 2 * WAVE) {                                            // wave-uniform: the usual, short list
         for (int e = l; e < cw; e += WAVE) {
             const u32 key = ordkey(__uint_as_float(list[e].x));
             mx = max(mx, key);
-            if (key >= gkey) atomicAdd(&H[min((key - gkey) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
+            if (key >= base) atomicAdd(&H[min((key - base) >> sh, (u32)(ROW_TBINS - 1))], 1u);   // (-0 listed under a threshold of +0 has a smaller key)
         }
     } else {
         // A long list is what a wave's own raise leaves behind: its entries lie close together next to the range, and
@@ -532,8 +541,8 @@ __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey,
         for (int e = l; e < cw; e += WAVE) {
             const u32 key = ordkey(__uint_as_float(list[e].x));
             mx = max(mx, key);
-            bool todo = key >= gkey;
-            const u32 bin = todo ? min((key - gkey) >> sh, (u32)(ROW_TBINS - 1)) : 0u;
+            bool todo = key >= base;
+            const u32 bin = todo ? min((key - base) >> sh, (u32)(ROW_TBINS - 1)) : 0u;
 #pragma unroll
             for (int turn = 0; turn < 2; turn++) {
                 const u64 open = __ballot(todo);
@@ -551,14 +560,17 @@ __device__ __forceinline__ void row_tighten(uint2 *list, u32 &count, u32 &twkey,
     if (l == 0 && mx) atomicMax(Mnext, mx);
     if (tid < ROW_TBINS) Hclear[tid] = 0u;
     lds_barrier();
-    const u32 nk = row_bins_crossing(H, want, gkey, sh);             // the same in every wave
-    if (nk <= gkey) return;
-    // (the top bin also holds every key beyond the range: a crossing there says nothing about how far above it lies)
-    if (span_out) *span_out = ((nk - gkey) >> sh) < (u32)(ROW_TBINS - 1) ? 1u << sh : 0u;
-    gkey = nk;
-    if (nk <= twkey) return;                                         // (this wave's own threshold is higher already)
-    row_list_compact<WCAP>(list, count, nk);
-    twkey = nk;
+    twlow = TW[(round + 1) % 3];
+    const u32 nk = row_bins_crossing(H, want, base, sh);             // the same in every wave
+    if (nk > gkey) {
+        // (the top bin also holds every key beyond the range: a crossing there says nothing about how far above it lies)
+        if (span_out) *span_out = ((nk - base) >> sh) < (u32)(ROW_TBINS - 1) ? 1u << sh : 0u;
+        gkey = nk;
+        if (nk > twkey) {                                            // (else this wave's own threshold is higher already)
+            row_list_compact<WCAP>(list, count, nk);
+            twkey = nk;
+        }
+    }
 }
 
 // Candidates with equal z (first wave only, after the rank sort by z).  They counted the same rank r0: one of them sits
@@ -621,7 +633,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     __shared__ u32 s_wthr[ROW_WAVES], s_wmax[ROW_WAVES];
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
     __shared__ __align__(16) u32 s_wbins[ROW_WAVES][ROW_TBINS];      // a wave's own bins, for a raise of its own threshold
-    __shared__ u32 s_max[2];
+    __shared__ u32 s_max[2], s_tw[3];                                // the largest key met, by round parity; the waves' lowest threshold, by round modulo 3
     __shared__ u32 s_kmax, s_kmin, s_zb;
     __shared__ int s_n, s_valid, s_over, s_next;
     __shared__ int s_x[1 + ROW_WAVES];
@@ -677,6 +689,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
         s_next = 0;
         s_max[0] = 0u;
         s_max[1] = 0u;
+        s_tw[0] = s_tw[1] = s_tw[2] = 0xFFFFFFFFu;
         s_kmax = 0u;
         s_kmin = 0xFFFFFFFFu;
         s_zb = 0u;
@@ -757,12 +770,12 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     uint2 *list = L + wave_id() * G::WCAP;
     u32 *const W = s_wbins[wave_id()];
     u32 count = 0;
-    u32 gkey = twkey;
+    u32 gkey = twkey, twlow = 0xFFFFFFFFu;
     int round = 0;
     auto tighten = [&]() {
         if (have_tw) {                                               // workgroup-uniform
             const u32 smax = max(max0, s_max[round & 1]);
-            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], s_tw, twlow, round, &s_over, tid);
             tw = ordkey_inv(twkey);
             round++;
         }
@@ -872,7 +885,7 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
             for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) tab[i] = 0u;
         {                                                            // (the round's barrier orders the clears before the joins)
             const u32 smax = span ? (u32)min((u64)gkey + (u64)(span - 1u), (u64)0xFFFFFFFFull) : max(max0, s_max[round & 1]);
-            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over,
+            row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], s_tw, twlow, round, &s_over,
                                  tid, &span);
             tw = ordkey_inv(twkey);
             round++;
@@ -1062,7 +1075,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
     u32 *const htab = reinterpret_cast<u32 *>(pool + G::OFF_HTAB);
     __shared__ u32 s_wmax[ROW_WAVES];
     __shared__ __align__(16) u32 s_bins[3][ROW_TBINS];
-    __shared__ u32 s_max[2];
+    __shared__ u32 s_max[2], s_tw[3];                                // the largest key met, by round parity; the waves' lowest threshold, by round modulo 3
     __shared__ int s_n, s_valid, s_over, s_next;
 
     const int tid = threadIdx.x, row = blockIdx.x;
@@ -1081,6 +1094,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         s_next = 0;
         s_max[0] = 0u;
         s_max[1] = 0u;
+        s_tw[0] = s_tw[1] = s_tw[2] = 0xFFFFFFFFu;
     }
     for (int i = tid; i < G::SLOTS; i += ROW_BLOCK) Khi[i] = 0u;
     for (int i = tid; i < ROW_HSLOTS; i += ROW_BLOCK) htab[i] = 0u;
@@ -1124,6 +1138,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
     uint2 *list = L + wave_id() * G::WCAP;
     u32 count = 0;
     int round = 0;
+    u32 twlow = 0xFFFFFFFFu;
     for (unsigned base = 0; base < cnt; base += ROW_BLOCK) {         // workgroup-uniform
         const unsigned e = base + tid;
         uint2 c = make_uint2(0u, 0u);
@@ -1139,7 +1154,7 @@ __global__ __launch_bounds__(ROW_BLOCK) void cand_row_kernel(SampleArgs a, const
         }
         count += (u32)__popcll(m);
         const u32 smax = max(max0, s_max[round & 1]);
-        row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], &s_over, tid);
+        row_tighten<G::WCAP>(list, count, twkey, gkey, want, smax, s_bins[round % 3], s_bins[(round + 1) % 3], &s_max[(round + 1) & 1], s_tw, twlow, round, &s_over, tid);
         round++;
     }
     if (count > (u32)G::WCAP && lane_id() == 0) s_over = 1;
