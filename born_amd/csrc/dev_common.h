@@ -330,26 +330,32 @@ struct BlockScratch {
     u64 bcast[4];
 };
 
-template <int BLOCK>
+// (LDSONLY: the barriers order LDS traffic only, so that global loads requested earlier stay in flight across them)
+template <bool LDSONLY>
+__device__ __forceinline__ void block_barrier() {
+    if (LDSONLY) lds_barrier();
+    else __syncthreads();
+}
+template <int BLOCK, bool LDSONLY = false>
 __device__ __forceinline__ float block_max_f32(float v, BlockScratch *s) {
     constexpr int NW = BLOCK / WAVE;
     v = wave_max_f32(v);
-    __syncthreads();
+    block_barrier<LDSONLY>();
     if (lane_id() == 0) ((float *)s->w)[wave_id()] = v;
-    __syncthreads();
+    block_barrier<LDSONLY>();
     float r = ((float *)s->w)[0];
 #pragma unroll
     for (int i = 1; i < NW; i++) r = fmaxf(r, ((float *)s->w)[i]);
     return r;
 }
 
-template <int BLOCK>
+template <int BLOCK, bool LDSONLY = false>
 __device__ __forceinline__ u32 block_sum_u32(u32 v, BlockScratch *s) {
     constexpr int NW = BLOCK / WAVE;
     v = wave_sum_u32(v);
-    __syncthreads();
+    block_barrier<LDSONLY>();
     if (lane_id() == 0) ((u32 *)s->w)[wave_id()] = v;
-    __syncthreads();
+    block_barrier<LDSONLY>();
     u32 r = 0;
 #pragma unroll
     for (int i = 0; i < NW; i++) r += ((u32 *)s->w)[i];
@@ -357,13 +363,13 @@ __device__ __forceinline__ u32 block_sum_u32(u32 v, BlockScratch *s) {
 }
 
 // Inclusive scan of one u64 per thread across the block; *total receives the block sum.
-template <int BLOCK>
+template <int BLOCK, bool LDSONLY = false>
 __device__ __forceinline__ u64 block_inclusive_scan_u64(u64 v, BlockScratch *s, u64 *total) {
     constexpr int NW = BLOCK / WAVE;
     u64 inc = wave_inclusive_scan_u64(v);
-    __syncthreads();
+    block_barrier<LDSONLY>();
     if (lane_id() == WAVE - 1) s->w[wave_id()] = inc;
-    __syncthreads();
+    block_barrier<LDSONLY>();
     u64 off = 0, tot = 0;
 #pragma unroll
     for (int i = 0; i < NW; i++) {

@@ -102,8 +102,12 @@ __device__ __forceinline__ nuc_f32x4 nuc_load4(const nuc_f32x4 *p) {
 }
 // PLAIN: the caller knows that the row has no penalties (a loop of its own without the penalty code: the visitor's
 // test of r.penal at every visit cost the single-sweep kernel 5 %).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F4, class F1, class PRE = NucNoPre>
-__device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE()) {
+// FIRST (AHEAD instances only): `first` holds the row's first stage, requested earlier with nuc_request_first.
+struct NucNoFirst {};
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F4, class F1, class PRE = NucNoPre,
+          class FIRST = NucNoFirst>
+__device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 f4, F1 f1, PRE pre = PRE(),
+                                             const FIRST &first = FIRST()) {
     const int tid = threadIdx.x;
     auto visit4 = [&](const nuc_f32x4 &q, int j) {
         float y[4] = {q[0], q[1], q[2], q[3]};
@@ -186,8 +190,13 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
                 // the compiler wait for every load in flight); only the visits of the last stage ask whether the block exists.
                 nuc_f32x4 va[NUC_U], vb[NUC_U];
                 const int lastb = n4 - 1;
+                if constexpr (!std::is_same<FIRST, NucNoFirst>::value) {
 #pragma unroll
-                for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + tid, lastb));
+                    for (int u = 0; u < NUC_U; u++) va[u] = first[u];
+                } else {
+#pragma unroll
+                    for (int u = 0; u < NUC_U; u++) va[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + tid, lastb));
+                }
                 pre();
                 for (int s = 0; s + 1 < nst; s++) {
 #pragma unroll
@@ -212,13 +221,25 @@ __device__ __forceinline__ void nuc_foreach4(const NucRow &r, const u32 *bm, F4 
         for (int j = tid; j < r.V; j += NUC_BLOCK) visit1(j);
     }
 }
+// Requests the first stage of an aligned row's next sweep (the same loads the AHEAD visitor starts with): issued at the
+// end of one sweep, they are in flight through the reductions and scans between the sweeps, which on a batch that leaves
+// CUs idle are otherwise a memory latency each.
+template <int NUC_BLOCK, bool NT>
+__device__ __forceinline__ void nuc_request_first(const NucRow &r, nuc_f32x4 (&first)[NucGeom<NUC_BLOCK>::U]) {
+    const int n4 = r.V >> 2;
+    if (r.vec && n4 > 0) {
+        const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(r.x);
+#pragma unroll
+        for (int u = 0; u < NucGeom<NUC_BLOCK>::U; u++) first[u] = nuc_load4<NT>(x4 + min(u * NUC_BLOCK + (int)threadIdx.x, n4 - 1));
+    }
+}
 // Visits every element of the row as f(id, penalised logit).
-template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F, class PRE = NucNoPre>
-__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f, PRE pre = PRE()) {
+template <int NUC_BLOCK, bool NT = false, bool AHEAD = false, bool PLAIN = false, class F, class PRE = NucNoPre, class FIRST = NucNoFirst>
+__device__ __forceinline__ void nuc_foreach(const NucRow &r, const u32 *bm, F f, PRE pre = PRE(), const FIRST &first = FIRST()) {
     nuc_foreach4<NUC_BLOCK, NT, AHEAD, PLAIN>(r, bm, [&](int j, const float (&y)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; t++) f(j + t, y[t]);
-    }, f, pre);
+    }, f, pre, first);
 }
 
 // smallest bin whose inclusive cumulative mass reaches target (the last bin if none does); called by whole waves.
@@ -371,8 +392,12 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         }
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
-    auto sweep = [&](auto nt, auto f, auto pre) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f, pre);
+    // (1024 threads: the first stage of sweeps 2 and 3 is requested ahead, into `ahead`)
+    constexpr bool REQ = NUC_BLOCK == 1024;
+    typename std::conditional<REQ, nuc_f32x4[NucGeom<NUC_BLOCK>::U], NucNoFirst>::type ahead;
+    auto &first = ahead;
+    auto sweep = [&](auto nt, auto f, auto pre, const auto &first) {
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024>(r, bm, f, pre, first);
         if (r.masked) {
 #pragma unroll
             for (int k = 0; k < NUC_SEEN; k++)
@@ -380,8 +405,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         }
     };
     // every element of the row as f(id, logit as stored): no penalty, no look at the history bitmap
-    auto sweep_plain = [&](auto nt, auto f) {
-        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, true>(r, bm, f, NucNoPre());
+    auto sweep_plain = [&](auto nt, auto f, const auto &first) {
+        nuc_foreach<NUC_BLOCK, decltype(nt)::value, NUC_BLOCK == 1024, true>(r, bm, f, NucNoPre(), first);
     };
     typedef std::integral_constant<bool, false> Cached;             // the row is read again: ordinary loads
     typedef std::integral_constant<bool, true> Streamed;             // the row's last sweep: non-temporal loads
@@ -394,9 +419,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
         sweep(Cached(), [&](int j, float y) {
             mx = fmaxf(mx, y);
             if ((j & 3) == 0) mn = fminf(mn, y > -3.402823466e+38f ? y : INFINITY);
-        }, prologue);
-        mx = block_max_f32<NUC_BLOCK>(mx, &scr);
-        mn = -block_max_f32<NUC_BLOCK>(-mn, &scr);
+        }, prologue, NucNoFirst());
+        // (sweep 2's first stage travels while the row's maximum is found; the barriers until then order LDS traffic only)
+        if constexpr (REQ) nuc_request_first<NUC_BLOCK, false>(r, ahead);
+        mx = block_max_f32<NUC_BLOCK, true>(mx, &scr);
+        mn = -block_max_f32<NUC_BLOCK, true>(-mn, &scr);
         r.m = uniform_f32(nuc_z(r, mx));
         r.degenerate = r.m == -INFINITY;                             // nothing finite: every d is 0 by definition
         const float zmin = mn < INFINITY ? nuc_z(r, mn) : r.m;
@@ -455,8 +482,8 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 #endif
     // ---- sweep 2: integer masses by bin
     if (lin) {
-        if (r.T == 1.0f) sweep_plain(Cached(), [&](int, float y) { lin_put(y, Plus()); });
-        else sweep_plain(Cached(), [&](int, float y) { lin_put(nuc_z_shortcut(r, y), Plus()); });
+        if (r.T == 1.0f) sweep_plain(Cached(), [&](int, float y) { lin_put(y, Plus()); }, first);
+        else sweep_plain(Cached(), [&](int, float y) { lin_put(nuc_z_shortcut(r, y), Plus()); }, first);
     } else if (r.T == 1.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
             float z = y;                                             // a logit of ordinary magnitude is its own canonical form
@@ -466,21 +493,23 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             }
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        }, NucNoPre());
+        }, NucNoPre(), first);
     } else if (r.rcp != 0.0f && !r.degenerate) {
         sweep(Cached(), [&](int, float y) {
             float z = nuc_z_shortcut(r, y);
             if (!nuc_ordinary(y)) z = nuc_z(r, y);                   // zeros, masked (-inf) and other unusual logits: the division
             const float d = r.m - z;
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        }, NucNoPre());
+        }, NucNoPre(), first);
     } else {
         sweep(Cached(), [&](int, float y) {
             const float d = nuc_d(r, nuc_z(r, y));
             atomicAdd(&mass[nuc_bin(r, d)], qfix(expneg(d, r.dcut), r.scale));
-        }, NucNoPre());
+        }, NucNoPre(), first);
     }
-    __syncthreads();
+    // (sweep 3's first stage travels while the bins are summed and the wanted ones found)
+    if constexpr (REQ) nuc_request_first<NUC_BLOCK, true>(r, ahead);
+    lds_barrier();
     BORN_STAMP(a, row, 3);
 #if defined(BORN_NUC_STOP_AFTER) && BORN_NUC_STOP_AFTER == 2
     if (tid == 0) a.tokens[row] = (int)(mass[0] & 1ull);
@@ -494,11 +523,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             local += mass[tid * NUC_PER + t];
             v[t] = local;
         }
-        const u64 excl = block_inclusive_scan_u64<NUC_BLOCK>(local, &scr, &Zk) - local;
+        const u64 excl = block_inclusive_scan_u64<NUC_BLOCK, true>(local, &scr, &Zk) - local;
 #pragma unroll
         for (int t = 0; t < NUC_PER; t++) mass[tid * NUC_PER + t] = v[t] + excl;
     }
-    __syncthreads();
+    lds_barrier();
     const u64 *cum = mass;
 
     // ---- the bins to gather: the top-p cut's, and the draw's predicted from the interval [tp, cum[bp]]
@@ -535,7 +564,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                 }
             }
             // (summed in sixteenths, each thread's share rounded up)
-            const u32 total = block_sum_u32<NUC_BLOCK>((u32)fminf(ceilf(bound * 16.0f), 1048576.0f), &scr);
+            const u32 total = block_sum_u32<NUC_BLOCK, true>((u32)fminf(ceilf(bound * 16.0f), 1048576.0f), &scr);
             whole = total <= (u32)(16 * NUC_CAP / 2);                 // (half the capacity: the lists are per wave, the logits fall as they may)
         }
     }
@@ -589,11 +618,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
             // (the stored logits; a seen id's stored logit that passes is dropped below, its penalised logit is offered
             // here under the id with the top bit set)
             if (nint == 1) {
-                sweep_plain(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); });
+                sweep_plain(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); }, first);
             } else {
                 sweep_plain(Streamed(), [&](int j, float y) {
                     append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
-                });
+                }, first);
             }
             if (r.penal) {
 #pragma unroll
@@ -605,11 +634,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
                     }
             }
         } else if (nint == 1) {
-            sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); }, NucNoPre());
+            sweep(Streamed(), [&](int j, float y) { append(!(y < lo0) & !(y > hi0), y, j); }, NucNoPre(), first);
         } else {
             sweep(Streamed(), [&](int j, float y) {
                 append((!(y < lo0) & !(y > hi0)) | (!(y < lo1) & !(y > hi1)) | (!(y < lo2) & !(y > hi2)), y, j);
-            }, NucNoPre());
+            }, NucNoPre(), first);
         }
         const u32 count = __hip_atomic_load(wcount, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
         if (count > (u32)NUC_WCAP && lane_id() == 0) s_over = 1;
