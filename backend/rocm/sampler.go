@@ -294,7 +294,7 @@ type RowConfigs struct {
 }
 
 const (
-	RowsSmallTopK uint32 = 1 // 1 <= top_k <= 512, no penalty that raises a logit
+	RowsSmallTopK uint32 = 1 // 1 <= top_k <= 512; a penalty that raises a logit only with a history stride <= 1024
 	RowsNoTopK    uint32 = 2 // top_k disabled
 	RowsOther     uint32 = 4 // everything else
 )

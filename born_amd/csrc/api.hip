@@ -382,9 +382,11 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
                                      per_row->min_p || per_row->frequency_penalty || per_row->presence_penalty);
     const bool counted = (counts_history(s->cfg) || (per_row && (per_row->frequency_penalty || per_row->presence_penalty))) &&
                          history && hist_stride > 0;
-    // The single-pass kernel relies on the penalties never raising a logit (per-row values are judged on the device).
+    // Penalties that raise a logit (a negative frequency / presence penalty; a repetition penalty below 1 raises the
+    // positive logits): the single-pass kernel takes them with a history short enough for its hash, which then names
+    // every id whose logit may have been raised (per-row values are judged on the device, by the same rule).
     const bool raises = counted && (a.freq < 0.0f || a.pres < 0.0f);
-    const bool boosts = (history && a.rep < 1.0f) || raises;       // (repetition_penalty < 1 raises the positive logits)
+    const bool boosts = ((history && a.rep < 1.0f) || raises) && hist_stride > TOPK_BOOST_HISTORY;   // ... beyond that hash
     // which kernels run.  One configuration: the one it selects.  Per-row arrays: all that the shape and the handle's
     // kernel selection allow, or those the caller's promise about the kinds of row leaves (mapped through the same
     // rules: under path 1 every row is the general kernel's); each workgroup takes its row only if the row's

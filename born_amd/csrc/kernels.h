@@ -7,6 +7,7 @@ namespace born {
 
 // The single-pass top-k kernel (one workgroup per row).
 constexpr int TOPK_LOCAL_COUNT_HISTORY = 4096;   // longest history whose occurrences it counts in LDS
+constexpr int TOPK_BOOST_HISTORY = 1024;   // longest history with which it takes penalties that raise logits (its hash names every seen id)
 constexpr int TOPK_MAX_K = 512;            // largest top_k it serves (its last wave holds up to eight survivors per lane)
 constexpr int LM_MAX_K = 128;              // largest top_k of the sampling step fused into the LM head
 constexpr int ROW_MAX_VOCAB = 393216;      // largest vocabulary it takes (its history bitmap is 48 KiB of LDS)

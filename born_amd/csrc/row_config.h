@@ -1,8 +1,8 @@
 // Per-row sampling configurations: when the caller passes arrays of temperature / top_k / top_p /
 // repetition_penalty / min_p / frequency_penalty / presence_penalty (one value per row, any of them optional), the three sampling kernels are all launched
 // over the whole batch and every workgroup first decides whether its row is its own: the single-pass kernel
-// takes 1 <= top_k <= 128 with a penalty that never raises a logit, the three-sweep kernel the rows without a
-// top-k cut, the general kernel everything else — the same rule the host applies to a uniform configuration.
+// takes 1 <= top_k <= 512 (penalties that raise a logit only over a history of at most 1024 tokens), the three-sweep
+// kernel the rows without a top-k cut, the general kernel everything else — the same rule the host applies to a uniform configuration.
 #pragma once
 #include "dev_common.h"
 #include "kernels.h"
@@ -58,8 +58,9 @@ __device__ __forceinline__ bool row_config_values(const SampleArgs &a, const Row
     if (!row_config_valid(v, min_p)) {
         invalid = true;
         route = ROUTE_GENERAL;
-    } else if (rc.path != 1 && v.top_k >= 1 && v.top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB && !(a.history && v.rep < 1.0f) &&
-               !((a.hist_counts || a.local_counts) && (v.freq < 0.0f || v.pres < 0.0f))) {
+    } else if (rc.path != 1 && v.top_k >= 1 && v.top_k <= TOPK_MAX_K && a.V <= ROW_MAX_VOCAB &&
+               (a.hist_stride <= TOPK_BOOST_HISTORY ||                // (penalties that raise a logit: only with a history that its hash holds)
+                (!(a.history && v.rep < 1.0f) && !((a.hist_counts || a.local_counts) && (v.freq < 0.0f || v.pres < 0.0f))))) {
         route = ROUTE_TOPK;
     } else if (rc.path != 1 && v.top_k == 0) {
         route = ROUTE_NUCLEUS;

@@ -21,8 +21,10 @@
 //       so the bound of the proof is the largest threshold any wave ended with.
 //   After the last load the lists hold a few times top_k entries; final rounds of T' (each refining inside the bin
 //   the boundary fell into) bring them down to what the rank sort takes.
-//   Any logit outside the lists is below T, and so is its z after a penalty (repetition_penalty >= 1
-//   only lowers a logit) and the monotone division by the temperature.  Every wave turns its own entries into rank
+//   Any logit outside the lists is below T, and so is its z after a penalty that only lowers logits (a
+//   repetition_penalty >= 1, frequency / presence penalties >= 0) and the monotone division by the temperature.
+//   Penalties that raise logits: the ids of the history, each once from its hash, join the candidates where their
+//   penalised z lies above the bound (histories of at most 1024 tokens).  Every wave turns its own entries into rank
 //   keys (probing its hash of the history) and appends them to one array; the row is proven if top_k candidates
 //   end up with z strictly above that bound.  A rank sort orders them (by counting for top_k <= 128, by buckets of
 //   the key above that; candidates of equal z are ranked among themselves from a short list) and one wave computes
@@ -62,6 +64,7 @@ static_assert(FB_HSLOTS == (1 << 13), "fb_hhash produces 13 bits");
 // The id + 1 of a slot; slots hold nothing else unless the kernel counts (LOCAL).
 template <bool LOCAL>
 __device__ __forceinline__ u32 hslot_id(u32 e) { return LOCAL ? (e & HSLOT_ID_MASK) : e; }
+static_assert(TOPK_BOOST_HISTORY == ROW_BLOCK, "a history of that length is hashed by the workgroup");
 static_assert(ROW_HSLOTS == (1 << 11) && ROW_HSLOTS >= 2 * ROW_BLOCK, "row_hhash produces 11 bits; load factor <= 0.5");
 
 constexpr int FB_BITMAP = 6144;               // words of history bitmap: 48 KiB, one bit per id
@@ -898,6 +901,50 @@ __device__ __forceinline__ void topk_row_body(SampleArgs &a) {
     }
     const u32 zb = s_zb;                                             // the largest of the waves' bounds
     bool ok = have_tw && !s_over && n >= k && n <= G::CAP;
+    // Penalties that raise a logit (a repetition penalty below 1, a negative frequency or presence penalty): an id of the
+    // history may have its z above the bound although its stored logit is below every threshold.  The hashed history
+    // names those ids, each once: the candidates flag their own slots, and every other slot's id joins the candidates
+    // (with its stored logit, like a list entry) if its penalised z lies above the bound.  After that a logit outside
+    // the candidates is either unseen and below its wave's threshold or seen with a z at or below the bound, as the
+    // proof needs.  A history too long for the hash leaves the row to the exact selection.
+    const bool boosts = penal && (a.rep < 1.0f || (counted && (a.freq < 0.0f || a.pres < 0.0f)));
+    if (boosts) {                                                    // workgroup-uniform
+        if (!hfast) ok = false;
+        if (ok) {
+            if (tid < n) {
+                const u32 id = C[tid].y;
+                u32 slot = row_hhash(id);
+                for (;;) {
+                    const u32 en = htab[slot];
+                    if (en == 0u) break;
+                    if (hslot_id<LOCAL>(en & 0x7FFFFFFFu) == id + 1u) {
+                        atomicOr(&htab[slot], 0x80000000u);          // (free: a count in a slot is at most ROW_BLOCK)
+                        break;
+                    }
+                    slot = (slot + 1) & (ROW_HSLOTS - 1);
+                }
+            }
+            __syncthreads();
+            for (int slot = tid; slot < ROW_HSLOTS; slot += ROW_BLOCK) {
+                const u32 en = htab[slot];
+                if (en & 0x80000000u) {
+                    htab[slot] = en & 0x7FFFFFFFu;
+                } else if (en != 0u) {
+                    const u32 id = hslot_id<LOCAL>(en) - 1u;
+                    const float y = x[id];
+                    const u32 occ = local ? en >> HSLOT_ID_BITS : counts ? counts[id] : 0u;
+                    const float z = z_of(penalise_counted(y, a.rep, counted, occ, a.freq, a.pres), a.T);
+                    if (z == z && ordkey(z) > zb) {                  // (a NaN has no place in any top_k)
+                        const int pos = atomicAdd(&s_n, 1);
+                        if (pos < G::CAP) C[pos] = make_uint2(__float_as_uint(y), id);
+                    }
+                }
+            }
+            __syncthreads();
+            n = s_n;
+            ok = n <= G::CAP;
+        }
+    }
     // top_k beyond TOPK_SMALL_K: the candidates are ranked through buckets of z (below), whose counters take the
     // threshold rounds' first set of bins (no round runs any more)
     const bool bucketed = KC == 1 && k > TOPK_SMALL_K;
@@ -1250,9 +1297,11 @@ constexpr size_t row_pool_bytes() { return (size_t)RowGeom<KC>::POOL * sizeof(u6
 template <bool VEC, bool LOCAL>
 static void launch_topk_row_as(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
     const dim3 gr((unsigned)a.B), bl(ROW_BLOCK);
+    // (penalties that raise logits add seen ids to the candidates: the instance with room for 1024 of them)
+    const bool boosts = a.history && (a.rep < 1.0f || ((a.hist_counts || a.local_counts) && (a.freq < 0.0f || a.pres < 0.0f)));
     if (rows)
         hipLaunchKernelGGL((topk_row_rows_kernel<VEC, LOCAL>), gr, bl, row_pool_bytes<1>(), st, a, *rows);
-    else if (a.top_k > TOPK_SMALL_K)
+    else if (a.top_k > TOPK_SMALL_K || boosts)
         hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL, 1>), gr, bl, row_pool_bytes<1>(), st, a);
     else
         hipLaunchKernelGGL((topk_row_kernel<VEC, LOCAL, 0>), gr, bl, row_pool_bytes<0>(), st, a);

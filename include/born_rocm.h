@@ -90,7 +90,8 @@ int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows
                                int64_t *general_rows);
 
 /* Diagnostics.  0 = choose the kernel from the configuration (default: the single-pass kernel for
- * 1 <= top_k <= 512 with a penalty >= 1 and a vocabulary of at most 393216, the general kernel otherwise).
+ * 1 <= top_k <= 512 and a vocabulary of at most 393216, with penalties that raise a logit (a repetition penalty below
+ * 1, a negative frequency or presence penalty) only over a history of at most 1024 tokens; the general kernel otherwise).
  * 1 = always the general kernel.  2 = as 0, but the kernel for top_k 0 runs 512 threads per row (two rows to a CU
  * at a time) whatever the batch; by default it does so only for batches of more rows than the device has CUs.
  * All implement the same fixed-point pipeline and must return identical results; tests compare them. */
@@ -164,9 +165,9 @@ typedef struct born_sampler_row_configs {
      * may occur.  A row of a kind that was not promised gets token 0 and BORN_ROCM_ERR_DATA, like an invalid one. */
     uint32_t       row_kinds;
 } born_sampler_row_configs;
-#define BORN_ROCM_ROWS_SMALL_TOP_K  1u   /* 1 <= top_k <= 512, no penalty that raises a logit, vocab <= 393216 */
+#define BORN_ROCM_ROWS_SMALL_TOP_K  1u   /* 1 <= top_k <= 512, vocab <= 393216; a penalty that raises a logit only with hist_stride <= 1024 */
 #define BORN_ROCM_ROWS_NO_TOP_K     2u   /* top_k disabled (<= 0 or >= vocab) */
-#define BORN_ROCM_ROWS_OTHER        4u   /* everything else (top_k > 512, a penalty that raises logits with a top-k cut, ...) */
+#define BORN_ROCM_ROWS_OTHER        4u   /* everything else (top_k > 512, a penalty that raises logits with a top-k cut and a longer history, ...) */
 
 int born_rocm_sample_rows(born_sampler *s, const float *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                           const int32_t *history, const int32_t *hist_len, int64_t hist_stride, const float *uniforms,

@@ -189,6 +189,10 @@ TOPK_PATHS = [0]
     (9, 777, 0.9, 300, 0.99, 1.5, 2000),
     (4, 600, 0.8, 512, 0.7, 1.0, 0),             # a row of three waves: no first-stage threshold
     (6, 16385, 0.7, 333, 0.9, 1.3, 64),          # one element in the second stage
+    (32, 128256, 0.7, 50, 0.9, 0.8, 512),        # a penalty < 1 raises logits: seen ids join the candidates from the history's hash
+    (16, 32000, 1.0, 100, 0.95, 0.5, 1000),
+    (16, 32000, 1.3, 300, 0.9, 0.25, 1024),      # the longest history the hash takes
+    (16, 50257, 1.1, 256, 0.95, 0.7, 1500),      # beyond it: the general kernel
 ])
 def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
     rng = np.random.default_rng(B * 1000003 + V)
@@ -197,10 +201,39 @@ def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
     hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
     got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, nuc=min(512, max(k, 1)), path=path)
     c = got["counters"]
-    if rep < 1.0 and H:          # a boosting penalty is served by the general kernel
+    if rep < 1.0 and H > 1024:   # a boosting penalty over a history longer than the workgroup's hash is served by the general kernel
         assert c["general_rows"] == B
     else:
         assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
+
+
+@pytest.mark.parametrize("V,H", [(128256, 512), (32000, 1000), (5003, 64), (777, 1024)])
+def test_topk_kernel_penalties_that_raise_logits(oracle, rocm, V, H):
+    # A repetition penalty below 1 and negative frequency / presence penalties lift seen ids from far below the
+    # streamed threshold into the top_k (and past the maximum); each seen id must be ranked by its penalised logit
+    # exactly once, whether its stored logit was listed or not.
+    rng = np.random.default_rng(V + H)
+    B = 24
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.0)).astype(np.float32)
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.2, size=(B, H)) - 1) % V).astype(np.int32)
+    hist[:, : H // 4] = rng.integers(0, V, size=(B, H // 4))            # a quarter spread over the vocabulary
+    for r in range(B):                                                   # some rows: the history holds the row's largest logits too
+        if r % 3 == 0:
+            hist[r, :8] = np.argsort(-x[r])[:8]
+    x[1, hist[1, :50]] = -np.inf                                         # seen ids that stay impossible
+    x[2, hist[2, :50]] = np.nan
+    hl = rng.integers(0, H + 1, size=B).astype(np.int32)
+    hl[:4] = H
+    for (T, k, p, rep, freq, pres) in [(0.8, 50, 0.9, 0.5, 0.0, 0.0), (1.0, 128, 1.0, 0.1, 0.0, 0.0), (1.2, 300, 0.95, 1.0, -0.5, -1.0),
+                                       (0.7, 40, 0.9, 1.3, -3.0, 0.0), (1.0, 1, 1.0, 0.7, 0.0, -2.0), (1.0, 64, 0.99, 0.9, -0.1, 0.3)]:
+        if k >= V:
+            continue
+        got, _, _ = _check_against_oracle(oracle, rocm, x, u, T, k, p, rep, hist, hl, nuc=min(512, k), freq=freq, pres=pres)
+        c = got["counters"]
+        assert c["general_rows"] == 0 and c["topk_rows"] + c["fallback_rows"] == B
+        if V > 20000:
+            assert c["fallback_rows"] <= 2, (T, k, p, rep, freq, pres, c)   # (the NaN / -inf rows may need the exact selection)
 
 
 @pytest.mark.parametrize("path", TOPK_PATHS)
@@ -456,7 +489,9 @@ def test_min_p_is_validated(rocm):
     (16, 32000, 1.0, 40, 0.95, 1.0, 64, 0.5, 0.0, "topk"),       # frequency alone, no repetition penalty
     (16, 32000, 1.0, 40, 0.95, 1.0, 64, 0.0, 1.5, "topk"),       # presence alone
     (9, 8000, 0.9, 64, 0.99, 1.2, 3000, 0.2, 0.3, "topk"),       # history longer than 1024: candidates are hashed instead
-    (16, 32000, 1.0, 20, 0.9, 1.1, 128, -0.4, 0.2, "general"),   # a negative penalty raises logits: general kernel
+    (16, 32000, 1.0, 20, 0.9, 1.1, 128, -0.4, 0.2, "topk"),      # a negative penalty raises logits: seen ids join the candidates
+    (16, 32000, 1.0, 20, 0.9, 1.1, 1024, -0.4, -0.2, "topk"),
+    (16, 32000, 1.0, 20, 0.9, 1.1, 1025, -0.4, 0.2, "general"),  # ... a history beyond the hash: the general kernel
     (16, 32000, 1.0, 0, 1.0, 1.0, 256, 0.4, 0.4, "nucleus"),     # no top-k: three-sweep kernel
     (16, 152064, 1.2, 0, 0.99, 1.05, 2048, 0.1, 0.6, "nucleus"), # C5 shape
     (16, 32000, 0.9, 500, 0.9, 1.1, 64, 0.25, 0.25, "topk"),       # beyond 128: the single-pass kernel's larger sizes
@@ -1055,7 +1090,8 @@ def test_per_row_configurations_with_handle_wide_extras(oracle, rocm, path, freq
         assert tok[b] == want["tokens"][0], (b, Ts[b], ks[b], ps[b], reps[b])
         assert pr[b:b + 1].view(np.uint32)[0] == want["probs"].view(np.uint32)[0], b
     if path != 1 and freq < 0:
-        assert s.Counters()["topk_rows"] == 0                            # a penalty that raises logits: never the single-pass kernel
+        # a penalty that raises logits, a history that the single-pass kernel's hash holds: its rows stay its own
+        assert s.Counters()["topk_rows"] == int(((ks >= 1) & (ks <= 512)).sum())
     s.Close()
 
 
