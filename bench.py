@@ -484,6 +484,9 @@ def main_extras(args, torch, S, synth, dev):
 
     if args.config == "C3x":
         base, minp, fp = mk(), mk(MinP=0.05), mk(FrequencyPenalty=0.3, PresencePenalty=0.5)
+        # penalties that raise logits (seen ids join the single-pass kernel's candidates from the history's hash)
+        fneg = mk(FrequencyPenalty=-0.2, PresencePenalty=-0.1)
+        rlow = S.NewSampler(S.SamplerConfig(Temperature=w.temperature, TopK=w.top_k, TopP=w.top_p, RepetitionPenalty=0.87), max_batch=B, max_vocab=V)
         k100, k128, k129, k256, k512, k513, k0 = mk(top_k=100), mk(top_k=128), mk(top_k=129), mk(top_k=256), mk(top_k=512), mk(top_k=513), mk(top_k=0)
         # rows whose large logits sit where a threshold drawn from the row's first logits does not look (same shape, same
         # history and uniforms): sorted ascending; a step up in the last tenth; a bump around the middle
@@ -520,6 +523,8 @@ def main_extras(args, torch, S, synth, dev):
             "C3 shape, top_k 0 (top-p alone: the three-sweep kernel)": lambda: k0.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + min_p 0.05": lambda: minp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 + frequency 0.3 + presence 0.5": lambda: fp.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 + frequency -0.2 + presence -0.1": lambda: fneg.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
+            "C3 with repetition penalty 0.87 instead of 1.15": lambda: rlow.Sample(nxt(), B, V, h, None, u, tok, pr, hist_stride=H, stream=stream),
             "C3 with per-row arrays (same values in every row)":
                 lambda: base.SampleRows(nxt(), B, V, h, None, u, Ts, ks, ps, rs, tok, pr, hist_stride=H, stream=stream),
             "C3 with per-row arrays and the promise that every row has a small top-k":
@@ -540,7 +545,8 @@ def main_extras(args, torch, S, synth, dev):
     if args.config == "C3x":
         # rows the single-pass kernel handed to its exact selection, over every step of every case above (0: none did)
         out["exact_selection_rows_total"] = {name: smp.Counters(stream)["fallback_rows"] for name, smp in
-                                             (("handle of the C3 settings (all its cases)", base), ("top_k 256", k256), ("top_k 512", k512))}
+                                             (("handle of the C3 settings (all its cases)", base), ("top_k 256", k256), ("top_k 512", k512),
+                                              ("frequency -0.2 + presence -0.1", fneg), ("repetition penalty 0.87", rlow))}
     out["algorithmic_bytes_per_step"] = w.algorithmic_bytes()
     print(json.dumps(out))
 
