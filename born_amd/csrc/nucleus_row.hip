@@ -274,7 +274,8 @@ __device__ __forceinline__ void nuc_range(const NucRow &r, int w, float &ylo, fl
 // cfg_T, cfg_p, cfg_rep: the row's temperature, top_p and repetition penalty (the handle's, or the row's own).
 // COUNTED: a frequency or presence penalty is on (the table of occurrence counts is read for ids the history holds);
 // its own instance, so that the usual one carries none of it.
-template <int NUC_BLOCK, bool COUNTED>
+// REQUEST (1024 threads only): the first stage of sweeps 2 and 3 is requested before the reductions between the sweeps.
+template <int NUC_BLOCK, bool COUNTED, bool REQUEST = true>
 __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const float cfg_T, const float cfg_p, const float cfg_rep,
                                                  const float cfg_dcut, const float cfg_freq, const float cfg_pres,
                                                  const float cfg_rcp) {
@@ -393,7 +394,7 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
     };
     // every element of the row as f(id, penalised logit): the sweep, then the seen ids when the sweep masked them
     // (1024 threads: the first stage of sweeps 2 and 3 is requested ahead, into `ahead`)
-    constexpr bool REQ = NUC_BLOCK == 1024;
+    constexpr bool REQ = REQUEST && NUC_BLOCK == 1024;
     typename std::conditional<REQ, nuc_f32x4[NucGeom<NUC_BLOCK>::U], NucNoFirst>::type ahead;
     auto &first = ahead;
     auto sweep = [&](auto nt, auto f, auto pre, const auto &first) {
@@ -874,9 +875,11 @@ __device__ __forceinline__ void nucleus_row_body(const SampleArgs &a, const floa
 }
 
 // (at most 128 registers either way: 512 threads are launched two workgroups to a CU)
-template <int BLOCK, bool COUNTED>
+// REQUEST: see the body; off for a batch small enough to be re-read from the L2s, where there is no memory latency to
+// hide and holding the requested stage in registers only costs (64 x 32 000: 21.1 us with it, 20.8 without).
+template <int BLOCK, bool COUNTED, bool REQUEST = true>
 __global__ __launch_bounds__(BLOCK, 4) void nucleus_row_kernel(SampleArgs a) {
-    nucleus_row_body<BLOCK, COUNTED>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres, a.rcp_T);
+    nucleus_row_body<BLOCK, COUNTED, REQUEST>(a, a.T, a.top_p, a.rep, a.dcut, a.freq, a.pres, a.rcp_T);
 }
 // The batch carries a configuration per row (row_config.h): the workgroup takes the row only if it is its own.
 template <int BLOCK, bool COUNTED>
@@ -1073,6 +1076,8 @@ static int cu_count() {
     return known[dev];
 }
 
+// A batch of at most this many bytes of logits is re-read from the L2s by sweeps 2 and 3 (eight L2s of 4 MiB).
+constexpr long long NUC_L2_RESIDENT_BYTES = 16ll << 20;
 template <int BLOCK>
 static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConfigs *rows) {
     const dim3 gr((unsigned)a.B), bl(BLOCK);
@@ -1080,6 +1085,9 @@ static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConf
     if (rows) {
         if (a.hist_counts) hipLaunchKernelGGL((nucleus_row_rows_kernel<BLOCK, true>), gr, bl, lds, st, a, *rows);
         else hipLaunchKernelGGL((nucleus_row_rows_kernel<BLOCK, false>), gr, bl, lds, st, a, *rows);
+    } else if (BLOCK == 1024 && (long long)a.B * a.V * (long long)sizeof(float) <= NUC_L2_RESIDENT_BYTES) {
+        if (a.hist_counts) hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, true, false>), gr, bl, lds, st, a);
+        else hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, false, false>), gr, bl, lds, st, a);
     } else {
         if (a.hist_counts) hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, true>), gr, bl, lds, st, a);
         else hipLaunchKernelGGL((nucleus_row_kernel<BLOCK, false>), gr, bl, lds, st, a);
@@ -1118,6 +1126,8 @@ hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConf
 hipError_t configure_nucleus() {
     const int lds = (int)nucleus_lds_bytes((int)WIDE_MAX_VOCAB);
     const void *kernels[] = {reinterpret_cast<const void *>(nucleus_row_kernel<1024, false>), reinterpret_cast<const void *>(nucleus_row_kernel<1024, true>),
+                             reinterpret_cast<const void *>(nucleus_row_kernel<1024, false, false>),
+                             reinterpret_cast<const void *>(nucleus_row_kernel<1024, true, false>),
                              reinterpret_cast<const void *>(nucleus_row_rows_kernel<1024, false>),
                              reinterpret_cast<const void *>(nucleus_row_rows_kernel<1024, true>)};
     for (const void *k : kernels) {
