@@ -454,7 +454,7 @@ static int sample_impl(born_sampler *s, const float *logits, int64_t batch, int6
             if (launched & 4u) keep_first(launch_sample_wide(a, st, &rows));
         }
     } else if (launched == 1u) {
-        keep_first(launch_topk_row(a, st));
+        keep_first(launch_topk_row(a, st, nullptr, s->path == 2));
     } else {
         // the kernels that divide every logit by the temperature take the shortcut where it is exact for this temperature
         // (host arithmetic only: nothing is launched or waited for; per-row temperatures, above, always divide)

@@ -159,7 +159,9 @@ hipError_t launch_exp(const float *x, float *out, long long n, hipStream_t st);
 hipError_t launch_hist_counts(const int *history, const int *hist_len, long long hist_stride, int B, int V, unsigned *counts,
                               bool clear, hipStream_t st);
 hipError_t launch_uniforms(unsigned long long seed, unsigned long long step, float *u, long long n, hipStream_t st);
-hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr);
+// two_per_cu: the 512-thread instance whatever the batch (by default: batches of more rows than the device has CUs)
+hipError_t launch_topk_row(const SampleArgs &a, hipStream_t st, const RowConfigs *rows = nullptr, bool two_per_cu = false);
+int device_cu_count();                      // compute units of the current device (256 if it cannot be asked)
 hipError_t configure_topk_row();   // one-time function attributes (dynamic LDS above 64 KiB)
 // Sampling fused into the LM head, in three steps around the GEMM that lists the candidates:
 //   thr[row] = the kth largest of samp[row][0..nsamp) + bias[j * sstep] (-inf if there are fewer); cand_cnt[row] = 0

@@ -1064,7 +1064,7 @@ size_t nucleus_lds_bytes(int V) { return nucleus_lds_bytes_of<1024>(V); }
 constexpr size_t LDS_PER_CU = 160 * 1024;
 
 // CUs of the current device (asked once per device)
-static int cu_count() {
+int device_cu_count() {
     static int known[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
@@ -1096,7 +1096,7 @@ static void launch_nucleus_of(const SampleArgs &a, hipStream_t st, const RowConf
 
 // Whether launch_nucleus_row would give this batch 512 threads per row.
 static bool nucleus_two_per_cu(const SampleArgs &a, bool two_per_cu) {
-    return (two_per_cu || a.B > cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU;
+    return (two_per_cu || a.B > device_cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU;
 }
 // The rows without a top-k cut and the general kernel's rows of a batch with per-row configurations: one launch where
 // the former would get a workgroup of 1024 threads anyway, else the two kernels one after the other.
@@ -1117,7 +1117,7 @@ hipError_t launch_nucleus_row(const SampleArgs &a, hipStream_t st, const RowConf
 #ifdef BORN_NUC_FORCE_1024
     if (false) launch_nucleus_of<512>(a, st, rows);                  // (measurement builds only)
 #else
-    if ((two_per_cu || a.B > cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU) launch_nucleus_of<512>(a, st, rows);
+    if ((two_per_cu || a.B > device_cu_count()) && 2 * nucleus_lds_bytes_of<512>(a.V) <= LDS_PER_CU) launch_nucleus_of<512>(a, st, rows);
 #endif
     else launch_nucleus_of<1024>(a, st, rows);
     return hipGetLastError();

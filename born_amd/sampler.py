@@ -160,7 +160,8 @@ class Sampler:
 
     def SetPath(self, path):
         """Diagnostics: 0 = kernel chosen from TopK, 1 = always the general kernel, 2 = as 0 with 512 threads per row in
-        the kernel for TopK 0 whatever the batch (by default: for batches of more rows than the device has CUs)."""
+        the kernel for TopK 0 and in the single-pass kernel for TopK <= 128 whatever the batch (by default: for batches of
+        more rows than the device has CUs)."""
         _check(_capi.lib().born_rocm_sampler_set_path(self._h, int(path)))
 
     def Step(self):

@@ -92,8 +92,9 @@ int born_rocm_sampler_counters(born_sampler *s, void *stream, int64_t *topk_rows
 /* Diagnostics.  0 = choose the kernel from the configuration (default: the single-pass kernel for
  * 1 <= top_k <= 512 and a vocabulary of at most 393216, with penalties that raise a logit (a repetition penalty below
  * 1, a negative frequency or presence penalty) only over a history of at most 1024 tokens; the general kernel otherwise).
- * 1 = always the general kernel.  2 = as 0, but the kernel for top_k 0 runs 512 threads per row (two rows to a CU
- * at a time) whatever the batch; by default it does so only for batches of more rows than the device has CUs.
+ * 1 = always the general kernel.  2 = as 0, but the kernel for top_k 0 and the single-pass kernel for top_k <= 128 run
+ * 512 threads per row (two rows to a CU at a time) whatever the batch; by default they do so only for batches of more
+ * rows than the device has CUs.
  * All implement the same fixed-point pipeline and must return identical results; tests compare them. */
 int born_rocm_sampler_set_path(born_sampler *s, int32_t path);
 

@@ -158,9 +158,10 @@ def test_softmax_operators(oracle, rocm):
 
 
 # ---------------------------------------------------------------- sampling: single-pass top-k kernel
-# path 0 = the default kernel selection (1 <= top_k <= 512: one workgroup per row, one launch)
+# path 0 = the default kernel selection (1 <= top_k <= 512: one workgroup per row, one launch); path 2 = the same with
+# the 512-thread instance (top_k <= 128) whatever the batch, which by default only batches of more rows than CUs get
 
-TOPK_PATHS = [0]
+TOPK_PATHS = [0, 2]
 
 
 @pytest.mark.parametrize("path", TOPK_PATHS)
@@ -205,6 +206,20 @@ def test_topk_kernel_against_oracle(oracle, rocm, B, V, T, k, p, rep, H, path):
         assert c["general_rows"] == B
     else:
         assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
+
+
+@pytest.mark.parametrize("B,V,k,H", [(300, 20000, 50, 64), (257, 8193, 128, 700), (600, 3001, 7, 0), (520, 16384, 100, 512)])
+def test_topk_kernel_more_rows_than_compute_units(oracle, rocm, B, V, k, H):
+    # Batches of more rows than the device has CUs run the 512-thread instance of the kernel (two rows to a CU at a
+    # time) by the default selection; same tokens, same probabilities, every row settled by the single-pass kernel.
+    rng = np.random.default_rng(B + V)
+    x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(1.5)).astype(np.float32)
+    x[::7] = np.sort(x[::7], axis=1)                                     # some rows ascending: thresholds raised by the waves
+    u = rng.random(B, dtype=np.float32)
+    hist = ((rng.zipf(1.1, size=(B, H)) - 1) % V).astype(np.int32) if H else None
+    got, _, _ = _check_against_oracle(oracle, rocm, x, u, 0.7, k, 0.9, 1.15, hist, nuc=k)
+    c = got["counters"]
+    assert c["topk_rows"] + c["fallback_rows"] == B and c["general_rows"] == 0
 
 
 @pytest.mark.parametrize("V,H", [(128256, 512), (32000, 1000), (5003, 64), (777, 1024)])
