@@ -514,7 +514,7 @@ int born_rocm_token_logprobs(born_sampler *s, const float *logits, int64_t batch
     a.hist_counts = counted ? s->hist_counts : nullptr;
     hipStream_t st = (hipStream_t)stream;
     if (counted) HIP_TRY(launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, false, st));
-    hipError_t e = launch_token_logprobs(a, tokens, logprobs_out, st);
+    hipError_t e = launch_token_logprobs(a, tokens, logprobs_out, st, s->path == 2);
     if (counted) {
         const hipError_t ce = launch_hist_counts(history, hist_len, hist_stride, a.B, a.V, s->hist_counts, true, st);
         if (e == hipSuccess) e = ce;

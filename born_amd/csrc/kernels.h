@@ -145,7 +145,7 @@ hipError_t launch_argmax(const float *logits, int B, int V, long long stride, in
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
                           hipStream_t st);
 // out[row] = log_softmax(z of the row)[tokens[row]] (penalties and temperature applied, no truncation)
-hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st);
+hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st, bool two_per_cu = false);
 // history[b][hist_len[b]] = tokens[b]; hist_len[b] += 1 (a full row: unchanged, status bit 4; a token outside [0, V): bit 0)
 hipError_t launch_history_append(int *history, int *hist_len, long long hist_stride, const int *tokens, int B, int V, int *status,
                                  hipStream_t st);

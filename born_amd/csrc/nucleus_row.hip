@@ -935,9 +935,12 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
-__global__ __launch_bounds__(NUC_BLOCK_MAX) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
-                                                                  float *__restrict__ out) {
-    constexpr int NUC_BLOCK = NUC_BLOCK_MAX, NUC_WAVES = NUC_BLOCK / WAVE;
+// NUC_BLOCK: 1024 threads per row, or 512 for batches of more rows than the device has CUs (two rows to a CU at a time: a
+// CU holds one 1024-thread workgroup of this kernel, and the rows beyond the first round would wait for a free CU).
+template <int NUC_BLOCK>
+__global__ __launch_bounds__(NUC_BLOCK, 4) void token_logprob_kernel(SampleArgs a, const int *__restrict__ tokens,
+                                                                     float *__restrict__ out) {
+    constexpr int NUC_WAVES = NUC_BLOCK / WAVE;
     extern __shared__ __align__(16) u64 nuc_dyn[];
     __shared__ BlockScratch scr;
     __shared__ double s_part[NUC_WAVES];
@@ -1049,8 +1052,11 @@ __global__ __launch_bounds__(NUC_BLOCK_MAX) void token_logprob_kernel(SampleArgs
 
 size_t token_logprob_lds_bytes(int V) { return sizeof(u32) * (size_t)((V + 31) / 32) + 16; }
 
-hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st) {
-    hipLaunchKernelGGL(token_logprob_kernel, dim3((unsigned)a.B), dim3(NUC_BLOCK_MAX), token_logprob_lds_bytes(a.V), st, a, tokens, out);
+hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st, bool two_per_cu) {
+    if (two_per_cu || a.B > device_cu_count())
+        hipLaunchKernelGGL(token_logprob_kernel<512>, dim3((unsigned)a.B), dim3(512), token_logprob_lds_bytes(a.V), st, a, tokens, out);
+    else
+        hipLaunchKernelGGL(token_logprob_kernel<1024>, dim3((unsigned)a.B), dim3(1024), token_logprob_lds_bytes(a.V), st, a, tokens, out);
     return hipGetLastError();
 }
 
@@ -1149,7 +1155,10 @@ hipError_t configure_nucleus() {
         const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_both);
         if (e != hipSuccess) return e;
     }
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel<512>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)token_logprob_lds_bytes((int)WIDE_MAX_VOCAB));
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(token_logprob_kernel<1024>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                (int)token_logprob_lds_bytes((int)WIDE_MAX_VOCAB));
 }
 

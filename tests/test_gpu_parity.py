@@ -610,8 +610,11 @@ def test_frequency_and_presence_penalties_are_validated(rocm):
     (9, 1001, 0.5, 0.8, 300, -0.1, 0.4),          # unaligned rows, boosting penalties
     (5, 3, 1.0, 1.0, 0, 0.0, 0.0),
     (5, 1, 2.0, 1.0, 0, 0.0, 0.0),
+    (300, 8193, 1.0, 1.0, 0, 0.0, 0.0),           # more rows than CUs: the 512-thread instance by the default selection
+    (520, 5000, 0.8, 1.2, 100, 0.1, 0.0),
 ])
-def test_token_logprobs_against_oracle(oracle, rocm, B, V, T, rep, H, freq, pres):
+@pytest.mark.parametrize("path", [0, 2])          # 2: the 512-thread instance (two rows to a CU) whatever the batch
+def test_token_logprobs_against_oracle(oracle, rocm, B, V, T, rep, H, freq, pres, path):
     rng = np.random.default_rng(B * 31 + V)
     x = (rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.5)).astype(np.float32)
     tok = rng.integers(0, V, B).astype(np.int32)
@@ -623,6 +626,7 @@ def test_token_logprobs_against_oracle(oracle, rocm, B, V, T, rep, H, freq, pres
     s = rocm.NewSampler(rocm.SamplerConfig(Temperature=T, RepetitionPenalty=rep, FrequencyPenalty=freq, PresencePenalty=pres,
                                            TopK=5, TopP=0.5, MinP=0.1),     # truncation settings do not enter
                         max_batch=B, max_vocab=V)
+    s.SetPath(path)
     got = rocm.token_logprobs_host(s, x, tok, hist, hist_len)
     s.Status()
     s.Close()

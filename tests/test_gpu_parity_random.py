@@ -89,6 +89,7 @@ def test_random_token_logprobs_against_oracle(oracle, rocm, chunk):
         tok = rng.integers(0, V, B).astype(np.int32)
         s = rocm.NewSampler(rocm.SamplerConfig(Temperature=c["T"], RepetitionPenalty=c["rep"], FrequencyPenalty=c["freq"],
                                                PresencePenalty=c["pres"]), max_batch=B, max_vocab=V)
+        s.SetPath(2 * (i & 1))                                                           # every other case: 512 threads per row
         got = rocm.token_logprobs_host(s, x, tok, hist, hist_len)
         s.Status()
         s.Close()
