@@ -162,44 +162,176 @@ hipError_t launch_argmax(const float *logits, int B, int V, long long stride, in
 }
 
 // ---------------------------------------------------------------------------
-// softmax / log-softmax: one workgroup (1024 threads) per row, three sweeps
-// (max, integer mass sum, write); sweeps two and three hit L2.
+// softmax / log-softmax over the rows of a [batch, vocab] matrix.
+//   m = max z, z = canon(x);  e = emass(z, m);  Z = sum of trunc(e * 2^S) as integers (order-free, so the result does
+//   not depend on how a row is spread over lanes);  softmax = fl32(fl64(e) / (Z * 2^-S)),  log-softmax =
+//   fl32((fl64(z) - fl64(m)) - ln(Z * 2^-S)).
+// Rows of up to 32 768 elements are held in registers between the three steps (one read of the row, one write):
+// 64, 256 or 1024 lanes per row by its length, eight 128-bit loads per lane at most; a row of a single wave needs no
+// LDS and no barrier, and four of them share a workgroup.  Longer rows are swept three times by 1024 threads.
 // ---------------------------------------------------------------------------
+typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
 
-template <bool LOG>
-__global__ __launch_bounds__(1024) void softmax_kernel(const float *__restrict__ logits, int V, long long stride,
-                                                       float *__restrict__ out, int S) {
+// fl32(fl64(e) / Zd).  The quotient by a reciprocal is within two units of the fp64 quotient's last place, so the two
+// round to the same fp32 unless the product lies that close to the middle between two fp32 values (or the result is
+// subnormal in fp32): only then is the division itself carried out.
+__device__ __forceinline__ float softmax_quotient(float e, double Zd, double rZ) {
+    const double q = (double)e * rZ;
+    const u32 low = (u32)__double2loint(q) & 0x1FFFFFFFu;            // the 29 bits below an fp32's last place
+    if ((low - 0x0FFFFFF8u) <= 0x10u || (q < 0x1p-120 && q != 0.0)) return (float)((double)e / Zd);
+    return (float)q;
+}
+__device__ __forceinline__ u64 wave_sum_u64(u64 v) { return shfl_u64(wave_inclusive_scan_u64(v), WAVE - 1); }
+
+// TPR lanes per row, U 128-bit loads per lane: TPR * U * 4 >= V.
+template <int TPR, int U, bool LOG>
+__global__ __launch_bounds__(TPR == 64 ? 256 : TPR) void softmax_resident_kernel(const float *__restrict__ logits, int B, int V,
+                                                                              long long stride, float *__restrict__ out, int S) {
+    constexpr int BLOCK = TPR == 64 ? 256 : TPR;
     __shared__ BlockScratch scr;
-    const int row = blockIdx.x;
+    const int t = TPR == 64 ? lane_id() : (int)threadIdx.x;
+    const int row = TPR == 64 ? (int)blockIdx.x * (BLOCK / WAVE) + wave_id() : (int)blockIdx.x;
+    if (row >= B) return;                                            // (whole waves, and no barrier where rows share a workgroup)
     const float *x = logits + (long long)row * stride;
     float *o = out + (long long)row * V;
+    const bool vin = (((uintptr_t)x) & 15) == 0, vout = (((uintptr_t)o) & 15) == 0;
+    float v[U][4];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int j = (u * TPR + t) * 4;
+        if (vin && j + 3 < V) {
+            const sm_f32x4 f = __builtin_nontemporal_load(reinterpret_cast<const sm_f32x4 *>(x + j));
+#pragma unroll
+            for (int c = 0; c < 4; c++) v[u][c] = f[c];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++) v[u][c] = j + c < V ? x[j + c] : 0.0f;
+        }
+    }
     float mx = -INFINITY;
-    for (int j = threadIdx.x; j < V; j += 1024) mx = fmaxf(mx, canon(x[j]));
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            v[u][c] = canon(v[u][c]);
+            if ((u * TPR + t) * 4 + c < V) mx = fmaxf(mx, v[u][c]);
+        }
+    const float m = TPR == 64 ? wave_max_f32(mx) : block_max_f32<BLOCK>(mx, &scr);
+    const float scale = mass_scale(S);
+    u64 acc = 0;
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float e = emass(v[u][c], m);
+            if ((u * TPR + t) * 4 + c < V) acc += qfix(e, scale);
+            if (!LOG) v[u][c] = e;
+        }
+    u64 Z;
+    if (TPR == 64) Z = wave_sum_u64(acc);
+    else block_inclusive_scan_u64<BLOCK>(acc, &scr, &Z);
+    const double Zd = ldexp((double)Z, -S);
+    const double lz = LOG ? log(Zd) : 0.0, rZ = LOG ? 0.0 : 1.0 / Zd;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int j = (u * TPR + t) * 4;
+        float r[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) r[c] = LOG ? (float)(((double)v[u][c] - (double)m) - lz) : softmax_quotient(v[u][c], Zd, rZ);
+        if (vout && j + 3 < V) {
+            sm_f32x4 f;
+#pragma unroll
+            for (int c = 0; c < 4; c++) f[c] = r[c];
+            __builtin_nontemporal_store(f, reinterpret_cast<sm_f32x4 *>(o + j));
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                if (j + c < V) o[j + c] = r[c];
+        }
+    }
+}
+
+// Rows beyond 32 768 elements: one workgroup of 1024 threads per row, three sweeps (the second and third re-read the
+// row from the caches where it still is), four 128-bit loads in flight per thread.
+template <bool LOG>
+__global__ __launch_bounds__(1024) void softmax_sweep_kernel(const float *__restrict__ logits, int V, long long stride,
+                                                             float *__restrict__ out, int S) {
+    __shared__ BlockScratch scr;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float *x = logits + (long long)row * stride;
+    float *o = out + (long long)row * V;
+    const bool vin = (((uintptr_t)x) & 15) == 0, vout = (((uintptr_t)o) & 15) == 0;
+    const int n4 = vin ? V >> 2 : 0;                                 // 128-bit blocks of the row; the rest element by element
+    const sm_f32x4 *x4 = reinterpret_cast<const sm_f32x4 *>(x);
+    // every element of the row as f(index, value): four blocks in flight, then single blocks, then the ragged end
+    auto sweep = [&](auto f) {
+        int i = tid;
+        for (; i + 3 * 1024 < n4; i += 4 * 1024) {
+            sm_f32x4 q[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) q[u] = x4[i + u * 1024];
+#pragma unroll
+            for (int u = 0; u < 4; u++) f((i + u * 1024) << 2, q[u]);
+        }
+        for (; i < n4; i += 1024) f(i << 2, x4[i]);
+    };
+    float mx = -INFINITY;
+    sweep([&](int, const sm_f32x4 &q) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) mx = fmaxf(mx, canon(q[c]));
+    });
+    for (int j = (n4 << 2) + tid; j < V; j += 1024) mx = fmaxf(mx, canon(x[j]));
     const float m = block_max_f32<1024>(mx, &scr);
     const float scale = mass_scale(S);
     u64 acc = 0;
-    for (int j = threadIdx.x; j < V; j += 1024) acc += qfix(emass(canon(x[j]), m), scale);
+    sweep([&](int, const sm_f32x4 &q) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc += qfix(emass(canon(q[c]), m), scale);
+    });
+    for (int j = (n4 << 2) + tid; j < V; j += 1024) acc += qfix(emass(canon(x[j]), m), scale);
     u64 Z;
     block_inclusive_scan_u64<1024>(acc, &scr, &Z);
     const double Zd = ldexp((double)Z, -S);
-    if (LOG) {
-        const double lz = log(Zd);
-        for (int j = threadIdx.x; j < V; j += 1024) {
-            float z = canon(x[j]);
-            o[j] = (float)(((double)z - (double)m) - lz);
+    const double lz = LOG ? log(Zd) : 0.0, rZ = LOG ? 0.0 : 1.0 / Zd;
+    auto result = [&](float xv) {
+        const float z = canon(xv);
+        return LOG ? (float)(((double)z - (double)m) - lz) : softmax_quotient(emass(z, m), Zd, rZ);
+    };
+    sweep([&](int j, const sm_f32x4 &q) {
+        sm_f32x4 r;
+#pragma unroll
+        for (int c = 0; c < 4; c++) r[c] = result(q[c]);
+        if (vout) {
+            __builtin_nontemporal_store(r, reinterpret_cast<sm_f32x4 *>(o + j));
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[j + c] = r[c];
         }
-    } else {
-        for (int j = threadIdx.x; j < V; j += 1024) o[j] = (float)((double)emass(canon(x[j]), m) / Zd);
-    }
+    });
+    for (int j = (n4 << 2) + tid; j < V; j += 1024) o[j] = result(x[j]);
+}
+
+template <bool LOG>
+static void launch_softmax_as(const float *logits, int B, int V, long long stride, float *out, int S, hipStream_t st) {
+    // the fewest lanes that hold the row in at most eight loads each, and no more loads per lane than the row needs (a
+    // load slot past the row's end still costs its arithmetic)
+    const dim3 waves((unsigned)((B + 3) / 4)), rows((unsigned)B);
+    if (V <= 256) hipLaunchKernelGGL((softmax_resident_kernel<64, 1, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 512) hipLaunchKernelGGL((softmax_resident_kernel<64, 2, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 1024) hipLaunchKernelGGL((softmax_resident_kernel<64, 4, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 2048) hipLaunchKernelGGL((softmax_resident_kernel<64, 8, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 4096) hipLaunchKernelGGL((softmax_resident_kernel<256, 4, LOG>), rows, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 8192) hipLaunchKernelGGL((softmax_resident_kernel<256, 8, LOG>), rows, dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 16384) hipLaunchKernelGGL((softmax_resident_kernel<1024, 4, LOG>), rows, dim3(1024), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 32768) hipLaunchKernelGGL((softmax_resident_kernel<1024, 8, LOG>), rows, dim3(1024), 0, st, logits, B, V, stride, out, S);
+    else hipLaunchKernelGGL(softmax_sweep_kernel<LOG>, rows, dim3(1024), 0, st, logits, V, stride, out, S);
 }
 
 hipError_t launch_softmax(const float *logits, int B, int V, long long stride, float *out, bool log_form,
                           hipStream_t st) {
-    int S = mass_shift(V);
-    if (log_form)
-        hipLaunchKernelGGL(softmax_kernel<true>, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, out, S);
-    else
-        hipLaunchKernelGGL(softmax_kernel<false>, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, out, S);
+    const int S = mass_shift(V);
+    if (log_form) launch_softmax_as<true>(logits, B, V, stride, out, S, st);
+    else launch_softmax_as<false>(logits, B, V, stride, out, S, st);
     return hipGetLastError();
 }
 

@@ -157,6 +157,44 @@ def test_softmax_operators(oracle, rocm):
     assert np.max(np.abs(lg - np.log(want))) < 1e-5
 
 
+@pytest.mark.parametrize("B,V,pad", [(5, 1, 0), (7, 3, 0), (33, 64, 0), (6, 256, 0), (600, 257, 0), (9, 512, 4), (9, 513, 1), (300, 1000, 0),
+                                     (17, 1024, 0), (17, 1025, 0), (9, 2048, 0), (9, 2049, 3), (260, 4096, 8), (7, 4097, 0), (5, 8192, 4),
+                                     (5, 8193, 0), (3, 16384, 0), (3, 16385, 2), (3, 32768, 0), (3, 32769, 1), (4, 70001, 0), (2, 128256, 0)])
+def test_softmax_every_row_length_and_layout(oracle, rocm, B, V, pad):
+    # One wave, 256 or 1024 lanes per row with the row held in registers, or three sweeps, by the row's length; rows that
+    # start unaligned (a pitch that is no multiple of four) and ragged ends take the element-wise loads and stores.
+    # Held to 1e-5 of the fp64 softmax; and equal, bit for bit, to the kernel's own definition put together from the
+    # oracle's pieces: fl32(fl64(e) / Z) with e the oracle's expneg of (max - z) and Z the sum of trunc(e * 2^S) * 2^-S.
+    rng = np.random.default_rng(B * 7919 + V)
+    x = (rng.standard_normal((B, V + pad)) * 3.0).astype(np.float32)
+    if V > 8:
+        x[0, rng.integers(0, V, size=3)] = -np.inf
+        x[B - 1, rng.integers(0, V, size=2)] = np.float32(-3e38)
+        x[B // 2, :V] = np.round(x[B // 2, :V])                             # ties at the maximum
+    s = rocm.NewSampler(max_batch=B, max_vocab=V)
+    d, o = rocm.DeviceBuffer.from_numpy(x), rocm.DeviceBuffer(4 * B * V)
+    rows = x[:, :V]
+    for log in (False, True):
+        s.Softmax(d, B, V, o, row_stride=V + pad, log=log)
+        got = o.to_numpy(np.float32, (B, V))
+        want = oracle.softmax_f64(np.ascontiguousarray(rows))
+        if log:
+            fin = want > 0
+            assert np.max(np.abs(got[fin].astype(np.float64) - np.log(want[fin]))) < 2e-5 and np.all(got[~fin] < -80.0)
+            continue
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-30)
+        assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
+        m, Zi = oracle.row_stats(np.ascontiguousarray(rows))                # the oracle's maximum and integer normaliser
+        assert np.array_equal(m, rows.max(axis=1))
+        with np.errstate(invalid="ignore"):
+            dist = (m[:, None] - rows).astype(np.float32)
+        dist[rows == m[:, None]] = 0.0
+        e = oracle.expneg(dist)
+        Z = Zi.astype(np.float64) * 2.0 ** -(62 - int(V).bit_length())       # (2^S with S = 62 - bits(V): a row sums below 2^62)
+        assert np.array_equal(got.view(np.uint32), (e.astype(np.float64) / Z[:, None]).astype(np.float32).view(np.uint32))
+    s.Close()
+
+
 # ---------------------------------------------------------------- sampling: single-pass top-k kernel
 # path 0 = the default kernel selection (1 <= top_k <= 512: one workgroup per row, one launch); path 2 = the same with
 # the 512-thread instance (top_k <= 128) whatever the batch, which by default only batches of more rows than CUs get
