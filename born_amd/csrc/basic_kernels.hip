@@ -171,6 +171,8 @@ hipError_t launch_argmax(const float *logits, int B, int V, long long stride, in
 // LDS and no barrier, and four of them share a workgroup.  Longer rows are swept three times by 1024 threads.
 // ---------------------------------------------------------------------------
 typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
+// canon() without its last step (-0 -> +0 only matters where z is turned into a sort key)
+__device__ __forceinline__ float sm_canon(float z) { return fminf((z != z) ? -INFINITY : z, 3.402823466e+38f); }
 
 // fl32(fl64(e) / Zd).  The quotient by a reciprocal is within two units of the fp64 quotient's last place, so the two
 // round to the same fp32 unless the product lies that close to the middle between two fp32 values (or the result is
@@ -178,8 +180,9 @@ typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float softmax_quotient(float e, double Zd, double rZ) {
     const double q = (double)e * rZ;
     const u32 low = (u32)__double2loint(q) & 0x1FFFFFFFu;            // the 29 bits below an fp32's last place
-    if ((low - 0x0FFFFFF8u) <= 0x10u || (q < 0x1p-120 && q != 0.0)) return (float)((double)e / Zd);
-    return (float)q;
+    const float f = (float)q;
+    if ((low - 0x0FFFFFF8u) <= 0x10u || (f < 0x1p-100f && e != 0.0f)) return (float)((double)e / Zd);
+    return f;
 }
 __device__ __forceinline__ u64 wave_sum_u64(u64 v) { return shfl_u64(wave_inclusive_scan_u64(v), WAVE - 1); }
 
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(TPR == 64 ? 256 : TPR) void softmax_resident_kernel
     for (int u = 0; u < U; u++)
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-            v[u][c] = canon(v[u][c]);
+            v[u][c] = sm_canon(v[u][c]);
             if ((u * TPR + t) * 4 + c < V) mx = fmaxf(mx, v[u][c]);
         }
     const float m = TPR == 64 ? wave_max_f32(mx) : block_max_f32<BLOCK>(mx, &scr);
@@ -278,23 +281,23 @@ __global__ __launch_bounds__(1024) void softmax_sweep_kernel(const float *__rest
     float mx = -INFINITY;
     sweep([&](int, const sm_f32x4 &q) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) mx = fmaxf(mx, canon(q[c]));
+        for (int c = 0; c < 4; c++) mx = fmaxf(mx, sm_canon(q[c]));
     });
-    for (int j = (n4 << 2) + tid; j < V; j += 1024) mx = fmaxf(mx, canon(x[j]));
+    for (int j = (n4 << 2) + tid; j < V; j += 1024) mx = fmaxf(mx, sm_canon(x[j]));
     const float m = block_max_f32<1024>(mx, &scr);
     const float scale = mass_scale(S);
     u64 acc = 0;
     sweep([&](int, const sm_f32x4 &q) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc += qfix(emass(canon(q[c]), m), scale);
+        for (int c = 0; c < 4; c++) acc += qfix(emass(sm_canon(q[c]), m), scale);
     });
-    for (int j = (n4 << 2) + tid; j < V; j += 1024) acc += qfix(emass(canon(x[j]), m), scale);
+    for (int j = (n4 << 2) + tid; j < V; j += 1024) acc += qfix(emass(sm_canon(x[j]), m), scale);
     u64 Z;
     block_inclusive_scan_u64<1024>(acc, &scr, &Z);
     const double Zd = ldexp((double)Z, -S);
     const double lz = LOG ? log(Zd) : 0.0, rZ = LOG ? 0.0 : 1.0 / Zd;
     auto result = [&](float xv) {
-        const float z = canon(xv);
+        const float z = sm_canon(xv);
         return LOG ? (float)(((double)z - (double)m) - lz) : softmax_quotient(emass(z, m), Zd, rZ);
     };
     sweep([&](int j, const sm_f32x4 &q) {
