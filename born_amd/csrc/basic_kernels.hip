@@ -95,13 +95,19 @@ __global__ __launch_bounds__(64) void argmax_merge_kernel(const float *__restric
     if (threadIdx.x == 0) tokens[row] = argmax_token(b, logits[(long long)row * stride]);
 }
 
-// Batches that fill a fair part of the device on their own: one workgroup of 1024 threads per row, one launch
+// Batches that fill a fair part of the device on their own: a row per workgroup in one launch
 // (64 rows x 32000: 7.1 us as two launches, of which the second only merges four partials per row).
+// TPR lanes per row by its length: 1024, 256, or one wave (four rows to a workgroup, no LDS and no barrier) - a row of
+// 1024 logits gives 1024 threads one logit each and spends its time in the reduction.
 typedef float argmax_f32x4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(1024) void argmax_row_kernel(const float *__restrict__ logits, int V, long long stride,
-                                                          int *__restrict__ tokens) {
-    __shared__ ArgPair sh[16];
-    const int row = blockIdx.x, tid = threadIdx.x;
+template <int TPR>
+__global__ __launch_bounds__(TPR == 64 ? 256 : TPR) void argmax_row_kernel(const float *__restrict__ logits, int B, int V, long long stride,
+                                                                        int *__restrict__ tokens) {
+    constexpr int NW = TPR / WAVE;
+    __shared__ ArgPair sh[NW];
+    const int row = TPR == 64 ? (int)blockIdx.x * 4 + wave_id() : (int)blockIdx.x;
+    const int tid = TPR == 64 ? lane_id() : (int)threadIdx.x;
+    if (row >= B) return;                                            // (whole waves; no barrier where rows share a workgroup)
     const float *x = logits + (long long)row * stride;
     const bool vec = ((stride & 3) == 0) && ((((uintptr_t)logits) & 15) == 0);
     ArgPair best = {-INFINITY, 0x7FFFFFFF};
@@ -116,30 +122,34 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const float *__restric
         const int n4 = V >> 2;
         const argmax_f32x4 *x4 = reinterpret_cast<const argmax_f32x4 *>(x);
         int i = tid;
-        for (; i + 3 * 1024 < n4; i += 4 * 1024) {                    // four loads in flight per thread
+        for (; i + 3 * TPR < n4; i += 4 * TPR) {                      // four loads in flight per thread
             argmax_f32x4 f[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) f[u] = __builtin_nontemporal_load(x4 + i + u * 1024);
+            for (int u = 0; u < 4; u++) f[u] = __builtin_nontemporal_load(x4 + i + u * TPR);
 #pragma unroll
             for (int u = 0; u < 4; u++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) take(f[u][c], ((i + u * 1024) << 2) + c);
+                for (int c = 0; c < 4; c++) take(f[u][c], ((i + u * TPR) << 2) + c);
         }
-        for (; i < n4; i += 1024) {
+        for (; i < n4; i += TPR) {
             const argmax_f32x4 f = __builtin_nontemporal_load(x4 + i);
 #pragma unroll
             for (int c = 0; c < 4; c++) take(f[c], (i << 2) + c);
         }
-        for (int j = (n4 << 2) + tid; j < V; j += 1024) take(x[j], j);
+        for (int j = (n4 << 2) + tid; j < V; j += TPR) take(x[j], j);
     } else {
-        for (int j = tid; j < V; j += 1024) take(x[j], j);
+        for (int j = tid; j < V; j += TPR) take(x[j], j);
     }
     best = wave_best(best);
+    if (TPR == 64) {
+        if (tid == 0) tokens[row] = argmax_token(best, x[0]);
+        return;
+    }
     if (lane_id() == 0) sh[wave_id()] = best;
     __syncthreads();
     if (tid == 0) {
         ArgPair b = sh[0];
-        for (int w = 1; w < 16; w++) b = better(b, sh[w]);
+        for (int w = 1; w < NW; w++) b = better(b, sh[w]);
         tokens[row] = argmax_token(b, x[0]);
     }
 }
@@ -149,7 +159,9 @@ constexpr int ARGMAX_ROW_KERNEL_BATCH = 64;     // from this many rows on, a row
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st) {
     if (B >= ARGMAX_ROW_KERNEL_BATCH) {
-        hipLaunchKernelGGL(argmax_row_kernel, dim3((unsigned)B), dim3(1024), 0, st, logits, V, stride, tokens);
+        if (V <= 4096) hipLaunchKernelGGL(argmax_row_kernel<64>, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, logits, B, V, stride, tokens);
+        else if (V <= 16384) hipLaunchKernelGGL(argmax_row_kernel<256>, dim3((unsigned)B), dim3(256), 0, st, logits, B, V, stride, tokens);
+        else hipLaunchKernelGGL(argmax_row_kernel<1024>, dim3((unsigned)B), dim3(1024), 0, st, logits, B, V, stride, tokens);
         return hipGetLastError();
     }
     int S = (V + ARGMAX_SEG - 1) / ARGMAX_SEG;

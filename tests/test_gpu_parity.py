@@ -115,7 +115,9 @@ def test_argmax_reference_kats_and_tie_rule(oracle, rocm):
 
 @pytest.mark.parametrize("B,V,stride", [(64, 32000, None), (7, 8193, None), (5, 1001, 1003), (3, 128256, None), (2, 5, 8),
                                         (63, 32000, None), (64, 8193, None), (70, 1001, 1003), (65, 5, 8), (64, 16384, 16388),
-                                        (96, 128256, None), (64, 1, None), (64, 20001, 20004)])
+                                        (96, 128256, None), (64, 1, None), (64, 20001, 20004),
+                                        (67, 4096, None), (66, 4097, None), (301, 1024, None), (130, 16384, None), (65, 16385, 16388),
+                                        (1000, 63, 64), (70, 4095, 4095)])
 def test_argmax_random_and_ties(oracle, rocm, B, V, stride):
     rng = np.random.default_rng(V)
     x = rng.standard_normal((B, V), dtype=np.float32)
