@@ -543,6 +543,24 @@ def main_extras(args, torch, S, synth, dev):
     for name, fn in cases.items():
         out["us"][name] = timed(fn, args.steps, args.warmup)
     if args.config == "C3x":
+        # larger batches at the C3 settings: more rows than CUs run two rows to a CU at a time (512 threads per row)
+        out["larger_batches"] = {}
+        for rows in (512, 1024):
+            wl = synth.c3(rows=rows)
+            lg2 = [torch.from_numpy(wl.logits).to(dev) for _ in range(2)]
+            u2, h2 = torch.from_numpy(wl.uniforms).to(dev), torch.from_numpy(wl.history).to(dev)
+            t2, p2 = torch.empty(rows, dtype=torch.int32, device=dev), torch.empty(rows, device=dev)
+            s2 = S.NewSampler(S.SamplerConfig(Temperature=wl.temperature, TopK=wl.top_k, TopP=wl.top_p, RepetitionPenalty=wl.rep),
+                              max_batch=rows, max_vocab=V)
+
+            def big():
+                c[0] += 1
+                s2.Sample(lg2[c[0] % 2], rows, V, h2, None, u2, t2, p2, hist_stride=H, stream=stream)
+            us = timed(big, args.steps, args.warmup)
+            out["larger_batches"][f"{rows} rows"] = {"us": us, "tokens_per_s": rows / us * 1e6,
+                                                     "frac_of_8TBs": wl.algorithmic_bytes() / us / 1e3 / HBM_PEAK_GBS}
+            s2.Close()
+            del lg2
         # rows the single-pass kernel handed to its exact selection, over every step of every case above (0: none did)
         out["exact_selection_rows_total"] = {name: smp.Counters(stream)["fallback_rows"] for name, smp in
                                              (("handle of the C3 settings (all its cases)", base), ("top_k 256", k256), ("top_k 512", k512),
