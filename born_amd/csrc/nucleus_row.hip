@@ -1050,9 +1050,93 @@ __global__ __launch_bounds__(NUC_BLOCK, 4) void token_logprob_kernel(SampleArgs 
     }
 }
 
+// Short rows without a history (the cross-entropy term of a classifier: ten classes, a few thousand at most): a group
+// of G lanes per row, 64 / G rows to a wave, no LDS and no barrier; the same arithmetic per lane as above, the lanes of
+// a group combined by butterflies.  A workgroup of 1024 threads for a row of ten logits spends its time in launches:
+// 65 536 x 10 took 252 us.
+template <int G>
+__global__ __launch_bounds__(256) void token_logprob_small_kernel(SampleArgs a, const int *__restrict__ tokens, float *__restrict__ out) {
+    const int V = a.V;
+    const int gl = (int)threadIdx.x & (G - 1);                       // lane within the row's group
+    const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / G;
+    const bool live = row < (long long)a.B;
+    const float *x = a.logits + (live ? row : 0ll) * a.row_stride;
+    const float T = a.T, rT = 1.0f / T;
+    const bool unit = T == 1.0f;
+    auto zof = [&](float y) {
+        if (unit) return canon(y);
+        const float q0 = y * rT;
+        const float q1 = fmaf(fmaf(-q0, T, y), rT, q0);
+        return canon(fabsf(y) <= 3.402823466e+38f ? q1 : q0);
+    };
+    auto term = [](float z, float m) { return z == m ? 1.0f : __expf(z - m); };
+    int qt = -1;
+    float qy = 0.0f;
+    if (live && gl == 0) {
+        qt = tokens[row];
+        if (qt >= 0 && qt < V) qy = x[qt];
+    }
+    float mt = -INFINITY;
+    double st = 0.0;
+    auto one = [&](float y) {
+        const float z = zof(y);
+        if (z > mt) {
+            st *= (double)__expf(mt - z);
+            mt = z;
+        }
+        st += (double)term(z, mt);
+    };
+    if (live) {
+        const bool vec = G == 64 && ((a.row_stride & 3) == 0) && ((((uintptr_t)a.logits) & 15) == 0);
+        int done = 0;
+        if (vec) {
+            const int n4 = V >> 2;
+            const nuc_f32x4 *x4 = reinterpret_cast<const nuc_f32x4 *>(x);
+            for (int i = gl; i < n4; i += G) {
+                const nuc_f32x4 q = __builtin_nontemporal_load(x4 + i);
+                float z[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) z[t] = zof(q[t]);
+                const float m4 = fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3]));
+                if (m4 > mt) {
+                    st *= (double)__expf(mt - m4);
+                    mt = m4;
+                }
+                st += (double)((term(z[0], mt) + term(z[1], mt)) + (term(z[2], mt) + term(z[3], mt)));
+            }
+            done = n4 << 2;
+        }
+        for (int j = done + gl; j < V; j += G) one(x[j]);
+    }
+    // the group's maximum, then the sums brought to it (a lane without elements: st = 0)
+    float m = mt;
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, WAVE));
+    double part = mt == m ? st : st * exp((double)mt - (double)m);
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) part += __shfl_xor(part, o, WAVE);
+    if (live && gl == 0) {
+        if (qt < 0 || qt >= V) {
+            atomicOr(a.status, 1);
+            out[row] = __uint_as_float(0x7FC00000u);                 // not a token of this vocabulary
+        } else {
+            const float z = zof(qy);
+            const double d = z == m ? 0.0 : (double)m - (double)z;
+            out[row] = (float)(-d - log(part));
+        }
+    }
+}
+
 size_t token_logprob_lds_bytes(int V) { return sizeof(u32) * (size_t)((V + 31) / 32) + 16; }
 
 hipError_t launch_token_logprobs(const SampleArgs &a, const int *tokens, float *out, hipStream_t st, bool two_per_cu) {
+    if (!a.history && a.V <= 4096) {                                 // short rows, nothing to penalise: lanes per row by length
+        const long long rows = a.B;
+        if (a.V <= 16) hipLaunchKernelGGL(token_logprob_small_kernel<4>, dim3((unsigned)((rows * 4 + 255) / 256)), dim3(256), 0, st, a, tokens, out);
+        else if (a.V <= 128) hipLaunchKernelGGL(token_logprob_small_kernel<16>, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st, a, tokens, out);
+        else hipLaunchKernelGGL(token_logprob_small_kernel<64>, dim3((unsigned)((rows * 64 + 255) / 256)), dim3(256), 0, st, a, tokens, out);
+        return hipGetLastError();
+    }
     if (two_per_cu || a.B > device_cu_count())
         hipLaunchKernelGGL(token_logprob_kernel<512>, dim3((unsigned)a.B), dim3(512), token_logprob_lds_bytes(a.V), st, a, tokens, out);
     else

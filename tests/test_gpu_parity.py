@@ -650,6 +650,11 @@ def test_frequency_and_presence_penalties_are_validated(rocm):
     (9, 1001, 0.5, 0.8, 300, -0.1, 0.4),          # unaligned rows, boosting penalties
     (5, 3, 1.0, 1.0, 0, 0.0, 0.0),
     (5, 1, 2.0, 1.0, 0, 0.0, 0.0),
+    (4096, 10, 1.0, 1.0, 0, 0.0, 0.0),            # short rows without a history: a group of lanes per row (4, 16 or 64 by length)
+    (300, 100, 0.7, 1.0, 0, 0.0, 0.0),
+    (70, 4096, 1.3, 1.0, 0, 0.0, 0.0),
+    (9, 4095, 1.0, 1.0, 0, 0.0, 0.0),
+    (33, 17, 2.0, 1.0, 0, 0.0, 0.0),
     (300, 8193, 1.0, 1.0, 0, 0.0, 0.0),           # more rows than CUs: the 512-thread instance by the default selection
     (520, 5000, 0.8, 1.2, 100, 0.1, 0.0),
 ])
