@@ -154,12 +154,39 @@ __global__ __launch_bounds__(TPR == 64 ? 256 : TPR) void argmax_row_kernel(const
     }
 }
 
+// Rows of at most 64 logits (the classes of a classifier): a group of G lanes per row, 64 / G rows to a wave.
+template <int G>
+__global__ __launch_bounds__(256) void argmax_group_kernel(const float *__restrict__ logits, int B, int V, long long stride,
+                                                           int *__restrict__ tokens) {
+    const int gl = (int)threadIdx.x & (G - 1);
+    const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / G;
+    const bool live = row < (long long)B;
+    const float *x = logits + (live ? row : 0ll) * stride;
+    ArgPair best = {-INFINITY, 0x7FFFFFFF};
+    if (live)
+        for (int j = gl; j < V; j += G) {
+            const float v = x[j];
+            if (v > best.v) {
+                best.v = v;
+                best.i = j;
+            }
+        }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) {
+        ArgPair t = {__shfl_xor(best.v, o, WAVE), __shfl_xor(best.i, o, WAVE)};
+        best = better(best, t);
+    }
+    if (live && gl == 0) tokens[row] = argmax_token(best, x[0]);
+}
+
 constexpr int ARGMAX_ROW_KERNEL_BATCH = 64;     // from this many rows on, a row per workgroup
 
 hipError_t launch_argmax(const float *logits, int B, int V, long long stride, int *tokens, float *part_val,
                          int *part_idx, hipStream_t st) {
     if (B >= ARGMAX_ROW_KERNEL_BATCH) {
-        if (V <= 4096) hipLaunchKernelGGL(argmax_row_kernel<64>, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, logits, B, V, stride, tokens);
+        if (V <= 16) hipLaunchKernelGGL(argmax_group_kernel<4>, dim3((unsigned)(((long long)B * 4 + 255) / 256)), dim3(256), 0, st, logits, B, V, stride, tokens);
+        else if (V <= 64) hipLaunchKernelGGL(argmax_group_kernel<16>, dim3((unsigned)(((long long)B * 16 + 255) / 256)), dim3(256), 0, st, logits, B, V, stride, tokens);
+        else if (V <= 4096) hipLaunchKernelGGL(argmax_row_kernel<64>, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, logits, B, V, stride, tokens);
         else if (V <= 16384) hipLaunchKernelGGL(argmax_row_kernel<256>, dim3((unsigned)B), dim3(256), 0, st, logits, B, V, stride, tokens);
         else hipLaunchKernelGGL(argmax_row_kernel<1024>, dim3((unsigned)B), dim3(1024), 0, st, logits, B, V, stride, tokens);
         return hipGetLastError();
@@ -266,6 +293,49 @@ __global__ __launch_bounds__(TPR == 64 ? 256 : TPR) void softmax_resident_kernel
     }
 }
 
+// Rows of at most 64 elements: a group of G lanes per row (four elements per lane at most), 64 / G rows to a wave.
+template <int G, bool LOG>
+__global__ __launch_bounds__(256) void softmax_group_kernel(const float *__restrict__ logits, int B, int V, long long stride,
+                                                            float *__restrict__ out, int S) {
+    const int gl = (int)threadIdx.x & (G - 1);
+    const long long row = ((long long)blockIdx.x * 256 + threadIdx.x) / G;
+    const bool live = row < (long long)B;
+    const float *x = logits + (live ? row : 0ll) * stride;
+    float *o = out + (live ? row : 0ll) * V;
+    float v[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int j = gl + t * G;
+        const bool in = live && j < V;
+        v[t] = sm_canon(in ? x[j] : 0.0f);
+        if (in) mx = fmaxf(mx, v[t]);
+    }
+#pragma unroll
+    for (int w = G / 2; w > 0; w >>= 1) mx = fmaxf(mx, __shfl_xor(mx, w, WAVE));
+    const float m = mx, scale = mass_scale(S);
+    u64 acc = 0;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const float e = emass(v[t], m);
+        if (live && gl + t * G < V) acc += qfix(e, scale);
+        if (!LOG) v[t] = e;
+    }
+#pragma unroll
+    for (int w = G / 2; w > 0; w >>= 1) {
+        const u32 lo = __shfl_xor((u32)acc, w, WAVE), hi = __shfl_xor((u32)(acc >> 32), w, WAVE);
+        acc += ((u64)hi << 32) | (u64)lo;
+    }
+    if (!live) return;
+    const double Zd = ldexp((double)acc, -S);
+    const double lz = LOG ? log(Zd) : 0.0, rZ = LOG ? 0.0 : 1.0 / Zd;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int j = gl + t * G;
+        if (j < V) o[j] = LOG ? (float)(((double)v[t] - (double)m) - lz) : softmax_quotient(v[t], Zd, rZ);
+    }
+}
+
 // Rows beyond 32 768 elements: one workgroup of 1024 threads per row, three sweeps (the second and third re-read the
 // row from the caches where it still is), four 128-bit loads in flight per thread.
 template <bool LOG>
@@ -331,7 +401,9 @@ static void launch_softmax_as(const float *logits, int B, int V, long long strid
     // the fewest lanes that hold the row in at most eight loads each, and no more loads per lane than the row needs (a
     // load slot past the row's end still costs its arithmetic)
     const dim3 waves((unsigned)((B + 3) / 4)), rows((unsigned)B);
-    if (V <= 256) hipLaunchKernelGGL((softmax_resident_kernel<64, 1, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
+    if (V <= 16) hipLaunchKernelGGL((softmax_group_kernel<4, LOG>), dim3((unsigned)(((long long)B * 4 + 255) / 256)), dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 64) hipLaunchKernelGGL((softmax_group_kernel<16, LOG>), dim3((unsigned)(((long long)B * 16 + 255) / 256)), dim3(256), 0, st, logits, B, V, stride, out, S);
+    else if (V <= 256) hipLaunchKernelGGL((softmax_resident_kernel<64, 1, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
     else if (V <= 512) hipLaunchKernelGGL((softmax_resident_kernel<64, 2, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
     else if (V <= 1024) hipLaunchKernelGGL((softmax_resident_kernel<64, 4, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);
     else if (V <= 2048) hipLaunchKernelGGL((softmax_resident_kernel<64, 8, LOG>), waves, dim3(256), 0, st, logits, B, V, stride, out, S);

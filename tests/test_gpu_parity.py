@@ -117,7 +117,8 @@ def test_argmax_reference_kats_and_tie_rule(oracle, rocm):
                                         (63, 32000, None), (64, 8193, None), (70, 1001, 1003), (65, 5, 8), (64, 16384, 16388),
                                         (96, 128256, None), (64, 1, None), (64, 20001, 20004),
                                         (67, 4096, None), (66, 4097, None), (301, 1024, None), (130, 16384, None), (65, 16385, 16388),
-                                        (1000, 63, 64), (70, 4095, 4095)])
+                                        (1000, 63, 64), (70, 4095, 4095), (4000, 10, None), (300, 16, 19), (77, 17, None), (129, 64, None),
+                                        (64, 65, None)])
 def test_argmax_random_and_ties(oracle, rocm, B, V, stride):
     rng = np.random.default_rng(V)
     x = rng.standard_normal((B, V), dtype=np.float32)
@@ -159,7 +160,7 @@ def test_softmax_operators(oracle, rocm):
     assert np.max(np.abs(lg - np.log(want))) < 1e-5
 
 
-@pytest.mark.parametrize("B,V,pad", [(5, 1, 0), (7, 3, 0), (33, 64, 0), (6, 256, 0), (600, 257, 0), (9, 512, 4), (9, 513, 1), (300, 1000, 0),
+@pytest.mark.parametrize("B,V,pad", [(5, 1, 0), (7, 3, 0), (33, 64, 0), (1000, 10, 0), (300, 16, 1), (77, 17, 0), (129, 63, 2), (64, 65, 0), (6, 256, 0), (600, 257, 0), (9, 512, 4), (9, 513, 1), (300, 1000, 0),
                                      (17, 1024, 0), (17, 1025, 0), (9, 2048, 0), (9, 2049, 3), (260, 4096, 8), (7, 4097, 0), (5, 8192, 4),
                                      (5, 8193, 0), (3, 16384, 0), (3, 16385, 2), (3, 32768, 0), (3, 32769, 1), (4, 70001, 0), (2, 128256, 0)])
 def test_softmax_every_row_length_and_layout(oracle, rocm, B, V, pad):
