@@ -195,8 +195,12 @@ __global__ __launch_bounds__(TOPS_BLOCK) void transpose_general_kernel(TensorInd
 // Conv2D (internal/backend/cpu/conv2d.go:35-203): input [N, C, H, W], kernel [CO, C, KH, KW], zero padding;
 // out[n, co, oh, ow] = sum over (c, kh, kw), in that order, of kernel * input, one fp32 accumulator per output,
 // product and sum each rounded (the reference's im2col + row-by-row dot product adds the terms in exactly this
-// order, the padded positions as a multiplication by 0), so results equal the CPU's bit for bit.  One output per
-// thread; neighbouring threads read neighbouring input columns and share the kernel values through the caches.
+// order, the padded positions as a multiplication by 0), so results equal the CPU's bit for bit.
+// conv2d_kernel: one output per thread; neighbouring threads read neighbouring input columns and share the kernel values
+// through the caches.  conv2d_group_kernel (below), which the launcher prefers: a workgroup takes 256 consecutive
+// positions (n, oh, ow) and CONV_COG output channels, so the kernel values are the same for every thread - scalar
+// loads, one per channel and product - and an input value is loaded once for CONV_COG products; every output still
+// has its own accumulator and the same order of terms.
 __global__ __launch_bounds__(TOPS_BLOCK) void conv2d_kernel(const float *in, const float *ker, float *out, int N, int C,
                                                             int H, int W, int CO, int KH, int KW, int HO, int WO, int stride,
                                                             int padding) {
@@ -319,8 +323,111 @@ hipError_t launch_tensor_transpose(const TensorIndexArgs &t, const float *in, fl
     return hipGetLastError();
 }
 
+// KWT: the kernel's width when it is 1, 3, 5 or 7 (the row of products is unrolled, its loads in flight together), else 0.
+// SQUARE: the kernel's height is KWT too, and a whole channel's patch is unrolled.
+// CONV_COG: output channels per thread (4; 2 or 1 where the launch would otherwise leave the SIMDs a wave or two each).
+template <int KWT, bool SQUARE, int CONV_COG>
+__global__ __launch_bounds__(TOPS_BLOCK) void conv2d_group_kernel(const float *__restrict__ in, const float *__restrict__ ker,
+                                                                  float *__restrict__ out, int N, int C, int H, int W, int CO, int KH,
+                                                                  int KW, int HO, int WO, int stride, int padding) {
+    const long long P = (long long)N * HO * WO;                      // positions
+    const long long p = (long long)blockIdx.x * TOPS_BLOCK + threadIdx.x;
+    const int co0 = (int)blockIdx.y * CONV_COG;                      // uniform: the kernel values come through scalar loads
+    const bool live = p < P;
+    const long long pc = live ? p : 0;
+    const int ow = (int)(pc % WO), oh = (int)((pc / WO) % HO), n = (int)(pc / ((long long)WO * HO));
+    const int h0 = oh * stride - padding, w0 = ow * stride - padding;
+    const long long ksz = (long long)C * KH * KW;
+    const float *kp[CONV_COG];
+#pragma unroll
+    for (int g = 0; g < CONV_COG; g++) kp[g] = ker + (long long)min(co0 + g, CO - 1) * ksz;   // (a channel past the last: computed, not stored)
+    float sum[CONV_COG];
+#pragma unroll
+    for (int g = 0; g < CONV_COG; g++) sum[g] = 0.0f;
+    const float *ip = in + (long long)n * C * H * W;
+    int kidx = 0;
+    for (int c = 0; c < C; c++, ip += (long long)H * W) {
+        if (SQUARE) {
+            float x[KWT > 0 ? KWT * KWT : 1];
+#pragma unroll
+            for (int kh = 0; kh < KWT; kh++) {
+                const int h = h0 + kh;
+                const bool hin = h >= 0 && h < H;
+                const float *rowp = ip + (long long)(hin ? h : 0) * W;
+#pragma unroll
+                for (int kw = 0; kw < KWT; kw++) {
+                    const int w = w0 + kw;
+                    x[kh * KWT + kw] = (hin && w >= 0 && w < W) ? rowp[w] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < KWT * KWT; t++)
+#pragma unroll
+                for (int g = 0; g < CONV_COG; g++) sum[g] += kp[g][kidx + t] * x[t];
+            kidx += KWT * KWT;
+            continue;
+        }
+        for (int kh = 0; kh < KH; kh++) {
+            const int h = h0 + kh;
+            const bool hin = h >= 0 && h < H;
+            const float *rowp = ip + (long long)(hin ? h : 0) * W;
+            if (KWT > 0) {
+                float x[KWT > 0 ? KWT : 1];
+#pragma unroll
+                for (int kw = 0; kw < KWT; kw++) {
+                    const int w = w0 + kw;
+                    x[kw] = (hin && w >= 0 && w < W) ? rowp[w] : 0.0f;
+                }
+#pragma unroll
+                for (int kw = 0; kw < KWT; kw++)
+#pragma unroll
+                    for (int g = 0; g < CONV_COG; g++) sum[g] += kp[g][kidx + kw] * x[kw];
+                kidx += KWT;
+            } else {
+                for (int kw = 0; kw < KW; kw++, kidx++) {
+                    const int w = w0 + kw;
+                    const bool win = hin && w >= 0 && w < W;
+                    const float x = win ? rowp[w] : 0.0f;
+#pragma unroll
+                    for (int g = 0; g < CONV_COG; g++) sum[g] += kp[g][kidx] * x;
+                }
+            }
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int g = 0; g < CONV_COG; g++)
+            if (co0 + g < CO) out[(((long long)n * CO + co0 + g) * HO + oh) * WO + ow] = sum[g];
+    }
+}
+
+template <int KWT, bool SQUARE>
+static void launch_conv2d_group(int cog, dim3 block, long long blocks, int CO, hipStream_t st, const float *in, const float *ker, float *out, int N,
+                                int C, int H, int W, int KH, int KW, int HO, int WO, int stride, int padding) {
+    const dim3 grid((unsigned)blocks, (unsigned)((CO + cog - 1) / cog));
+    if (cog == 4) hipLaunchKernelGGL((conv2d_group_kernel<KWT, SQUARE, 4>), grid, block, 0, st, in, ker, out, N, C, H, W, CO, KH, KW, HO, WO, stride, padding);
+    else if (cog == 2) hipLaunchKernelGGL((conv2d_group_kernel<KWT, SQUARE, 2>), grid, block, 0, st, in, ker, out, N, C, H, W, CO, KH, KW, HO, WO, stride, padding);
+    else hipLaunchKernelGGL((conv2d_group_kernel<KWT, SQUARE, 1>), grid, block, 0, st, in, ker, out, N, C, H, W, CO, KH, KW, HO, WO, stride, padding);
+}
+
 hipError_t launch_conv2d(const float *in, const float *ker, float *out, int N, int C, int H, int W, int CO, int KH, int KW,
                          int HO, int WO, int stride, int padding, hipStream_t st) {
+    const long long P = (long long)N * HO * WO, blocks = (P + TOPS_BLOCK - 1) / TOPS_BLOCK;
+    // four output channels per thread share every input load; fewer where that would leave fewer than eight waves to a CU
+    // (2048 on the device) to hide the loads behind
+    const long long waves1 = blocks * (TOPS_BLOCK / 64) * CO;
+    const int cog = waves1 >= 4 * 2048 ? 4 : waves1 >= 2 * 2048 ? 2 : 1;
+    if (blocks <= 0x7FFFFFFFll && (CO + cog - 1) / cog <= 65535) {
+        const dim3 block(TOPS_BLOCK);
+        if (KW == 3 && KH == 3) launch_conv2d_group<3, true>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else if (KW == 5 && KH == 5) launch_conv2d_group<5, true>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else if (KW == 1) launch_conv2d_group<1, false>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else if (KW == 3) launch_conv2d_group<3, false>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else if (KW == 5) launch_conv2d_group<5, false>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else if (KW == 7) launch_conv2d_group<7, false>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        else launch_conv2d_group<0, false>(cog, block, blocks, CO, st, in, ker, out, N, C, H, W, KH, KW, HO, WO, stride, padding);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(conv2d_kernel, dim3(tensor_grid((long long)N * CO * HO * WO)), dim3(TOPS_BLOCK), 0, st, in, ker, out, N, C, H,
                        W, CO, KH, KW, HO, WO, stride, padding);
     return hipGetLastError();
