@@ -669,7 +669,14 @@ hipError_t launch_lm_threshold(const float *samp, long long ld, int B, int nsamp
 }
 
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
-    const int bm = g.bm ? g.bm : g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
+    int bm = g.bm ? g.bm : g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
+    // A product of few tiles leaves most of the device idle (1024 x 1024 x 1024 is 64 tiles of 128 x 128 for 256 CUs):
+    // shorter tiles until about two thirds of the CUs have one.  (Whatever the epilogue: the LM head fused with the greedy
+    // or sampling step must add its products in the order of the plain head, which the tile height decides.)
+    if (!g.bm) {
+        const long long nt = (g.N + GN - 1) / GN;
+        while (bm > 16 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
+    }
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
