@@ -23,9 +23,12 @@ The other configurations of BASELINE.json run through the same script for their 
 headline): --config C1 | C2 (multinomial) | C2g (greedy argmax) | C4 (speculative verify, 64 x 5 positions;
 "tokens" are verified draft positions) | C5; and three sets of secondary timings at the C3 shape:
 --config C3x (the step with min-p, with the frequency / presence penalties, with per-row arrays) | LP (token
-log-probabilities) | GEN (the generation loop: embedding lookup, LM head, sampling, history append).
+log-probabilities) | GEN (the generation loop: embedding lookup, LM head, sampling, history append); and
+--config OPS: the reference's operators on the path (softmax, log-softmax, argmax, token log-probabilities, conv2d,
+matmul) at shapes from a classifier's ten classes to an LLM's vocabulary, each beside the vendor library's time
+through torch.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C2g|C4|C5|C3x|LP|GEN] [--no-cpu] [--no-producer]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C3|C1|C2|C2g|C4|C5|C3x|LP|GEN|OPS] [--no-cpu] [--no-producer]
 """
 import argparse
 import json
@@ -271,6 +274,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.config == "OPS":
+        return main_ops(args, torch, S, dev)
     if args.config in ("C3x", "LP", "GEN"):
         return main_extras(args, torch, S, synth, dev)
     gen = {"C1": synth.c1, "C2": synth.c2, "C2g": synth.c2, "C3": synth.c3, "C4": synth.c4, "C5": synth.c5}[args.config]
@@ -420,6 +425,77 @@ def main():
     if not args.no_cpu:
         out["parity"] = parity_block(w, tok_host, probs.cpu().numpy())
         out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+def main_ops(args, torch, S, dev):
+    """The operators at several shapes, us per call through the C ABI with every buffer allocated beforehand (best of three
+    regions of --steps calls), and the same operation through torch (the vendor libraries) beside it.  One JSON line."""
+    import ctypes as C
+    from born_amd import _capi
+    lib = _capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    steps = max(5, min(args.steps, 50))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+
+    def best(fn):
+        res = []
+        for _ in range(3):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            res.append(e0.elapsed_time(e1) / steps * 1e3)
+        return min(res)
+
+    def ptr(t):
+        return C.c_void_p(t.data_ptr())
+
+    out = {"metric": "operators of the path, us per call (not the headline)", "config": {"workload": "OPS"}, "n_gpus": 1, "steps": steps,
+           "data": "synthetic", "dtype": "f32", "us": {}}
+    smp = S.NewSampler(S.SamplerConfig(), max_batch=65536, max_vocab=152064)
+    for rows, V in ((65536, 10), (8192, 1024), (4096, 4096), (1024, 32000), (256, 128256)):
+        x = torch.randn(rows, V, device=dev, generator=gen) * 1.5
+        y = torch.empty(rows, V, device=dev)
+        tok = torch.randint(0, V, (rows,), device=dev, dtype=torch.int32)
+        tok64 = tok.long()
+        o32 = torch.empty(rows, dtype=torch.int32, device=dev)
+        lp = torch.empty(rows, device=dev)
+        shape = f"{rows} x {V}"
+        out["us"][f"softmax {shape}"] = {"born": best(lambda: smp.Softmax(x, rows, V, y, stream=stream)),
+                                         "torch": best(lambda: torch.softmax(x, dim=1, out=y))}
+        out["us"][f"log_softmax {shape}"] = {"born": best(lambda: smp.Softmax(x, rows, V, y, stream=stream, log=True)),
+                                             "torch": best(lambda: torch.log_softmax(x, dim=1, out=y))}
+        out["us"][f"argmax {shape}"] = {"born": best(lambda: smp.Argmax(x, rows, V, o32, stream=stream)),
+                                        "torch": best(lambda: torch.argmax(x, dim=1))}
+        out["us"][f"token log-probabilities {shape}"] = {
+            "born": best(lambda: smp.TokenLogprobs(x, rows, V, None, None, tok, lp, stream=stream)),
+            "torch": best(lambda: torch.nn.functional.cross_entropy(x, tok64, reduction="none"))}
+        del x, y
+    smp.Close()
+    for (m, k, n) in ((64, 784, 128), (64, 128, 10), (256, 784, 512), (1024, 1024, 1024), (512, 4096, 512), (4096, 4096, 4096)):
+        a, b, c = torch.randn(m, k, device=dev, generator=gen), torch.randn(k, n, device=dev, generator=gen), torch.empty(m, n, device=dev)
+
+        def mm():
+            _capi.check(lib.born_rocm_matmul(ptr(a), ptr(b), ptr(c), m, k, n, k, n, n, None))
+        out["us"][f"matmul [{m},{k}] @ [{k},{n}]"] = {"born": best(mm), "torch": best(lambda: torch.matmul(a, b, out=c))}
+    for (xs, ks, stride, pad) in (((64, 1, 28, 28), (32, 1, 5, 5), 1, 0), ((64, 32, 12, 12), (64, 32, 5, 5), 1, 0),
+                                  ((256, 64, 56, 56), (64, 64, 3, 3), 1, 1)):
+        x, w = torch.randn(*xs, device=dev, generator=gen), torch.randn(*ks, device=dev, generator=gen)
+        ho, wo = (xs[2] + 2 * pad - ks[2]) // stride + 1, (xs[3] + 2 * pad - ks[3]) // stride + 1
+        y = torch.empty(xs[0], ks[0], ho, wo, device=dev)
+        xsa, ksa, osh = (C.c_int64 * 4)(*xs), (C.c_int64 * 4)(*ks), (C.c_int64 * 4)()
+
+        def conv():
+            _capi.check(lib.born_rocm_conv2d(ptr(x), xsa, ptr(w), ksa, stride, pad, ptr(y), osh, None))
+        out["us"][f"conv2d {list(xs)} * {list(ks)} stride {stride} padding {pad}"] = {
+            "born": best(conv), "torch": best(lambda: torch.nn.functional.conv2d(x, w, stride=stride, padding=pad))}
     print(json.dumps(out))
 
 
