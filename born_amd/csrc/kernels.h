@@ -117,6 +117,10 @@ struct GemmArgs {
     uint2 *cand;                  // [M][cand_cap]
     int cand_cap;
     int bm;                       // 0: tile height chosen from M; else 16, 32, 64 or 128 (a narrow product wants more, lower tiles)
+    // set by the launcher for a product of few tiles and a long K (plain [K,N] products only): blockIdx.y = slice of K,
+    // kslice values of k each (a multiple of 32); slice z writes its partial product, without bias, to ws + z * M * N
+    int ksplit, kslice;
+    float *ws;
 };
 constexpr int LM_BEST_PITCH = 16;
 constexpr int LM_CAND_PITCH = 32;          // u32 words between the candidate counters of consecutive rows (a 128-byte line each)

@@ -20,6 +20,9 @@
 // Workgroup ids are dealt round-robin to the 8 XCDs; the tile order makes the workgroups that share a tile
 // column of B (all M-tiles of that column) land on the same XCD back to back, so that B is fetched from HBM
 // once and re-read from that XCD's L2.
+#include <algorithm>
+#include <mutex>
+#include <vector>
 #include "dev_common.h"
 #include "kernels.h"
 
@@ -261,6 +264,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_f32_kernel(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) float As[2][AROWS * GPITCH];
     __shared__ __attribute__((aligned(16))) float Bs[2][B_WORDS];
 
+    if (g.ksplit > 1) {                                              // this workgroup's slice of K, as a product of its own
+        const int k0z = (int)blockIdx.y * g.kslice;
+        g.a += k0z;
+        g.b += BT ? (long long)k0z : (long long)k0z * g.ldb;
+        g.K = min(g.kslice, g.K - k0z);
+        g.c = g.ws + (long long)blockIdx.y * g.M * g.N;
+        g.ldc = g.N;
+        g.bias = nullptr;
+    }
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
     const int wave = tid >> 6;
@@ -556,14 +568,72 @@ template <bool BT, bool FAST, int EPI>
 static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
     const long long nt = (g.N + GN - 1) / GN;
     const dim3 bl(GEMM_THREADS);
+    const unsigned ky = g.ksplit > 1 ? (unsigned)g.ksplit : 1u;
     if (bm == 16)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 16, EPI>), dim3((unsigned)(nt * ((g.M + 15) / 16))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 16, EPI>), dim3((unsigned)(nt * ((g.M + 15) / 16)), ky), bl, 0, st, g);
     else if (bm == 32)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32, EPI>), dim3((unsigned)(nt * ((g.M + 31) / 32))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 32, EPI>), dim3((unsigned)(nt * ((g.M + 31) / 32)), ky), bl, 0, st, g);
     else if (bm == 64)
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64, EPI>), dim3((unsigned)(nt * ((g.M + 63) / 64))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 64, EPI>), dim3((unsigned)(nt * ((g.M + 63) / 64)), ky), bl, 0, st, g);
     else
-        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 128, EPI>), dim3((unsigned)(nt * ((g.M + 127) / 128))), bl, 0, st, g);
+        hipLaunchKernelGGL((gemm_f32_kernel<BT, FAST, 128, EPI>), dim3((unsigned)(nt * ((g.M + 127) / 128)), ky), bl, 0, st, g);
+}
+
+// The sum of the partial products of a split K, slice by slice in ascending order (so the result does not depend on
+// which workgroup finished first), plus the bias.
+__global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float *__restrict__ ws, int slices, long long mn, int N,
+                                                              float *__restrict__ c, long long ldc, const float *__restrict__ bias) {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < mn; i += (long long)gridDim.x * 256) {
+        float sum = ws[i];
+        for (int z = 1; z < slices; z++) sum += ws[(long long)z * mn + i];
+        const long long row = i / N;
+        const int col = (int)(i - row * N);
+        c[row * ldc + col] = bias ? sum + bias[col] : sum;
+    }
+}
+
+// Workspace for the partial products: one buffer per (device, stream) that ever needed one, kept until the process
+// ends (calls on one stream are ordered, so they can share; calls on different streams cannot).  Null when none can be
+// had now (the stream is being captured, too many streams, out of memory): the product is then computed unsplit.
+constexpr size_t GEMM_WS_MAX = (size_t)64 << 20, GEMM_WS_MIN = (size_t)8 << 20;
+static float *gemm_workspace(hipStream_t st, size_t bytes) {
+    struct Entry {
+        int dev;
+        hipStream_t st;
+        float *p;
+        size_t bytes;
+    };
+    static std::mutex mu;
+    static std::vector<Entry> cache;
+    int dev = 0;
+    if (bytes > GEMM_WS_MAX || hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    Entry *found = nullptr;
+    for (Entry &e : cache)
+        if (e.dev == dev && e.st == st) found = &e;
+    if (found && found->bytes >= bytes) return found->p;
+    if (!found && cache.size() >= 16) return nullptr;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return nullptr;
+    if (found) {                                                     // a larger one: the old buffer may still be in use on the stream
+        if (hipStreamSynchronize(st) != hipSuccess) return nullptr;
+        (void)hipFree(found->p);
+        found->p = nullptr;
+        found->bytes = 0;
+    }
+    const size_t want = bytes < GEMM_WS_MIN ? GEMM_WS_MIN : GEMM_WS_MAX;
+    float *p = nullptr;
+    if (hipMalloc((void **)&p, want) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (found) {
+        found->p = p;
+        found->bytes = want;
+    } else {
+        cache.push_back(Entry{dev, st, p, want});
+    }
+    return p;
 }
 
 template <int EPI>
@@ -675,7 +745,13 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     // or sampling step must add its products in the order of the plain head, which the tile height decides.)
     if (!g.bm) {
         const long long nt = (g.N + GN - 1) / GN;
-        while (bm > 16 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
+        // (a [K,N] product with a long K keeps its tall tiles where slices of K alone can fill the device: below)
+        const long long tiles0 = nt * ((g.M + bm - 1) / bm);
+        // (measured: 1024^3, 64 tall tiles, is faster as 256 short tiles than as 64 x 4 slices; [512,4096] @ [4096,512],
+        // 16 tall tiles, is faster as 16 x 16 slices than as 128 short tiles)
+        const bool split_fills = !b_transposed && !g.cand && !g.best && tiles0 <= 32 && g.K >= 1024 &&
+                                 tiles0 * std::min<long long>(std::min<long long>(16, 256 / tiles0), g.K / 128) >= 128;
+        while (!split_fills && bm > 16 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
     }
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
@@ -690,10 +766,35 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     } else if (b_transposed) {
         launch_gemm_nt<0>(g, bm, grid, fast, st);
     } else {
+        // A product of few tiles and a long K: the slices of K go to workgroups of their own, each writes a partial
+        // product to the workspace, and one more launch adds them in order.  ([K,N] products only: the head of a
+        // linear layer must add its products in the order of the heads fused with the greedy and sampling steps.)
+        GemmArgs gs = g;
+        gs.ksplit = 0;
+        const long long tiles = grid;
+        if (tiles < 128 && g.K >= 256 && (long long)g.M * g.N <= (long long)(GEMM_WS_MAX / sizeof(float) / 2)) {
+            int slices = (int)std::min<long long>(std::min<long long>(16, 256 / tiles), g.K / 128);
+            if (slices >= 2) {
+                const int kslice = (((g.K + slices - 1) / slices + GK - 1) / GK) * GK;
+                slices = (g.K + kslice - 1) / kslice;
+                const size_t bytes = (size_t)slices * (size_t)g.M * (size_t)g.N * sizeof(float);
+                float *ws = slices >= 2 ? gemm_workspace(st, bytes) : nullptr;
+                if (ws) {
+                    gs.ksplit = slices;
+                    gs.kslice = kslice;
+                    gs.ws = ws;
+                }
+            }
+        }
         if (fast)
-            launch_gemm_bm<false, true, 0>(g, bm, st);
+            launch_gemm_bm<false, true, 0>(gs, bm, st);
         else
-            launch_gemm_bm<false, false, 0>(g, bm, st);
+            launch_gemm_bm<false, false, 0>(gs, bm, st);
+        if (gs.ksplit > 1) {
+            const long long mn = (long long)g.M * g.N;
+            hipLaunchKernelGGL(gemm_splitk_sum_kernel, dim3((unsigned)std::min<long long>((mn + 255) / 256, 4096)), dim3(256), 0, st, gs.ws,
+                               gs.ksplit, mn, g.N, g.c, g.ldc, g.bias);
+        }
     }
     return hipGetLastError();
 }

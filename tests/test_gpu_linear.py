@@ -70,7 +70,9 @@ def test_reference_kats(rocm, lin):
 SHAPES = [(1, 1, 1), (1, 3, 2), (2, 2, 2), (3, 5, 7), (7, 16, 5), (33, 17, 65), (64, 64, 64), (127, 100, 129),
           (128, 128, 128), (129, 15, 127), (130, 257, 300), (256, 512, 1000), (5, 1000, 1), (300, 33, 31),
           # every tile height (16, 32, 64, 128 rows) on the unguarded-load route (K a multiple of 32)
-          (1, 64, 300), (16, 128, 260), (17, 96, 132), (32, 256, 100), (48, 64, 256), (65, 32, 128), (12, 4096, 520)]
+          (1, 64, 300), (16, 128, 260), (17, 96, 132), (32, 256, 100), (48, 64, 256), (65, 32, 128), (12, 4096, 520),
+          # few tiles and a long K: the [K,N] product splits K over workgroups (ragged last slice, unaligned K, one row)
+          (64, 784, 128), (64, 790, 10), (512, 4096, 512), (100, 1000, 260), (1, 5000, 7), (33, 257, 129), (200, 2048, 300)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
