@@ -33,7 +33,7 @@ def test_random_linear_and_matmul_shapes(oracle, rocm, lin, chunk):
     rng = np.random.default_rng(555 + chunk)
     for i in range(8):
         M = int(rng.choice([1, 2, 15, 16, 17, 31, 33, 64, 65, 100, 128, 129, 200]))
-        K = int(rng.choice([1, 3, 8, 31, 32, 33, 64, 96, 100, 256, 260]))
+        K = int(rng.choice([1, 3, 8, 31, 32, 33, 64, 96, 100, 256, 260, 777, 1024, 2050]))    # (from 256 on a [K,N] product of few tiles splits K)
         N = int(rng.choice([1, 2, 4, 7, 127, 128, 129, 130, 255, 300, 512, 1001]))
         x = rng.standard_normal((M, K)).astype(np.float32)
         w = rng.standard_normal((N, K)).astype(np.float32)
