@@ -580,15 +580,21 @@ static void launch_gemm_bm(const GemmArgs &g, int bm, hipStream_t st) {
 }
 
 // The sum of the partial products of a split K, slice by slice in ascending order (so the result does not depend on
-// which workgroup finished first), plus the bias.
-__global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float *__restrict__ ws, int slices, long long mn, int N,
-                                                              float *__restrict__ c, long long ldc, const float *__restrict__ bias) {
+// which workgroup finished first), plus the bias; then what the product's own epilogue would have done with the
+// result (EPI as in the tiles' epilogues: stored, offered as its row's largest, or listed as a candidate), so that the
+// fused forms of a head see the very numbers its plain form stores.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(GemmArgs g, long long mn) {
+    const float *__restrict__ ws = g.ws;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < mn; i += (long long)gridDim.x * 256) {
         float sum = ws[i];
-        for (int z = 1; z < slices; z++) sum += ws[(long long)z * mn + i];
-        const long long row = i / N;
-        const int col = (int)(i - row * N);
-        c[row * ldc + col] = bias ? sum + bias[col] : sum;
+        for (int z = 1; z < g.ksplit; z++) sum += ws[(long long)z * mn + i];
+        const int row = (int)(i / g.N);
+        const int col = (int)(i - (long long)row * g.N);
+        const float val = g.bias ? sum + g.bias[col] : sum;
+        if (EPI == 0) g.c[(long long)row * g.ldc + col] = val;
+        else if (EPI == 1) gemm_offer_key(g.best, row, gemm_argmax_key(val, col));
+        else gemm_offer_candidate(g, row, col, val, g.thr[row]);
     }
 }
 
@@ -745,56 +751,62 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     // or sampling step must add its products in the order of the plain head, which the tile height decides.)
     if (!g.bm) {
         const long long nt = (g.N + GN - 1) / GN;
-        // (a [K,N] product with a long K keeps its tall tiles where slices of K alone can fill the device: below)
+        // (a product with a long K keeps its tall tiles where slices of K alone can fill the device: below)
         const long long tiles0 = nt * ((g.M + bm - 1) / bm);
         // (measured: 1024^3, 64 tall tiles, is faster as 256 short tiles than as 64 x 4 slices; [512,4096] @ [4096,512],
         // 16 tall tiles, is faster as 16 x 16 slices than as 128 short tiles)
-        const bool split_fills = !b_transposed && !g.cand && !g.best && tiles0 <= 32 && g.K >= 1024 &&
+        const bool split_fills = tiles0 <= 32 && g.K >= 1024 &&
                                  tiles0 * std::min<long long>(std::min<long long>(16, 256 / tiles0), g.K / 128) >= 128;
         while (!split_fills && bm > 16 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
     }
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
     const bool fast = g.vec_a && g.vec_b && g.K % GK == 0 && (b_transposed || (g.N % 4 == 0));
-    if (g.cand) {                                                    // candidate epilogue: W[N,K] form only
-        if (!b_transposed || !g.thr || !g.cand_cnt || g.cand_cap <= 0) return hipErrorInvalidValue;
+    if (g.cand && (!b_transposed || !g.thr || !g.cand_cnt || g.cand_cap <= 0)) return hipErrorInvalidValue;   // candidate epilogue: W[N,K] form only
+    if (g.best && (!b_transposed || !g.tokens)) return hipErrorInvalidValue;                                    // argmax epilogue: W[N,K] form only
+    // A product of few tiles and a long K: the slices of K go to workgroups of their own, each writes a partial
+    // product to the workspace, and one more launch adds them in order and does what the product's epilogue does.
+    GemmArgs gs = g;
+    gs.ksplit = 0;
+    if (grid < 128 && g.K >= 256 && (long long)g.M * g.N <= (long long)(GEMM_WS_MAX / sizeof(float) / 2)) {
+        int slices = (int)std::min<long long>(std::min<long long>(16, 256 / grid), g.K / 128);
+        if (slices >= 2) {
+            const int kslice = (((g.K + slices - 1) / slices + GK - 1) / GK) * GK;
+            slices = (g.K + kslice - 1) / kslice;
+            float *ws = slices >= 2 ? gemm_workspace(st, (size_t)slices * (size_t)g.M * (size_t)g.N * sizeof(float)) : nullptr;
+            if (ws) {
+                gs.ksplit = slices;
+                gs.kslice = kslice;
+                gs.ws = ws;
+            }
+        }
+    }
+    if (gs.ksplit > 1) {
+        if (b_transposed) {
+            if (fast) launch_gemm_bm<true, true, 0>(gs, bm, st); else launch_gemm_bm<true, false, 0>(gs, bm, st);
+        } else {
+            if (fast) launch_gemm_bm<false, true, 0>(gs, bm, st); else launch_gemm_bm<false, false, 0>(gs, bm, st);
+        }
+        const long long mn = (long long)g.M * g.N;
+        const dim3 sg((unsigned)std::min<long long>((mn + 255) / 256, 4096)), sb(256);
+        if (g.cand) hipLaunchKernelGGL(gemm_splitk_sum_kernel<2>, sg, sb, 0, st, gs, mn);
+        else if (g.best) hipLaunchKernelGGL(gemm_splitk_sum_kernel<1>, sg, sb, 0, st, gs, mn);
+        else hipLaunchKernelGGL(gemm_splitk_sum_kernel<0>, sg, sb, 0, st, gs, mn);
+        if (g.best) hipLaunchKernelGGL(argmax_keys_token_kernel, dim3((unsigned)((g.M + 255) / 256)), dim3(256), 0, st, g.best, g.tokens, g.M);
+        return hipGetLastError();
+    }
+    if (g.cand) {
         launch_gemm_nt<2>(g, bm, grid, fast, st);
-    } else if (g.best) {                                             // argmax epilogue: W[N,K] form only
-        if (!b_transposed || !g.tokens) return hipErrorInvalidValue;
+    } else if (g.best) {
         launch_gemm_nt<1>(g, bm, grid, fast, st);
         hipLaunchKernelGGL(argmax_keys_token_kernel, dim3((unsigned)((g.M + 255) / 256)), dim3(256), 0, st, g.best, g.tokens, g.M);
     } else if (b_transposed) {
         launch_gemm_nt<0>(g, bm, grid, fast, st);
     } else {
-        // A product of few tiles and a long K: the slices of K go to workgroups of their own, each writes a partial
-        // product to the workspace, and one more launch adds them in order.  ([K,N] products only: the head of a
-        // linear layer must add its products in the order of the heads fused with the greedy and sampling steps.)
-        GemmArgs gs = g;
-        gs.ksplit = 0;
-        const long long tiles = grid;
-        if (tiles < 128 && g.K >= 256 && (long long)g.M * g.N <= (long long)(GEMM_WS_MAX / sizeof(float) / 2)) {
-            int slices = (int)std::min<long long>(std::min<long long>(16, 256 / tiles), g.K / 128);
-            if (slices >= 2) {
-                const int kslice = (((g.K + slices - 1) / slices + GK - 1) / GK) * GK;
-                slices = (g.K + kslice - 1) / kslice;
-                const size_t bytes = (size_t)slices * (size_t)g.M * (size_t)g.N * sizeof(float);
-                float *ws = slices >= 2 ? gemm_workspace(st, bytes) : nullptr;
-                if (ws) {
-                    gs.ksplit = slices;
-                    gs.kslice = kslice;
-                    gs.ws = ws;
-                }
-            }
-        }
         if (fast)
-            launch_gemm_bm<false, true, 0>(gs, bm, st);
+            launch_gemm_bm<false, true, 0>(g, bm, st);
         else
-            launch_gemm_bm<false, false, 0>(gs, bm, st);
-        if (gs.ksplit > 1) {
-            const long long mn = (long long)g.M * g.N;
-            hipLaunchKernelGGL(gemm_splitk_sum_kernel, dim3((unsigned)std::min<long long>((mn + 255) / 256, 4096)), dim3(256), 0, st, gs.ws,
-                               gs.ksplit, mn, g.N, g.c, g.ldc, g.bias);
-        }
+            launch_gemm_bm<false, false, 0>(g, bm, st);
     }
     return hipGetLastError();
 }

@@ -259,7 +259,7 @@ int born_rocm_spec_verify_bonus(born_sampler *s, const float *target, int64_t ta
 int born_rocm_linear(const float *x, int64_t batch, int64_t in_features, int64_t x_stride, const float *weight,
                      int64_t out_features, int64_t w_stride, const float *bias, float *out, int64_t out_stride,
                      void *stream);
-/* (born_rocm_matmul: a product of few output tiles and a long k is computed in slices of k that are added in a fixed order;
+/* (born_rocm_matmul, born_rocm_linear and the fused heads below: a product of few output tiles and a long k is computed in slices of k that are added in a fixed order;
  * the first such call on a stream allocates the library's workspace for that stream, 8 or 64 MiB kept until the process
  * ends - outside a stream capture; a call under capture that finds no workspace computes the product unsplit.) */
 int born_rocm_matmul(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int64_t lda,
