@@ -747,17 +747,16 @@ hipError_t launch_lm_threshold(const float *samp, long long ld, int B, int nsamp
 hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st) {
     int bm = g.bm ? g.bm : g.M <= 16 ? 16 : g.M <= 32 ? 32 : g.M <= 64 ? 64 : 128;
     // A product of few tiles leaves most of the device idle (1024 x 1024 x 1024 is 64 tiles of 128 x 128 for 256 CUs):
-    // shorter tiles until about two thirds of the CUs have one.  (Whatever the epilogue: the LM head fused with the greedy
-    // or sampling step must add its products in the order of the plain head, which the tile height decides.)
+    // shorter tiles, down to 32 rows, until about two thirds of the CUs have one; 16 rows only for a product that is
+    // still a handful of tiles then.  What is missing after that comes from slices of K (below).  Measured over tile
+    // heights and slice counts on seven shapes: [512,4096] @ [4096,512] 32.3 us as 64 tiles of 32 rows x 8 slices, 39.3
+    // as 16 tiles of 128 rows x 16 slices, 64.9 as 128 tiles of 16 rows unsplit; 1024^3 27.9 as 256 tiles of 32 rows, 38.4
+    // as 64 tall tiles x 4 slices.  (Whatever the epilogue: the LM head fused with the greedy or sampling step must add
+    // its products in the order of the plain head, which the tile height and the slices decide.)
     if (!g.bm) {
         const long long nt = (g.N + GN - 1) / GN;
-        // (a product with a long K keeps its tall tiles where slices of K alone can fill the device: below)
-        const long long tiles0 = nt * ((g.M + bm - 1) / bm);
-        // (measured: 1024^3, 64 tall tiles, is faster as 256 short tiles than as 64 x 4 slices; [512,4096] @ [4096,512],
-        // 16 tall tiles, is faster as 16 x 16 slices than as 128 short tiles)
-        const bool split_fills = tiles0 <= 32 && g.K >= 1024 &&
-                                 tiles0 * std::min<long long>(std::min<long long>(16, 256 / tiles0), g.K / 128) >= 128;
-        while (!split_fills && bm > 16 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
+        while (bm > 32 && nt * ((g.M + bm - 1) / bm) < 160) bm >>= 1;
+        if (bm == 32 && nt * ((g.M + 31) / 32) < 16) bm = 16;
     }
     const long long grid = (long long)((g.M + bm - 1) / bm) * ((g.N + GN - 1) / GN);
     if (grid <= 0 || grid > 0x7FFFFFFFll) return hipErrorInvalidValue;
@@ -769,7 +768,7 @@ hipError_t launch_gemm_f32(const GemmArgs &g, bool b_transposed, hipStream_t st)
     GemmArgs gs = g;
     gs.ksplit = 0;
     if (grid < 128 && g.K >= 256 && (long long)g.M * g.N <= (long long)(GEMM_WS_MAX / sizeof(float) / 2)) {
-        int slices = (int)std::min<long long>(std::min<long long>(16, 256 / grid), g.K / 128);
+        int slices = (int)std::min<long long>(std::min<long long>(16, 512 / grid), g.K / 128);   // (two workgroups to a CU)
         if (slices >= 2) {
             const int kslice = (((g.K + slices - 1) / slices + GK - 1) / GK) * GK;
             slices = (g.K + kslice - 1) / kslice;
