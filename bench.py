@@ -52,13 +52,13 @@ MFMA_FP32_PEAK_TFLOPS = 157.3
 # file under profiles/ that holds the counters; a run whose dominant kernel is not listed prints null.
 PMC_TRAFFIC = {
     ("C3", "topk_row_kernel"): {
-        "bytes": int(64681.0 * (128256 / 64139.6) * 1024 + 24.0 * 1024),
+        "bytes": int(64680.2 * (128256 / 64139.6) * 1024 + 24.0 * 1024),
         "measured_on": "born::topk_row_kernel<true, false, 0>, workload C3",
         "source": "profiles/topk_row_kernel_c3_hbm_traffic.txt",
     },
     # (the probe of that run copied a C5 logits buffer: 608 256 KiB read and written)
     ("C5", "nucleus_row_kernel"): {
-        "bytes": int(1014065.9 * (608256 / 304141.8) * 1024 + 102.5 * 1024),
+        "bytes": int(1013983.9 * (608256 / 304141.8) * 1024 + 102.9 * 1024),
         "measured_on": "born::nucleus_row_kernel<512, false, true>, workload C5 (what the L2s fetch, the Infinity Cache's share included)",
         "source": "profiles/nucleus_row_kernel_c5_counters.txt",
     },
