@@ -792,9 +792,9 @@ int born_rocm_linear_argmax(born_sampler *s, const float *x, int64_t batch, int6
                       out_features, true, stream, s->lm_best, tokens_out);
 }
 
-// LM head and sampling step in one call: x[batch, in] @ weight[out, in]^T + bias is never written.  Four launches:
-// the same product over a strided sample of at most 1024 weight rows (a small GEMM into the handle's workspace), the
-// per-row thresholds from it, the full product whose epilogue lists the logits at or above each row's threshold, and
+// LM head and sampling step in one call: x[batch, in] @ weight[out, in]^T + bias is never written.  Four steps:
+// the same product over a strided sample of at most 1024 weight rows (a small GEMM into the handle's workspace: few
+// tiles, so its K is split over workgroups and summed by a launch of its own), the per-row thresholds from it, the full product whose epilogue lists the logits at or above each row's threshold, and
 // the sampling step over the lists.
 int born_rocm_linear_sample(born_sampler *s, const float *x, int64_t batch, int64_t in_features, int64_t x_stride,
                             const float *weight, int64_t out_features, int64_t w_stride, const float *bias,
