@@ -485,6 +485,14 @@ def main_ops(args, torch, S, dev):
         def mm():
             _capi.check(lib.born_rocm_matmul(ptr(a), ptr(b), ptr(c), m, k, n, k, n, n, None))
         out["us"][f"matmul [{m},{k}] @ [{k},{n}]"] = {"born": best(mm), "torch": best(lambda: torch.matmul(a, b, out=c))}
+    for (m, k, n) in ((64, 784, 128), (64, 4096, 4096), (512, 4096, 512), (32, 4096, 128256)):
+        x, w, b = torch.randn(m, k, device=dev, generator=gen), torch.randn(n, k, device=dev, generator=gen), torch.randn(n, device=dev, generator=gen)
+        y = torch.empty(m, n, device=dev)
+
+        def lin():
+            _capi.check(lib.born_rocm_linear(ptr(x), m, k, k, ptr(w), n, k, ptr(b), ptr(y), n, None))
+        out["us"][f"linear [{m},{k}] -> {n}"] = {"born": best(lin), "torch": best(lambda: torch.nn.functional.linear(x, w, b))}
+        del x, w, y
     for (xs, ks, stride, pad) in (((64, 1, 28, 28), (32, 1, 5, 5), 1, 0), ((64, 32, 12, 12), (64, 32, 5, 5), 1, 0),
                                   ((256, 64, 56, 56), (64, 64, 3, 3), 1, 1)):
         x, w = torch.randn(*xs, device=dev, generator=gen), torch.randn(*ks, device=dev, generator=gen)
